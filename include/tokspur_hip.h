@@ -1,0 +1,170 @@
+/*
+ * tokspur_hip — C ABI of the MI355X (gfx950) quantized-matmul / MoE kernels.
+ *
+ * This is the layer a tokspur maintainer binds underneath the native engine's graph executor:
+ * every device entry point below replaces one `tokspur::MetalGraph` operator encoder (cited per
+ * function, paths relative to the reference tree's native/ directory) and every host entry point
+ * replaces one pure planner / layout routine. The reference has no C ABI of its own; its boundary
+ * is the C++ class in include/tokspur/graph.hpp:431-1168, which the host class in
+ * tokspur-public_amd/host/hip_graph.hpp mirrors on top of these functions.
+ *
+ * Conventions
+ *  - Plain pointers and sizes only. Device pointers are HIP device addresses; `stream` is a
+ *    hipStream_t passed as void* (NULL = the default stream). Calls enqueue and return; nothing
+ *    here synchronises or allocates device memory unless its comment says so.
+ *  - Return value: TSP_OK, or a refusal made on the host BEFORE anything was enqueued
+ *    (TSP_ERR_FORMAT = what the reference reports as tokspur::FormatError; TSP_ERR_HIP = a HIP
+ *    runtime error). tsp_last_error() returns the message for the calling thread.
+ *  - `error_word` is the device-side sticky error word of the reference's kernels (buffer index 7,
+ *    e.g. kernels/gemv.metal:114,213): kernels OR in TSP_ERRBIT_NONFINITE (1) when an output is
+ *    not finite and TSP_ERRBIT_INDEX (4) on a bad expert id or grouping geometry. The caller zeroes
+ *    it, reads it once per batch and refuses the batch when it is non-zero (src/graph.mm:3977-3978).
+ *  - Outputs must not overlap inputs; padding beyond `columns` of a strided row is never written.
+ */
+#ifndef TOKSPUR_HIP_H
+#define TOKSPUR_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TSP_OK 0
+#define TSP_ERR_FORMAT 1
+#define TSP_ERR_HIP 2
+
+#define TSP_ERRBIT_NONFINITE 1u
+#define TSP_ERRBIT_INDEX 4u
+
+/* GGUF tensor encodings the path decodes (src/gguf.cpp:21-32, src/numeric.cpp:93-95). */
+#define TSP_F32 0u
+#define TSP_F16 1u
+#define TSP_Q5_1 7u
+#define TSP_Q8_0 8u
+#define TSP_Q4_K 12u
+#define TSP_Q5_K 13u
+#define TSP_Q6_K 14u
+#define TSP_IQ4_NL 20u
+#define TSP_BF16 30u
+
+/* Row layouts of a dense matrix (include/tokspur/grouped_mm.hpp:6; planar = one Pack v3 expert). */
+#define TSP_LAYOUT_GGUF 0u
+#define TSP_LAYOUT_Q8_LANES_V1 1u
+#define TSP_LAYOUT_PLANAR_V3 3u
+
+/* Pack v3 planar kinds (include/tokspur/planar_pack_v3.hpp:29-40). Kind 10 is this library's
+ * extension: Q6_K experts in planes [ql 128][qh 64][sc 16][d 2] per block, for down projections. */
+#define TSP_KIND_PLAIN 0u
+#define TSP_KIND_Q8_LANES_V1 1u
+#define TSP_KIND_Q4K_COLOC_GATE 2u
+#define TSP_KIND_Q4K_COLOC_UP 3u
+#define TSP_KIND_Q5K_COLOC_GATE 4u
+#define TSP_KIND_Q5K_COLOC_UP 5u
+#define TSP_KIND_Q8_COLOC_GATE 6u
+#define TSP_KIND_Q8_COLOC_UP 7u
+#define TSP_KIND_Q51_PLANAR 8u
+#define TSP_KIND_Q8_PLANAR 9u
+#define TSP_KIND_Q6K_PLANAR_X 10u
+
+const char* tsp_last_error(void);
+/* ABI revision of this header; bumped on any incompatible change. */
+uint32_t tsp_abi_version(void);
+
+/* ------------------------------------------------------------------ host: formats and layouts */
+
+/* src/gguf.cpp:21-32, 157-160 `encoding()`: block geometry of a GGUF type. */
+int tsp_encoding(uint32_t type, uint32_t* elements_per_block, uint32_t* bytes_per_block);
+/* src/numeric.cpp:93-95 `can_decode()`. */
+int tsp_can_decode(uint32_t type);
+
+/* include/tokspur/planar_pack_v3.hpp:48-61 `PlanarExpertSpec` (field for field). */
+typedef struct tsp_planar_spec {
+    uint32_t source_type, columns, rows, blocks_per_row;
+    uint64_t source_row_bytes, planar_row_bytes, source_expert_bytes, planar_expert_bytes;
+    uint64_t qs_offset, qh_offset, sm_offset, dm_offset;
+} tsp_planar_spec;
+/* src/planar_pack_v3.cpp:601-650 `make_expert_spec` (+ type 14 for TSP_KIND_Q6K_PLANAR_X:
+ * qs = ql plane, qh = qh plane, sm = int8 sub-scale plane, dm = f16 d plane). */
+int tsp_make_expert_spec(uint32_t source_type, uint32_t columns, uint32_t rows, tsp_planar_spec* spec);
+/* src/planar_pack_v3.cpp:652-674 `pack_sm16` / `unpack_sm16`. */
+void tsp_pack_sm16(const uint8_t scales12[12], uint8_t sm16[16]);
+int tsp_unpack_sm16(const uint8_t sm16[16], uint8_t scales12[12]);
+/* src/planar_pack_v3.cpp:676-758 `pack_expert_planar_v3` / `unpack_expert_planar_v3` (host memory). */
+int tsp_pack_expert_planar_v3(const tsp_planar_spec* spec, const uint8_t* gguf_expert, uint64_t gguf_bytes,
+                              uint8_t* planar_expert, uint64_t planar_bytes);
+int tsp_unpack_expert_planar_v3(const tsp_planar_spec* spec, const uint8_t* planar_expert, uint64_t planar_bytes,
+                                uint8_t* gguf_expert, uint64_t gguf_bytes);
+/* src/planar_pack_v3.cpp:1061-1123 co-location: half 0 ("pair_lo", stored under the gate tensor's
+ * name) holds experts 0..E/2-1 as interleaved [gate_e, up_e]; half 1 ("pair_hi") holds the rest. */
+int tsp_pack_coloc_half(const tsp_planar_spec* spec, const uint8_t* gate_gguf, const uint8_t* up_gguf,
+                        uint32_t experts, uint32_t half, uint8_t* out, uint64_t out_bytes);
+/* src/expert_lanes.cpp:83-119 `packed_quant_offset` / `pack_rows` / `unpack_rows` for Q8_0. */
+int tsp_q8_lanes_quant_offset(uint32_t columns, uint32_t block, uint32_t index, uint64_t* offset);
+int tsp_q8_lanes_pack_rows(uint32_t columns, const uint8_t* original, uint8_t* packed, uint64_t bytes);
+int tsp_q8_lanes_unpack_rows(uint32_t columns, const uint8_t* packed, uint8_t* original, uint64_t bytes);
+
+/* ------------------------------------------------------------------ host: planners */
+
+/* include/tokspur/grouped_mm.hpp:8-21 `GroupedMmArgs` (56 bytes) and `GroupedMmPlan`. */
+typedef struct tsp_grouped_mm_args_t {
+    uint32_t columns, rows, row_bytes, experts, selected, tokens, broadcast, maximum_tasks;
+    uint64_t expert_stride_bytes, input_stride_bytes, output_stride_bytes;
+} tsp_grouped_mm_args_t;
+typedef struct tsp_grouped_mm_plan_t {
+    tsp_grouped_mm_args_t args;
+    uint64_t matrix_bytes, indices_bytes, input_bytes, output_bytes, token_map_bytes, counts_bytes, tasks_bytes;
+    uint32_t grid_x, grid_y;
+} tsp_grouped_mm_plan_t;
+/* src/grouped_mm.cpp:24-47 `grouped_mm_plan`; 48-54 `dense_mm_q8_plan`. */
+int tsp_grouped_mm_plan(uint32_t encoding, uint32_t layout, uint32_t columns, uint32_t rows, uint32_t experts,
+                        uint32_t selected, uint32_t tokens, uint64_t input_stride_bytes, uint64_t output_stride_bytes,
+                        int broadcast, int allow_nax_2k, tsp_grouped_mm_plan_t* plan);
+int tsp_dense_mm_q8_plan(uint32_t layout, uint32_t columns, uint32_t rows, uint32_t tokens, uint64_t input_stride_bytes,
+                         uint64_t output_stride_bytes, int allow_nax_2k, tsp_grouped_mm_plan_t* plan);
+/* src/moe_mm_many_plan.cpp:28-52 `moe_mm_many_bytes`: the 13 scratch views and their total. */
+int tsp_moe_mm_many_bytes(uint32_t channels, uint32_t hidden, uint32_t experts, uint32_t selected, uint32_t capacity,
+                          int allow_nax_2k, uint64_t views[13], uint64_t* total);
+/* src/q8_many.cpp:20-35 `q8_many_width` / `q8_many_chunks`. */
+int tsp_q8_many_width(uint32_t remaining, uint32_t* width);
+int tsp_q8_many_chunks(uint32_t rows, uint32_t* chunks);
+
+/* ------------------------------------------------------------------ device: dequantisation */
+
+/* src/numeric.cpp:97-148 `dequantize` on the device: raw GGUF blocks -> f32, bit-identical to the
+ * reference's double-then-one-cast value for every block whose double arithmetic is exact (all
+ * blocks with finite f16 fields of ordinary magnitude). Non-finite results set TSP_ERRBIT_NONFINITE. */
+int tsp_dequantize(uint32_t type, const void* blocks, uint64_t nbytes, float* out, uint64_t nelem,
+                   uint32_t* error_word, void* stream);
+/* src/planar_pack_v3.cpp:829-896 `dequantize_expert_planar_v3_f32` on the device, one planar expert. */
+int tsp_dequantize_planar(const tsp_planar_spec* spec, const void* planar_expert, float* out,
+                          uint32_t* error_word, void* stream);
+
+/* ------------------------------------------------------------------ device: GEMV family */
+
+/* include/tokspur/graph.hpp:730 `MetalGraph::gemv` (src/graph.mm:4182-4270; kernels/gemv.metal:99-117,
+ * 232-266): y[r] = sum_c dec(W[r,c]) * x[c], f32 decode and accumulate. `layout` selects raw GGUF
+ * rows, q8_lanes_v1 rows (Q8_0 only) or one planar v3 expert (Q4_K, Q8_0, Q6_K planes). */
+int tsp_gemv(uint32_t encoding, uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* x, float* y,
+             uint32_t columns, uint32_t rows, uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:733 `gemv_rows` (src/graph.mm:4271-4336): gemv once per token row of a
+ * strided f32 row set; strides in bytes. */
+int tsp_gemv_rows(uint32_t encoding, uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* x,
+                  uint64_t x_stride_bytes, float* y, uint64_t y_stride_bytes, uint32_t count, uint32_t columns,
+                  uint32_t rows, uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:745 `q8_matvec_many` (kernels/q8_many.metal:7-46): Q8_0 GEMV for
+ * width in {1,2,4,8} token rows, x token-major [width, columns], y token-major [width, rows]; each
+ * weight is decoded once for all rows. */
+int tsp_q8_matvec_many(uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* x, float* y,
+                       uint32_t columns, uint32_t rows, uint32_t width, uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:1093 `routed_gemv` (kernels/gemv.metal:198-227): per selected expert s,
+ * y[s, :] = W[ids[s]] * x (x broadcast, or one x row per route). Raw GGUF expert stacks. */
+int tsp_routed_gemv(uint32_t encoding, const void* matrices, uint64_t matrices_bytes, const uint32_t* ids, const float* x,
+                    float* y, uint32_t columns, uint32_t rows, uint32_t experts, uint32_t selected, int broadcast_input,
+                    uint32_t* error_word, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

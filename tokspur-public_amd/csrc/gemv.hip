@@ -1,0 +1,259 @@
+// Decode / verify GEMV over block-quantised rows: y[r] = sum_c dec(W[r,c]) * x[c], f32 decode and
+// f32 accumulate. HBM-bound work: every kernel streams each weight byte exactly once with 16-byte
+// coalesced loads, keeps the activation slice a lane needs in registers across rows, unpacks
+// nibbles and scales in registers and finishes with DPP reductions inside the wave.
+//
+//  gemv_generic   wave per row, any decodable encoding and any K: the scalar control arm.
+//  gemv_q4k       Q4_K, raw GGUF rows or one planar v3 expert; a lane owns one 32-byte nibble pair
+//                 (two 32-weight sub-blocks), 4 lanes per super-block.
+//  gemv_q8        Q8_0 raw rows as a flat dword stream (row bytes are a multiple of 4).
+//  gemv_q6k       Q6_K planar expert planes.
+#include "decode.hpp"
+
+using namespace tsp;
+
+namespace {
+
+struct GemvArgs {
+    const uint8_t* matrix;       // first row of expert 0
+    const float* x;
+    float* y;
+    const uint32_t* ids;         // per blockIdx.y expert id, or nullptr
+    uint64_t expert_stride;      // bytes between experts
+    uint64_t x_stride, y_stride; // bytes between blockIdx.y slices of x / y
+    uint32_t columns, rows, experts, count;
+    uint32_t* error_word;
+    tsp_planar_spec spec;        // planar layouts only
+};
+
+// Resolves the blockIdx.y slice: returns false (after zero-filling and flagging) for a bad expert id.
+__device__ __forceinline__ bool resolve(const GemvArgs& a, const uint8_t*& w, const float*& x, float*& y) {
+    const uint32_t slice = blockIdx.y;
+    w = a.matrix;
+    x = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(a.x) + slice * a.x_stride);
+    y = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.y) + slice * a.y_stride);
+    if (a.ids) {
+        const uint32_t e = a.ids[slice];
+        if (e >= a.experts) {
+            if (threadIdx.x == 0 && blockIdx.x == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+            for (uint32_t r = blockIdx.x * blockDim.x + threadIdx.x; r < a.rows; r += gridDim.x * blockDim.x) y[r] = 0;
+            return false;
+        }
+        w += e * a.expert_stride;
+    }
+    return true;
+}
+
+// ------------------------------------------------------------------------------------ generic
+template <uint32_t T>
+__global__ __launch_bounds__(256) void gemv_generic(GemvArgs a) {
+    constexpr uint32_t E = BlockGeometry<T>::elements, B = BlockGeometry<T>::bytes;
+    const uint8_t* w; const float* x; float* y;
+    if (!resolve(a, w, x, y)) return;
+    const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const uint64_t row_bytes = uint64_t(a.columns / E) * B;
+    for (uint32_t row = blockIdx.x * 4 + wave; row < a.rows; row += gridDim.x * 4) {
+        const uint8_t* data = w + row * row_bytes;
+        float acc = 0;
+        for (uint32_t c = lane; c < a.columns; c += kWave) acc = __builtin_fmaf(decode_element<T>(data + (c / E) * B, c % E), x[c], acc);
+        const float total = wave_sum(acc);
+        if (lane == 0) {
+            if (nonfinite(total)) atomicOr(a.error_word, TSP_ERRBIT_NONFINITE);
+            y[row] = total;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------ Q4_K
+__device__ __forceinline__ float ub(uint32_t w, int i) { return float((w >> (8 * i)) & 0xffu); }
+
+// Sum over aligned groups of N lanes (N = 8, 16, 32, 64); every lane of a group gets the sum.
+template <int N>
+__device__ __forceinline__ float group_sum(float v) {
+    v = dpp_add<0xB1>(v);
+    v = dpp_add<0x4E>(v);
+    v = dpp_add<0x141>(v);
+    if constexpr (N >= 16) v = dpp_add<0x140>(v);
+    if constexpr (N >= 32) v += __shfl_xor(v, 16, kWave);
+    if constexpr (N >= 64) v += __shfl_xor(v, 32, kWave);
+    return v;
+}
+
+// BPR = super-blocks per row (K / 256), one of 2, 4, 8, 16. A wave covers 16 super-blocks per step
+// (16 / BPR rows); lane = (block-in-step, pair) owns 64 weights and keeps their 64 activations in
+// registers for every row it visits.
+template <int BPR, bool PLANAR>
+__global__ __launch_bounds__(256) void gemv_q4k(GemvArgs a) {
+    constexpr int LPR = 4 * BPR;        // lanes per row
+    constexpr int RPS = kWave / LPR;    // rows per wave step
+    __shared__ float xs[BPR * 256];
+    const uint8_t* w; const float* x; float* y;
+    if (!resolve(a, w, x, y)) return;
+    for (uint32_t i = threadIdx.x; i < BPR * 256; i += blockDim.x) xs[i] = x[i];
+    __syncthreads();
+
+    const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const uint32_t pair = lane % 4, blk_in_row = (lane / 4) % BPR, row_in_step = lane / LPR;
+    float xa[32], xb[32];
+    float sxa = 0, sxb = 0;
+    {
+        const float* src = xs + blk_in_row * 256 + pair * 64;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) { xa[i] = src[i]; sxa += xa[i]; }
+#pragma unroll
+        for (int i = 0; i < 32; ++i) { xb[i] = src[32 + i]; sxb += xb[i]; }
+    }
+
+    const uint32_t steps = (a.rows + RPS - 1) / RPS;
+    const uint32_t waves = gridDim.x * (blockDim.x / kWave);
+    for (uint32_t step = blockIdx.x * (blockDim.x / kWave) + wave; step < steps; step += waves) {
+        const uint32_t row = step * RPS + row_in_step;
+        const bool live = row < a.rows;
+        const uint64_t blk = uint64_t(live ? row : a.rows - 1) * BPR + blk_in_row;
+        uint4 q0, q1;
+        float d, dmin;
+        uint32_t sc_a, sc_b, mn_a, mn_b;
+        if constexpr (PLANAR) {
+            const uint8_t* qs = w + a.spec.qs_offset + blk * 128 + pair * 32;
+            q0 = *reinterpret_cast<const uint4*>(qs);
+            q1 = *reinterpret_cast<const uint4*>(qs + 16);
+            const uint8_t* sm = w + a.spec.sm_offset + blk * 16 + pair * 2;
+            const uint32_t sc = *reinterpret_cast<const uint16_t*>(sm), mn = *reinterpret_cast<const uint16_t*>(sm + 8);
+            const uint32_t dm = *reinterpret_cast<const uint32_t*>(w + a.spec.dm_offset + blk * 4);
+            sc_a = sc & 0xffu; sc_b = sc >> 8; mn_a = mn & 0xffu; mn_b = mn >> 8;
+            d = half_bits_to_float(dm & 0xffffu); dmin = half_bits_to_float(dm >> 16);
+        } else {
+            const uint8_t* block = w + blk * 144;
+            const uint4 hdr = *reinterpret_cast<const uint4*>(block);
+            q0 = *reinterpret_cast<const uint4*>(block + 16 + pair * 32);
+            q1 = *reinterpret_cast<const uint4*>(block + 32 + pair * 32);
+            d = half_bits_to_float(hdr.x & 0xffffu); dmin = half_bits_to_float(hdr.x >> 16);
+            // sub-blocks 2*pair and 2*pair+1: byte j = (2*pair) & 3 (and j+1) of the three header words
+            const uint32_t sh = (pair & 1u) * 16u;
+            const uint32_t s2 = (hdr.y >> sh) & 0xffffu, m2 = (hdr.z >> sh) & 0xffffu, e2 = (hdr.w >> sh) & 0xffffu;
+            if (pair < 2) {
+                sc_a = s2 & 63u; sc_b = (s2 >> 8) & 63u; mn_a = m2 & 63u; mn_b = (m2 >> 8) & 63u;
+            } else {
+                sc_a = (e2 & 15u) | (((s2 >> 6) & 3u) << 4);
+                sc_b = ((e2 >> 8) & 15u) | (((s2 >> 14) & 3u) << 4);
+                mn_a = ((e2 >> 4) & 15u) | (((m2 >> 6) & 3u) << 4);
+                mn_b = ((e2 >> 12) & 15u) | (((m2 >> 14) & 3u) << 4);
+            }
+        }
+        const uint32_t words[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        float dot_a0 = 0, dot_a1 = 0, dot_b0 = 0, dot_b1 = 0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t lo = words[k] & 0x0f0f0f0fu, hi = (words[k] >> 4) & 0x0f0f0f0fu;
+            dot_a0 = __builtin_fmaf(ub(lo, 0), xa[4 * k + 0], dot_a0);
+            dot_a1 = __builtin_fmaf(ub(lo, 1), xa[4 * k + 1], dot_a1);
+            dot_a0 = __builtin_fmaf(ub(lo, 2), xa[4 * k + 2], dot_a0);
+            dot_a1 = __builtin_fmaf(ub(lo, 3), xa[4 * k + 3], dot_a1);
+            dot_b0 = __builtin_fmaf(ub(hi, 0), xb[4 * k + 0], dot_b0);
+            dot_b1 = __builtin_fmaf(ub(hi, 1), xb[4 * k + 1], dot_b1);
+            dot_b0 = __builtin_fmaf(ub(hi, 2), xb[4 * k + 2], dot_b0);
+            dot_b1 = __builtin_fmaf(ub(hi, 3), xb[4 * k + 3], dot_b1);
+        }
+        // sum_c ((d*sc)*q - dmin*mn) * x = (d*sc) * sum q x - (dmin*mn) * sum x, per sub-block
+        float part = (d * float(sc_a)) * (dot_a0 + dot_a1) - (dmin * float(mn_a)) * sxa;
+        part += (d * float(sc_b)) * (dot_b0 + dot_b1) - (dmin * float(mn_b)) * sxb;
+        const float total = group_sum<LPR>(part);
+        if (live && lane % LPR == 0) {
+            if (nonfinite(total)) atomicOr(a.error_word, TSP_ERRBIT_NONFINITE);
+            y[row] = total;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------ launch
+uint32_t grid_rows(uint32_t work_items, uint32_t per_block) {
+    const uint32_t blocks = (work_items + per_block - 1) / per_block;
+    return blocks < 1 ? 1 : blocks > 2048 ? 2048 : blocks;
+}
+
+int launch_gemv(uint32_t encoding, uint32_t layout, GemvArgs a, hipStream_t stream) {
+    const bool aligned = reinterpret_cast<uintptr_t>(a.matrix) % 16 == 0 && a.expert_stride % 16 == 0;
+    if (encoding == 12 && aligned && (layout == TSP_LAYOUT_GGUF || layout == TSP_LAYOUT_PLANAR_V3)) {
+        const uint32_t bpr = a.columns / 256;
+        const bool planar = layout == TSP_LAYOUT_PLANAR_V3;
+#define TSP_Q4K_CASE(N)                                                                                                   \
+    if (bpr == N) {                                                                                                       \
+        const dim3 grid(grid_rows((a.rows + 64 / (4 * N) - 1) / (64 / (4 * N)), 4), a.count);                             \
+        if (planar) gemv_q4k<N, true><<<grid, 256, 0, stream>>>(a);                                                       \
+        else gemv_q4k<N, false><<<grid, 256, 0, stream>>>(a);                                                             \
+        return launch_status("gemv_q4k");                                                                                 \
+    }
+        TSP_Q4K_CASE(2) TSP_Q4K_CASE(4) TSP_Q4K_CASE(8) TSP_Q4K_CASE(16)
+#undef TSP_Q4K_CASE
+    }
+    TSP_REQUIRE(layout == TSP_LAYOUT_GGUF, "no GEMV kernel for this layout/encoding/shape");
+    const dim3 grid(grid_rows(a.rows, 4), a.count);
+    const bool ok = dispatch_encoding(encoding, [&]<uint32_t T>() { gemv_generic<T><<<grid, 256, 0, stream>>>(a); });
+    TSP_REQUIRE(ok, "no owned numerical decoder for this encoding");
+    return launch_status("gemv_generic");
+}
+
+int check_shape(uint32_t encoding, uint32_t layout, uint64_t matrix_bytes, uint32_t columns, uint32_t rows, uint32_t experts,
+                tsp_planar_spec* spec, uint64_t* expert_stride) {
+    TSP_REQUIRE(tsp_can_decode(encoding) && columns && columns <= 65536 && rows && rows <= 1000000, "unsupported graph GEMV shape/type");
+    const auto* enc = find_encoding(encoding);
+    TSP_REQUIRE(columns % enc->elements == 0, "GEMV row is not block-aligned");
+    std::memset(spec, 0, sizeof *spec);
+    if (layout == TSP_LAYOUT_PLANAR_V3) {
+        const int rc = tsp_make_expert_spec(encoding, columns, rows, spec);
+        if (rc != TSP_OK) return rc;
+        *expert_stride = spec->planar_expert_bytes;
+    } else {
+        TSP_REQUIRE(layout == TSP_LAYOUT_GGUF || (layout == TSP_LAYOUT_Q8_LANES_V1 && encoding == 8), "layout/encoding mismatch");
+        *expert_stride = uint64_t(columns / enc->elements) * enc->bytes * rows;
+    }
+    TSP_REQUIRE(!mul_overflows(*expert_stride, experts) && *expert_stride * experts == matrix_bytes, "graph GEMV buffer shape mismatch");
+    return TSP_OK;
+}
+
+}  // namespace
+
+extern "C" int tsp_gemv_rows(uint32_t encoding, uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* x,
+                             uint64_t x_stride_bytes, float* y, uint64_t y_stride_bytes, uint32_t count, uint32_t columns,
+                             uint32_t rows, uint32_t* error_word, void* stream) {
+    GemvArgs a{};
+    if (encoding == 8 && count == 1 && layout != TSP_LAYOUT_PLANAR_V3)
+        return tsp_q8_matvec_many(layout, matrix, matrix_bytes, x, y, columns, rows, 1, error_word, stream);
+    const int rc = check_shape(encoding, layout, matrix_bytes, columns, rows, 1, &a.spec, &a.expert_stride);
+    if (rc != TSP_OK) return rc;
+    TSP_REQUIRE(matrix && x && y && error_word, "null device pointer");
+    TSP_REQUIRE(count && count <= 65535 && x_stride_bytes % 4 == 0 && y_stride_bytes % 4 == 0 &&
+                    (count == 1 || (x_stride_bytes >= uint64_t(columns) * 4 && y_stride_bytes >= uint64_t(rows) * 4)),
+                "graph GEMV row extent mismatch");
+    const uint64_t x_span = uint64_t(count - 1) * x_stride_bytes + uint64_t(columns) * 4;
+    const uint64_t y_span = uint64_t(count - 1) * y_stride_bytes + uint64_t(rows) * 4;
+    TSP_REQUIRE(!ranges_overlap(y, y_span, matrix, matrix_bytes) && !ranges_overlap(y, y_span, x, x_span),
+                "GEMV output overlaps an input");
+    a.matrix = static_cast<const uint8_t*>(matrix); a.x = x; a.y = y; a.ids = nullptr;
+    a.x_stride = x_stride_bytes; a.y_stride = y_stride_bytes;
+    a.columns = columns; a.rows = rows; a.experts = 1; a.count = count; a.error_word = error_word;
+    return launch_gemv(encoding, layout, a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tsp_gemv(uint32_t encoding, uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* x, float* y,
+                        uint32_t columns, uint32_t rows, uint32_t* error_word, void* stream) {
+    return tsp_gemv_rows(encoding, layout, matrix, matrix_bytes, x, 0, y, 0, 1, columns, rows, error_word, stream);
+}
+
+extern "C" int tsp_routed_gemv(uint32_t encoding, const void* matrices, uint64_t matrices_bytes, const uint32_t* ids, const float* x,
+                               float* y, uint32_t columns, uint32_t rows, uint32_t experts, uint32_t selected, int broadcast_input,
+                               uint32_t* error_word, void* stream) {
+    GemvArgs a{};
+    TSP_REQUIRE(experts && experts <= 4096 && selected && selected <= 64, "invalid routed GEMV routing shape");
+    const int rc = check_shape(encoding, TSP_LAYOUT_GGUF, matrices_bytes, columns, rows, experts, &a.spec, &a.expert_stride);
+    if (rc != TSP_OK) return rc;
+    TSP_REQUIRE(matrices && ids && x && y && error_word, "null device pointer");
+    const uint64_t x_span = uint64_t(broadcast_input ? 1 : selected) * columns * 4, y_span = uint64_t(selected) * rows * 4;
+    TSP_REQUIRE(!ranges_overlap(y, y_span, matrices, matrices_bytes) && !ranges_overlap(y, y_span, x, x_span) &&
+                    !ranges_overlap(y, y_span, ids, uint64_t(selected) * 4),
+                "routed GEMV output overlaps an input");
+    a.matrix = static_cast<const uint8_t*>(matrices); a.x = x; a.y = y; a.ids = ids;
+    a.x_stride = broadcast_input ? 0 : uint64_t(columns) * 4; a.y_stride = uint64_t(rows) * 4;
+    a.columns = columns; a.rows = rows; a.experts = experts; a.count = selected; a.error_word = error_word;
+    return launch_gemv(encoding, TSP_LAYOUT_GGUF, a, static_cast<hipStream_t>(stream));
+}
