@@ -164,6 +164,80 @@ int tsp_routed_gemv(uint32_t encoding, const void* matrices, uint64_t matrices_b
                     float* y, uint32_t columns, uint32_t rows, uint32_t experts, uint32_t selected, int broadcast_input,
                     uint32_t* error_word, void* stream);
 
+/* ------------------------------------------------------------------ device: router, combine, SwiGLU */
+
+/* include/tokspur/graph.hpp:1091 `route` (kernels/graph.metal:466-526; CPU: src/routing.cpp:11-40):
+ * top-`selected` of `experts` f32 logits by (logit desc, id asc); weights = softmax (mode 0) or
+ * sigmoid (mode 1), renormalised over the selected when normalize_selected. ids are exact. */
+int tsp_route(const float* logits, uint32_t* indices, float* weights, uint32_t experts, uint32_t selected, uint32_t mode,
+              int normalize_selected, uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:852 `prefill_route_batch` / 837 `moe_route_rows` (kernels/graph.metal:551-638):
+ * the same per token row; logits [tokens, experts], outputs [tokens, selected]. */
+int tsp_route_batch(const float* logits, uint32_t* indices, float* weights, uint32_t experts, uint32_t selected,
+                    uint32_t tokens, uint32_t mode, int normalize_selected, uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:1102 `mixture` (kernels/graph.metal:528-544; CPU: src/routing.cpp:42-60):
+ * y[c] = sigmoid(shared_logit) * shared[c] + sum_r w[r] * experts[r, c], r in route order. */
+int tsp_mixture(const float* expert_outputs, const float* weights, const float* shared_output, const float* shared_logit,
+                float* output, uint32_t channels, uint32_t selected, uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:853 `prefill_mixture_batch` (kernels/graph.metal:654-691): per token row;
+ * expert_outputs [tokens, selected, channels], output rows `output_stride_bytes` apart. */
+int tsp_mixture_batch(const float* expert_outputs, const float* weights, const float* shared_output, const float* shared_logit,
+                      float* output, uint64_t output_stride_bytes, uint32_t channels, uint32_t selected, uint32_t tokens,
+                      uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:990 `swiglu` (kernels/graph.metal:312-326): out = silu(gate*scale) * up. */
+int tsp_swiglu(const float* gate, const float* up, float* output, uint64_t count, float scale, uint32_t* error_word, void* stream);
+
+/* ------------------------------------------------------------------ device: expert permutation */
+
+/* kernels/grouped_mpp.metal:12-37 `graph_grouped_routes` (encoded inside `grouped_mm`, src/graph.mm:4571,
+ * and `planar_nax_grouped_moe`, src/graph.mm:9383): token_map[e*tokens + k] = t*selected + slot for the
+ * k-th token in ascending order that routes to expert e; counts[e]. Tails of token_map rows are not
+ * written. TSP_ERRBIT_INDEX on id >= experts or an expert repeated within one token. */
+int tsp_grouped_routes(const uint32_t* ids, uint32_t* token_map, uint32_t* counts, uint32_t experts, uint32_t selected,
+                       uint32_t tokens, uint32_t* error_word, void* stream);
+/* kernels/grouped_mpp.metal:41-64 `graph_grouped_tasks` / kernels/nax_prefill.metal:4057-4091: tasks[0] =
+ * tiles, tasks[1] = routes, tasks[2+2i] = expert, tasks[3+2i] = first row of the tile; unused slots up to
+ * tokens*selected/tile + experts are 0xFFFFFFFF. (The Metal indirect-grid words have no HIP counterpart.) */
+int tsp_grouped_tasks(const uint32_t* counts, uint32_t* tasks, uint32_t experts, uint32_t selected, uint32_t tokens,
+                      uint32_t tile, uint32_t* error_word, void* stream);
+/* kernels/planar_moe_v3.metal:413-509 `planar_moe_build_union_m8`: the 9 280-byte union block for
+ * tokens <= 8 (layout src/graph.mm:9091, kernels/planar_moe_v3.metal:439-442): [0..7] header,
+ * +8 experts[128], +136 counts[128], +264 tokens[128][8], +1288 routes[128][8] (32-bit words). */
+int tsp_planar_union_build(const uint32_t* ids, uint32_t* meta, uint32_t experts, uint32_t selected, uint32_t tokens,
+                           uint32_t hidden, uint32_t channels, uint32_t* error_word, void* stream);
+
+/* ------------------------------------------------------------------ device: routed MoE, 1..8 token rows */
+
+/* The operands of `planar_moe_gate_up_swiglu_m8` / `planar_moe_routed_m8`
+ * (include/tokspur/graph.hpp:472-477; src/graph.mm:9134-9291). pair_lo / pair_hi are the two
+ * co-located gate/up tensors (kinds 2/3, 4/5 or 6/7), `down` is [experts] planar experts of kind
+ * 8 (Q5_1), 9 (Q8_0) or 10 (Q6_K, this library's extension). x holds `tokens` f32 rows of
+ * `channels`; h and y hold tokens*selected rows (route rid = t*selected + slot) of `hidden` and
+ * `channels` floats. Strides are bytes. union_meta is the caller's 9 280-byte union block
+ * (required when tokens > 1; the entry points rebuild it from ids on every call). */
+typedef struct tsp_small_moe {
+    const void* pair_lo;
+    const void* pair_hi;
+    const void* down;
+    uint32_t gate_kind, up_kind, down_kind;
+    uint32_t channels, hidden, experts, selected, tokens;
+    const uint32_t* ids;
+    const float* x;
+    uint64_t x_stride_bytes;
+    float* h;
+    uint64_t h_stride_bytes;
+    float* y;
+    uint64_t y_stride_bytes;
+    uint32_t* union_meta;
+    uint32_t* error_word;
+} tsp_small_moe;
+/* include/tokspur/graph.hpp:472 `planar_moe_gate_up_swiglu_m8` (kernels/planar_moe_v3.metal:513-1090):
+ * h[rid, r] = silu(Wg[e] x_t)[r] * (Wu[e] x_t)[r], f32 throughout. `down`, `y` are ignored. */
+int tsp_planar_moe_gate_up_swiglu_m8(const tsp_small_moe* moe, void* stream);
+/* include/tokspur/graph.hpp:475 `planar_moe_routed_m8` (kernels/planar_moe_v3.metal:1572-1803):
+ * the above followed by y[rid, :] = Wd[e] h[rid, :]. */
+int tsp_planar_moe_routed_m8(const tsp_small_moe* moe, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -56,9 +56,36 @@ def tsp():
 
 
 @pytest.fixture(scope="session")
-def gpu(tsp):
+def _device(tsp):
     import torch
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     torch.cuda.set_device(0)
     return tsp.Device()
+
+
+@pytest.fixture
+def gpu(_device):
+    """The device with a clean sticky error word, so one failing test cannot poison the next."""
+    _device.clear_error()
+    return _device
+
+
+def nmse(got, ref):
+    """Normalised mean squared error, the engine's bound for MoE outputs (native/tests/test_planar_pack_v3.cpp:181-192)."""
+    import numpy as np
+    got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
+    assert np.isfinite(got).all() and np.isfinite(ref).all()
+    return float(((got - ref) ** 2).sum() / max((ref ** 2).sum(), 1e-300))
+
+
+def max_rel_error(got, ref):
+    """max |a - e| / max(1, |e|, rms(e_row)): element-wise error in units of the row's own scale. With f32
+    accumulation the absolute error grows with sum |w||x|, so an element that cancels to near zero in a row of
+    large values cannot be judged against its own magnitude."""
+    import numpy as np
+    got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
+    ref2 = ref.reshape(-1, ref.shape[-1]) if ref.ndim > 1 else ref.reshape(1, -1)
+    got2 = got.reshape(ref2.shape)
+    rms = np.sqrt((ref2 ** 2).mean(axis=1, keepdims=True))
+    return float(np.max(np.abs(got2 - ref2) / np.maximum(np.maximum(1.0, np.abs(ref2)), rms)))

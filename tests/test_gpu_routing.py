@@ -1,0 +1,183 @@
+"""GPU parity for the router (ids bit-exact), the expert permutation and prefix-sum offsets
+(bit-exact), the T <= 8 union records (bit-exact), and the mixture / SwiGLU operators."""
+import numpy as np
+import pytest
+
+from test_oracle_pack import union_spec
+from test_oracle_routing import std_mt19937
+
+pytestmark = pytest.mark.gpu
+
+
+def u32(t):
+    return t.cpu().numpy().view(np.uint32)
+
+
+# ---------------------------------------------------------------------------------- router
+
+def test_route_reference_trials(gpu, orc):
+    # native/tests/test_routing.cpp:24-48 trials, pushed through the device router; logits are multiples of 0.01
+    # rounded to f32, so the f32 order (with its ties) is what the oracle sees too.
+    bg = std_mt19937(0x726F7574)
+    for trial in range(300):
+        count = 1 + int(bg.random_raw()) % 1024
+        selected = 1 + int(bg.random_raw()) % min(64, count)
+        logits = ((bg.random_raw(count).astype(np.int64) % 2001 - 1000) / 100.0).astype(np.float32)
+        mode, normalize = trial % 2, (trial // 2) % 2 == 0
+        ids, w = gpu.route(gpu.upload(logits), selected, mode, normalize)
+        want_ids, want_w = orc.route_reference(logits.astype(np.float64), selected, mode, normalize)
+        assert np.array_equal(u32(ids)[0], want_ids), trial
+        assert np.allclose(w.cpu().numpy()[0], want_w, rtol=2e-5, atol=1e-7), trial
+    assert gpu.error() == 0
+
+
+def test_route_goldens(gpu, orc):
+    # native/tests/test_routing.cpp:49-51 tie golden; native/tests/test_moe_mm_many_gpu.cpp:252-253 all-zero logits.
+    ids, _ = gpu.route(gpu.upload(np.array([3, 3, 2, 1, 3], dtype=np.float32)), 3, 0, True)
+    assert list(u32(ids)[0]) == [0, 1, 4]
+    ids, w = gpu.route(gpu.upload(np.zeros((4, 512), dtype=np.float32)), 10, 0, True, tokens=4)
+    assert (u32(ids) == np.arange(10)).all() and np.allclose(w.cpu().numpy(), 0.1, rtol=1e-6)
+    # -0.0 and +0.0 compare equal: ties go to the lower id
+    ids, _ = gpu.route(gpu.upload(np.array([-0.0, 0.0, -0.0, 0.0], dtype=np.float32)), 2, 0, True)
+    assert list(u32(ids)[0]) == [0, 1]
+    # underflow cases, native/tests/test_routing.cpp:60-64
+    _, w = gpu.route(gpu.upload(np.array([-1000.0], dtype=np.float32)), 1, 1, True)
+    assert w.cpu().numpy()[0, 0] == 1.0
+    _, w = gpu.route(gpu.upload(np.array([-1000.0], dtype=np.float32)), 1, 0, True)
+    assert w.cpu().numpy()[0, 0] == 1.0 and gpu.error() == 0
+
+
+@pytest.mark.parametrize("tokens,experts,selected", [(8, 512, 10), (2048, 512, 10), (33, 64, 4), (5, 200, 64)])
+def test_route_batch_ids_bit_exact(gpu, orc, synth, tokens, experts, selected):
+    """Configs 2 and 3: softmax, top-10 renormalised over 512 experts; Zipf-biased logits at T = 2048."""
+    seed = synth.tensor_seed(3, 10 + tokens)
+    logits = synth.zipf_router_logits(seed, tokens, experts) if tokens == 2048 else synth.activations_f32(seed, (tokens, experts))
+    if tokens == 33:
+        logits = np.round(logits * 2) / 2  # plenty of exact ties
+    ids, w = gpu.route(gpu.upload(logits), selected, 0, True, tokens=tokens)
+    ids, w = u32(ids), w.cpu().numpy()
+    for t in range(tokens):
+        want_ids, want_w = orc.route_reference(logits[t].astype(np.float64), selected, 0, True)
+        assert np.array_equal(ids[t], want_ids), t
+        assert np.allclose(w[t], want_w, rtol=2e-5, atol=1e-9), t
+    assert gpu.error() == 0
+    assert np.allclose(w.sum(axis=1), 1.0, rtol=1e-5)
+
+
+def test_route_errors(gpu, tsp):
+    logits = np.zeros(16, dtype=np.float32)
+    logits[3] = np.nan
+    ids, _ = gpu.route(gpu.upload(logits), 2, 0, True)
+    assert gpu.error() & tsp.ERRBIT_NONFINITE and list(u32(ids)[0]) == [0, 1]
+    for args in ((0, 0, True), (17, 0, True), (2, 2, True)):
+        with pytest.raises(tsp.FormatError):
+            gpu.route(gpu.upload(np.zeros(16, dtype=np.float32)), *args)
+    with pytest.raises(tsp.FormatError):
+        gpu.route(gpu.upload(np.zeros((2, 600), dtype=np.float32)), 2, 0, True, tokens=2)
+
+
+# ---------------------------------------------------------------------------------- permutation
+
+def random_ids(rng, tokens, selected, experts, skew=False):
+    out = np.empty((tokens, selected), dtype=np.uint32)
+    p = None
+    if skew:
+        p = 1.0 / np.arange(1, experts + 1) ** 1.1
+        p /= p.sum()
+    for t in range(tokens):
+        out[t] = rng.choice(experts, size=selected, replace=False, p=p)
+    return out.reshape(-1)
+
+
+@pytest.mark.parametrize("tokens,selected,experts", [(1, 1, 2), (5, 3, 8), (33, 4, 16), (100, 10, 64), (64, 2, 4), (257, 10, 512),
+                                                     (2048, 10, 512), (544, 4, 8)])
+def test_grouped_routes_and_tasks_bit_exact(gpu, orc, tokens, selected, experts):
+    rng = np.random.default_rng(tokens * 31 + selected)
+    ids = random_ids(rng, tokens, selected, experts, skew=tokens == 2048)
+    want_map, want_counts, err = orc.grouped_routes(ids, experts, selected, tokens)
+    assert err == 0
+    token_map, counts = gpu.grouped_routes(gpu.upload(ids), experts, selected, tokens)
+    assert np.array_equal(u32(counts), want_counts)
+    assert np.array_equal(u32(token_map).reshape(-1), want_map)  # untouched tails keep the caller's fill on both sides
+    want_tasks, err = orc.grouped_tasks(want_counts, experts, selected, tokens, 32)
+    tasks = gpu.grouped_tasks(counts, experts, selected, tokens, 32)
+    assert err == 0 and np.array_equal(u32(tasks), want_tasks) and gpu.error() == 0
+    # size-independent invariants of the permutation
+    tm = u32(token_map).reshape(experts, tokens)
+    seen = np.concatenate([tm[e, :want_counts[e]] for e in range(experts)])
+    assert np.array_equal(np.sort(seen), np.arange(tokens * selected))
+    for e in range(experts):
+        row = tm[e, :want_counts[e]]
+        assert (ids[row] == e).all() and (np.diff(row.astype(np.int64)) > 0).all()
+
+
+def test_grouping_error_bits(gpu, tsp):
+    for ids in ([0, 9], [1, 1]):
+        gpu.grouped_routes(gpu.upload(np.array(ids, dtype=np.uint32)), 4, 2, 1)
+        assert gpu.error() == tsp.ERRBIT_INDEX
+    gpu.grouped_tasks(gpu.upload(np.array([1, 0, 0, 0], dtype=np.uint32)), 4, 2, 1)
+    assert gpu.error() == tsp.ERRBIT_INDEX
+    gpu.grouped_tasks(gpu.upload(np.array([9, 0, 0, 0], dtype=np.uint32)), 4, 2, 4)
+    assert gpu.error() == tsp.ERRBIT_INDEX
+
+
+def test_union_metadata_all_cases_bit_exact(gpu, orc):
+    # native/tests/test_planar_union_metadata.mm:105-124: T = 1..8 x S = 1..16, four id patterns each; untouched
+    # words must keep the caller's poison and invalid ids must zero the header and raise bit 4.
+    bg = std_mt19937(1729)
+    for tokens in range(1, 9):
+        for selected in range(1, 17):
+            n = tokens * selected
+            mixed = [int(bg.random_raw()) % 7 if i % 3 else 511 for i in range(n)]
+            for ids in ([511] * n, [(511 - i) % 512 for i in range(n)], mixed, mixed[:-1] + [512]):
+                got = u32(gpu.union_build(gpu.upload(np.array(ids, dtype=np.uint32)), 512, selected, tokens, 639, 2559))
+                want, want_err = union_spec(512, selected, tokens, 639, 2559, ids)
+                assert gpu.error() == want_err and np.array_equal(got, want), (tokens, selected)
+                assert np.array_equal(got, orc.union_metadata(512, selected, tokens, 639, 2559, ids)[0])
+    for shape, ids in (((3, 1, 1, 640, 2560), [0]), ((2, 3, 1, 640, 2560), [0, 1, 0])):
+        got = u32(gpu.union_build(gpu.upload(np.array(ids, dtype=np.uint32)), *shape))
+        assert gpu.error() == 4 and not got[:8].any() and (got[8:] == 0xBAADF00D).all()
+
+
+# ---------------------------------------------------------------------------------- mixture / SwiGLU
+
+def test_mixture_golden_and_rows(gpu, orc, synth):
+    # native/tests/test_routing.cpp:52-55
+    out = gpu.mixture(gpu.upload(np.array([1, 2, 3, 4], dtype=np.float32)), gpu.upload(np.array([0.25, 0.75], dtype=np.float32)),
+                      gpu.upload(np.array([5, 6], dtype=np.float32)), gpu.upload(np.zeros(1, dtype=np.float32)), 2, 2)
+    assert list(out.cpu().numpy()[0]) == [5.0, 6.5]
+    tokens, selected, channels = 37, 10, 2048
+    ex = synth.activations_f32(1, (tokens, selected, channels))
+    w = np.abs(synth.activations_f32(2, (tokens, selected))) / 10
+    sh = synth.activations_f32(3, (tokens, channels))
+    sl = synth.activations_f32(4, tokens)
+    out = gpu.full((tokens, channels + 16), -3.0)
+    gpu.mixture(gpu.upload(ex), gpu.upload(w), gpu.upload(sh), gpu.upload(sl), channels, selected, tokens, out=out, out_stride=(channels + 16) * 4)
+    out = out.cpu().numpy()
+    for t in range(tokens):
+        want = orc.mixture_reference(ex[t].astype(np.float64), w[t].astype(np.float64), sh[t].astype(np.float64), float(sl[t]))
+        assert np.max(np.abs(out[t, :channels] - want) / np.maximum(1, np.abs(want))) <= 5e-6
+    assert (out[:, channels:] == -3.0).all() and gpu.error() == 0
+
+
+def test_mixture_errors(gpu, tsp):
+    one = gpu.upload(np.ones(4, dtype=np.float32))
+    gpu.mixture(gpu.upload(np.ones(8, dtype=np.float32)), gpu.upload(np.array([0.5, -0.5], dtype=np.float32)), one,
+                gpu.upload(np.zeros(1, dtype=np.float32)), 4, 2)
+    assert gpu.error() == tsp.ERRBIT_NONFINITE
+    gpu.mixture(gpu.upload(np.ones(8, dtype=np.float32)), gpu.upload(np.array([0.5, 0.5], dtype=np.float32)), one,
+                gpu.upload(np.array([np.inf], dtype=np.float32)), 4, 2)
+    assert gpu.error() == tsp.ERRBIT_NONFINITE
+
+
+def test_swiglu(gpu, tsp, orc):
+    g = np.linspace(-30, 30, 4001).astype(np.float32)
+    u = np.cos(np.arange(4001)).astype(np.float32) * 3
+    out = gpu.swiglu(gpu.upload(g), gpu.upload(u), 0.5).cpu().numpy()
+    want = np.array([orc.stable_silu(float(np.float32(a) * np.float32(0.5))) * float(b) for a, b in zip(g, u)])
+    assert np.max(np.abs(out - want) / np.maximum(1, np.abs(want))) <= 2e-6 and gpu.error() == 0
+    assert gpu.swiglu(gpu.upload(np.zeros(3, dtype=np.float32)), gpu.upload(np.ones(3, dtype=np.float32))).cpu().numpy().tolist() == [0, 0, 0]
+    bad = g.copy()
+    bad[5] = np.nan
+    gpu.swiglu(gpu.upload(bad), gpu.upload(u))
+    assert gpu.error() == tsp.ERRBIT_NONFINITE

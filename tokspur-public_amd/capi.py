@@ -212,6 +212,8 @@ class Device:
         return self.torch.zeros(shape, dtype=getattr(self.torch, dtype), device=self.dev)
 
     def full(self, shape, value, dtype="float32"):
+        shape = tuple(shape) if isinstance(shape, (tuple, list)) else (int(shape),)
+        value = value.item() if hasattr(value, "item") else value
         return self.torch.full(shape, value, dtype=getattr(self.torch, dtype), device=self.dev)
 
     @staticmethod
@@ -274,3 +276,110 @@ class Device:
                                     self.ptr(y), C.c_uint32(columns), C.c_uint32(rows), C.c_uint32(experts), C.c_uint32(selected),
                                     C.c_int(bool(broadcast)), self.ptr(self.err), self.stream()))
         return y
+
+    def route(self, logits, selected, mode=0, normalize=True, tokens=None):
+        """logits [experts] (tokens=None: the single-row operator) or [tokens, experts]."""
+        experts = logits.shape[-1]
+        n = 1 if tokens is None else tokens
+        ids = self.zeros((n, selected), "int32")
+        w = self.zeros((n, selected))
+        if tokens is None:
+            check(dll().tsp_route(self.ptr(logits), self.ptr(ids), self.ptr(w), C.c_uint32(experts), C.c_uint32(selected), C.c_uint32(mode),
+                                  C.c_int(bool(normalize)), self.ptr(self.err), self.stream()))
+        else:
+            check(dll().tsp_route_batch(self.ptr(logits), self.ptr(ids), self.ptr(w), C.c_uint32(experts), C.c_uint32(selected),
+                                        C.c_uint32(tokens), C.c_uint32(mode), C.c_int(bool(normalize)), self.ptr(self.err), self.stream()))
+        return ids, w
+
+    def mixture(self, expert_out, weights, shared, shared_logit, channels, selected, tokens=1, out=None, out_stride=None):
+        out = self.empty((tokens, channels)) if out is None else out
+        stride = channels * 4 if out_stride is None else out_stride
+        check(dll().tsp_mixture_batch(self.ptr(expert_out), self.ptr(weights), self.ptr(shared), self.ptr(shared_logit), self.ptr(out),
+                                      C.c_uint64(stride), C.c_uint32(channels), C.c_uint32(selected), C.c_uint32(tokens),
+                                      self.ptr(self.err), self.stream()))
+        return out
+
+    def swiglu(self, gate, up, scale=1.0, out=None):
+        out = self.empty(gate.shape) if out is None else out
+        check(dll().tsp_swiglu(self.ptr(gate), self.ptr(up), self.ptr(out), C.c_uint64(gate.numel()), C.c_float(scale),
+                               self.ptr(self.err), self.stream()))
+        return out
+
+    def grouped_routes(self, ids, experts, selected, tokens, fill=0xDEADBEEF):
+        token_map = self.full((experts, tokens), np.int32(np.uint32(fill).view(np.int32)), "int32")
+        counts = self.zeros(experts, "int32")
+        check(dll().tsp_grouped_routes(self.ptr(ids), self.ptr(token_map), self.ptr(counts), C.c_uint32(experts), C.c_uint32(selected),
+                                       C.c_uint32(tokens), self.ptr(self.err), self.stream()))
+        return token_map, counts
+
+    def grouped_tasks(self, counts, experts, selected, tokens, tile=32):
+        bound = tokens * selected // tile + experts
+        tasks = self.zeros(2 + 2 * bound, "int32")
+        check(dll().tsp_grouped_tasks(self.ptr(counts), self.ptr(tasks), C.c_uint32(experts), C.c_uint32(selected), C.c_uint32(tokens),
+                                      C.c_uint32(tile), self.ptr(self.err), self.stream()))
+        return tasks
+
+    def union_build(self, ids, experts, selected, tokens, hidden, channels, poison=0xBAADF00D):
+        meta = self.full(2320, np.int32(np.uint32(poison).view(np.int32)), "int32")
+        check(dll().tsp_planar_union_build(self.ptr(ids), self.ptr(meta), C.c_uint32(experts), C.c_uint32(selected), C.c_uint32(tokens),
+                                           C.c_uint32(hidden), C.c_uint32(channels), self.ptr(self.err), self.stream()))
+        return meta
+
+
+class SmallMoe(C.Structure):
+    _fields_ = [("pair_lo", C.c_void_p), ("pair_hi", C.c_void_p), ("down", C.c_void_p),
+                ("gate_kind", C.c_uint32), ("up_kind", C.c_uint32), ("down_kind", C.c_uint32),
+                ("channels", C.c_uint32), ("hidden", C.c_uint32), ("experts", C.c_uint32), ("selected", C.c_uint32),
+                ("tokens", C.c_uint32), ("ids", C.c_void_p), ("x", C.c_void_p), ("x_stride_bytes", C.c_uint64),
+                ("h", C.c_void_p), ("h_stride_bytes", C.c_uint64), ("y", C.c_void_p), ("y_stride_bytes", C.c_uint64),
+                ("union_meta", C.c_void_p), ("error_word", C.c_void_p)]
+
+
+COLOC_KINDS = {12: (2, 3), 13: (4, 5), 8: (6, 7)}
+DOWN_KINDS = {7: 8, 8: 9, 14: 10}
+
+
+class PlanarMoeWeights:
+    """Device-resident planar v3 expert tensors of one MoE sublayer: pair_lo / pair_hi (co-located
+    gate/up halves) and the [experts] down tensor, built from raw GGUF expert stacks on the host."""
+
+    def __init__(self, dev, gu_type, dn_type, channels, hidden, experts, gate_raw, up_raw, down_raw):
+        self.gu_type, self.dn_type = gu_type, dn_type
+        self.channels, self.hidden, self.experts = channels, hidden, experts
+        self.gu_spec = make_expert_spec(gu_type, channels, hidden)
+        self.dn_spec = make_expert_spec(dn_type, hidden, channels)
+        self.pair_lo = dev.upload(pack_coloc_half(self.gu_spec, gate_raw, up_raw, experts, 0))
+        self.pair_hi = dev.upload(pack_coloc_half(self.gu_spec, gate_raw, up_raw, experts, 1))
+        self.down = dev.upload(pack_experts(self.dn_spec, down_raw, experts))
+        self.union_meta = dev.zeros(2320, "int32")
+
+
+def _small_moe(dev, w, ids, x, tokens, selected, h, y, x_stride=None, h_stride=None, y_stride=None):
+    gate_kind, up_kind = COLOC_KINDS[w.gu_type]
+    m = SmallMoe(w.pair_lo.data_ptr(), w.pair_hi.data_ptr(), w.down.data_ptr() if y is not None else None,
+                 gate_kind, up_kind, DOWN_KINDS[w.dn_type], w.channels, w.hidden, w.experts, selected, tokens,
+                 ids.data_ptr(), x.data_ptr(), w.channels * 4 if x_stride is None else x_stride,
+                 h.data_ptr(), w.hidden * 4 if h_stride is None else h_stride,
+                 y.data_ptr() if y is not None else None, w.channels * 4 if y_stride is None else y_stride,
+                 w.union_meta.data_ptr(), dev.err.data_ptr())
+    return m
+
+
+def planar_moe_gate_up_swiglu_m8(dev, w, ids, x, tokens, selected, h=None, **strides):
+    h = dev.empty((tokens * selected, w.hidden)) if h is None else h
+    m = _small_moe(dev, w, ids, x, tokens, selected, h, None, **strides)
+    check(dll().tsp_planar_moe_gate_up_swiglu_m8(C.byref(m), dev.stream()))
+    return h
+
+
+def planar_moe_routed_m8(dev, w, ids, x, tokens, selected, h=None, y=None, **strides):
+    h = dev.empty((tokens * selected, w.hidden)) if h is None else h
+    y = dev.empty((tokens * selected, w.channels)) if y is None else y
+    m = _small_moe(dev, w, ids, x, tokens, selected, h, y, **strides)
+    check(dll().tsp_planar_moe_routed_m8(C.byref(m), dev.stream()))
+    return h, y
+
+
+def as_u32(t):
+    """Device int32 tensor -> host uint32 array."""
+    return t.cpu().numpy().view(np.uint32)

@@ -1,0 +1,185 @@
+// Deterministic expert permutation, prefix-sum tile offsets, and the T <= 8 union records.
+// Integer work only; every output word is a pure function of the route ids, so results are
+// bit-identical run to run and identical to the sequential specification.
+//
+//  grouped_routes  token_map[e*T + k] = t*S + slot for the k-th token (ascending) that routes to e;
+//                  counts[e] = number of such tokens. No atomics on the map: one block per expert
+//                  compacts with ballots and a running base, so order is the token order.
+//  grouped_tasks   tiles(e) = ceil(min(counts[e], T) / tile); exclusive scan over experts; task i of
+//                  expert e is (e, i*tile); unused slots up to the bound are 0xFFFFFFFF.
+//  union_build     for T*S <= 128 routes: records (expert, <= cap routes) in first-use order.
+#include "tsp_common.hpp"
+
+using namespace tsp;
+
+namespace {
+
+__global__ __launch_bounds__(256) void grouped_routes_kernel(const uint32_t* __restrict__ ids, uint32_t* __restrict__ token_map,
+                                                             uint32_t* __restrict__ counts, uint32_t experts, uint32_t selected,
+                                                             uint32_t tokens, uint32_t* error_word) {
+    __shared__ uint32_t wave_totals[4];
+    const uint32_t expert = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    uint32_t accumulated = 0, bad = 0;
+    for (uint32_t base = 0; base < tokens; base += 256) {
+        const uint32_t token = base + tid;
+        uint32_t slot = 0xffffffffu, matches = 0;
+        if (token < tokens) {
+            for (uint32_t i = 0; i < selected; ++i) {
+                const uint32_t id = ids[uint64_t(token) * selected + i];
+                if (id >= experts) bad = TSP_ERRBIT_INDEX;
+                if (id == expert) { slot = i; ++matches; }
+            }
+        }
+        if (matches > 1) bad = TSP_ERRBIT_INDEX;
+        const bool found = matches == 1;
+        const uint64_t mask = __builtin_amdgcn_ballot_w64(found);
+        const uint32_t prefix = __builtin_popcountll(mask & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_totals[wave] = __builtin_popcountll(mask);
+        __syncthreads();
+        uint32_t before = 0, chunk = 0;
+        for (uint32_t w = 0; w < 4; ++w) { if (w < wave) before += wave_totals[w]; chunk += wave_totals[w]; }
+        if (found) token_map[uint64_t(expert) * tokens + accumulated + before + prefix] = token * selected + slot;
+        accumulated += chunk;
+        __syncthreads();
+    }
+    if (tid == 0) counts[expert] = accumulated;
+    publish_error(bad, error_word);
+}
+
+// One block of 512 threads; experts <= 512.
+__global__ __launch_bounds__(512) void grouped_tasks_kernel(const uint32_t* __restrict__ counts, uint32_t* __restrict__ tasks,
+                                                            uint32_t experts, uint32_t selected, uint32_t tokens, uint32_t tile,
+                                                            uint32_t* error_word) {
+    __shared__ uint32_t tiles_scan[512];
+    __shared__ uint32_t routes_scan[512];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t bound = tokens * selected / tile + experts;
+    uint32_t bad = 0;
+    const uint32_t count = tid < experts ? counts[tid] : 0;
+    if (count > tokens) bad = TSP_ERRBIT_INDEX;
+    const uint32_t n = ((count < tokens ? count : tokens) + tile - 1) / tile;
+    tiles_scan[tid] = n;
+    routes_scan[tid] = count;
+    __syncthreads();
+    for (uint32_t step = 1; step < 512; step <<= 1) {  // inclusive Hillis-Steele scan
+        const uint32_t a = tid >= step ? tiles_scan[tid - step] : 0, b = tid >= step ? routes_scan[tid - step] : 0;
+        __syncthreads();
+        tiles_scan[tid] += a;
+        routes_scan[tid] += b;
+        __syncthreads();
+    }
+    const uint32_t total = tiles_scan[511], routes = routes_scan[511];
+    const uint32_t offset = tiles_scan[tid] - n;
+    for (uint32_t i = tid; i < bound; i += 512) { tasks[2 + 2 * i] = 0xffffffffu; tasks[3 + 2 * i] = 0xffffffffu; }
+    __syncthreads();
+    if (tid < experts)
+        for (uint32_t i = 0; i < n; ++i)
+            if (offset + i < bound) { tasks[2 + 2 * (offset + i)] = tid; tasks[3 + 2 * (offset + i)] = i * tile; }
+    if (tid == 0) {
+        tasks[0] = total < bound ? total : bound;
+        tasks[1] = routes;
+        if (total > bound || routes != tokens * selected) bad = TSP_ERRBIT_INDEX;
+    }
+    publish_error(bad, error_word);
+}
+
+// 128 threads, one per flat route (T*S <= 128). meta layout in 32-bit words: [0..7] header,
+// +8 experts[128], +136 counts[128], +264 tokens[128][8], +1288 routes[128][8].
+__global__ __launch_bounds__(128) void union_build_kernel(const uint32_t* __restrict__ ids, uint32_t* __restrict__ meta,
+                                                          uint32_t experts, uint32_t selected, uint32_t tokens, uint32_t hidden,
+                                                          uint32_t channels, uint32_t* error_word) {
+    __shared__ uint32_t sid[128];
+    __shared__ uint32_t record_of[128];
+    __shared__ uint32_t wave_leaders[2];
+    __shared__ uint32_t any_bad;
+    const uint32_t f = threadIdx.x, total = tokens * selected;
+    const bool shape_ok = experts && experts <= 512 && experts % 2 == 0 && selected && selected <= 16 && selected <= experts &&
+                          tokens && tokens <= 8 && hidden && channels;
+    if (f == 0) any_bad = shape_ok ? 0u : 1u;
+    __syncthreads();
+    const bool live = shape_ok && f < total;
+    const uint32_t mine = live ? ids[f] : 0xffffffffu;
+    if (live && mine >= experts) any_bad = 1u;
+    sid[f] = mine;
+    __syncthreads();
+    if (any_bad) {
+        if (f < 8) meta[f] = 0;
+        if (f == 0) atomicOr(error_word, TSP_ERRBIT_INDEX);
+        return;
+    }
+    const uint32_t cap = tokens <= 4 ? 4u : 8u;
+    uint32_t rank = 0, same = 0;
+    if (live) {
+        for (uint32_t g = 0; g < total; ++g) {
+            const bool eq = sid[g] == mine;
+            rank += (eq && g < f) ? 1u : 0u;
+            same += eq ? 1u : 0u;
+        }
+    }
+    const bool leader = live && rank % cap == 0;
+    const uint64_t mask = __builtin_amdgcn_ballot_w64(leader);
+    const uint32_t lane = f % kWave, wave = f / kWave;
+    if (lane == 0) wave_leaders[wave] = __builtin_popcountll(mask);
+    __syncthreads();
+    const uint32_t record = (wave ? wave_leaders[0] : 0u) + __builtin_popcountll(mask & ((1ull << lane) - 1ull));
+    const uint32_t records = wave_leaders[0] + wave_leaders[1];
+    record_of[f] = leader ? record : 0xffffffffu;
+    __syncthreads();
+    if (live) {
+        // my record is the one opened by the route of my expert whose rank is rank - rank % cap
+        const uint32_t want = rank - rank % cap;
+        uint32_t seen = 0, rec = record;
+        if (!leader) {
+            for (uint32_t g = 0; g < f; ++g) {
+                if (sid[g] == mine) {
+                    if (seen == want) { rec = record_of[g]; break; }
+                    ++seen;
+                }
+            }
+        }
+        const uint32_t slot = rank % cap;
+        meta[264 + rec * 8 + slot] = f / selected;
+        meta[1288 + rec * 8 + slot] = f;
+        if (leader) {
+            const uint32_t members = same - rank < cap ? same - rank : cap;
+            meta[8 + rec] = mine;
+            meta[136 + rec] = members;
+            for (uint32_t k = members; k < 8; ++k) { meta[264 + rec * 8 + k] = f / selected; meta[1288 + rec * 8 + k] = f; }
+        }
+    }
+    if (f == 0) {
+        meta[0] = (hidden + 7) / 8; meta[1] = records; meta[2] = 1;
+        meta[3] = (channels + 15) / 16; meta[4] = records; meta[5] = 1;
+        meta[6] = records; meta[7] = 0;
+    }
+}
+
+}  // namespace
+
+extern "C" int tsp_grouped_routes(const uint32_t* ids, uint32_t* token_map, uint32_t* counts, uint32_t experts, uint32_t selected,
+                                  uint32_t tokens, uint32_t* error_word, void* stream) {
+    TSP_REQUIRE(experts && experts <= 512 && selected && selected <= 16 && selected <= experts && tokens && tokens <= 2048,
+                "grouped routes geometry");
+    TSP_REQUIRE(ids && token_map && counts && error_word, "null device pointer");
+    grouped_routes_kernel<<<experts, 256, 0, static_cast<hipStream_t>(stream)>>>(ids, token_map, counts, experts, selected, tokens, error_word);
+    return launch_status("grouped_routes");
+}
+
+extern "C" int tsp_grouped_tasks(const uint32_t* counts, uint32_t* tasks, uint32_t experts, uint32_t selected, uint32_t tokens,
+                                 uint32_t tile, uint32_t* error_word, void* stream) {
+    TSP_REQUIRE(experts && experts <= 512 && selected && selected <= 16 && tokens && tokens <= 2048 && tile && tile <= 256,
+                "grouped tasks geometry");
+    TSP_REQUIRE(counts && tasks && error_word, "null device pointer");
+    grouped_tasks_kernel<<<1, 512, 0, static_cast<hipStream_t>(stream)>>>(counts, tasks, experts, selected, tokens, tile, error_word);
+    return launch_status("grouped_tasks");
+}
+
+extern "C" int tsp_planar_union_build(const uint32_t* ids, uint32_t* meta, uint32_t experts, uint32_t selected, uint32_t tokens,
+                                      uint32_t hidden, uint32_t channels, uint32_t* error_word, void* stream) {
+    // Shape validity is decided on the device like the engine's kernel (it flags and zeroes the header);
+    // only what would index outside the 128-route staging is refused here.
+    TSP_REQUIRE(uint64_t(tokens) * selected <= 128 || !(tokens <= 8 && selected <= 16), "union build route bound");
+    TSP_REQUIRE(ids && meta && error_word, "null device pointer");
+    union_build_kernel<<<1, 128, 0, static_cast<hipStream_t>(stream)>>>(ids, meta, experts, selected, tokens, hidden, channels, error_word);
+    return launch_status("planar_union_build");
+}

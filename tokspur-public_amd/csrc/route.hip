@@ -1,0 +1,216 @@
+// Router top-k with softmax / sigmoid weights, the weighted mixture (combine) and SwiGLU.
+//
+// Top-k is integer-exact: k rounds of arg-max over f32 logits compared as given, exact ties to the
+// lower expert id. One 64-lane wave owns one token row and keeps the row's logits in registers
+// (lane i holds experts i, i+64, ...), so a round is a per-lane scan plus two wave reductions and
+// no barrier. Weights use accurate expf/logf; their association differs from a sequential sum but
+// they are compared to the double reference under tolerance, never bit for bit.
+#include "tsp_common.hpp"
+
+using namespace tsp;
+
+namespace {
+
+__device__ __forceinline__ float sigmoid_f(float x) {
+    if (x >= 0) return 1.0f / (1.0f + expf(-x));
+    const float e = expf(x);
+    return e / (1.0f + e);
+}
+
+__device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x))); }
+
+__device__ __forceinline__ float route_activation(float logit, float maximum, uint32_t mode, uint32_t normalize) {
+    if (!mode) return expf(logit - maximum);
+    if (normalize) return expf(-softplus_f(-logit) + softplus_f(-maximum));
+    return sigmoid_f(logit);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+    for (int m = 1; m < kWave; m <<= 1) v = fmaxf(v, __shfl_xor(v, m, kWave));
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_min(uint32_t v) {
+    for (int m = 1; m < kWave; m <<= 1) { const uint32_t o = __shfl_xor(v, m, kWave); v = o < v ? o : v; }
+    return v;
+}
+__device__ __forceinline__ float wave_sum_shfl(float v) {
+    for (int m = 1; m < kWave; m <<= 1) v += __shfl_xor(v, m, kWave);
+    return v;
+}
+
+// CAND = ceil(experts / 64) register slots per lane (8 covers 512 experts, 64 covers 4096).
+template <int CAND>
+__global__ __launch_bounds__(64) void route_rows(const float* __restrict__ logits, uint32_t* __restrict__ indices,
+                                                 float* __restrict__ weights, uint32_t experts, uint32_t selected,
+                                                 uint32_t mode, uint32_t normalize, uint32_t tokens, uint32_t* error_word) {
+    const uint32_t row = blockIdx.x, lane = threadIdx.x;
+    if (row >= tokens) return;
+    const float* row_logits = logits + uint64_t(row) * experts;
+    float cand[CAND];
+    uint32_t bad = 0;
+#pragma unroll
+    for (int k = 0; k < CAND; ++k) {
+        const uint32_t i = lane + k * kWave;
+        float v = -INFINITY;
+        if (i < experts) {
+            v = row_logits[i];
+            if (nonfinite(v)) { bad |= TSP_ERRBIT_NONFINITE; v = -INFINITY; }
+        }
+        cand[k] = v;
+    }
+    // chosen logit j is kept by lane j (selected <= 64)
+    float chosen_mine = 0, chosen_first = 0;
+    for (uint32_t s = 0; s < selected; ++s) {
+        float best = -INFINITY;
+        uint32_t expert = 0xffffffffu;
+#pragma unroll
+        for (int k = 0; k < CAND; ++k) {
+            const uint32_t i = lane + k * kWave;
+            if (i < experts && (cand[k] > best || (cand[k] == best && i < expert))) { best = cand[k]; expert = i; }
+        }
+        const float score = wave_max(best);
+        uint32_t chosen = wave_min(best == score ? expert : 0xffffffffu);
+        if (chosen >= experts) { bad |= TSP_ERRBIT_INDEX; chosen = 0; }
+        if (lane == 0) indices[uint64_t(row) * selected + s] = chosen;
+        const float value = nonfinite(score) ? row_logits[chosen] : score;
+        if (s == 0) chosen_first = value;
+        if (s == lane) chosen_mine = value;
+#pragma unroll
+        for (int k = 0; k < CAND; ++k) if (chosen == lane + k * kWave) cand[k] = -INFINITY;
+    }
+    const float act = lane < selected ? route_activation(chosen_mine, chosen_first, mode, normalize) : 0.0f;
+    float sum = mode ? 1.0f : 0.0f;
+    if (normalize) {
+        sum = wave_sum_shfl(act);
+    } else if (!mode) {
+        float part = 0;
+        for (uint32_t i = lane; i < experts; i += kWave) part += expf(row_logits[i] - chosen_first);
+        sum = wave_sum_shfl(part);
+    }
+    if (nonfinite(sum) || !(sum > 0.0f)) { bad |= TSP_ERRBIT_NONFINITE; sum = 1.0f; }
+    if (lane < selected) {
+        const float w = act / sum;
+        if (nonfinite(w)) bad |= TSP_ERRBIT_NONFINITE;
+        weights[uint64_t(row) * selected + lane] = w;
+    }
+    publish_error(bad, error_word);
+}
+
+struct MixtureArgs {
+    const float* experts;       // [tokens, selected, channels]
+    const float* weights;       // [tokens, selected]
+    const float* shared;        // [tokens, channels]
+    const float* shared_logit;  // [tokens]
+    float* output;
+    uint64_t output_stride_bytes;
+    uint32_t channels, selected, tokens;
+    uint32_t* error_word;
+};
+
+__global__ __launch_bounds__(256) void mixture_rows(MixtureArgs a) {
+    const uint32_t channel = blockIdx.x * blockDim.x + threadIdx.x, row = blockIdx.y;
+    uint32_t bad = 0;
+    if (channel < a.channels && row < a.tokens) {
+        const float slogit = a.shared_logit[row];
+        if (nonfinite(slogit)) {
+            bad = TSP_ERRBIT_NONFINITE;
+        } else {
+            const float* ex = a.experts + uint64_t(row) * a.selected * a.channels + channel;
+            const float* w = a.weights + uint64_t(row) * a.selected;
+            float value = a.shared[uint64_t(row) * a.channels + channel] * sigmoid_f(slogit);
+            for (uint32_t r = 0; r < a.selected; ++r) {
+                const float wr = w[r];
+                if (nonfinite(wr) || wr < 0.0f) bad = TSP_ERRBIT_NONFINITE;
+                value = __builtin_fmaf(wr, ex[uint64_t(r) * a.channels], value);
+            }
+            if (nonfinite(value)) bad = TSP_ERRBIT_NONFINITE;
+            reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(a.output) + row * a.output_stride_bytes)[channel] = value;
+        }
+    }
+    publish_error(bad, a.error_word);
+}
+
+__global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                     float* __restrict__ out, uint64_t count, float scale, uint32_t* error_word) {
+    uint32_t bad = 0;
+    for (uint64_t i = blockIdx.x * uint64_t(blockDim.x) + threadIdx.x; i < count; i += uint64_t(gridDim.x) * blockDim.x) {
+        const float x = gate[i] * scale, u = up[i];
+        float r;
+        if (nonfinite(x)) {
+            r = x;
+            bad = TSP_ERRBIT_NONFINITE;
+        } else {
+            const float activated = x * sigmoid_f(x);
+            if (nonfinite(activated) || nonfinite(u)) { bad = TSP_ERRBIT_NONFINITE; continue; }
+            r = activated * u;
+            if (nonfinite(r)) bad = TSP_ERRBIT_NONFINITE;
+        }
+        out[i] = r;
+    }
+    publish_error(bad, error_word);
+}
+
+int route_common(const float* logits, uint32_t* indices, float* weights, uint32_t experts, uint32_t selected, uint32_t tokens,
+                 uint32_t mode, int normalize, uint32_t* error_word, void* stream) {
+    TSP_REQUIRE(logits && indices && weights && error_word, "null device pointer");
+    const uint64_t lb = uint64_t(tokens) * experts * 4, ob = uint64_t(tokens) * selected * 4;
+    TSP_REQUIRE(!ranges_overlap(indices, ob, logits, lb) && !ranges_overlap(weights, ob, logits, lb) &&
+                    !ranges_overlap(indices, ob, weights, ob),
+                "router outputs overlap");
+    const auto s = static_cast<hipStream_t>(stream);
+    if (experts <= 512) route_rows<8><<<tokens, 64, 0, s>>>(logits, indices, weights, experts, selected, mode, normalize != 0, tokens, error_word);
+    else route_rows<64><<<tokens, 64, 0, s>>>(logits, indices, weights, experts, selected, mode, normalize != 0, tokens, error_word);
+    return launch_status("route");
+}
+
+}  // namespace
+
+extern "C" int tsp_route(const float* logits, uint32_t* indices, float* weights, uint32_t experts, uint32_t selected,
+                         uint32_t mode, int normalize_selected, uint32_t* error_word, void* stream) {
+    TSP_REQUIRE(experts && experts <= 4096 && selected && selected <= 64 && selected <= experts && mode <= 1,
+                "graph router shape/mode mismatch");
+    return route_common(logits, indices, weights, experts, selected, 1, mode, normalize_selected, error_word, stream);
+}
+
+extern "C" int tsp_route_batch(const float* logits, uint32_t* indices, float* weights, uint32_t experts, uint32_t selected,
+                               uint32_t tokens, uint32_t mode, int normalize_selected, uint32_t* error_word, void* stream) {
+    TSP_REQUIRE(experts && experts <= 512 && selected && selected <= 64 && selected <= experts && tokens >= 1 && tokens <= 2048 &&
+                    mode <= 1,
+                "prefill route batch geometry/mode mismatch");
+    return route_common(logits, indices, weights, experts, selected, tokens, mode, normalize_selected, error_word, stream);
+}
+
+extern "C" int tsp_mixture_batch(const float* experts, const float* weights, const float* shared, const float* shared_logit,
+                                 float* output, uint64_t output_stride_bytes, uint32_t channels, uint32_t selected, uint32_t tokens,
+                                 uint32_t* error_word, void* stream) {
+    TSP_REQUIRE(channels && channels <= 65536 && selected && selected <= 64 && tokens && tokens <= 2048 &&
+                    output_stride_bytes >= uint64_t(channels) * 4 && output_stride_bytes % 4 == 0,
+                "mixture shape mismatch");
+    TSP_REQUIRE(experts && weights && shared && shared_logit && output && error_word, "null device pointer");
+    const uint64_t out_span = uint64_t(tokens - 1) * output_stride_bytes + uint64_t(channels) * 4;
+    TSP_REQUIRE(!ranges_overlap(output, out_span, experts, uint64_t(tokens) * selected * channels * 4) &&
+                    !ranges_overlap(output, out_span, weights, uint64_t(tokens) * selected * 4) &&
+                    !ranges_overlap(output, out_span, shared, uint64_t(tokens) * channels * 4) &&
+                    !ranges_overlap(output, out_span, shared_logit, uint64_t(tokens) * 4),
+                "mixture output overlaps an input");
+    const MixtureArgs a{experts, weights, shared, shared_logit, output, output_stride_bytes, channels, selected, tokens, error_word};
+    mixture_rows<<<dim3((channels + 255) / 256, tokens), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+    return launch_status("mixture");
+}
+
+extern "C" int tsp_mixture(const float* experts, const float* weights, const float* shared, const float* shared_logit,
+                           float* output, uint32_t channels, uint32_t selected, uint32_t* error_word, void* stream) {
+    return tsp_mixture_batch(experts, weights, shared, shared_logit, output, uint64_t(channels) * 4, channels, selected, 1,
+                             error_word, stream);
+}
+
+extern "C" int tsp_swiglu(const float* gate, const float* up, float* output, uint64_t count, float scale, uint32_t* error_word,
+                          void* stream) {
+    TSP_REQUIRE(count && count <= (1ull << 32) && scale == scale && scale - scale == 0.0f, "graph SwiGLU shape/scale mismatch");
+    TSP_REQUIRE(gate && up && output && error_word, "null device pointer");
+    TSP_REQUIRE(!ranges_overlap(output, count * 4, up, count * 4) && (output == gate || !ranges_overlap(output, count * 4, gate, count * 4)),
+                "SwiGLU output overlaps an input");
+    const uint64_t blocks = (count + 255) / 256;
+    swiglu_kernel<<<uint32_t(blocks > 4096 ? 4096 : blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(gate, up, output, count, scale, error_word);
+    return launch_status("swiglu");
+}
