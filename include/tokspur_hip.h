@@ -238,6 +238,50 @@ int tsp_planar_moe_gate_up_swiglu_m8(const tsp_small_moe* moe, void* stream);
  * the above followed by y[rid, :] = Wd[e] h[rid, :]. */
 int tsp_planar_moe_routed_m8(const tsp_small_moe* moe, void* stream);
 
+/* ------------------------------------------------------------------ device: prefill dequant-GEMM (matrix cores) */
+
+/* include/tokspur/graph.hpp:750-753 `grouped_mm` with experts = selected = 1, broadcast (the dense case,
+ * kernels/grouped_mm.metal:159-243) and 859-860 `dense_mm_q8`: out[t, r] = sum_c x[t, c] * dec(W[r, c]) for
+ * `tokens` rows. Declared precision as in the engine: weights dequantised in f32 and staged as f16,
+ * activations staged as bf16-valued f16, f32 accumulation. Input rows are f32 or bf16, output rows f32 or
+ * bf16 (RNE); strides in bytes. Q4_K raw GGUF rows or planar planes, Q6_K planes. `workspace` is caller
+ * owned scratch of tsp_dense_mm_workspace_bytes(tokens, columns) bytes, 16-byte aligned. */
+uint64_t tsp_dense_mm_workspace_bytes(uint32_t tokens, uint32_t columns);
+int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matrix, uint64_t matrix_bytes, const void* input,
+                 uint64_t input_stride_bytes, int input_is_bf16, void* output, uint64_t output_stride_bytes, int output_is_bf16,
+                 uint32_t tokens, uint32_t columns, uint32_t rows, void* workspace, uint64_t workspace_bytes,
+                 uint32_t* error_word, void* stream);
+
+/* The operands of `planar_nax_grouped_moe` (include/tokspur/graph.hpp:478-481; src/graph.mm:9293-9420).
+ * x holds `tokens` f32 rows of `channels`; y (the engine's expert_down) holds tokens*selected f32 rows
+ * of `channels`, row rid = t*selected + slot. token_map [experts*tokens], counts [experts] and tasks
+ * [2 + 2*(tokens*selected/32 + experts)] are outputs with the engine's layouts (tile = 32). workspace is
+ * caller-owned scratch (the engine's nax_bf16_scratch, src/graph.mm:9100-9126) of
+ * tsp_planar_nax_workspace_bytes(...) bytes, 256-byte aligned. */
+typedef struct tsp_grouped_moe {
+    const void* pair_lo;
+    const void* pair_hi;
+    const void* down;
+    uint32_t gate_kind, up_kind, down_kind;
+    uint32_t channels, hidden, experts, selected, tokens;
+    const uint32_t* ids;
+    const float* x;
+    uint64_t x_stride_bytes;
+    float* y;
+    uint64_t y_stride_bytes;
+    uint32_t* token_map;
+    uint32_t* counts;
+    uint32_t* tasks;
+    void* workspace;
+    uint64_t workspace_bytes;
+    uint32_t* error_word;
+} tsp_grouped_moe;
+uint64_t tsp_planar_nax_workspace_bytes(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t channels, uint32_t hidden);
+/* include/tokspur/graph.hpp:478 `planar_nax_grouped_moe` (kernels/planar_moe_v3.metal:2406-2621): expert
+ * permutation -> prefix-sum tasks -> gather -> ragged grouped gate/up GEMM with fused SwiGLU (h carried as
+ * bf16) -> grouped down GEMM -> scatter of f32 rows to y[rid]. */
+int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* moe, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -296,6 +296,29 @@ class Oracle(_Lib):
         bad = C.c_uint32(0)
         return int(self.dll.orc_round_bf16_bits(C.c_float(v), C.byref(bad))), bad.value
 
+    def round_f16(self, a):
+        """float32 -> float16 (RNE) -> float32, element-wise through the C routine."""
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        out = np.empty_like(a)
+        f = self.dll.orc_round_f16
+        f.restype, f.argtypes = C.c_float, [C.c_float]
+        flat_in, flat_out = a.reshape(-1), out.reshape(-1)
+        for i in range(flat_in.size):
+            flat_out[i] = f(float(flat_in[i]))
+        return out
+
+    def staged_gemm(self, t, matrix, columns, x, rows_sel=None, nrows=None, stage_f16=True, threads=8):
+        """out[m][i] = sum_k half(dec(W[rows_sel[i], k])) * x[m, k] in double; x is [tokens, columns] float32."""
+        matrix = _u8(matrix)
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        sel = None if rows_sel is None else np.ascontiguousarray(rows_sel, dtype=np.uint32)
+        nsel = int(sel.size) if sel is not None else int(nrows)
+        out = np.empty((x.shape[0], nsel), dtype=np.float64)
+        _check(self.dll.orc_staged_gemm(C.c_uint32(t), _p(matrix, _u8p), C.c_uint32(columns), _p(sel, _u32p) if sel is not None else None,
+                                        C.c_uint32(nsel), _p(x, _f32p), C.c_uint64(x.shape[1]), C.c_uint32(x.shape[0]), C.c_int(bool(stage_f16)),
+                                        _p(out, _f64p), C.c_uint32(threads)))
+        return out
+
     def fixture_weights(self, t, k, r, e):
         epb, bpb = self.encoding(t)
         out = np.empty((k // epb) * bpb * r * e, dtype=np.uint8)
@@ -303,7 +326,7 @@ class Oracle(_Lib):
         return out
 
     def moe_routed_reference(self, gu_type, dn_type, gate, up, down, channels, hidden, experts, ids, tokens, selected, x,
-                             silu_f32=True, stage_bf16=False, threads=1, want_down=True):
+                             silu_f32=True, stage=0, threads=1, want_down=True):
         gate, up = _u8(gate), _u8(up)
         down = _u8(down) if down is not None else None
         ids = np.ascontiguousarray(ids, dtype=np.uint32)
@@ -314,7 +337,7 @@ class Oracle(_Lib):
         _check(self.dll.orc_moe_routed_reference(
             C.c_uint32(gu_type), C.c_uint32(dn_type), _p(gate, _u8p), _p(up, _u8p), _p(down, _u8p) if down is not None else None,
             C.c_uint32(channels), C.c_uint32(hidden), C.c_uint32(experts), _p(ids, _u32p), C.c_uint32(tokens), C.c_uint32(selected),
-            _p(x, _f32p), C.c_uint64(x.shape[-1] if x.ndim > 1 else channels), C.c_int(bool(silu_f32)), C.c_int(bool(stage_bf16)),
+            _p(x, _f32p), C.c_uint64(x.shape[-1] if x.ndim > 1 else channels), C.c_int(bool(silu_f32)), C.c_int(int(stage)),
             _p(h, _f64p), _p(y, _f64p) if y is not None else None, C.c_uint32(threads)))
         return h, y
 

@@ -781,21 +781,24 @@ static void* moe_worker(void* arg) {
     for (uint32_t rid = j->route_begin; rid < j->route_end; ++rid) {
         const uint32_t e = j->ids[rid];
         const float* x = j->input + (uint64_t)(rid / j->selected) * j->input_stride;
-        for (uint32_t c = 0; c < j->channels; ++c) xs[c] = stage(x[c], j->stage_bf16);
+        for (uint32_t c = 0; c < j->channels; ++c) xs[c] = stage(x[c], j->stage_bf16 & 1);
         for (uint32_t r = 0; r < j->hidden; ++r) {
             double dg = 0, du = 0;
             if (orc_dequantize(j->gu_type, j->gate + ((uint64_t)e * j->hidden + r) * gu_row, gu_row, wrow, j->channels)) goto done;
+            if (j->stage_bf16 & 2) for (uint32_t c = 0; c < j->channels; ++c) wrow[c] = orc_round_f16(wrow[c]);
             for (uint32_t c = 0; c < j->channels; ++c) dg += (double)wrow[c] * xs[c];
             if (orc_dequantize(j->gu_type, j->up + ((uint64_t)e * j->hidden + r) * gu_row, gu_row, wrow, j->channels)) goto done;
+            if (j->stage_bf16 & 2) for (uint32_t c = 0; c < j->channels; ++c) wrow[c] = orc_round_f16(wrow[c]);
             for (uint32_t c = 0; c < j->channels; ++c) du += (double)wrow[c] * xs[c];
             if (j->silu_f32) h[r] = silu_f32((float)dg) * (float)du;
             else { double s; orc_stable_silu(dg, &s); h[r] = s * du; }
-            if (j->stage_bf16) h[r] = stage((float)h[r], 1);
+            if (j->stage_bf16 & 1) h[r] = stage((float)h[r], 1);
             if (j->hidden_out) j->hidden_out[(uint64_t)rid * j->hidden + r] = h[r];
         }
         if (j->down && j->down_out) for (uint32_t r = 0; r < j->channels; ++r) {
             double dd = 0;
             if (orc_dequantize(j->dn_type, j->down + ((uint64_t)e * j->channels + r) * dn_row, dn_row, wrow, j->hidden)) goto done;
+            if (j->stage_bf16 & 2) for (uint32_t c = 0; c < j->hidden; ++c) wrow[c] = orc_round_f16(wrow[c]);
             for (uint32_t c = 0; c < j->hidden; ++c) dd += (double)wrow[c] * h[c];
             j->down_out[(uint64_t)rid * j->channels + r] = dd;
         }
@@ -847,4 +850,71 @@ int orc_fixture_weights(uint32_t type, uint32_t k, uint32_t r, uint32_t e, uint8
         if (type != 8) { out[at + 2] = 0x03; out[at + 3] = 0x1c; }
     }
     return ORC_OK;
+}
+
+/* ------------------------------------------------------------------------- */
+/* IEEE binary32 -> binary16 with round-to-nearest-even, returned as the float the half represents.
+ * This is the `half(value)` staging of kernels/grouped_mm.metal:214-216 and
+ * kernels/planar_moe_v3.metal:160-166. Overflow gives +-inf like the hardware conversion. */
+float orc_round_f16(float v) {
+    const uint32_t b = f32_bits(v), sign = b & 0x80000000u, mag = b & 0x7fffffffu;
+    if (mag >= 0x7f800000u) return v;                         /* inf / nan */
+    if (mag >= 0x477ff000u) return bits_f32(sign | 0x7f800000u); /* rounds to >= 65520 -> inf */
+    if (mag < 0x33000001u) return bits_f32(sign);             /* below half of the smallest subnormal (ties to even -> 0) */
+    if (mag < 0x38800000u) {                                  /* subnormal half: quantum 2^-24 */
+        const float q = bits_f32(mag) * 16777216.0f;          /* exact scaling */
+        const float r = nearbyintf(q);                        /* default rounding mode: nearest even */
+        return bits_f32(sign | f32_bits(r * 5.9604644775390625e-8f));
+    }
+    const uint32_t rounded = (mag + 0xfffu + ((mag >> 13) & 1u)) & 0xffffe000u;
+    return bits_f32(sign | rounded);
+}
+
+/* Declared-precision dense reference (tests/test_moe_mm_many_gpu.cpp:54-63 `dot(..., half)`):
+ * out[m][n] = sum_k double(half(dec(W[n,k]))) * double(x[m,k]), sequential double accumulation.
+ * `rows_sel` (may be NULL) lists which weight rows to evaluate. */
+typedef struct {
+    uint32_t type, columns, tokens, begin, end, stage_f16; uint64_t x_stride;
+    const uint8_t* matrix; const uint32_t* rows_sel; const float* x; double* out; uint32_t nsel; int status;
+} sg_job;
+
+static void* sg_worker(void* arg) {
+    sg_job* j = (sg_job*)arg;
+    uint32_t epb, bpb;
+    j->status = ORC_FORMAT_ERROR;
+    if (orc_encoding(j->type, &epb, &bpb)) return NULL;
+    const uint64_t row_bytes = (uint64_t)(j->columns / epb) * bpb;
+    float* w = (float*)malloc(sizeof(float) * j->columns);
+    if (!w) return NULL;
+    for (uint32_t i = j->begin; i < j->end; ++i) {
+        const uint32_t n = j->rows_sel ? j->rows_sel[i] : i;
+        if (orc_dequantize(j->type, j->matrix + (uint64_t)n * row_bytes, row_bytes, w, j->columns)) { free(w); return NULL; }
+        if (j->stage_f16) for (uint32_t c = 0; c < j->columns; ++c) w[c] = orc_round_f16(w[c]);
+        for (uint32_t m = 0; m < j->tokens; ++m) {
+            const float* x = j->x + (uint64_t)m * j->x_stride;
+            double sum = 0;
+            for (uint32_t c = 0; c < j->columns; ++c) sum += (double)w[c] * (double)x[c];
+            j->out[(uint64_t)m * j->nsel + i] = sum;
+        }
+    }
+    free(w);
+    j->status = ORC_OK;
+    return NULL;
+}
+
+int orc_staged_gemm(uint32_t type, const uint8_t* matrix, uint32_t columns, const uint32_t* rows_sel, uint32_t nsel,
+                    const float* x, uint64_t x_stride_floats, uint32_t tokens, int stage_f16, double* out, uint32_t threads) {
+    REQUIRE(nsel && tokens && columns);
+    if (threads < 1) threads = 1;
+    if (threads > 256) threads = 256;
+    if (threads > nsel) threads = nsel;
+    pthread_t tids[256]; sg_job jobs[256];
+    for (uint32_t t = 0; t < threads; ++t) {
+        jobs[t] = (sg_job){type, columns, tokens, (uint32_t)((uint64_t)nsel * t / threads), (uint32_t)((uint64_t)nsel * (t + 1) / threads),
+                           (uint32_t)(stage_f16 != 0), x_stride_floats, matrix, rows_sel, x, out, nsel, 0};
+        if (threads == 1 || pthread_create(&tids[t], NULL, sg_worker, &jobs[t])) { sg_worker(&jobs[t]); tids[t] = 0; }
+    }
+    int status = ORC_OK;
+    for (uint32_t t = 0; t < threads; ++t) { if (tids[t]) pthread_join(tids[t], NULL); if (jobs[t].status) status = ORC_FORMAT_ERROR; }
+    return status;
 }

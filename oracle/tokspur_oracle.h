@@ -155,6 +155,15 @@ int orc_moe_routed_reference(uint32_t gate_up_type, uint32_t down_type, const ui
                              uint64_t input_stride_floats, int silu_f32, int stage_bf16,
                              double* hidden_out, double* down_out, uint32_t threads);
 
+/* binary32 -> binary16 (RNE) -> binary32: the half staging of kernels/grouped_mm.metal:214-216. */
+float orc_round_f16(float v);
+/* Declared-precision dense reference, tests/test_moe_mm_many_gpu.cpp:54-63: weights optionally staged to
+ * half, sequential double accumulation; evaluates the weight rows listed in rows_sel (NULL = first nsel).
+ * out is [tokens][nsel]. `stage` in orc_moe_routed_reference: bit 0 = activations and h as bf16
+ * (kernels/planar_moe_v3.metal:82-94, 2406-2483), bit 1 = weights as half. */
+int orc_staged_gemm(uint32_t type, const uint8_t* matrix, uint32_t columns, const uint32_t* rows_sel, uint32_t nsel,
+                    const float* x, uint64_t x_stride_floats, uint32_t tokens, int stage_f16, double* out, uint32_t threads);
+
 /* tests/grouped_mm_fixture.hpp:10-19 — the reference tests' LCG weight fixture generator. */
 int orc_fixture_weights(uint32_t type, uint32_t k, uint32_t r, uint32_t e, uint8_t* out, uint64_t nbytes);
 

@@ -51,7 +51,7 @@ def test_route_goldens(gpu, orc):
 def test_route_batch_ids_bit_exact(gpu, orc, synth, tokens, experts, selected):
     """Configs 2 and 3: softmax, top-10 renormalised over 512 experts; Zipf-biased logits at T = 2048."""
     seed = synth.tensor_seed(3, 10 + tokens)
-    logits = synth.zipf_router_logits(seed, tokens, experts) if tokens == 2048 else synth.activations_f32(seed, (tokens, experts))
+    logits = synth.zipf_router_logits(seed, tokens, experts, scale=synth.ZIPF_BIAS_SCALE) if tokens == 2048 else synth.activations_f32(seed, (tokens, experts))
     if tokens == 33:
         logits = np.round(logits * 2) / 2  # plenty of exact ties
     ids, w = gpu.route(gpu.upload(logits), selected, 0, True, tokens=tokens)

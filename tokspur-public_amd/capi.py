@@ -380,6 +380,66 @@ def planar_moe_routed_m8(dev, w, ids, x, tokens, selected, h=None, y=None, **str
     return h, y
 
 
+class GroupedMoe(C.Structure):
+    _fields_ = [("pair_lo", C.c_void_p), ("pair_hi", C.c_void_p), ("down", C.c_void_p),
+                ("gate_kind", C.c_uint32), ("up_kind", C.c_uint32), ("down_kind", C.c_uint32),
+                ("channels", C.c_uint32), ("hidden", C.c_uint32), ("experts", C.c_uint32), ("selected", C.c_uint32),
+                ("tokens", C.c_uint32), ("ids", C.c_void_p), ("x", C.c_void_p), ("x_stride_bytes", C.c_uint64),
+                ("y", C.c_void_p), ("y_stride_bytes", C.c_uint64), ("token_map", C.c_void_p), ("counts", C.c_void_p),
+                ("tasks", C.c_void_p), ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("error_word", C.c_void_p)]
+
+
+def dense_mm_workspace_bytes(tokens, columns):
+    f = dll().tsp_dense_mm_workspace_bytes
+    f.restype = C.c_uint64
+    return f(C.c_uint32(tokens), C.c_uint32(columns))
+
+
+def planar_nax_workspace_bytes(tokens, selected, experts, channels, hidden):
+    f = dll().tsp_planar_nax_workspace_bytes
+    f.restype = C.c_uint64
+    return f(C.c_uint32(tokens), C.c_uint32(selected), C.c_uint32(experts), C.c_uint32(channels), C.c_uint32(hidden))
+
+
+def dense_mm(dev, encoding, layout, matrix, x, tokens, columns, rows, out=None, out_bf16=False, workspace=None,
+             x_stride=None, out_stride=None):
+    """x: f32 or bf16 rows. Returns out rows (f32, or bf16 bits as int16 when out_bf16)."""
+    in_bf16 = x.dtype == dev.torch.bfloat16 or x.dtype == dev.torch.int16
+    if out is None:
+        out = dev.empty((tokens, rows), "int16" if out_bf16 else "float32")
+    if workspace is None:
+        workspace = dev.empty(dense_mm_workspace_bytes(tokens, columns), "uint8")
+    xs = (columns * (2 if in_bf16 else 4)) if x_stride is None else x_stride
+    os_ = (rows * (2 if out_bf16 else 4)) if out_stride is None else out_stride
+    check(dll().tsp_dense_mm(C.c_uint32(encoding), C.c_uint32(layout), dev.ptr(matrix), C.c_uint64(dev.nbytes(matrix)), dev.ptr(x),
+                             C.c_uint64(xs), C.c_int(bool(in_bf16)), dev.ptr(out), C.c_uint64(os_), C.c_int(bool(out_bf16)),
+                             C.c_uint32(tokens), C.c_uint32(columns), C.c_uint32(rows), dev.ptr(workspace),
+                             C.c_uint64(dev.nbytes(workspace)), dev.ptr(dev.err), dev.stream()))
+    return out
+
+
+class GroupedScratch:
+    """Caller-owned outputs and scratch of planar_nax_grouped_moe for a given capacity."""
+
+    def __init__(self, dev, tokens, selected, experts, channels, hidden):
+        self.token_map = dev.zeros(experts * tokens, "int32")
+        self.counts = dev.zeros(experts, "int32")
+        self.tasks = dev.zeros(2 + 2 * (tokens * selected // 32 + experts), "int32")
+        self.workspace = dev.empty(planar_nax_workspace_bytes(tokens, selected, experts, channels, hidden), "uint8")
+
+
+def planar_nax_grouped_moe(dev, w, ids, x, tokens, selected, scratch, y=None, x_stride=None, y_stride=None):
+    y = dev.empty((tokens * selected, w.channels)) if y is None else y
+    gate_kind, up_kind = COLOC_KINDS[w.gu_type]
+    m = GroupedMoe(w.pair_lo.data_ptr(), w.pair_hi.data_ptr(), w.down.data_ptr(), gate_kind, up_kind, DOWN_KINDS[w.dn_type],
+                   w.channels, w.hidden, w.experts, selected, tokens, ids.data_ptr(), x.data_ptr(),
+                   w.channels * 4 if x_stride is None else x_stride, y.data_ptr(), w.channels * 4 if y_stride is None else y_stride,
+                   scratch.token_map.data_ptr(), scratch.counts.data_ptr(), scratch.tasks.data_ptr(), scratch.workspace.data_ptr(),
+                   dev.nbytes(scratch.workspace), dev.err.data_ptr())
+    check(dll().tsp_planar_nax_grouped_moe(C.byref(m), dev.stream()))
+    return y
+
+
 def as_u32(t):
     """Device int32 tensor -> host uint32 array."""
     return t.cpu().numpy().view(np.uint32)
