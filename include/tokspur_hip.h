@@ -72,6 +72,19 @@ const char* tsp_last_error(void);
 /* ABI revision of this header; bumped on any incompatible change. */
 uint32_t tsp_abi_version(void);
 
+/* Per-kernel timing, the engine's `configure_profiling` / `GraphProfile{KernelTiming}`
+ * (include/tokspur/graph.hpp:353-400; src/graph.mm:2669): between begin and end every kernel launched
+ * through this library is bracketed by a pair of events on its stream. tsp_profile_end waits for them,
+ * closes the window and returns one row per kernel name. Not for use while other threads launch. */
+typedef struct tsp_kernel_time {
+    char name[48];
+    uint32_t launches;
+    float total_ms;
+    float min_ms;
+} tsp_kernel_time;
+int tsp_profile_begin(void);
+int tsp_profile_end(tsp_kernel_time* rows, uint32_t capacity, uint32_t* count);
+
 /* ------------------------------------------------------------------ host: formats and layouts */
 
 /* src/gguf.cpp:21-32, 157-160 `encoding()`: block geometry of a GGUF type. */

@@ -277,12 +277,11 @@ class Device:
                                     C.c_int(bool(broadcast)), self.ptr(self.err), self.stream()))
         return y
 
-    def route(self, logits, selected, mode=0, normalize=True, tokens=None):
+    def route(self, logits, selected, mode=0, normalize=True, tokens=None, out=None):
         """logits [experts] (tokens=None: the single-row operator) or [tokens, experts]."""
         experts = logits.shape[-1]
         n = 1 if tokens is None else tokens
-        ids = self.zeros((n, selected), "int32")
-        w = self.zeros((n, selected))
+        ids, w = out if out is not None else (self.zeros((n, selected), "int32"), self.zeros((n, selected)))
         if tokens is None:
             check(dll().tsp_route(self.ptr(logits), self.ptr(ids), self.ptr(w), C.c_uint32(experts), C.c_uint32(selected), C.c_uint32(mode),
                                   C.c_int(bool(normalize)), self.ptr(self.err), self.stream()))
@@ -438,6 +437,22 @@ def planar_nax_grouped_moe(dev, w, ids, x, tokens, selected, scratch, y=None, x_
                    dev.nbytes(scratch.workspace), dev.err.data_ptr())
     check(dll().tsp_planar_nax_grouped_moe(C.byref(m), dev.stream()))
     return y
+
+
+class KernelTime(C.Structure):
+    _fields_ = [("name", C.c_char * 48), ("launches", C.c_uint32), ("total_ms", C.c_float), ("min_ms", C.c_float)]
+
+
+def profile_begin():
+    check(dll().tsp_profile_begin())
+
+
+def profile_end():
+    """{kernel name: (launches, total ms, min ms)} for every launch since profile_begin()."""
+    rows = (KernelTime * 64)()
+    n = C.c_uint32()
+    check(dll().tsp_profile_end(rows, C.c_uint32(64), C.byref(n)))
+    return {rows[i].name.decode(): (rows[i].launches, rows[i].total_ms, rows[i].min_ms) for i in range(min(n.value, 64))}
 
 
 def as_u32(t):

@@ -79,8 +79,7 @@ extern "C" int tsp_dequantize(uint32_t type, const void* blocks, uint64_t nbytes
     TSP_REQUIRE(blocks && out && error_word, "null device pointer");
     TSP_REQUIRE(!ranges_overlap(blocks, nbytes, out, nelem * 4), "dequantize output overlaps its input");
     dispatch_encoding(type, [&]<uint32_t T>() {
-        dequant_kernel<T><<<grid_for(nelem), 256, 0, static_cast<hipStream_t>(stream)>>>(
-            static_cast<const uint8_t*>(blocks), out, nelem, error_word);
+        TSP_LAUNCH("dequant", static_cast<hipStream_t>(stream), dequant_kernel<T><<<grid_for(nelem), 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const uint8_t*>(blocks), out, nelem, error_word));
     });
     return launch_status("dequantize");
 }
@@ -97,11 +96,11 @@ extern "C" int tsp_dequantize_planar(const tsp_planar_spec* spec, const void* pl
     const auto* base = static_cast<const uint8_t*>(planar);
     const auto s = static_cast<hipStream_t>(stream);
     switch (spec->source_type) {
-    case 12: dequant_planar_kernel<12><<<grid_for(nelem), 256, 0, s>>>(base, *spec, out, nelem, error_word); break;
-    case 13: dequant_planar_kernel<13><<<grid_for(nelem), 256, 0, s>>>(base, *spec, out, nelem, error_word); break;
-    case 14: dequant_planar_kernel<14><<<grid_for(nelem), 256, 0, s>>>(base, *spec, out, nelem, error_word); break;
-    case 7: dequant_planar_kernel<7><<<grid_for(nelem), 256, 0, s>>>(base, *spec, out, nelem, error_word); break;
-    default: dequant_planar_kernel<8><<<grid_for(nelem), 256, 0, s>>>(base, *spec, out, nelem, error_word); break;
+    case 12: TSP_LAUNCH("dequant_planar", s, dequant_planar_kernel<12><<<grid_for(nelem), 256, 0, s>>>(base, *spec, out, nelem, error_word)); break;
+    case 13: TSP_LAUNCH("dequant_planar", s, dequant_planar_kernel<13><<<grid_for(nelem), 256, 0, s>>>(base, *spec, out, nelem, error_word)); break;
+    case 14: TSP_LAUNCH("dequant_planar", s, dequant_planar_kernel<14><<<grid_for(nelem), 256, 0, s>>>(base, *spec, out, nelem, error_word)); break;
+    case 7: TSP_LAUNCH("dequant_planar", s, dequant_planar_kernel<7><<<grid_for(nelem), 256, 0, s>>>(base, *spec, out, nelem, error_word)); break;
+    default: TSP_LAUNCH("dequant_planar", s, dequant_planar_kernel<8><<<grid_for(nelem), 256, 0, s>>>(base, *spec, out, nelem, error_word)); break;
     }
     return launch_status("dequantize_planar");
 }

@@ -367,15 +367,16 @@ __global__ __launch_bounds__(256) void to_f16_rows(const void* __restrict__ src,
 
 template <int BKIND, int EPI, int ROWS>
 int launch(const GemmArgs& a, uint32_t col_tiles, uint32_t tasks, hipStream_t s) {
-    gemm_kernel<BKIND, EPI, ROWS><<<dim3(col_tiles, tasks), 256, 0, s>>>(a);
+    constexpr const char* name = EPI == EPI_SWIGLU ? "gemm_gate_up_swiglu" : ROWS == ROWS_TASK_SLOTS ? "gemm_down" : "gemm_dense";
+    TSP_LAUNCH(name, s, gemm_kernel<BKIND, EPI, ROWS><<<dim3(col_tiles, tasks), 256, 0, s>>>(a));
     return launch_status("dequant_gemm");
 }
 
 int convert_rows(const void* src, uint64_t stride, int from_bf16, _Float16* dst, uint32_t rows, uint32_t columns, uint32_t* err, hipStream_t s) {
     const uint64_t total = uint64_t(rows) * columns;
     const uint32_t grid = uint32_t((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
-    if (from_bf16) to_f16_rows<true><<<grid, 256, 0, s>>>(src, stride, dst, rows, columns, err);
-    else to_f16_rows<false><<<grid, 256, 0, s>>>(src, stride, dst, rows, columns, err);
+    if (from_bf16) TSP_LAUNCH("to_f16_rows", s, to_f16_rows<true><<<grid, 256, 0, s>>>(src, stride, dst, rows, columns, err));
+    else TSP_LAUNCH("to_f16_rows", s, to_f16_rows<false><<<grid, 256, 0, s>>>(src, stride, dst, rows, columns, err));
     return launch_status("to_f16_rows");
 }
 

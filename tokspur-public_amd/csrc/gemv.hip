@@ -179,8 +179,8 @@ int launch_gemv(uint32_t encoding, uint32_t layout, GemvArgs a, hipStream_t stre
 #define TSP_Q4K_CASE(N)                                                                                                   \
     if (bpr == N) {                                                                                                       \
         const dim3 grid(grid_rows((a.rows + 64 / (4 * N) - 1) / (64 / (4 * N)), 4), a.count);                             \
-        if (planar) gemv_q4k<N, true><<<grid, 256, 0, stream>>>(a);                                                       \
-        else gemv_q4k<N, false><<<grid, 256, 0, stream>>>(a);                                                             \
+        if (planar) TSP_LAUNCH("gemv_q4k", stream, gemv_q4k<N, true><<<grid, 256, 0, stream>>>(a));                                                       \
+        else TSP_LAUNCH("gemv_q4k", stream, gemv_q4k<N, false><<<grid, 256, 0, stream>>>(a));                                                             \
         return launch_status("gemv_q4k");                                                                                 \
     }
         TSP_Q4K_CASE(2) TSP_Q4K_CASE(4) TSP_Q4K_CASE(8) TSP_Q4K_CASE(16)
@@ -188,7 +188,7 @@ int launch_gemv(uint32_t encoding, uint32_t layout, GemvArgs a, hipStream_t stre
     }
     TSP_REQUIRE(layout == TSP_LAYOUT_GGUF, "no GEMV kernel for this layout/encoding/shape");
     const dim3 grid(grid_rows(a.rows, 4), a.count);
-    const bool ok = dispatch_encoding(encoding, [&]<uint32_t T>() { gemv_generic<T><<<grid, 256, 0, stream>>>(a); });
+    const bool ok = dispatch_encoding(encoding, [&]<uint32_t T>() { TSP_LAUNCH("gemv_generic", stream, gemv_generic<T><<<grid, 256, 0, stream>>>(a)); });
     TSP_REQUIRE(ok, "no owned numerical decoder for this encoding");
     return launch_status("gemv_generic");
 }

@@ -161,7 +161,7 @@ extern "C" int tsp_grouped_routes(const uint32_t* ids, uint32_t* token_map, uint
     TSP_REQUIRE(experts && experts <= 512 && selected && selected <= 16 && selected <= experts && tokens && tokens <= 2048,
                 "grouped routes geometry");
     TSP_REQUIRE(ids && token_map && counts && error_word, "null device pointer");
-    grouped_routes_kernel<<<experts, 256, 0, static_cast<hipStream_t>(stream)>>>(ids, token_map, counts, experts, selected, tokens, error_word);
+    TSP_LAUNCH("grouped_routes", static_cast<hipStream_t>(stream), grouped_routes_kernel<<<experts, 256, 0, static_cast<hipStream_t>(stream)>>>(ids, token_map, counts, experts, selected, tokens, error_word));
     return launch_status("grouped_routes");
 }
 
@@ -170,7 +170,7 @@ extern "C" int tsp_grouped_tasks(const uint32_t* counts, uint32_t* tasks, uint32
     TSP_REQUIRE(experts && experts <= 512 && selected && selected <= 16 && tokens && tokens <= 2048 && tile && tile <= 256,
                 "grouped tasks geometry");
     TSP_REQUIRE(counts && tasks && error_word, "null device pointer");
-    grouped_tasks_kernel<<<1, 512, 0, static_cast<hipStream_t>(stream)>>>(counts, tasks, experts, selected, tokens, tile, error_word);
+    TSP_LAUNCH("grouped_tasks", static_cast<hipStream_t>(stream), grouped_tasks_kernel<<<1, 512, 0, static_cast<hipStream_t>(stream)>>>(counts, tasks, experts, selected, tokens, tile, error_word));
     return launch_status("grouped_tasks");
 }
 
@@ -180,6 +180,6 @@ extern "C" int tsp_planar_union_build(const uint32_t* ids, uint32_t* meta, uint3
     // only what would index outside the 128-route staging is refused here.
     TSP_REQUIRE(uint64_t(tokens) * selected <= 128 || !(tokens <= 8 && selected <= 16), "union build route bound");
     TSP_REQUIRE(ids && meta && error_word, "null device pointer");
-    union_build_kernel<<<1, 128, 0, static_cast<hipStream_t>(stream)>>>(ids, meta, experts, selected, tokens, hidden, channels, error_word);
+    TSP_LAUNCH("union_build", static_cast<hipStream_t>(stream), union_build_kernel<<<1, 128, 0, static_cast<hipStream_t>(stream)>>>(ids, meta, experts, selected, tokens, hidden, channels, error_word));
     return launch_status("planar_union_build");
 }

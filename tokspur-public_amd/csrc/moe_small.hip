@@ -418,8 +418,8 @@ int launch_gate_up(const SmallMoeArgs& a, hipStream_t s) {
         const dim3 grid(a.tokens == 1 ? (steps + 3) / 4 : steps, records);
 #define TSP_GU(N)                                                             \
     if (bpr == N) {                                                           \
-        if (a.tokens == 1) gate_up_q4k<N, 1><<<grid, 256, 0, s>>>(a);         \
-        else gate_up_q4k<N, 2><<<grid, 256, 0, s>>>(a);                       \
+        if (a.tokens == 1) TSP_LAUNCH("gate_up_q4k", s, gate_up_q4k<N, 1><<<grid, 256, 0, s>>>(a));         \
+        else TSP_LAUNCH("gate_up_q4k", s, gate_up_q4k<N, 2><<<grid, 256, 0, s>>>(a));                       \
         return launch_status("gate_up_q4k");                                  \
     }
         TSP_GU(2) TSP_GU(4) TSP_GU(8)
@@ -427,9 +427,9 @@ int launch_gate_up(const SmallMoeArgs& a, hipStream_t s) {
     }
     const dim3 grid((a.hidden + 3) / 4, records);
     switch (a.gu.source_type) {
-    case 12: gate_up_generic<12><<<grid, 256, 0, s>>>(a); break;
-    case 13: gate_up_generic<13><<<grid, 256, 0, s>>>(a); break;
-    default: gate_up_generic<8><<<grid, 256, 0, s>>>(a); break;
+    case 12: TSP_LAUNCH("gate_up_generic", s, gate_up_generic<12><<<grid, 256, 0, s>>>(a)); break;
+    case 13: TSP_LAUNCH("gate_up_generic", s, gate_up_generic<13><<<grid, 256, 0, s>>>(a)); break;
+    default: TSP_LAUNCH("gate_up_generic", s, gate_up_generic<8><<<grid, 256, 0, s>>>(a)); break;
     }
     return launch_status("gate_up_generic");
 }
@@ -444,8 +444,8 @@ int launch_down(const SmallMoeArgs& a, hipStream_t s) {
         const dim3 grid(a.tokens == 1 ? (steps + 3) / 4 : steps, records);
 #define TSP_DN(N)                                                          \
     if (bpr == N) {                                                        \
-        if (a.tokens == 1) down_q6k<N, 1><<<grid, 256, 0, s>>>(a);         \
-        else down_q6k<N, 2><<<grid, 256, 0, s>>>(a);                       \
+        if (a.tokens == 1) TSP_LAUNCH("down_q6k", s, down_q6k<N, 1><<<grid, 256, 0, s>>>(a));         \
+        else TSP_LAUNCH("down_q6k", s, down_q6k<N, 2><<<grid, 256, 0, s>>>(a));                       \
         return launch_status("down_q6k");                                  \
     }
         TSP_DN(1) TSP_DN(2) TSP_DN(4)
@@ -453,9 +453,9 @@ int launch_down(const SmallMoeArgs& a, hipStream_t s) {
     }
     const dim3 grid((a.channels + 3) / 4, records);
     switch (a.dn.source_type) {
-    case 7: down_generic<7><<<grid, 256, 0, s>>>(a); break;
-    case 8: down_generic<8><<<grid, 256, 0, s>>>(a); break;
-    default: down_generic<14><<<grid, 256, 0, s>>>(a); break;
+    case 7: TSP_LAUNCH("down_generic", s, down_generic<7><<<grid, 256, 0, s>>>(a)); break;
+    case 8: TSP_LAUNCH("down_generic", s, down_generic<8><<<grid, 256, 0, s>>>(a)); break;
+    default: TSP_LAUNCH("down_generic", s, down_generic<14><<<grid, 256, 0, s>>>(a)); break;
     }
     return launch_status("down_generic");
 }

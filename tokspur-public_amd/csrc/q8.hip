@@ -149,7 +149,7 @@ template <int M>
 int launch(uint32_t layout, const Q8Args& a, hipStream_t stream) {
     const uint32_t grid = (a.rows + 3) / 4 > 4096 ? 4096 : (a.rows + 3) / 4;
     if (layout == TSP_LAYOUT_Q8_LANES_V1) {
-        q8_lanes<M><<<grid, 256, 0, stream>>>(a);
+        TSP_LAUNCH("q8_lanes", stream, q8_lanes<M><<<grid, 256, 0, stream>>>(a));
         return launch_status("q8_lanes");
     }
     const uint64_t lds_bytes = uint64_t(M) * (a.columns + 4) * 4;
@@ -159,10 +159,10 @@ int launch(uint32_t layout, const Q8Args& a, hipStream_t stream) {
             TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_flat<M>), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
             raised[M] = true;
         }
-        q8_flat<M><<<grid, 256, lds_bytes, stream>>>(a);
+        TSP_LAUNCH("q8_flat", stream, q8_flat<M><<<grid, 256, lds_bytes, stream>>>(a));
         return launch_status("q8_flat");
     }
-    q8_blocks<M><<<grid, 256, 0, stream>>>(a);
+    TSP_LAUNCH("q8_blocks", stream, q8_blocks<M><<<grid, 256, 0, stream>>>(a));
     return launch_status("q8_blocks");
 }
 

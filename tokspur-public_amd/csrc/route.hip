@@ -158,8 +158,8 @@ int route_common(const float* logits, uint32_t* indices, float* weights, uint32_
                     !ranges_overlap(indices, ob, weights, ob),
                 "router outputs overlap");
     const auto s = static_cast<hipStream_t>(stream);
-    if (experts <= 512) route_rows<8><<<tokens, 64, 0, s>>>(logits, indices, weights, experts, selected, mode, normalize != 0, tokens, error_word);
-    else route_rows<64><<<tokens, 64, 0, s>>>(logits, indices, weights, experts, selected, mode, normalize != 0, tokens, error_word);
+    if (experts <= 512) TSP_LAUNCH("route_rows", s, route_rows<8><<<tokens, 64, 0, s>>>(logits, indices, weights, experts, selected, mode, normalize != 0, tokens, error_word));
+    else TSP_LAUNCH("route_rows", s, route_rows<64><<<tokens, 64, 0, s>>>(logits, indices, weights, experts, selected, mode, normalize != 0, tokens, error_word));
     return launch_status("route");
 }
 
@@ -194,7 +194,7 @@ extern "C" int tsp_mixture_batch(const float* experts, const float* weights, con
                     !ranges_overlap(output, out_span, shared_logit, uint64_t(tokens) * 4),
                 "mixture output overlaps an input");
     const MixtureArgs a{experts, weights, shared, shared_logit, output, output_stride_bytes, channels, selected, tokens, error_word};
-    mixture_rows<<<dim3((channels + 255) / 256, tokens), 256, 0, static_cast<hipStream_t>(stream)>>>(a);
+    TSP_LAUNCH("mixture_rows", static_cast<hipStream_t>(stream), mixture_rows<<<dim3((channels + 255) / 256, tokens), 256, 0, static_cast<hipStream_t>(stream)>>>(a));
     return launch_status("mixture");
 }
 
@@ -211,6 +211,6 @@ extern "C" int tsp_swiglu(const float* gate, const float* up, float* output, uin
     TSP_REQUIRE(!ranges_overlap(output, count * 4, up, count * 4) && (output == gate || !ranges_overlap(output, count * 4, gate, count * 4)),
                 "SwiGLU output overlaps an input");
     const uint64_t blocks = (count + 255) / 256;
-    swiglu_kernel<<<uint32_t(blocks > 4096 ? 4096 : blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(gate, up, output, count, scale, error_word);
+    TSP_LAUNCH("swiglu", static_cast<hipStream_t>(stream), swiglu_kernel<<<uint32_t(blocks > 4096 ? 4096 : blocks), 256, 0, static_cast<hipStream_t>(stream)>>>(gate, up, output, count, scale, error_word));
     return launch_status("swiglu");
 }

@@ -36,6 +36,25 @@ inline bool ranges_overlap(const void* a, uint64_t an, const void* b, uint64_t b
 
 int launch_status(const char* what);
 
+// Per-kernel timing (the engine's GraphProfile / KernelTiming, include/tokspur/graph.hpp:353-400): while a
+// profile window is open every launch is bracketed by a pair of events on its own stream.
+struct KernelTimer {
+    KernelTimer(const char* name, hipStream_t stream);
+    ~KernelTimer();
+    int slot;
+    hipStream_t stream;
+};
+extern bool g_profiling;
+#define TSP_LAUNCH(name, stream, ...)                                  \
+    do {                                                               \
+        if (::tsp::g_profiling) {                                      \
+            ::tsp::KernelTimer timer_(name, stream);                   \
+            __VA_ARGS__;                                               \
+        } else {                                                       \
+            __VA_ARGS__;                                               \
+        }                                                              \
+    } while (0)
+
 struct Encoding { uint32_t id, elements, bytes; };
 const Encoding* find_encoding(uint32_t type);
 
