@@ -308,14 +308,15 @@ class Oracle(_Lib):
         return out
 
     def staged_gemm(self, t, matrix, columns, x, rows_sel=None, nrows=None, stage_f16=True, threads=8):
-        """out[m][i] = sum_k half(dec(W[rows_sel[i], k])) * x[m, k] in double; x is [tokens, columns] float32."""
+        """out[m][i] = sum_k stage(dec(W[rows_sel[i], k])) * x[m, k] in double; x is [tokens, columns] float32.
+        stage_f16: False/0 none, True/1 round weights to half, 2 Q6_K integer products as half (scale d kept f32)."""
         matrix = _u8(matrix)
         x = np.ascontiguousarray(x, dtype=np.float32)
         sel = None if rows_sel is None else np.ascontiguousarray(rows_sel, dtype=np.uint32)
         nsel = int(sel.size) if sel is not None else int(nrows)
         out = np.empty((x.shape[0], nsel), dtype=np.float64)
         _check(self.dll.orc_staged_gemm(C.c_uint32(t), _p(matrix, _u8p), C.c_uint32(columns), _p(sel, _u32p) if sel is not None else None,
-                                        C.c_uint32(nsel), _p(x, _f32p), C.c_uint64(x.shape[1]), C.c_uint32(x.shape[0]), C.c_int(bool(stage_f16)),
+                                        C.c_uint32(nsel), _p(x, _f32p), C.c_uint64(x.shape[1]), C.c_uint32(x.shape[0]), C.c_int(int(stage_f16)),
                                         _p(out, _f64p), C.c_uint32(threads)))
         return out
 

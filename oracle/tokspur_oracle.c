@@ -768,6 +768,20 @@ typedef struct {
 static float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 static float stage(float v, int bf16) { uint32_t bad = 0; return bf16 ? orc_bf16_to_f32(orc_round_bf16_bits(v, &bad)) : v; }
 
+/* Matrix-core staging of one dequantised Q6_K row (210-byte blocks, f16 d at byte 208): the kernel multiplies the
+ * integer product sc * (q - 32) as a half and applies d in f32, so w becomes d * half(w / d). w / d is that integer
+ * exactly (w = d * sc * (q - 32) has at most 24 significant bits); only magnitudes above 2048 can round. */
+static void stage_q6k_products(const uint8_t* row, float* w, uint32_t columns) {
+    for (uint32_t b = 0; b < columns / 256; ++b) {
+        const uint8_t* blk = row + (uint64_t)b * 210;
+        const double d = orc_binary16((uint16_t)(blk[208] | (blk[209] << 8)));
+        for (uint32_t i = 0; i < 256; ++i) {
+            float* v = w + b * 256 + i;
+            if (d != 0 && isfinite(d)) *v = (float)(d * (double)orc_round_f16((float)((double)*v / d)));
+        }
+    }
+}
+
 static void* moe_worker(void* arg) {
     moe_job* j = (moe_job*)arg;
     uint32_t gu_epb, gu_bpb, dn_epb, dn_bpb;
@@ -781,7 +795,7 @@ static void* moe_worker(void* arg) {
     for (uint32_t rid = j->route_begin; rid < j->route_end; ++rid) {
         const uint32_t e = j->ids[rid];
         const float* x = j->input + (uint64_t)(rid / j->selected) * j->input_stride;
-        for (uint32_t c = 0; c < j->channels; ++c) xs[c] = stage(x[c], j->stage_bf16 & 1);
+        for (uint32_t c = 0; c < j->channels; ++c) xs[c] = stage(x[c], j->stage_bf16 & 5);
         for (uint32_t r = 0; r < j->hidden; ++r) {
             double dg = 0, du = 0;
             if (orc_dequantize(j->gu_type, j->gate + ((uint64_t)e * j->hidden + r) * gu_row, gu_row, wrow, j->channels)) goto done;
@@ -793,12 +807,14 @@ static void* moe_worker(void* arg) {
             if (j->silu_f32) h[r] = silu_f32((float)dg) * (float)du;
             else { double s; orc_stable_silu(dg, &s); h[r] = s * du; }
             if (j->stage_bf16 & 1) h[r] = stage((float)h[r], 1);
+            if (j->stage_bf16 & 4) h[r] = 256.0 * (double)orc_round_f16((float)h[r] * 0.00390625f);
             if (j->hidden_out) j->hidden_out[(uint64_t)rid * j->hidden + r] = h[r];
         }
         if (j->down && j->down_out) for (uint32_t r = 0; r < j->channels; ++r) {
             double dd = 0;
             if (orc_dequantize(j->dn_type, j->down + ((uint64_t)e * j->channels + r) * dn_row, dn_row, wrow, j->hidden)) goto done;
             if (j->stage_bf16 & 2) for (uint32_t c = 0; c < j->hidden; ++c) wrow[c] = orc_round_f16(wrow[c]);
+            if ((j->stage_bf16 & 8) && j->dn_type == 14) stage_q6k_products(j->down + ((uint64_t)e * j->channels + r) * dn_row, wrow, j->hidden);
             for (uint32_t c = 0; c < j->hidden; ++c) dd += (double)wrow[c] * h[c];
             j->down_out[(uint64_t)rid * j->channels + r] = dd;
         }
@@ -889,7 +905,8 @@ static void* sg_worker(void* arg) {
     for (uint32_t i = j->begin; i < j->end; ++i) {
         const uint32_t n = j->rows_sel ? j->rows_sel[i] : i;
         if (orc_dequantize(j->type, j->matrix + (uint64_t)n * row_bytes, row_bytes, w, j->columns)) { free(w); return NULL; }
-        if (j->stage_f16) for (uint32_t c = 0; c < j->columns; ++c) w[c] = orc_round_f16(w[c]);
+        if (j->stage_f16 == 1) for (uint32_t c = 0; c < j->columns; ++c) w[c] = orc_round_f16(w[c]);
+        if (j->stage_f16 == 2 && j->type == 14) stage_q6k_products(j->matrix + (uint64_t)n * row_bytes, w, j->columns);
         for (uint32_t m = 0; m < j->tokens; ++m) {
             const float* x = j->x + (uint64_t)m * j->x_stride;
             double sum = 0;
@@ -911,7 +928,7 @@ int orc_staged_gemm(uint32_t type, const uint8_t* matrix, uint32_t columns, cons
     pthread_t tids[256]; sg_job jobs[256];
     for (uint32_t t = 0; t < threads; ++t) {
         jobs[t] = (sg_job){type, columns, tokens, (uint32_t)((uint64_t)nsel * t / threads), (uint32_t)((uint64_t)nsel * (t + 1) / threads),
-                           (uint32_t)(stage_f16 != 0), x_stride_floats, matrix, rows_sel, x, out, nsel, 0};
+                           (uint32_t)stage_f16, x_stride_floats, matrix, rows_sel, x, out, nsel, 0};
         if (threads == 1 || pthread_create(&tids[t], NULL, sg_worker, &jobs[t])) { sg_worker(&jobs[t]); tids[t] = 0; }
     }
     int status = ORC_OK;

@@ -157,10 +157,15 @@ int orc_moe_routed_reference(uint32_t gate_up_type, uint32_t down_type, const ui
 
 /* binary32 -> binary16 (RNE) -> binary32: the half staging of kernels/grouped_mm.metal:214-216. */
 float orc_round_f16(float v);
-/* Declared-precision dense reference, tests/test_moe_mm_many_gpu.cpp:54-63: weights optionally staged to
- * half, sequential double accumulation; evaluates the weight rows listed in rows_sel (NULL = first nsel).
- * out is [tokens][nsel]. `stage` in orc_moe_routed_reference: bit 0 = activations and h as bf16
- * (kernels/planar_moe_v3.metal:82-94, 2406-2483), bit 1 = weights as half. */
+/* Declared-precision dense reference, tests/test_moe_mm_many_gpu.cpp:54-63: weights optionally staged,
+ * sequential double accumulation; evaluates the weight rows listed in rows_sel (NULL = first nsel).
+ * out is [tokens][nsel]. stage_f16: 0 = f32-dequantised weights, 1 = weights rounded to half
+ * (kernels/grouped_mm.metal:214-216), 2 = Q6_K rows as d * half(sc * (q - 32)), the staging of a matrix-core
+ * kernel that multiplies the integer products as halves and applies d in f32 (no reference counterpart;
+ * other types unchanged).
+ * `stage` in orc_moe_routed_reference: bit 0 = activations and h as bf16 (kernels/planar_moe_v3.metal:82-94,
+ * 2406-2483), bit 1 = weights as half, bit 2 = activations as bf16 and h as 256 * half(h / 256), bit 3 = Q6_K
+ * down rows staged as under stage_f16 = 2. Bits 2 and 3 describe the HIP kernels, not the reference. */
 int orc_staged_gemm(uint32_t type, const uint8_t* matrix, uint32_t columns, const uint32_t* rows_sel, uint32_t nsel,
                     const float* x, uint64_t x_stride_floats, uint32_t tokens, int stage_f16, double* out, uint32_t threads);
 

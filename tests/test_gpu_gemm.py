@@ -4,8 +4,17 @@ The engine's declared precision for this path is half-staged weights, bf16 activ
 accumulation (kernels/grouped_mm.metal:214-216, kernels/planar_moe_v3.metal:118-166, 2406-2483), and
 its tests compare against a CPU reference staged the same way (native/tests/test_moe_mm_many_gpu.cpp:
 54-63, limits scaled <= 1e-3 and rel-L2 <= 5e-3) plus NMSE <= 2e-3 against the unstaged reference
-(native/tests/test_planar_pack_v3.cpp:693). Both comparisons are made here; the bar for the staged
-comparison is max error <= 2e-3 in units of the row's scale."""
+(native/tests/test_planar_pack_v3.cpp:693).
+
+The kernels here keep the bf16 activations but do not round weights to half: they multiply the exact
+integer factors of the K-quant formats (sc*q for Q4_K, sc*(q-32) for Q6_K) as halves on the matrix cores
+and apply the block scales in f32; the intermediate h travels as the half nearest to h/256 (11 bits,
+bf16 in the engine). That is the kernels' declared precision, restated by the oracle's stage bits 2|3
+(= 12) and stage_f16 = 2, and the tight comparisons (<= 2e-5 of the row's scale for one GEMM) are made
+against it. Q4_K products always fit a half exactly; Q6_K products above 2048 lose their lowest bit.
+The f32-dequantised reference fed the same bf16 activations has to be met within the path's tolerance
+of 2e-3 (max error in units of the row's scale); the half-staged reference itself sits ~2e-3 away from
+that one, so against it the engine's own rel-L2 limit of 5e-3 applies."""
 import numpy as np
 import pytest
 
@@ -40,7 +49,7 @@ def test_dense_mm_q4k(gpu, tsp, orc, synth, layout, tokens, rows, cols):
         dw, lay = gpu.upload(w), tsp.LAYOUT_GGUF
     got = tsp.dense_mm(gpu, 12, lay, dw, gpu.upload(x), tokens, cols, rows).cpu().numpy()
     assert gpu.error() == 0
-    assert max_rel_error(got, want) <= 2e-5 and nmse(got, unstaged) <= 1e-6
+    assert max_rel_error(got, unstaged) <= 2e-5 and rel_l2(got, want) <= 5e-3 and nmse(got, unstaged) <= 1e-9
     # bf16 activations in, bf16 rows out (configuration 1's interface): same values, one more rounding
     xb = gpu.upload(synth.bf16_bits(x))
     got_b = bf16_to_f32(tsp.dense_mm(gpu, 12, lay, dw, xb, tokens, cols, rows, out_bf16=True).cpu().numpy()).reshape(tokens, rows)
@@ -53,7 +62,13 @@ def test_dense_mm_q6k_planar(gpu, tsp, orc, synth):
     x = synth.round_bf16(synth.activations_f32(2101, (tokens, cols)))
     dw = gpu.upload(tsp.pack_expert(tsp.make_expert_spec(14, cols, rows), w))
     got = tsp.dense_mm(gpu, 14, tsp.LAYOUT_PLANAR_V3, dw, gpu.upload(x), tokens, cols, rows).cpu().numpy()
-    assert gpu.error() == 0 and max_rel_error(got, orc.staged_gemm(14, w, cols, x, nrows=rows)) <= 2e-5
+    assert gpu.error() == 0
+    # Q6_K integer products sc * (q - 32) above 2048 (|sc| > 64) lose their lowest bit in f16: a 2^-12 step on those
+    # weights only, against 2^-11 on every weight for half staging. The synthetic scales span all of int8.
+    assert max_rel_error(got, orc.staged_gemm(14, w, cols, x, nrows=rows, stage_f16=2)) <= 2e-5
+    exact = orc.staged_gemm(14, w, cols, x, nrows=rows, stage_f16=False)
+    assert max_rel_error(got, exact) <= 2e-3 and nmse(got, exact) <= 1e-6
+    assert rel_l2(got, orc.staged_gemm(14, w, cols, x, nrows=rows)) <= 5e-3
 
 
 def test_dense_mm_strides_canaries_and_errors(gpu, tsp, orc, synth):
@@ -64,7 +79,7 @@ def test_dense_mm_strides_canaries_and_errors(gpu, tsp, orc, synth):
     dw = gpu.upload(w)
     tsp.dense_mm(gpu, 12, tsp.LAYOUT_GGUF, dw, gpu.upload(x), tokens, cols, rows, out=out, x_stride=(cols + 32) * 4, out_stride=(rows + 8) * 4)
     out = out.cpu().numpy()
-    want = orc.staged_gemm(12, w, cols, np.ascontiguousarray(x[:, :cols]), nrows=rows)
+    want = orc.staged_gemm(12, w, cols, np.ascontiguousarray(x[:, :cols]), nrows=rows, stage_f16=False)
     assert max_rel_error(out[:, :rows], want) <= 2e-5 and (out[:, rows:] == -9.0).all() and gpu.error() == 0
     bad = x.copy()
     bad[3, 7] = np.inf
@@ -100,9 +115,9 @@ def test_config1_dense_q4k_gemm(gpu, tsp, orc, synth, tokens):
     want = orc.staged_gemm(12, w, cols, x, rows_sel=sel)
     unstaged = orc.staged_gemm(12, w, cols, x, rows_sel=sel, stage_f16=False)
     err, err_un = max_rel_error(out_f32[:, sel], want), max_rel_error(out_f32[:, sel], unstaged)
-    print(f"config1 M={tokens}: max rel error vs declared-precision reference {err:.2e}, vs unstaged {err_un:.2e}, "
-          f"NMSE vs unstaged {nmse(out_f32[:, sel], unstaged):.2e}")
-    assert err <= 2e-5 and err_un <= 2e-3
+    print(f"config1 M={tokens}: max rel error vs half-staged reference {err:.2e}, vs f32-dequantised {err_un:.2e}, "
+          f"NMSE vs f32-dequantised {nmse(out_f32[:, sel], unstaged):.2e}")
+    assert err_un <= 2e-5 and rel_l2(out_f32[:, sel], want) <= 5e-3
     # every column: permuting the token rows permutes the output rows bit for bit (tiles hold no row state)
     perm = np.random.default_rng(1).permutation(tokens)
     out_p = tsp.dense_mm(gpu, 12, tsp.LAYOUT_GGUF, dw, gpu.upload(x[perm]), tokens, cols, rows).cpu().numpy()
@@ -174,9 +189,38 @@ def test_grouped_moe_reference_cases(gpu, tsp, orc, synth, n):
         assert np.array_equal(tm[e, :counts[e]], want_map.reshape(experts, n)[e, :counts[e]])
     assert np.array_equal(scratch.tasks.cpu().numpy().view(np.uint32), orc.grouped_tasks(want_counts, experts, selected, n, 32)[0])
     _, staged = orc.moe_routed_reference(12, 14, gate, up, down, channels, hidden, experts, ids, n, selected, x, stage=3, threads=8)
+    _, declared = orc.moe_routed_reference(12, 14, gate, up, down, channels, hidden, experts, ids, n, selected, x, stage=12, threads=8)
     _, plain = orc.moe_routed_reference(12, 14, gate, up, down, channels, hidden, experts, ids, n, selected, x, stage=0, threads=8)
     assert nmse(y, plain) <= 2e-3
-    assert max_rel_error(y, staged) <= 2e-3 and rel_l2(y, staged) <= 5e-3
+    assert rel_l2(y, staged) <= 5e-3
+    # the kernels' own staging: what is left is f32 accumulation and the odd tie of half(h / 256) falling the other way
+    assert max_rel_error(y, declared) <= 2e-3 and nmse(y, declared) <= 1e-7
+
+
+def test_grouped_moe_exact_when_products_fit_half(gpu, tsp, orc, synth):
+    """With Q6_K sub-scales in [-64, 63] every integer product sc * (q - 32) is exact in f16, and the grouped MoE
+    then differs from the f32-dequantised CPU reference (bf16 x, h as half(h / 256)) only by f32 accumulation and
+    rare ties of h. Against the reference that rounds nothing, the 2^-12 step of the carried h on heavy-tailed
+    rows (|h| up to 7 sigma here) already costs up to ~3e-3 of the row scale at the worst output (1.8e-2 with the
+    engine's bf16 h), so that comparison is made in NMSE, as the engine's own test does."""
+    channels, hidden, experts, selected, n = 512, 256, 8, 4, 150
+    gate = synth.matrix(12, 3201, hidden * experts, channels)
+    up = synth.matrix(12, 3202, hidden * experts, channels)
+    down = synth.matrix(14, 3203, channels * experts, hidden).reshape(-1, 210).copy()
+    down[:, 192:208] = (down[:, 192:208].view(np.int8) >> 1).view(np.uint8)
+    down = down.reshape(-1)
+    w = tsp.PlanarMoeWeights(gpu, 12, 14, channels, hidden, experts, gate, up, down)
+    rng = np.random.default_rng(5)
+    ids = np.stack([rng.permutation(experts)[:selected] for _ in range(n)]).astype(np.uint32).reshape(-1)
+    x = synth.round_bf16(synth.activations_f32(3204, (n, channels)))
+    scratch = tsp.GroupedScratch(gpu, n, selected, experts, channels, hidden)
+    y = tsp.planar_nax_grouped_moe(gpu, w, gpu.upload(ids), gpu.upload(x), n, selected, scratch).cpu().numpy()
+    assert gpu.error() == 0
+    _, carried = orc.moe_routed_reference(12, 14, gate, up, down, channels, hidden, experts, ids, n, selected, x, stage=4, threads=8)
+    _, plain = orc.moe_routed_reference(12, 14, gate, up, down, channels, hidden, experts, ids, n, selected, x, stage=0, threads=8)
+    print(f"exact-products case: max rel error {max_rel_error(y, carried):.2e} (NMSE {nmse(y, carried):.2e}), "
+          f"vs unrounded reference {max_rel_error(y, plain):.2e}")
+    assert max_rel_error(y, carried) <= 2e-3 and nmse(y, carried) <= 1e-7 and nmse(y, plain) <= 1e-6
 
 
 def test_grouped_moe_sticky_errors(gpu, tsp, synth):
@@ -231,7 +275,7 @@ def test_config3_moe_grouped_prefill(gpu, tsp, orc, synth):
     for e in range(E):
         assert np.array_equal(tm[e, :counts[e]], want_map.reshape(E, T)[e, :counts[e]])
     assert np.array_equal(scratch.tasks.cpu().numpy().view(np.uint32), orc.grouped_tasks(want_counts, E, S, T, 32)[0])
-    # sampled routes: the busiest expert's first and last rows (several 128-row tasks), a mid-size and the smallest experts
+    # sampled routes: the busiest expert's first and last rows (several tasks apart), a mid-size and the smallest experts
     order = np.argsort(-want_counts.astype(np.int64))
     picks = []
     busiest = int(order[0])
@@ -243,11 +287,14 @@ def test_config3_moe_grouped_prefill(gpu, tsp, orc, synth):
     sub_ids = ids[picks]
     sub_x = x[picks // S]
     _, staged = orc.moe_routed_reference(12, 14, gate, up, down, C, H, E, sub_ids, len(picks), 1, sub_x, stage=3, threads=8)
+    _, declared = orc.moe_routed_reference(12, 14, gate, up, down, C, H, E, sub_ids, len(picks), 1, sub_x, stage=12, threads=8)
     _, plain = orc.moe_routed_reference(12, 14, gate, up, down, C, H, E, sub_ids, len(picks), 1, sub_x, stage=0, threads=8)
     got = y[gpu.upload(picks.astype(np.int64))].cpu().numpy()
-    print(f"config3: {len(picks)} sampled routes, max rel error vs declared-precision reference {max_rel_error(got, staged):.2e}, "
-          f"NMSE vs unstaged {nmse(got, plain):.2e}")
-    assert max_rel_error(got, staged) <= 2e-3 and rel_l2(got, staged) <= 5e-3 and nmse(got, plain) <= 2e-3
+    print(f"config3: {len(picks)} sampled routes, max rel error vs half-staged reference {max_rel_error(got, staged):.2e}, "
+          f"vs the kernels' declared precision {max_rel_error(got, declared):.2e}, vs unrounded reference "
+          f"{max_rel_error(got, plain):.2e} (NMSE {nmse(got, plain):.2e})")
+    assert rel_l2(got, staged) <= 5e-3 and nmse(got, plain) <= 2e-3
+    assert max_rel_error(got, declared) <= 2e-3 and nmse(got, declared) <= 1e-7 and nmse(got, plain) <= 1e-6
     # weighted combine over the routes (shared expert left out here: it is the dense GEMM of config 1 at M = 2048)
     out = gpu.mixture(y, wts_d, gpu.zeros((T, C)), gpu.zeros(T), C, S, tokens=T).cpu().numpy()
     yh, wh = y.cpu().numpy().reshape(T, S, C), wts_d.cpu().numpy()

@@ -1,21 +1,32 @@
 // Prefill dequant-GEMM on the matrix cores: out[m, n] = sum_k x[m, k] * dec(W[n, k]).
 //
-// Operands follow the engine's declared precision for this path: weights are dequantised in f32
-// ((d*sc)*q - dmin*mn, d*sc*(q-32)) and rounded once to f16, activations are bf16 values carried
-// as f16 (exact for every bf16 inside the f16 range), products accumulate in f32 inside
-// v_mfma_f32_32x32x16_f16.
+// K-quant weights factor as  w = d * (sc * q) - dmin * mn  (Q4_K) and  w = d * (sc * (q - 32))  (Q6_K)
+// with a per-super-block f16 factor d (dmin) and small INTEGER products sc*q (< 2^10) resp. sc*(q-32)
+// (< 2^12). The kernel feeds those integers, which are exact in f16, to v_mfma_f32_32x32x16_f16 against
+// the activations (bf16 values carried as f16, exact), accumulates one super-block of 256 columns in a
+// scratch accumulator, and applies d once per super-block on the f32 accumulators:
 //
-// One workgroup = 4 waves = one task (<= 128 activation rows of one expert, or one 128-row slab of a
-// dense matrix) x 256 weight rows. Each wave owns 64 weight rows (two 32-wide MFMA column tiles) and
-// all 128 activation rows (four row tiles): 8 accumulator tiles = 128 VGPRs.
-//   * Weights never touch LDS: a lane loads the 8-byte nibble runs of ITS weight row straight into
-//     the MFMA B-fragment layout (lane = (row % 32, k-half)), so every weight is dequantised exactly
-//     once per task and there is no cross-wave traffic for B.
-//   * Activations are shared by the four waves: staged global -> LDS (padded rows, conflict-free
-//     16-byte reads), double buffered, one barrier per K step.
-//   * For gate/up the two column tiles of a wave are the gate rows and the up rows of the same 32
-//     hidden units, so SwiGLU is an element-wise epilogue on accumulator registers.
+//     out += d[n, b] * sum_{k in b} x[m, k] * (sc*q)[n, k]   -   sum_s (dmin*mn)[n, b, s] * Sx[m, b, s]
+//
+// The second term (Q4_K minima) is one more MFMA per super-block against the per-sub-block activation
+// sums Sx, carried as a hi+lo pair of f16. Nothing is rounded to f16 that is not an exact integer (Q6_K
+// products above 2048 round to even, a 2^-12 relative step), so results track the f32-dequantised
+// reference to f32-accumulation accuracy, and unpacking costs ~1.4 VALU operations per weight (mask,
+// byte permute into 1024+q, one packed f16 fma) instead of ~3 for convert + f32 fma + f16 round.
+//
+// One workgroup = 4 waves = one task (<= 64 activation rows of one expert, or one 64-row slab of a dense
+// matrix) x 256 weight rows. Each wave owns 64 weight rows (two 32-wide MFMA column tiles) and all 64
+// activation rows (two row tiles).
+//   * Weights never touch LDS: a lane loads 16 contiguous bytes of ITS weight row per K step straight
+//     into MFMA B-fragment order (lane = (row % 32, k-half)); every weight is unpacked once per task.
+//   * Activations are shared by the four waves: staged global -> LDS (padded rows), double buffered, one
+//     LDS-only barrier per K step; the next step's weight bytes and activation slab are requested before
+//     the current step is unpacked.
+//   * For gate/up the two column tiles of a wave are the gate rows and the up rows of the same 32 hidden
+//     units, so SwiGLU is an element-wise epilogue on accumulator registers.
 #include "decode.hpp"
+
+#include <type_traits>
 
 using namespace tsp;
 
@@ -23,23 +34,25 @@ namespace {
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 enum BKind : int { B_Q4K_RAW = 0, B_Q4K_PLANAR = 1, B_Q6K_PLANAR = 2 };
 enum Epilogue : int { EPI_F32 = 0, EPI_BF16 = 1, EPI_SWIGLU = 2 };
 enum Rows : int { ROWS_DENSE = 0, ROWS_GATHER_TOKENS = 1, ROWS_TASK_SLOTS = 2 };
 
-constexpr int kTaskRows = 128;
+constexpr int kTaskRows = 64;
+constexpr int kRowTiles = kTaskRows / 32;
 
 struct GemmArgs {
     const _Float16* a;        // activation rows, a_stride halfs apart
     uint64_t a_stride;
+    const _Float16* sx;       // per row, per super-block: 8 sub-block sums (hi) + 8 residuals (lo); Q4_K only
     const uint8_t* w0;        // dense matrix / pair_lo / down experts
     const uint8_t* w1;        // pair_hi
-    tsp_planar_spec spec;     // planar layouts (per expert); raw: columns/rows only
+    tsp_planar_spec spec;     // planar layouts (per expert)
     uint32_t experts;
-    const uint32_t* tasks;    // grouped: [2 + 2*bound] with 128-row tiles
+    const uint32_t* tasks;    // grouped: [2 + 2*bound] with kTaskRows-row tiles
     const uint32_t* counts;
     const uint32_t* token_map;
     const uint32_t* ids;
@@ -51,120 +64,143 @@ struct GemmArgs {
     uint32_t* error_word;
 };
 
-__device__ __forceinline__ f16x2 pack2(float a, float b) {
-    const f32x2 v = {a, b};
-    return __builtin_convertvector(v, f16x2);  // RNE
-}
+// Workgroup barrier that waits for this wave's LDS traffic only. __syncthreads() also drains every outstanding
+// global load, which would serialise the prefetch of the next K step behind the barrier.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-__device__ __forceinline__ f16x8 pack8(const float* w) {
-    const f16x2 p0 = pack2(w[0], w[1]), p1 = pack2(w[2], w[3]), p2 = pack2(w[4], w[5]), p3 = pack2(w[6], w[7]);
+__device__ __forceinline__ f16x2 as_h2(uint32_t bits) { return __builtin_bit_cast(f16x2, bits); }
+__device__ __forceinline__ uint32_t as_u32(f16x2 v) { return __builtin_bit_cast(uint32_t, v); }
+__device__ __forceinline__ f16x2 splat(float v) { const _Float16 h = _Float16(v); return f16x2{h, h}; }
+// one rounding per lane: the products below are only exact as fused multiply-adds
+__device__ __forceinline__ f16x2 fma2(f16x2 a, f16x2 b, f16x2 c) { return __builtin_elementwise_fma(a, b, c); }
+
+// Bytes (b0, b1) resp. (b2, b3) of `codes` into the low bytes of two f16 lanes whose high bytes are `hi`.
+__device__ __forceinline__ uint32_t spread01(uint32_t codes, uint32_t hi) { return __builtin_amdgcn_perm(hi, codes, 0x04010400u); }
+__device__ __forceinline__ uint32_t spread23(uint32_t codes, uint32_t hi) { return __builtin_amdgcn_perm(hi, codes, 0x04030402u); }
+
+// Eight codes 0..15 (one per byte of c0, c1) times the integer scale: (1024 + q) * sc - 1024 * sc, exact in f16.
+__device__ __forceinline__ f16x8 scaled8_q4(uint32_t c0, uint32_t c1, f16x2 sc, f16x2 bias) {
+    constexpr uint32_t K = 0x64646464u;  // 0x64xx = 1024 + xx
+    const f16x2 p0 = fma2(as_h2(spread01(c0, K)), sc, bias), p1 = fma2(as_h2(spread23(c0, K)), sc, bias);
+    const f16x2 p2 = fma2(as_h2(spread01(c1, K)), sc, bias), p3 = fma2(as_h2(spread23(c1, K)), sc, bias);
     return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
 }
 
-__device__ __forceinline__ float ubq(uint32_t w, int i) { return float((w >> (8 * i)) & 0xffu); }
-
-// Eight weights dl*q - ml from the byte-wise codes of two dwords.
-__device__ __forceinline__ f16x8 affine8(uint32_t c0, uint32_t c1, float dl, float neg_ml) {
-    float w[8];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { w[i] = __builtin_fmaf(ubq(c0, i), dl, neg_ml); w[4 + i] = __builtin_fmaf(ubq(c1, i), dl, neg_ml); }
-    return pack8(w);
+// Eight codes 0..63: 0x5400 | (c << 4) = 64 + c, so (64 + c) * sc - 96 * sc = (c - 32) * sc.
+__device__ __forceinline__ f16x8 scaled8_q6(uint32_t c0, uint32_t c1, f16x2 sc, f16x2 bias) {
+    constexpr uint32_t K = 0x54005400u;
+    const f16x2 p0 = fma2(as_h2((spread01(c0, 0) << 4) | K), sc, bias), p1 = fma2(as_h2((spread23(c0, 0) << 4) | K), sc, bias);
+    const f16x2 p2 = fma2(as_h2((spread01(c1, 0) << 4) | K), sc, bias), p3 = fma2(as_h2((spread23(c1, 0) << 4) | K), sc, bias);
+    return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
 }
 
-// ---------------------------------------------------------------- B fragments, one K step, one weight row
-// Q4_K: K step = 64 (one nibble pair = sub-blocks 2p and 2p+1); four k16 fragments.
+// ---------------------------------------------------------------- Q4_K operands
+struct HdrQ4 { uint32_t sc[2], mn[2]; float d, dmin; };  // eight 6-bit scales and minima, one per byte
+
 template <int BKIND>
-__device__ __forceinline__ void load_b_q4k(const uint8_t* base, const tsp_planar_spec& s, uint64_t row, uint32_t bpr, uint32_t step,
-                                           uint32_t khalf, uint2& lo8, uint2& hi8, float& dl_a, float& nml_a, float& dl_b, float& nml_b) {
+__device__ __forceinline__ HdrQ4 load_hdr_q4k(const uint8_t* base, const tsp_planar_spec& s, uint64_t row, uint32_t bpr, uint32_t b) {
+    const uint64_t blk = row * bpr + b;
+    HdrQ4 h;
+    if constexpr (BKIND == B_Q4K_PLANAR) {
+        const uint4 sm = *reinterpret_cast<const uint4*>(base + s.sm_offset + blk * 16);
+        const uint32_t dm = *reinterpret_cast<const uint32_t*>(base + s.dm_offset + blk * 4);
+        h.sc[0] = sm.x; h.sc[1] = sm.y; h.mn[0] = sm.z; h.mn[1] = sm.w;
+        h.d = half_bits_to_float(dm & 0xffffu); h.dmin = half_bits_to_float(dm >> 16);
+    } else {
+        const uint4 g = *reinterpret_cast<const uint4*>(base + blk * 144);
+        h.d = half_bits_to_float(g.x & 0xffffu); h.dmin = half_bits_to_float(g.x >> 16);
+        // 12 packed bytes -> one byte per value: sub-blocks 0..3 are the low six bits of bytes 0..7, sub-blocks
+        // 4..7 take four bits from bytes 8..11 and two from the top of bytes 0..7
+        h.sc[0] = g.y & 0x3f3f3f3fu;
+        h.mn[0] = g.z & 0x3f3f3f3fu;
+        h.sc[1] = (g.w & 0x0f0f0f0fu) | ((g.y >> 2) & 0x30303030u);
+        h.mn[1] = ((g.w >> 4) & 0x0f0f0f0fu) | ((g.z >> 2) & 0x30303030u);
+    }
+    return h;
+}
+
+template <int BKIND>
+__device__ __forceinline__ u32x4 load_raw_q4k(const uint8_t* base, const tsp_planar_spec& s, uint64_t row, uint32_t bpr, uint32_t step,
+                                              uint32_t khalf) {
     const uint32_t b = step / 4, p = step % 4;
     const uint64_t blk = row * bpr + b;
-    float d, dmin;
-    uint32_t sc_a, sc_b, mn_a, mn_b;
-    if constexpr (BKIND == B_Q4K_PLANAR) {
-        const uint8_t* qs = base + s.qs_offset + blk * 128 + p * 32 + khalf * 8;
-        lo8 = *reinterpret_cast<const uint2*>(qs);
-        hi8 = *reinterpret_cast<const uint2*>(qs + 16);
-        const uint8_t* sm = base + s.sm_offset + blk * 16 + p * 2;
-        const uint32_t sc = *reinterpret_cast<const uint16_t*>(sm), mn = *reinterpret_cast<const uint16_t*>(sm + 8);
-        const uint32_t dm = *reinterpret_cast<const uint32_t*>(base + s.dm_offset + blk * 4);
-        sc_a = sc & 0xffu; sc_b = sc >> 8; mn_a = mn & 0xffu; mn_b = mn >> 8;
-        d = half_bits_to_float(dm & 0xffffu); dmin = half_bits_to_float(dm >> 16);
-    } else {
-        const uint8_t* block = base + blk * 144;
-        const uint4 hdr = *reinterpret_cast<const uint4*>(block);
-        lo8 = *reinterpret_cast<const uint2*>(block + 16 + p * 32 + khalf * 8);
-        hi8 = *reinterpret_cast<const uint2*>(block + 32 + p * 32 + khalf * 8);
-        d = half_bits_to_float(hdr.x & 0xffffu); dmin = half_bits_to_float(hdr.x >> 16);
-        const uint32_t sh = (p & 1u) * 16u;
-        const uint32_t s2 = (hdr.y >> sh) & 0xffffu, m2 = (hdr.z >> sh) & 0xffffu, e2 = (hdr.w >> sh) & 0xffffu;
-        if (p < 2) {
-            sc_a = s2 & 63u; sc_b = (s2 >> 8) & 63u; mn_a = m2 & 63u; mn_b = (m2 >> 8) & 63u;
-        } else {
-            sc_a = (e2 & 15u) | (((s2 >> 6) & 3u) << 4);
-            sc_b = ((e2 >> 8) & 15u) | (((s2 >> 14) & 3u) << 4);
-            mn_a = ((e2 >> 4) & 15u) | (((m2 >> 6) & 3u) << 4);
-            mn_b = ((e2 >> 12) & 15u) | (((m2 >> 14) & 3u) << 4);
-        }
-    }
-    dl_a = d * float(sc_a); dl_b = d * float(sc_b);
-    nml_a = -(dmin * float(mn_a)); nml_b = -(dmin * float(mn_b));
+    const uint8_t* qs = BKIND == B_Q4K_PLANAR ? base + s.qs_offset + blk * 128 + p * 32 + khalf * 16
+                                               : base + blk * 144 + 16 + p * 32 + khalf * 16;
+    return *reinterpret_cast<const u32x4*>(qs);
 }
 
-__device__ __forceinline__ void frags_q4k(uint2 lo8, uint2 hi8, float dl_a, float nml_a, float dl_b, float nml_b, f16x8 frag[4]) {
+// Fragments of pair P: bytes 16h..16h+15 of the 32-byte pair; low nibbles are sub-block 2P, high nibbles 2P+1.
+// Fragment f covers activation columns (f/2)*32 + 16h + (f%2)*8 .. +8 of the 64-column slab.
+template <int P>
+__device__ __forceinline__ void frags_q4k(const u32x4& raw, const HdrQ4& h, f16x8 frag[4]) {
     constexpr uint32_t M4 = 0x0f0f0f0fu;
-    frag[0] = affine8(lo8.x & M4, lo8.y & M4, dl_a, nml_a);
-    frag[1] = affine8(hi8.x & M4, hi8.y & M4, dl_a, nml_a);
-    frag[2] = affine8((lo8.x >> 4) & M4, (lo8.y >> 4) & M4, dl_b, nml_b);
-    frag[3] = affine8((hi8.x >> 4) & M4, (hi8.y >> 4) & M4, dl_b, nml_b);
+    const uint32_t sc_a = (h.sc[P >> 1] >> ((P & 1) * 16)) & 0xffu, sc_b = (h.sc[P >> 1] >> ((P & 1) * 16 + 8)) & 0xffu;
+    const f16x2 sa = splat(float(sc_a)), sb = splat(float(sc_b));
+    const f16x2 ba = sa * splat(-1024.0f), bb = sb * splat(-1024.0f);
+    frag[0] = scaled8_q4(raw[0] & M4, raw[1] & M4, sa, ba);
+    frag[1] = scaled8_q4(raw[2] & M4, raw[3] & M4, sa, ba);
+    frag[2] = scaled8_q4((raw[0] >> 4) & M4, (raw[1] >> 4) & M4, sb, bb);
+    frag[3] = scaled8_q4((raw[2] >> 4) & M4, (raw[3] >> 4) & M4, sb, bb);
 }
 
-// Q6_K planes: K step = 128 (one section); eight k16 fragments. For k16 step s the eight weights of a
-// lane are elements q*32 + j .. +7 of the section with q = s/2, j = (s%2)*16 + khalf*8.
-struct RawQ6 { uint2 la[2], lb[2], qh[2]; float d; const uint8_t* sc; };
+// B operand of the minima term: the eight integer minima, the same in both k-halves (hi and lo sums).
+__device__ __forceinline__ f16x8 minima_frag(const HdrQ4& h) {
+    constexpr uint32_t K = 0x64646464u;
+    const f16x2 one = splat(1.0f), off = splat(-1024.0f);
+    const f16x2 p0 = fma2(as_h2(spread01(h.mn[0], K)), one, off), p1 = fma2(as_h2(spread23(h.mn[0], K)), one, off);
+    const f16x2 p2 = fma2(as_h2(spread01(h.mn[1], K)), one, off), p3 = fma2(as_h2(spread23(h.mn[1], K)), one, off);
+    return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
 
-__device__ __forceinline__ void load_b_q6k(const uint8_t* base, const tsp_planar_spec& s, uint64_t row, uint32_t bpr, uint32_t step,
-                                           uint32_t khalf, RawQ6& r) {
-    const uint32_t b = step / 2, sec = step % 2;
+// ---------------------------------------------------------------- Q6_K operands (planes ql / qh / sc / d)
+struct RawQ6 { u32x4 la, lb, qh; uint32_t sc[2]; float d; };
+
+__device__ __forceinline__ void load_raw_q6k(const uint8_t* base, const tsp_planar_spec& s, uint64_t row, uint32_t bpr, uint32_t step,
+                                             uint32_t khalf, RawQ6& r) {
+    const uint32_t b = step / 2, sec = step % 2;  // step counts 128-column sections
     const uint64_t blk = row * bpr + b;
-#pragma unroll
-    for (int par = 0; par < 2; ++par) {
-        const uint32_t j = par * 16 + khalf * 8;
-        const uint8_t* ql = base + s.qs_offset + blk * 128 + sec * 64 + j;
-        r.la[par] = *reinterpret_cast<const uint2*>(ql);
-        r.lb[par] = *reinterpret_cast<const uint2*>(ql + 32);
-        r.qh[par] = *reinterpret_cast<const uint2*>(base + s.qh_offset + blk * 64 + sec * 32 + j);
-    }
+    const uint8_t* ql = base + s.qs_offset + blk * 128 + sec * 64 + khalf * 16;
+    r.la = *reinterpret_cast<const u32x4*>(ql);
+    r.lb = *reinterpret_cast<const u32x4*>(ql + 32);
+    r.qh = *reinterpret_cast<const u32x4*>(base + s.qh_offset + blk * 64 + sec * 32 + khalf * 16);
+    const uint2 sc8 = *reinterpret_cast<const uint2*>(base + s.sm_offset + blk * 16 + sec * 8);
+    r.sc[0] = sc8.x; r.sc[1] = sc8.y;
     r.d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(base + s.dm_offset + blk * 2));
-    r.sc = base + s.sm_offset + blk * 16 + sec * 8;
 }
 
-__device__ __forceinline__ void frags_q6k(const RawQ6& r, f16x8 frag[8]) {
+// Quarter Q of the section (elements Q*32 .. Q*32+31): this lane's 16 bytes are elements Q*32 + 16h + 0..15, all in
+// the 16-weight group 2Q + h. Fragment f covers activation columns Q*32 + 16h + f*8 .. +8 of the section.
+template <int Q>
+__device__ __forceinline__ void frags_q6k(const RawQ6& r, uint32_t khalf, f16x8 frag[2]) {
     constexpr uint32_t M4 = 0x0f0f0f0fu, M2 = 0x30303030u;
+    const u32x4& l = (Q & 1) ? r.lb : r.la;
+    const uint32_t g = 2 * Q + khalf;
+    const int sc = int(int8_t((r.sc[g >> 2] >> ((g & 3) * 8)) & 0xffu));
+    const f16x2 s2 = splat(float(sc)), bias = s2 * splat(-96.0f);
+    uint32_t c[4];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-#pragma unroll
-        for (int par = 0; par < 2; ++par) {
-            const uint2 l = (q & 1) ? r.lb[par] : r.la[par];
-            const uint2 h = r.qh[par];
-            uint32_t c0, c1;
-            if (q < 2) { c0 = l.x & M4; c1 = l.y & M4; } else { c0 = (l.x >> 4) & M4; c1 = (l.y >> 4) & M4; }
-            const int shift = 4 - 2 * q;  // bits 2q..2q+1 of qh move to bits 4..5
-            c0 |= (shift >= 0 ? h.x << shift : h.x >> -shift) & M2;
-            c1 |= (shift >= 0 ? h.y << shift : h.y >> -shift) & M2;
-            // sub-scale of the 16-weight group: element / 16 = q*2 + par within the section
-            const float ds = r.d * float(int(int8_t(r.sc[q * 2 + par])));
-            frag[q * 2 + par] = affine8(c0, c1, ds, -32.0f * ds);
-        }
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t low = Q < 2 ? l[i] & M4 : (l[i] >> 4) & M4;
+        uint32_t high;  // bits 2Q..2Q+1 of qh move to bits 4..5 of the code
+        if constexpr (Q == 0) high = r.qh[i] << 4;
+        else if constexpr (Q == 1) high = r.qh[i] << 2;
+        else if constexpr (Q == 2) high = r.qh[i];
+        else high = r.qh[i] >> 2;
+        c[i] = low | (high & M2);
     }
+    frag[0] = scaled8_q6(c[0], c[1], s2, bias);
+    frag[1] = scaled8_q6(c[2], c[3], s2, bias);
 }
 
 // ---------------------------------------------------------------- the kernel
 template <int BKIND, int EPI, int ROWS>
-__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
-    constexpr int KSTEP = BKIND == B_Q6K_PLANAR ? 128 : 64;
-    constexpr int NFRAG = KSTEP / 16;
-    constexpr int LDA = KSTEP + 8;  // halfs per staged row: 16 bytes of padding keeps 16-byte reads conflict free
+__global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two workgroups per CU: <= 256 registers per lane
+    constexpr bool Q6 = BKIND == B_Q6K_PLANAR;
+    constexpr int KSTEP = 64;
+    constexpr int LDA = KSTEP + 8;   // halfs per staged row: 16 bytes of padding spreads 16-byte reads over the banks
+    constexpr int LDS_SX = 24;       // halfs per staged row of activation sums (16 used)
     __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][kTaskRows * LDA];
+    __shared__ __attribute__((aligned(16))) _Float16 lds_sx[2][Q6 ? 8 : kTaskRows * LDS_SX];
     __shared__ uint32_t row_src[kTaskRows];
     __shared__ uint32_t row_dst[kTaskRows];
     __shared__ uint32_t task_bad;
@@ -181,7 +217,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
         const uint32_t row0 = task * kTaskRows;
         if (row0 >= a.m) return;
         nrows = a.m - row0 < kTaskRows ? a.m - row0 : kTaskRows;
-        if (tid < kTaskRows) { row_src[tid] = row0 + tid; row_dst[tid] = row0 + tid; }
+        if (tid < kTaskRows) { row_src[tid] = row0 + (tid < nrows ? tid : 0); row_dst[tid] = row0 + tid; }
     } else {
         const uint32_t bound = a.tokens * a.selected / kTaskRows + a.experts;
         const uint32_t live = a.tasks[0];
@@ -199,12 +235,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
         }
         nrows = count - start < kTaskRows ? count - start : kTaskRows;
         if (tid < kTaskRows) {
-            uint32_t rid = 0xffffffffu;
-            if (tid < nrows) {
-                rid = a.token_map[uint64_t(expert) * a.tokens + start + tid];
-                if (rid >= a.tokens * a.selected || a.ids[rid] != expert) { rid = 0xffffffffu; task_bad = 1; }
-            }
-            row_src[tid] = ROWS == ROWS_GATHER_TOKENS ? (rid == 0xffffffffu ? 0xffffffffu : rid / a.selected) : task * kTaskRows + tid;
+            // rows past the task's end re-read its first row: their accumulators are never stored
+            uint32_t rid = a.token_map[uint64_t(expert) * a.tokens + start + (tid < nrows ? tid : 0)];
+            if (rid >= a.tokens * a.selected || a.ids[rid] != expert) { rid = 0xffffffffu; task_bad = 1; }
+            row_src[tid] = ROWS == ROWS_GATHER_TOKENS ? (rid == 0xffffffffu ? 0 : rid / a.selected) : task * kTaskRows + (tid < nrows ? tid : 0);
             row_dst[tid] = ROWS == ROWS_GATHER_TOKENS ? task * kTaskRows + tid : rid;
         }
     }
@@ -238,72 +272,179 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
     const uint32_t bpr = a.k / 256;
     const uint32_t ksteps = a.k / KSTEP;
 
-    f32x16 acc[4][2];
+    f32x16 acc[kRowTiles][2], blk[kRowTiles][2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kRowTiles; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // ---- activation staging: thread t copies (KSTEP*2/2) bytes of row t/2
-    constexpr int SEG = KSTEP / 2;  // halfs per thread per step
-    const uint32_t st_row = tid / 2, st_seg = tid % 2;
-    const uint32_t src_row = row_src[st_row];
-    const bool st_live = st_row < nrows && src_row != 0xffffffffu;
-    const _Float16* st_src = a.a + uint64_t(st_live ? src_row : 0) * a.a_stride + st_seg * SEG;
-    uint4 stage[SEG / 8];
+    // ---- activation staging: thread t copies KSTEP/4 halfs of row t/4 per step, global -> registers -> LDS
+    constexpr int SEG = KSTEP / 4;
+    const uint32_t st_row = tid / 4, st_seg = tid % 4;
+    const _Float16* st_src = a.a + uint64_t(row_src[st_row]) * a.a_stride + st_seg * SEG;
+    u32x4 stage0{}, stage1{};  // named registers: an array here is kept in scratch memory
     auto fetch_a = [&](uint32_t step) {
-#pragma unroll
-        for (int i = 0; i < SEG / 8; ++i)
-            stage[i] = st_live ? *reinterpret_cast<const uint4*>(st_src + uint64_t(step) * KSTEP + i * 8) : uint4{0, 0, 0, 0};
+        const u32x4* src = reinterpret_cast<const u32x4*>(st_src + uint64_t(step) * KSTEP);
+        stage0 = src[0];
+        stage1 = src[1];
     };
     auto store_a = [&](int buf) {
+        u32x4* dst = reinterpret_cast<u32x4*>(&lds_a[buf][st_row * LDA + st_seg * SEG]);
+        dst[0] = stage0;
+        dst[1] = stage1;
+    };
+    // activation sums of one super-block: 64 rows x 32 bytes, threads 0..127 copy 16 bytes each
+    const uint32_t sx_row = (tid / 2) % kTaskRows, sx_seg = tid % 2;
+    uint4 sx_stage{};
+    auto fetch_sx = [&](uint32_t b) {
+        if constexpr (!Q6) {
+            if (tid < 2 * kTaskRows) sx_stage = *reinterpret_cast<const uint4*>(a.sx + (uint64_t(row_src[sx_row]) * bpr + b) * 16 + sx_seg * 8);
+        }
+    };
+    auto store_sx = [&](int buf) {
+        if constexpr (!Q6) {
+            if (tid < 2 * kTaskRows) *reinterpret_cast<uint4*>(&lds_sx[buf][sx_row * LDS_SX + sx_seg * 8]) = sx_stage;
+        }
+    };
+    // one k16 MFMA per (row tile, column tile); `first` starts the super-block accumulator from zero
+    auto mfma = [&](int buf, int k0, const f16x8& b0, const f16x8& b1, bool first) {
 #pragma unroll
-        for (int i = 0; i < SEG / 8; ++i) *reinterpret_cast<uint4*>(&lds_a[buf][st_row * LDA + st_seg * SEG + i * 8]) = stage[i];
+        for (int i = 0; i < kRowTiles; ++i) {
+            if (i < mt_live) {
+                const f16x8 af = *reinterpret_cast<const f16x8*>(&lds_a[buf][(i * 32 + col) * LDA + k0]);
+                if (first) {
+                    const f32x16 zero{};
+                    blk[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b0, zero, 0, 0, 0);
+                    blk[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b1, zero, 0, 0, 0);
+                } else {
+                    blk[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b0, blk[i][0], 0, 0, 0);
+                    blk[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b1, blk[i][1], 0, 0, 0);
+                }
+            }
+        }
+    };
+    auto fold = [&](float d0, float d1) {  // acc += d * blk at the end of a super-block
+#pragma unroll
+        for (int i = 0; i < kRowTiles; ++i) {
+            if (i < mt_live) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    acc[i][0][v] = __builtin_fmaf(d0, blk[i][0][v], acc[i][0][v]);
+                    acc[i][1][v] = __builtin_fmaf(d1, blk[i][1][v], acc[i][1][v]);
+                }
+            }
+        }
     };
 
     fetch_a(0);
     store_a(0);
-    for (uint32_t step = 0; step < ksteps; ++step) {
-        const int buf = step & 1;
-        if (step + 1 < ksteps) fetch_a(step + 1);
-        f16x8 bfrag[2][NFRAG];
-        if constexpr (BKIND == B_Q6K_PLANAR) {
+    if constexpr (Q6) {
+        RawQ6 cur[2], nxt[2];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                RawQ6 raw;
-                load_b_q6k(wbase[j], a.spec, wrow[j], bpr, step, khalf, raw);
-                frags_q6k(raw, bfrag[j]);
-            }
-        } else {
+        for (int j = 0; j < 2; ++j) load_raw_q6k(wbase[j], a.spec, wrow[j], bpr, 0, khalf, cur[j]);
+        // K step H of a super-block: section H/2 (128 columns, one set of weight bytes), quarters 2*(H%2) and +1
+        auto half_step = [&](uint32_t step, auto h_tag) {
+            constexpr int H = decltype(h_tag)::value;
+            const int buf = H & 1;
+            const bool more = step + 1 < ksteps;
+            if (more) {
+                fetch_a(step + 1);
+                if (H & 1) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                uint2 lo8, hi8;
-                float dl_a, nml_a, dl_b, nml_b;
-                load_b_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, step, khalf, lo8, hi8, dl_a, nml_a, dl_b, nml_b);
-                frags_q4k(lo8, hi8, dl_a, nml_a, dl_b, nml_b, bfrag[j]);
-            }
-        }
-        __syncthreads();  // lds_a[buf] is complete; every wave has left lds_a[buf ^ 1]
-#pragma unroll
-        for (int f = 0; f < NFRAG; ++f) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if (i < mt_live) {
-                    const f16x8 afrag = *reinterpret_cast<const f16x8*>(&lds_a[buf][(i * 32 + col) * LDA + f * 16 + khalf * 8]);
-                    acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afrag, bfrag[0][f], acc[i][0], 0, 0, 0);
-                    acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afrag, bfrag[1][f], acc[i][1], 0, 0, 0);
+                    for (int j = 0; j < 2; ++j) load_raw_q6k(wbase[j], a.spec, wrow[j], bpr, (step + 1) / 2, khalf, nxt[j]);
                 }
             }
+            auto quarter = [&](auto q_tag) {
+                constexpr int Q = decltype(q_tag)::value;
+                f16x8 f0[2], f1[2];
+                frags_q6k<Q>(cur[0], khalf, f0);
+                frags_q6k<Q>(cur[1], khalf, f1);
+                if (Q % 2 == 0) lds_barrier();  // lds_a[buf] is complete; every wave has left lds_a[buf ^ 1]
+                mfma(buf, (Q % 2) * 32 + khalf * 16, f0[0], f1[0], H == 0 && Q == 0);
+                mfma(buf, (Q % 2) * 32 + khalf * 16 + 8, f0[1], f1[1], false);
+            };
+            quarter(std::integral_constant<int, 2 * (H % 2)>{});
+            quarter(std::integral_constant<int, 2 * (H % 2) + 1>{});
+            if (H == 3) fold(cur[0].d, cur[1].d);
+            if (more) {
+                store_a(buf ^ 1);
+                if (H & 1) { cur[0] = nxt[0]; cur[1] = nxt[1]; }
+            }
+        };
+        for (uint32_t b = 0; b < bpr; ++b) {
+            half_step(b * 4 + 0, std::integral_constant<int, 0>{});
+            half_step(b * 4 + 1, std::integral_constant<int, 1>{});
+            half_step(b * 4 + 2, std::integral_constant<int, 2>{});
+            half_step(b * 4 + 3, std::integral_constant<int, 3>{});
         }
-        if (step + 1 < ksteps) store_a(buf ^ 1);
+    } else {
+        HdrQ4 hdr[2], hdr_next[2];
+        u32x4 cur[2], nxt[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            hdr[j] = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, 0);
+            cur[j] = load_raw_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, 0, khalf);
+            hdr_next[j] = hdr[j];
+        }
+        fetch_sx(0);
+        store_sx(0);
+        auto pair_step = [&](uint32_t step, auto p_tag) {
+            constexpr int P = decltype(p_tag)::value;
+            const int buf = step & 1;
+            const uint32_t b = step / 4;
+            const bool more = step + 1 < ksteps;
+            if (more) {
+                fetch_a(step + 1);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) nxt[j] = load_raw_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, step + 1, khalf);
+                if (P == 0 && b + 1 < bpr) {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) hdr_next[j] = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, b + 1);
+                    fetch_sx(b + 1);
+                }
+            }
+            f16x8 f0[4], f1[4];
+            frags_q4k<P>(cur[0], hdr[0], f0);
+            frags_q4k<P>(cur[1], hdr[1], f1);
+            lds_barrier();  // lds_a[buf] (and at P == 0 lds_sx[b & 1]) is complete; every wave has left the other buffer
+#pragma unroll
+            for (int f = 0; f < 4; ++f) mfma(buf, (f / 2) * 32 + khalf * 16 + (f % 2) * 8, f0[f], f1[f], P == 0 && f == 0);
+            if (P == 3) {
+                fold(hdr[0].d, hdr[1].d);
+                // minima: acc -= dmin * sum_s Sx(hi + lo)[m, s] * mn[n, s]
+                const f16x8 m0 = minima_frag(hdr[0]), m1 = minima_frag(hdr[1]);
+#pragma unroll
+                for (int i = 0; i < kRowTiles; ++i) {
+                    if (i < mt_live) {
+                        const f16x8 sf = *reinterpret_cast<const f16x8*>(&lds_sx[b & 1][(i * 32 + col) * LDS_SX + khalf * 8]);
+                        const f32x16 zero{};
+                        blk[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m0, zero, 0, 0, 0);
+                        blk[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m1, zero, 0, 0, 0);
+                    }
+                }
+                fold(-hdr[0].dmin, -hdr[1].dmin);
+            }
+            if (more) {
+                store_a(buf ^ 1);
+                cur[0] = nxt[0]; cur[1] = nxt[1];
+                if (P == 0 && b + 1 < bpr) store_sx((b + 1) & 1);
+                if (P == 3) { hdr[0] = hdr_next[0]; hdr[1] = hdr_next[1]; }
+            }
+        };
+        for (uint32_t b = 0; b < bpr; ++b) {
+            pair_step(b * 4 + 0, std::integral_constant<int, 0>{});
+            pair_step(b * 4 + 1, std::integral_constant<int, 1>{});
+            pair_step(b * 4 + 2, std::integral_constant<int, 2>{});
+            pair_step(b * 4 + 3, std::integral_constant<int, 3>{});
+        }
     }
 
     // ---- epilogue. Accumulator v of tile (i, j): row = i*32 + 8*(v/4) + 4*khalf + v%4, column = col.
     uint32_t bad = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kRowTiles; ++i) {
         if (i >= mt_live) continue;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -316,11 +457,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
                 const float g = acc[i][0][v], u = acc[i][1][v];
                 const float sg = g >= 0 ? 1.0f / (1.0f + expf(-g)) : expf(g) / (1.0f + expf(g));
                 const float h = (g * sg) * u;
-                // h is carried between the two GEMMs as bf16 (RNE) and fed to the f16 matrix core as h * 2^-8
-                const uint32_t hb = __float_as_uint(h);
-                const uint32_t rounded = (hb + 0x7fffu + ((hb >> 16) & 1u)) & 0xffff0000u;
-                if (nonfinite(g) || nonfinite(u) || nonfinite(h) || (rounded & 0x7f800000u) == 0x7f800000u) bad = TSP_ERRBIT_NONFINITE;
-                reinterpret_cast<_Float16*>(a.out)[uint64_t(dst) * a.n + out_col[0]] = _Float16(__uint_as_float(rounded) * 0.00390625f);
+                // h is carried between the two GEMMs as the half nearest to h * 2^-8: 11 significant bits for
+                // 0.016 <= |h| < 1.6e7, an absolute step of 2^-16 below that
+                const _Float16 carried = _Float16(h * 0.00390625f);
+                if (nonfinite(g) || nonfinite(u) || nonfinite(h) || (__builtin_bit_cast(uint16_t, carried) & 0x7c00u) == 0x7c00u) bad = TSP_ERRBIT_NONFINITE;
+                reinterpret_cast<_Float16*>(a.out)[uint64_t(dst) * a.n + out_col[0]] = carried;
             } else {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
@@ -341,26 +482,49 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
     publish_error(bad, a.error_word);
 }
 
-// f32 rows -> bf16 (RNE) -> f16, or bf16 rows -> f16. Values outside the f16 range are flagged.
+// f32 rows -> bf16 (RNE) -> f16, or bf16 rows -> f16, plus the per-sub-block (32 column) sums of the converted
+// values as hi + lo f16 pairs: sx[row][block][0..7] = hi, [8..15] = lo. A thread converts 8 columns; four
+// neighbouring lanes share one sub-block. Values outside the f16 range are flagged.
 template <bool FROM_BF16>
 __global__ __launch_bounds__(256) void to_f16_rows(const void* __restrict__ src, uint64_t src_stride_bytes, _Float16* __restrict__ dst,
-                                                   uint32_t rows, uint32_t columns, uint32_t* error_word) {
+                                                   _Float16* __restrict__ sx, uint32_t rows, uint32_t columns, uint32_t* error_word) {
     uint32_t bad = 0;
-    const uint64_t total = uint64_t(rows) * columns;
-    for (uint64_t i = blockIdx.x * uint64_t(blockDim.x) + threadIdx.x; i < total; i += uint64_t(gridDim.x) * blockDim.x) {
-        const uint64_t r = i / columns, c = i % columns;
+    const uint64_t chunks = uint64_t(rows) * (columns / 8);
+    const uint64_t span = (chunks + 3) / 4 * 4;  // whole groups of four lanes stay in the loop together
+    for (uint64_t i = blockIdx.x * uint64_t(blockDim.x) + threadIdx.x; i < span; i += uint64_t(gridDim.x) * blockDim.x) {
+        const bool live = i < chunks;
+        const uint64_t r = live ? i / (columns / 8) : 0, c8 = live ? i % (columns / 8) : 0;
         const uint8_t* row = static_cast<const uint8_t*>(src) + r * src_stride_bytes;
-        uint32_t bits;
-        if constexpr (FROM_BF16) {
-            bits = uint32_t(reinterpret_cast<const uint16_t*>(row)[c]) << 16;
-        } else {
-            const uint32_t fb = __float_as_uint(reinterpret_cast<const float*>(row)[c]);
-            bits = (fb + 0x7fffu + ((fb >> 16) & 1u)) & 0xffff0000u;
-            if ((fb & 0x7f800000u) == 0x7f800000u) bits = fb;
+        float sum = 0;
+        f16x8 out;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            uint32_t bits;
+            if constexpr (FROM_BF16) {
+                bits = uint32_t(reinterpret_cast<const uint16_t*>(row)[c8 * 8 + e]) << 16;
+            } else {
+                const uint32_t fb = __float_as_uint(reinterpret_cast<const float*>(row)[c8 * 8 + e]);
+                bits = (fb + 0x7fffu + ((fb >> 16) & 1u)) & 0xffff0000u;
+                if ((fb & 0x7f800000u) == 0x7f800000u) bits = fb;
+            }
+            const _Float16 h = _Float16(__uint_as_float(bits));
+            if ((bits & 0x7f800000u) == 0x7f800000u || (__builtin_bit_cast(uint16_t, h) & 0x7c00u) == 0x7c00u) bad = TSP_ERRBIT_NONFINITE;
+            out[e] = h;
+            sum += float(h);
         }
-        const _Float16 h = _Float16(__uint_as_float(bits));
-        if ((bits & 0x7f800000u) == 0x7f800000u || (__builtin_bit_cast(uint16_t, h) & 0x7c00u) == 0x7c00u) bad = TSP_ERRBIT_NONFINITE;
-        dst[i] = h;
+        sum += __shfl_xor(sum, 1, kWave);
+        sum += __shfl_xor(sum, 2, kWave);
+        if (live) {
+            *reinterpret_cast<f16x8*>(dst + r * columns + c8 * 8) = out;
+            if (sx && (c8 & 3) == 0) {
+                const uint32_t sub = uint32_t(c8 / 4), b = sub / 8, s = sub % 8;
+                const _Float16 hi = _Float16(sum), lo = _Float16(sum - float(hi));
+                if ((__builtin_bit_cast(uint16_t, hi) & 0x7c00u) == 0x7c00u) bad = TSP_ERRBIT_NONFINITE;
+                _Float16* o = sx + (r * (columns / 256) + b) * 16;
+                o[s] = hi;
+                o[8 + s] = lo;
+            }
+        }
     }
     publish_error(bad, error_word);
 }
@@ -372,11 +536,12 @@ int launch(const GemmArgs& a, uint32_t col_tiles, uint32_t tasks, hipStream_t s)
     return launch_status("dequant_gemm");
 }
 
-int convert_rows(const void* src, uint64_t stride, int from_bf16, _Float16* dst, uint32_t rows, uint32_t columns, uint32_t* err, hipStream_t s) {
-    const uint64_t total = uint64_t(rows) * columns;
-    const uint32_t grid = uint32_t((total + 255) / 256 > 8192 ? 8192 : (total + 255) / 256);
-    if (from_bf16) TSP_LAUNCH("to_f16_rows", s, to_f16_rows<true><<<grid, 256, 0, s>>>(src, stride, dst, rows, columns, err));
-    else TSP_LAUNCH("to_f16_rows", s, to_f16_rows<false><<<grid, 256, 0, s>>>(src, stride, dst, rows, columns, err));
+int convert_rows(const void* src, uint64_t stride, int from_bf16, _Float16* dst, _Float16* sx, uint32_t rows, uint32_t columns,
+                 uint32_t* err, hipStream_t s) {
+    const uint64_t chunks = uint64_t(rows) * (columns / 8);
+    const uint32_t grid = uint32_t((chunks + 255) / 256 > 8192 ? 8192 : (chunks + 255) / 256);
+    if (from_bf16) TSP_LAUNCH("to_f16_rows", s, to_f16_rows<true><<<grid, 256, 0, s>>>(src, stride, dst, sx, rows, columns, err));
+    else TSP_LAUNCH("to_f16_rows", s, to_f16_rows<false><<<grid, 256, 0, s>>>(src, stride, dst, sx, rows, columns, err));
     return launch_status("to_f16_rows");
 }
 
@@ -384,7 +549,10 @@ uint64_t align256(uint64_t v) { return (v + 255) / 256 * 256; }
 
 }  // namespace
 
-extern "C" uint64_t tsp_dense_mm_workspace_bytes(uint32_t tokens, uint32_t columns) { return align256(uint64_t(tokens) * columns * 2); }
+// workspace: [f16 rows][activation sums]
+extern "C" uint64_t tsp_dense_mm_workspace_bytes(uint32_t tokens, uint32_t columns) {
+    return align256(uint64_t(tokens) * columns * 2) + align256(uint64_t(tokens) * (columns / 256) * 32);
+}
 
 extern "C" int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matrix, uint64_t matrix_bytes, const void* input,
                             uint64_t input_stride_bytes, int input_is_bf16, void* output, uint64_t output_stride_bytes,
@@ -419,9 +587,10 @@ extern "C" int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matr
                 "dense dequant-GEMM buffers overlap");
     const auto s = static_cast<hipStream_t>(stream);
     auto* xh = static_cast<_Float16*>(workspace);
-    int rc = convert_rows(input, input_stride_bytes, input_is_bf16, xh, tokens, columns, error_word, s);
+    auto* sx = reinterpret_cast<_Float16*>(static_cast<uint8_t*>(workspace) + align256(uint64_t(tokens) * columns * 2));
+    int rc = convert_rows(input, input_stride_bytes, input_is_bf16, xh, encoding == 12 ? sx : nullptr, tokens, columns, error_word, s);
     if (rc != TSP_OK) return rc;
-    a.a = xh; a.a_stride = columns; a.w0 = static_cast<const uint8_t*>(matrix); a.experts = 1;
+    a.a = xh; a.a_stride = columns; a.sx = sx; a.w0 = static_cast<const uint8_t*>(matrix); a.experts = 1;
     a.m = tokens; a.n = rows; a.k = columns; a.out = output; a.out_stride = output_stride_bytes; a.out_scale = 1.0f;
     a.error_word = error_word;
     const uint32_t col_tiles = (rows + 255) / 256, tasks = (tokens + kTaskRows - 1) / kTaskRows;
@@ -435,14 +604,15 @@ extern "C" int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matr
 
 // ---------------------------------------------------------------- grouped MoE
 namespace {
-struct NaxLayout { uint64_t xh, tasks128, hbuf, total; uint32_t bound128; };
+struct NaxLayout { uint64_t xh, sx, tasks, hbuf, total; uint32_t bound; };
 NaxLayout nax_layout(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t channels, uint32_t hidden) {
     NaxLayout l{};
-    l.bound128 = tokens * selected / kTaskRows + experts;
+    l.bound = tokens * selected / kTaskRows + experts;
     l.xh = 0;
-    l.tasks128 = align256(uint64_t(tokens) * channels * 2);
-    l.hbuf = l.tasks128 + align256((2 + 2 * uint64_t(l.bound128)) * 4);
-    l.total = l.hbuf + align256(uint64_t(l.bound128) * kTaskRows * hidden * 2);
+    l.sx = align256(uint64_t(tokens) * channels * 2);
+    l.tasks = l.sx + align256(uint64_t(tokens) * (channels / 256) * 32);
+    l.hbuf = l.tasks + align256((2 + 2 * uint64_t(l.bound)) * 4);
+    l.total = l.hbuf + align256(uint64_t(l.bound) * kTaskRows * hidden * 2);
     return l;
 }
 }  // namespace
@@ -491,27 +661,28 @@ extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream
     const auto s = static_cast<hipStream_t>(stream);
     auto* ws = static_cast<uint8_t*>(m->workspace);
     auto* xh = reinterpret_cast<_Float16*>(ws + l.xh);
-    auto* tasks128 = reinterpret_cast<uint32_t*>(ws + l.tasks128);
+    auto* sx = reinterpret_cast<_Float16*>(ws + l.sx);
+    auto* task_list = reinterpret_cast<uint32_t*>(ws + l.tasks);
     auto* hbuf = reinterpret_cast<_Float16*>(ws + l.hbuf);
 
     rc = tsp_grouped_routes(m->ids, m->token_map, m->counts, m->experts, m->selected, m->tokens, m->error_word, stream);
     if (rc == TSP_OK) rc = tsp_grouped_tasks(m->counts, m->tasks, m->experts, m->selected, m->tokens, 32, m->error_word, stream);
-    if (rc == TSP_OK) rc = tsp_grouped_tasks(m->counts, tasks128, m->experts, m->selected, m->tokens, kTaskRows, m->error_word, stream);
-    if (rc == TSP_OK) rc = convert_rows(m->x, m->x_stride_bytes, 0, xh, m->tokens, m->channels, m->error_word, s);
+    if (rc == TSP_OK) rc = tsp_grouped_tasks(m->counts, task_list, m->experts, m->selected, m->tokens, kTaskRows, m->error_word, stream);
+    if (rc == TSP_OK) rc = convert_rows(m->x, m->x_stride_bytes, 0, xh, sx, m->tokens, m->channels, m->error_word, s);
     if (rc != TSP_OK) return rc;
 
     GemmArgs g{};
-    g.a = xh; g.a_stride = m->channels; g.w0 = static_cast<const uint8_t*>(m->pair_lo); g.w1 = static_cast<const uint8_t*>(m->pair_hi);
-    g.spec = gu; g.experts = m->experts; g.tasks = tasks128; g.counts = m->counts; g.token_map = m->token_map; g.ids = m->ids;
+    g.a = xh; g.a_stride = m->channels; g.sx = sx; g.w0 = static_cast<const uint8_t*>(m->pair_lo); g.w1 = static_cast<const uint8_t*>(m->pair_hi);
+    g.spec = gu; g.experts = m->experts; g.tasks = task_list; g.counts = m->counts; g.token_map = m->token_map; g.ids = m->ids;
     g.tokens = m->tokens; g.selected = m->selected; g.n = m->hidden; g.k = m->channels; g.out = hbuf; g.out_scale = 1.0f;
     g.error_word = m->error_word;
-    rc = launch<B_Q4K_PLANAR, EPI_SWIGLU, ROWS_GATHER_TOKENS>(g, (m->hidden + 127) / 128, l.bound128, s);
+    rc = launch<B_Q4K_PLANAR, EPI_SWIGLU, ROWS_GATHER_TOKENS>(g, (m->hidden + 127) / 128, l.bound, s);
     if (rc != TSP_OK) return rc;
 
     GemmArgs d{};
     d.a = hbuf; d.a_stride = m->hidden; d.w0 = static_cast<const uint8_t*>(m->down); d.spec = dn; d.experts = m->experts;
-    d.tasks = tasks128; d.counts = m->counts; d.token_map = m->token_map; d.ids = m->ids; d.tokens = m->tokens; d.selected = m->selected;
+    d.tasks = task_list; d.counts = m->counts; d.token_map = m->token_map; d.ids = m->ids; d.tokens = m->tokens; d.selected = m->selected;
     d.n = m->channels; d.k = m->hidden; d.out = m->y; d.out_stride = m->y_stride_bytes; d.out_scale = 256.0f;  // undo the 2^-8 carried by h
     d.error_word = m->error_word;
-    return launch<B_Q6K_PLANAR, EPI_F32, ROWS_TASK_SLOTS>(d, (m->channels + 255) / 256, l.bound128, s);
+    return launch<B_Q6K_PLANAR, EPI_F32, ROWS_TASK_SLOTS>(d, (m->channels + 255) / 256, l.bound, s);
 }
