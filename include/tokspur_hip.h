@@ -84,6 +84,10 @@ typedef struct tsp_kernel_time {
 } tsp_kernel_time;
 int tsp_profile_begin(void);
 int tsp_profile_end(tsp_kernel_time* rows, uint32_t capacity, uint32_t* count);
+/* Measurement aid with no counterpart in the reference: a plain copy kernel ("calibration_copy") of `bytes`
+ * (a multiple of 16) from src to dst. Its HBM traffic is known, so the memory counters of a profiler read for
+ * it give the factor by which to scale the same counters read for the other kernels. */
+int tsp_calibration_copy(void* dst, const void* src, uint64_t bytes, void* stream);
 
 /* ------------------------------------------------------------------ host: formats and layouts */
 

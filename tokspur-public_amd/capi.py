@@ -455,6 +455,11 @@ def profile_end():
     return {rows[i].name.decode(): (rows[i].launches, rows[i].total_ms, rows[i].min_ms) for i in range(min(n.value, 64))}
 
 
+def calibration_copy(dev, dst, src):
+    """Plain copy kernel of a known size (scales a profiler's HBM byte counters)."""
+    check(dll().tsp_calibration_copy(dev.ptr(dst), dev.ptr(src), C.c_uint64(dev.nbytes(src)), dev.stream()))
+
+
 def as_u32(t):
     """Device int32 tensor -> host uint32 array."""
     return t.cpu().numpy().view(np.uint32)

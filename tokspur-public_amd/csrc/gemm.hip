@@ -62,6 +62,7 @@ struct GemmArgs {
     uint64_t out_stride;      // bytes
     float out_scale;
     uint32_t* error_word;
+    uint32_t col_tiles, task_slots;  // logical grid: column tiles x tasks, launched as one linear grid
 };
 
 // Workgroup barrier that waits for this wave's LDS traffic only. __syncthreads() also drains every outstanding
@@ -119,28 +120,15 @@ __device__ __forceinline__ HdrQ4 load_hdr_q4k(const uint8_t* base, const tsp_pla
     return h;
 }
 
-template <int BKIND>
-__device__ __forceinline__ u32x4 load_raw_q4k(const uint8_t* base, const tsp_planar_spec& s, uint64_t row, uint32_t bpr, uint32_t step,
-                                              uint32_t khalf) {
-    const uint32_t b = step / 4, p = step % 4;
-    const uint64_t blk = row * bpr + b;
-    const uint8_t* qs = BKIND == B_Q4K_PLANAR ? base + s.qs_offset + blk * 128 + p * 32 + khalf * 16
-                                               : base + blk * 144 + 16 + p * 32 + khalf * 16;
-    return *reinterpret_cast<const u32x4*>(qs);
-}
-
-// Fragments of pair P: bytes 16h..16h+15 of the 32-byte pair; low nibbles are sub-block 2P, high nibbles 2P+1.
-// Fragment f covers activation columns (f/2)*32 + 16h + (f%2)*8 .. +8 of the 64-column slab.
-template <int P>
-__device__ __forceinline__ void frags_q4k(const u32x4& raw, const HdrQ4& h, f16x8 frag[4]) {
+// Fragments of pair P: bytes 16h..16h+15 of the 32-byte pair; low nibbles (HI = 0) are sub-block 2P, high nibbles
+// sub-block 2P+1. Fragment f of a half covers activation columns HI*32 + 16h + f*8 .. +8 of the 64-column slab.
+template <int P, int HI>
+__device__ __forceinline__ void frags_q4k(const u32x4& raw, const HdrQ4& h, f16x8 frag[2]) {
     constexpr uint32_t M4 = 0x0f0f0f0fu;
-    const uint32_t sc_a = (h.sc[P >> 1] >> ((P & 1) * 16)) & 0xffu, sc_b = (h.sc[P >> 1] >> ((P & 1) * 16 + 8)) & 0xffu;
-    const f16x2 sa = splat(float(sc_a)), sb = splat(float(sc_b));
-    const f16x2 ba = sa * splat(-1024.0f), bb = sb * splat(-1024.0f);
-    frag[0] = scaled8_q4(raw[0] & M4, raw[1] & M4, sa, ba);
-    frag[1] = scaled8_q4(raw[2] & M4, raw[3] & M4, sa, ba);
-    frag[2] = scaled8_q4((raw[0] >> 4) & M4, (raw[1] >> 4) & M4, sb, bb);
-    frag[3] = scaled8_q4((raw[2] >> 4) & M4, (raw[3] >> 4) & M4, sb, bb);
+    const uint32_t sc = (h.sc[P >> 1] >> ((P & 1) * 16 + HI * 8)) & 0xffu;
+    const f16x2 s2 = splat(float(sc)), bias = s2 * splat(-1024.0f);
+    frag[0] = scaled8_q4((raw[0] >> (4 * HI)) & M4, (raw[1] >> (4 * HI)) & M4, s2, bias);
+    frag[1] = scaled8_q4((raw[2] >> (4 * HI)) & M4, (raw[3] >> (4 * HI)) & M4, s2, bias);
 }
 
 // B operand of the minima term: the eight integer minima, the same in both k-halves (hi and lo sums).
@@ -201,13 +189,30 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
     constexpr int LDS_SX = 24;       // halfs per staged row of activation sums (16 used)
     __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][kTaskRows * LDA];
     __shared__ __attribute__((aligned(16))) _Float16 lds_sx[2][Q6 ? 8 : kTaskRows * LDS_SX];
+    // Q4_K quant bytes, half a super-block at a time, double buffered, private to each wave:
+    // [wave][buffer][64 rows][4 chunks of 16 B], chunks swizzled so that the row-wise stores and the column-wise reads
+    // both spread over all banks
+    __shared__ __attribute__((aligned(16))) uint8_t lds_w[Q6 ? 16 : 4 * 2 * 64 * 64];
     __shared__ uint32_t row_src[kTaskRows];
     __shared__ uint32_t row_dst[kTaskRows];
     __shared__ uint32_t task_bad;
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const uint32_t col = lane % 32, khalf = lane / 32;
-    const uint32_t task = blockIdx.y;
+    // Logical (column tile, task) from the linear workgroup id. Workgroups go to the eight XCDs round-robin by id and
+    // each XCD has its own L2, so ids are dealt out in runs: XCD x gets the x-th eighth of the live (task, tile) pairs in
+    // order. All column tiles of a task, and the row slabs of one expert, then meet in one L2: the task's activation
+    // rows and the expert's weight bytes are fetched from memory once and hit in L2 for the other workgroups.
+    uint32_t live_tasks = a.task_slots;
+    if constexpr (ROWS != ROWS_DENSE) {
+        const uint32_t listed = a.tasks[0];
+        live_tasks = listed < a.task_slots ? listed : a.task_slots;
+        if (live_tasks == 0) live_tasks = 1;  // keeps workgroup (0, 0) alive to report a bad task list
+    }
+    const uint32_t live_groups = live_tasks * a.col_tiles, per_xcd = (live_groups + 7) / 8;
+    const uint32_t logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (blockIdx.x / 8 >= per_xcd || logical >= live_groups) return;
+    const uint32_t task = logical / a.col_tiles, bx = logical % a.col_tiles;
 
     // ---- task resolution
     uint32_t expert = 0, nrows = 0;
@@ -222,7 +227,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
         const uint32_t bound = a.tokens * a.selected / kTaskRows + a.experts;
         const uint32_t live = a.tasks[0];
         if (live > bound || a.tasks[1] != a.tokens * a.selected) {
-            if (tid == 0 && blockIdx.x == 0 && task == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+            if (tid == 0 && bx == 0 && task == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
             return;
         }
         if (task >= live) return;
@@ -230,7 +235,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
         const uint32_t start = a.tasks[3 + 2 * task];
         const uint32_t count = expert < a.experts ? a.counts[expert] : 0;
         if (expert >= a.experts || count > a.tokens || start >= count) {
-            if (tid == 0 && blockIdx.x == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+            if (tid == 0 && bx == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
             return;
         }
         nrows = count - start < kTaskRows ? count - start : kTaskRows;
@@ -243,7 +248,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
         }
     }
     __syncthreads();
-    if (task_bad && tid == 0 && blockIdx.x == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+    if (task_bad && tid == 0 && bx == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
     const int mt_live = (nrows + 31) / 32;
 
     // ---- weight rows of this wave
@@ -252,7 +257,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
     uint32_t out_col[2];
     bool col_live[2];
     if constexpr (EPI == EPI_SWIGLU) {
-        const uint32_t unit = blockIdx.x * 128 + wave * 32 + col;
+        const uint32_t unit = bx * 128 + wave * 32 + col;
         const uint32_t half_e = a.experts / 2;
         const uint8_t* pair = (expert < half_e ? a.w0 : a.w1) + uint64_t(expert < half_e ? expert : expert - half_e) * 2 * a.spec.planar_expert_bytes;
         wbase[0] = pair; wbase[1] = pair + a.spec.planar_expert_bytes;
@@ -262,7 +267,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
     } else {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const uint32_t n = blockIdx.x * 256 + wave * 64 + j * 32 + col;
+            const uint32_t n = bx * 256 + wave * 64 + j * 32 + col;
             col_live[j] = n < a.n;
             wrow[j] = col_live[j] ? n : a.n - 1;
             out_col[j] = n;
@@ -280,39 +285,47 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // ---- activation staging: thread t copies KSTEP/4 halfs of row t/4 per step, global -> registers -> LDS
-    constexpr int SEG = KSTEP / 4;
-    const uint32_t st_row = tid / 4, st_seg = tid % 4;
-    const _Float16* st_src = a.a + uint64_t(row_src[st_row]) * a.a_stride + st_seg * SEG;
-    u32x4 stage0{}, stage1{};  // named registers: an array here is kept in scratch memory
-    auto fetch_a = [&](uint32_t step) {
-        const u32x4* src = reinterpret_cast<const u32x4*>(st_src + uint64_t(step) * KSTEP);
-        stage0 = src[0];
-        stage1 = src[1];
-    };
-    auto store_a = [&](int buf) {
-        u32x4* dst = reinterpret_cast<u32x4*>(&lds_a[buf][st_row * LDA + st_seg * SEG]);
-        dst[0] = stage0;
-        dst[1] = stage1;
-    };
+    // ---- activation staging, global -> registers -> LDS: per step 64 rows x 128 bytes; instruction i of thread t takes
+    // the 16-byte chunk t % 8 of row t / 8 + 32 i, so one wave instruction reads eight rows' whole 128 bytes
+    const uint32_t st_row = tid / 8, st_chunk = tid % 8;
+    const _Float16* st_src0 = a.a + uint64_t(row_src[st_row]) * a.a_stride + st_chunk * 8;
+    const _Float16* st_src1 = a.a + uint64_t(row_src[st_row + 32]) * a.a_stride + st_chunk * 8;
+    u32x4 stage[1][2] = {};
+    using Slot0 = std::integral_constant<int, 0>;
+    using Slot1 = std::integral_constant<int, 1>;  // tags also used as tile / position indices below
     // activation sums of one super-block: 64 rows x 32 bytes, threads 0..127 copy 16 bytes each
     const uint32_t sx_row = (tid / 2) % kTaskRows, sx_seg = tid % 2;
     uint4 sx_stage{};
     auto fetch_sx = [&](uint32_t b) {
         if constexpr (!Q6) {
-            if (tid < 2 * kTaskRows) sx_stage = *reinterpret_cast<const uint4*>(a.sx + (uint64_t(row_src[sx_row]) * bpr + b) * 16 + sx_seg * 8);
+            // 64 rows x 32 bytes; threads 128..255 repeat the work of 0..127 so that no load sits under a branch
+            sx_stage = *reinterpret_cast<const uint4*>(a.sx + (uint64_t(row_src[sx_row]) * bpr + b) * 16 + sx_seg * 8);
         }
     };
     auto store_sx = [&](int buf) {
         if constexpr (!Q6) {
-            if (tid < 2 * kTaskRows) *reinterpret_cast<uint4*>(&lds_sx[buf][sx_row * LDS_SX + sx_seg * 8]) = sx_stage;
+            *reinterpret_cast<uint4*>(&lds_sx[buf][sx_row * LDS_SX + sx_seg * 8]) = sx_stage;
         }
     };
-    // one k16 MFMA per (row tile, column tile); `first` starts the super-block accumulator from zero
-    auto mfma = [&](int buf, int k0, const f16x8& b0, const f16x8& b1, bool first) {
-#pragma unroll
-        for (int i = 0; i < kRowTiles; ++i) {
-            if (i < mt_live) {
+    // The whole K loop is instantiated once per number of live 32-row tiles, so that its body is straight-line code:
+    // a branch per tile would cut every step into a dozen basic blocks, each waiting for its own LDS read before its
+    // two MFMAs, and nothing could be scheduled across them.
+    auto run = [&](auto mt_tag) {
+        constexpr int MT = decltype(mt_tag)::value;
+        auto fetch_a = [&](uint32_t step, auto slot_tag) {  // rows 32..63 only when the task has them
+            constexpr int SLOT = decltype(slot_tag)::value;
+            stage[SLOT][0] = *reinterpret_cast<const u32x4*>(st_src0 + uint64_t(step) * KSTEP);
+            if constexpr (MT == 2) stage[SLOT][1] = *reinterpret_cast<const u32x4*>(st_src1 + uint64_t(step) * KSTEP);
+        };
+        auto store_a = [&](int buf, auto slot_tag) {
+            constexpr int SLOT = decltype(slot_tag)::value;
+            *reinterpret_cast<u32x4*>(&lds_a[buf][st_row * LDA + st_chunk * 8]) = stage[SLOT][0];
+            if constexpr (MT == 2) *reinterpret_cast<u32x4*>(&lds_a[buf][(st_row + 32) * LDA + st_chunk * 8]) = stage[SLOT][1];
+        };
+        // one k16 MFMA per (row tile, column tile); `first` starts the super-block accumulator from zero
+        auto mfma = [&](int buf, int k0, const f16x8& b0, const f16x8& b1, bool first) {
+    #pragma unroll
+            for (int i = 0; i < MT; ++i) {
                 const f16x8 af = *reinterpret_cast<const f16x8*>(&lds_a[buf][(i * 32 + col) * LDA + k0]);
                 if (first) {
                     const f32x16 zero{};
@@ -323,123 +336,161 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
                     blk[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b1, blk[i][1], 0, 0, 0);
                 }
             }
-        }
-    };
-    auto fold = [&](float d0, float d1) {  // acc += d * blk at the end of a super-block
-#pragma unroll
-        for (int i = 0; i < kRowTiles; ++i) {
-            if (i < mt_live) {
-#pragma unroll
+        };
+        auto fold = [&](float d0, float d1) {  // acc += d * blk at the end of a super-block
+    #pragma unroll
+            for (int i = 0; i < MT; ++i) {
+    #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     acc[i][0][v] = __builtin_fmaf(d0, blk[i][0][v], acc[i][0][v]);
                     acc[i][1][v] = __builtin_fmaf(d1, blk[i][1][v], acc[i][1][v]);
                 }
             }
-        }
-    };
-
-    fetch_a(0);
-    store_a(0);
-    if constexpr (Q6) {
-        RawQ6 cur[2], nxt[2];
-#pragma unroll
-        for (int j = 0; j < 2; ++j) load_raw_q6k(wbase[j], a.spec, wrow[j], bpr, 0, khalf, cur[j]);
-        // K step H of a super-block: section H/2 (128 columns, one set of weight bytes), quarters 2*(H%2) and +1
-        auto half_step = [&](uint32_t step, auto h_tag) {
-            constexpr int H = decltype(h_tag)::value;
-            const int buf = H & 1;
-            const bool more = step + 1 < ksteps;
-            if (more) {
-                fetch_a(step + 1);
-                if (H & 1) {
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) load_raw_q6k(wbase[j], a.spec, wrow[j], bpr, (step + 1) / 2, khalf, nxt[j]);
-                }
-            }
-            auto quarter = [&](auto q_tag) {
-                constexpr int Q = decltype(q_tag)::value;
-                f16x8 f0[2], f1[2];
-                frags_q6k<Q>(cur[0], khalf, f0);
-                frags_q6k<Q>(cur[1], khalf, f1);
-                if (Q % 2 == 0) lds_barrier();  // lds_a[buf] is complete; every wave has left lds_a[buf ^ 1]
-                mfma(buf, (Q % 2) * 32 + khalf * 16, f0[0], f1[0], H == 0 && Q == 0);
-                mfma(buf, (Q % 2) * 32 + khalf * 16 + 8, f0[1], f1[1], false);
-            };
-            quarter(std::integral_constant<int, 2 * (H % 2)>{});
-            quarter(std::integral_constant<int, 2 * (H % 2) + 1>{});
-            if (H == 3) fold(cur[0].d, cur[1].d);
-            if (more) {
-                store_a(buf ^ 1);
-                if (H & 1) { cur[0] = nxt[0]; cur[1] = nxt[1]; }
-            }
         };
-        for (uint32_t b = 0; b < bpr; ++b) {
-            half_step(b * 4 + 0, std::integral_constant<int, 0>{});
-            half_step(b * 4 + 1, std::integral_constant<int, 1>{});
-            half_step(b * 4 + 2, std::integral_constant<int, 2>{});
-            half_step(b * 4 + 3, std::integral_constant<int, 3>{});
-        }
-    } else {
-        HdrQ4 hdr[2], hdr_next[2];
-        u32x4 cur[2], nxt[2];
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            hdr[j] = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, 0);
-            cur[j] = load_raw_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, 0, khalf);
-            hdr_next[j] = hdr[j];
-        }
-        fetch_sx(0);
-        store_sx(0);
-        auto pair_step = [&](uint32_t step, auto p_tag) {
-            constexpr int P = decltype(p_tag)::value;
-            const int buf = step & 1;
-            const uint32_t b = step / 4;
-            const bool more = step + 1 < ksteps;
-            if (more) {
-                fetch_a(step + 1);
-#pragma unroll
-                for (int j = 0; j < 2; ++j) nxt[j] = load_raw_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, step + 1, khalf);
-                if (P == 0 && b + 1 < bpr) {
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) hdr_next[j] = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, b + 1);
-                    fetch_sx(b + 1);
+
+        fetch_a(0, Slot0{});
+        store_a(0, Slot0{});
+        if constexpr (Q6) {
+            RawQ6 cur[2], nxt[2];
+    #pragma unroll
+            for (int j = 0; j < 2; ++j) load_raw_q6k(wbase[j], a.spec, wrow[j], bpr, 0, khalf, cur[j]);
+            // K step H of a super-block: section H/2 (128 columns, one set of weight bytes), quarters 2*(H%2) and +1
+            auto half_step = [&](uint32_t step, auto h_tag) {
+                constexpr int H = decltype(h_tag)::value;
+                const int buf = H & 1;
+                const bool more = step + 1 < ksteps;
+                if (more) {
+                    fetch_a(step + 1, Slot0{});
+                    if (H & 1) {
+    #pragma unroll
+                        for (int j = 0; j < 2; ++j) load_raw_q6k(wbase[j], a.spec, wrow[j], bpr, (step + 1) / 2, khalf, nxt[j]);
+                    }
                 }
+                auto quarter = [&](auto q_tag) {
+                    constexpr int Q = decltype(q_tag)::value;
+                    f16x8 f0[2], f1[2];
+                    frags_q6k<Q>(cur[0], khalf, f0);
+                    frags_q6k<Q>(cur[1], khalf, f1);
+                    if (Q % 2 == 0) lds_barrier();  // lds_a[buf] is complete; every wave has left lds_a[buf ^ 1]
+                    mfma(buf, (Q % 2) * 32 + khalf * 16, f0[0], f1[0], H == 0 && Q == 0);
+                    mfma(buf, (Q % 2) * 32 + khalf * 16 + 8, f0[1], f1[1], false);
+                };
+                quarter(std::integral_constant<int, 2 * (H % 2)>{});
+                quarter(std::integral_constant<int, 2 * (H % 2) + 1>{});
+                if (H == 3) fold(cur[0].d, cur[1].d);
+                if (more) {
+                    store_a(buf ^ 1, Slot0{});
+                    if (H & 1) { cur[0] = nxt[0]; cur[1] = nxt[1]; }
+                }
+            };
+            for (uint32_t b = 0; b < bpr; ++b) {
+                half_step(b * 4 + 0, std::integral_constant<int, 0>{});
+                half_step(b * 4 + 1, std::integral_constant<int, 1>{});
+                half_step(b * 4 + 2, std::integral_constant<int, 2>{});
+                half_step(b * 4 + 3, std::integral_constant<int, 3>{});
             }
-            f16x8 f0[4], f1[4];
-            frags_q4k<P>(cur[0], hdr[0], f0);
-            frags_q4k<P>(cur[1], hdr[1], f1);
-            lds_barrier();  // lds_a[buf] (and at P == 0 lds_sx[b & 1]) is complete; every wave has left the other buffer
-#pragma unroll
-            for (int f = 0; f < 4; ++f) mfma(buf, (f / 2) * 32 + khalf * 16 + (f % 2) * 8, f0[f], f1[f], P == 0 && f == 0);
-            if (P == 3) {
-                fold(hdr[0].d, hdr[1].d);
-                // minima: acc -= dmin * sum_s Sx(hi + lo)[m, s] * mn[n, s]
-                const f16x8 m0 = minima_frag(hdr[0]), m1 = minima_frag(hdr[1]);
-#pragma unroll
-                for (int i = 0; i < kRowTiles; ++i) {
-                    if (i < mt_live) {
+        } else {
+            // Q4_K. Quant bytes travel global -> registers -> LDS -> fragment registers, half a super-block (two K steps)
+            // ahead. The global loads are issued row-wise (one instruction = sixteen rows x 64 contiguous bytes, lane = 16-byte
+            // chunk), so cache lines are requested in whole halves by neighbouring lanes. In LDS lane (row, k-half) then picks
+            // its 16 bytes of the step. Headers (scales, minima, d, dmin: 16 + 4 bytes per lane) go straight to registers.
+            //
+            // Every load in the loop is unconditional (indices past the end are clamped, the data unused): with no branch
+            // around a load the compiler can count outstanding loads exactly and waits only for the oldest ones; a
+            // conditional load anywhere makes it drain all of them (s_waitcnt vmcnt(0)) at every step, which exposes a full
+            // memory round trip per step. Loads return in issue order, so each step requests its activation slab (awaited
+            // at the end of the same step) BEFORE the weight bytes (awaited a step later).
+            constexpr uint32_t BLK = BKIND == B_Q4K_PLANAR ? 128 : 144, QS_AT = BKIND == B_Q4K_PLANAR ? 0 : 16;
+            uint8_t* const my_w = lds_w + wave * (2 * 64 * 64);  // [2 buffers][64 rows][4 chunks of 16 B]
+            const uint32_t ld_row = lane / 4, ld_chunk = (lane % 4) ^ ((lane / 8) & 3);  // chunk c of row r sits at position c ^ ((r >> 1) & 3)
+            const uint32_t wave_row0 = EPI == EPI_SWIGLU ? bx * 128 + wave * 32 : bx * 256 + wave * 64;
+            const uint32_t row_bytes = bpr * BLK;
+            const uint32_t halves = 2 * bpr;
+            u32x4 wstage[4];
+            // instruction Q of a half-block: rows 16Q .. 16Q+15 of the wave's 64 (tile Q / 2)
+            auto fetch_w = [&](uint32_t half, auto q_tag) {
+                constexpr int Q = decltype(q_tag)::value, J = Q / 2;
+                uint32_t row = wave_row0 + (EPI == EPI_SWIGLU ? (Q % 2) * 16 : Q * 16) + ld_row;
+                row = row < a.n ? row : a.n - 1;
+                // uniform base + 32-bit lane offset (the host refuses matrices whose rows span 4 GiB or more)
+                const uint8_t* base = wbase[J] + (BKIND == B_Q4K_PLANAR ? a.spec.qs_offset : 0) + uint64_t(half / 2) * BLK + QS_AT + (half % 2) * 64;
+                wstage[Q] = *reinterpret_cast<const u32x4*>(base + (row * row_bytes + ld_chunk * 16));
+            };
+            auto fetch_w_all = [&](uint32_t half) {
+                half = half < halves ? half : halves - 1;
+                fetch_w(half, std::integral_constant<int, 0>{});
+                fetch_w(half, std::integral_constant<int, 1>{});
+                fetch_w(half, std::integral_constant<int, 2>{});
+                fetch_w(half, std::integral_constant<int, 3>{});
+            };
+            auto store_w = [&](int wbuf) {
+    #pragma unroll
+                for (int q = 0; q < 4; ++q) *reinterpret_cast<u32x4*>(my_w + wbuf * 4096 + (q * 64 + lane) * 16) = wstage[q];
+            };
+            auto read_w = [&](int wbuf, int j, int p2) {  // row j*32 + col, chunk 2*p2 + khalf
+                return *reinterpret_cast<const u32x4*>(my_w + wbuf * 4096 + ((j * 32 + col) * 4 + ((2 * p2 + khalf) ^ ((col >> 1) & 3))) * 16);
+            };
+            HdrQ4 hdr[2], hdr_next[2];
+    #pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                hdr[j] = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, 0);
+                hdr_next[j] = hdr[j];
+            }
+            fetch_w_all(0);
+            store_w(0);
+            fetch_sx(0);
+            store_sx(0);
+            auto pair_step = [&](uint32_t step, auto p_tag) {
+                constexpr int P = decltype(p_tag)::value;
+                constexpr int buf = P & 1, wbuf = P / 2;
+                const uint32_t b = step / 4;
+                fetch_a(step + 1 < ksteps ? step + 1 : step, Slot0{});
+                if (P == 0) fetch_sx(b + 1 < bpr ? b + 1 : b);
+                if (P == 0 || P == 2) fetch_w_all(step / 2 + 1);
+                if (P == 2) {
+    #pragma unroll
+                    for (int j = 0; j < 2; ++j) hdr_next[j] = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, b + 1 < bpr ? b + 1 : b);
+                }
+                lds_barrier();  // lds_a[buf], this wave's weight bytes (and at P == 0 lds_sx[b & 1]) are complete; every wave has left the other buffers
+                const u32x4 raw0 = read_w(wbuf, 0, P & 1), raw1 = read_w(wbuf, 1, P & 1);
+                f16x8 f0[2], f1[2];
+                frags_q4k<P, 0>(raw0, hdr[0], f0);
+                frags_q4k<P, 0>(raw1, hdr[1], f1);
+                mfma(buf, khalf * 16, f0[0], f1[0], P == 0);
+                mfma(buf, khalf * 16 + 8, f0[1], f1[1], false);
+                frags_q4k<P, 1>(raw0, hdr[0], f0);
+                frags_q4k<P, 1>(raw1, hdr[1], f1);
+                mfma(buf, 32 + khalf * 16, f0[0], f1[0], false);
+                mfma(buf, 32 + khalf * 16 + 8, f0[1], f1[1], false);
+                if (P == 3) {
+                    fold(hdr[0].d, hdr[1].d);
+                    // minima: acc -= dmin * sum_s Sx(hi + lo)[m, s] * mn[n, s]
+                    const f16x8 m0 = minima_frag(hdr[0]), m1 = minima_frag(hdr[1]);
+    #pragma unroll
+                    for (int i = 0; i < MT; ++i) {
                         const f16x8 sf = *reinterpret_cast<const f16x8*>(&lds_sx[b & 1][(i * 32 + col) * LDS_SX + khalf * 8]);
                         const f32x16 zero{};
                         blk[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m0, zero, 0, 0, 0);
                         blk[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m1, zero, 0, 0, 0);
                     }
+                    fold(-hdr[0].dmin, -hdr[1].dmin);
                 }
-                fold(-hdr[0].dmin, -hdr[1].dmin);
-            }
-            if (more) {
-                store_a(buf ^ 1);
-                cur[0] = nxt[0]; cur[1] = nxt[1];
-                if (P == 0 && b + 1 < bpr) store_sx((b + 1) & 1);
+                // the slab of the next step (and everything requested before it) has to have arrived now
+                store_a(buf ^ 1, Slot0{});
+                if (P == 0) store_sx((b + 1) & 1);
+                if (P == 1 || P == 3) store_w(wbuf ^ 1);  // read again two barriers from now; this buffer was last read a step ago
                 if (P == 3) { hdr[0] = hdr_next[0]; hdr[1] = hdr_next[1]; }
+            };
+            for (uint32_t b = 0; b < bpr; ++b) {
+                pair_step(b * 4 + 0, std::integral_constant<int, 0>{});
+                pair_step(b * 4 + 1, std::integral_constant<int, 1>{});
+                pair_step(b * 4 + 2, std::integral_constant<int, 2>{});
+                pair_step(b * 4 + 3, std::integral_constant<int, 3>{});
             }
-        };
-        for (uint32_t b = 0; b < bpr; ++b) {
-            pair_step(b * 4 + 0, std::integral_constant<int, 0>{});
-            pair_step(b * 4 + 1, std::integral_constant<int, 1>{});
-            pair_step(b * 4 + 2, std::integral_constant<int, 2>{});
-            pair_step(b * 4 + 3, std::integral_constant<int, 3>{});
         }
-    }
+    };
+    if (mt_live == 1) run(std::integral_constant<int, 1>{});
+    else run(std::integral_constant<int, 2>{});
 
     // ---- epilogue. Accumulator v of tile (i, j): row = i*32 + 8*(v/4) + 4*khalf + v%4, column = col.
     uint32_t bad = 0;
@@ -532,7 +583,11 @@ __global__ __launch_bounds__(256) void to_f16_rows(const void* __restrict__ src,
 template <int BKIND, int EPI, int ROWS>
 int launch(const GemmArgs& a, uint32_t col_tiles, uint32_t tasks, hipStream_t s) {
     constexpr const char* name = EPI == EPI_SWIGLU ? "gemm_gate_up_swiglu" : ROWS == ROWS_TASK_SLOTS ? "gemm_down" : "gemm_dense";
-    TSP_LAUNCH(name, s, gemm_kernel<BKIND, EPI, ROWS><<<dim3(col_tiles, tasks), 256, 0, s>>>(a));
+    GemmArgs g = a;
+    g.col_tiles = col_tiles;
+    g.task_slots = tasks;
+    const uint32_t groups = (col_tiles * tasks + 7) / 8 * 8;
+    TSP_LAUNCH(name, s, gemm_kernel<BKIND, EPI, ROWS><<<groups, 256, 0, s>>>(g));
     return launch_status("dequant_gemm");
 }
 
@@ -579,6 +634,7 @@ extern "C" int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matr
     TSP_REQUIRE(reinterpret_cast<uintptr_t>(matrix) % 16 == 0 && reinterpret_cast<uintptr_t>(workspace) % 16 == 0,
                 "dense dequant-GEMM needs 16-byte aligned weights and workspace");
     TSP_REQUIRE(workspace_bytes >= tsp_dense_mm_workspace_bytes(tokens, columns), "dense dequant-GEMM workspace too small");
+    TSP_REQUIRE(matrix_bytes < (1ull << 32), "dense dequant-GEMM addresses weight rows with 32-bit offsets: matrix must be under 4 GiB");
     const uint64_t in_span = uint64_t(tokens - 1) * input_stride_bytes + uint64_t(columns) * in_elem;
     const uint64_t out_span = uint64_t(tokens - 1) * output_stride_bytes + uint64_t(rows) * out_elem;
     TSP_REQUIRE(!ranges_overlap(output, out_span, matrix, matrix_bytes) && !ranges_overlap(output, out_span, input, in_span) &&
@@ -639,6 +695,8 @@ extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream
     int rc = tsp_make_expert_spec(12, m->channels, m->hidden, &gu);
     if (rc == TSP_OK) rc = tsp_make_expert_spec(14, m->hidden, m->channels, &dn);
     if (rc != TSP_OK) return rc;
+    TSP_REQUIRE(gu.planar_expert_bytes < (1ull << 32) && dn.planar_expert_bytes < (1ull << 32),
+                "planar v3 grouped MoE addresses weight rows with 32-bit offsets: one expert must be under 4 GiB");
     const NaxLayout l = nax_layout(m->tokens, m->selected, m->experts, m->channels, m->hidden);
     TSP_REQUIRE(m->workspace_bytes >= l.total, "planar v3 NAX scratch too small for requested batch");
     TSP_REQUIRE(reinterpret_cast<uintptr_t>(m->workspace) % 256 == 0 && reinterpret_cast<uintptr_t>(m->pair_lo) % 16 == 0 &&
