@@ -141,20 +141,7 @@ __device__ __forceinline__ f16x8 minima_frag(const HdrQ4& h) {
 }
 
 // ---------------------------------------------------------------- Q6_K operands (planes ql / qh / sc / d)
-struct RawQ6 { u32x4 la, lb, qh; uint32_t sc[2]; float d; };
-
-__device__ __forceinline__ void load_raw_q6k(const uint8_t* base, const tsp_planar_spec& s, uint64_t row, uint32_t bpr, uint32_t step,
-                                             uint32_t khalf, RawQ6& r) {
-    const uint32_t b = step / 2, sec = step % 2;  // step counts 128-column sections
-    const uint64_t blk = row * bpr + b;
-    const uint8_t* ql = base + s.qs_offset + blk * 128 + sec * 64 + khalf * 16;
-    r.la = *reinterpret_cast<const u32x4*>(ql);
-    r.lb = *reinterpret_cast<const u32x4*>(ql + 32);
-    r.qh = *reinterpret_cast<const u32x4*>(base + s.qh_offset + blk * 64 + sec * 32 + khalf * 16);
-    const uint2 sc8 = *reinterpret_cast<const uint2*>(base + s.sm_offset + blk * 16 + sec * 8);
-    r.sc[0] = sc8.x; r.sc[1] = sc8.y;
-    r.d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(base + s.dm_offset + blk * 2));
-}
+struct RawQ6 { u32x4 la, lb, qh; uint32_t sc[2]; };  // one section: low nibbles of quarters 0/2 and 1/3, high bit pairs, 8 sub-scales
 
 // Quarter Q of the section (elements Q*32 .. Q*32+31): this lane's 16 bytes are elements Q*32 + 16h + 0..15, all in
 // the 16-weight group 2Q + h. Fragment f covers activation columns Q*32 + 16h + f*8 .. +8 of the section.
@@ -189,10 +176,10 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
     constexpr int LDS_SX = 24;       // halfs per staged row of activation sums (16 used)
     __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][kTaskRows * LDA];
     __shared__ __attribute__((aligned(16))) _Float16 lds_sx[2][Q6 ? 8 : kTaskRows * LDS_SX];
-    // Q4_K quant bytes, half a super-block at a time, double buffered, private to each wave:
-    // [wave][buffer][64 rows][4 chunks of 16 B], chunks swizzled so that the row-wise stores and the column-wise reads
-    // both spread over all banks
-    __shared__ __attribute__((aligned(16))) uint8_t lds_w[Q6 ? 16 : 4 * 2 * 64 * 64];
+    // Quant bytes, half a super-block at a time, double buffered, private to each wave: Q4_K
+    // [wave][buffer][64 rows][4 chunks of 16 B], Q6_K the same for the low nibbles plus [64 rows][2 chunks] of high bits.
+    // Chunks are swizzled so that the row-wise stores and the column-wise reads both spread over all banks
+    __shared__ __attribute__((aligned(16))) uint8_t lds_w[Q6 ? 4 * 2 * 64 * 96 : 4 * 2 * 64 * 64];
     __shared__ uint32_t row_src[kTaskRows];
     __shared__ uint32_t row_dst[kTaskRows];
     __shared__ uint32_t task_bad;
@@ -351,37 +338,79 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
         fetch_a(0, Slot0{});
         store_a(0, Slot0{});
         if constexpr (Q6) {
-            RawQ6 cur[2], nxt[2];
+            // Q6_K planes. Low nibbles (64 B) and high bit pairs (32 B) of one 128-column section per row travel
+            // global -> registers -> LDS -> fragment registers one section (two K steps) ahead, loaded row-wise like
+            // the Q4_K bytes below; sub-scales (16 B) and d (2 B) per super-block go straight to registers. All loads
+            // are unconditional (clamped past the end) so that outstanding loads are counted exactly.
+            uint8_t* const my_w = lds_w + wave * (2 * 64 * 96);  // [2 buffers]{[64 rows][4 chunks] low nibbles, [64 rows][2 chunks] high bits}
+            const uint32_t row_ql = bpr * 128, row_qh = bpr * 64;
+            const uint32_t sections = 2 * bpr;
+            const uint32_t wave_row0 = bx * 256 + wave * 64;
+            const uint32_t ql_row = lane / 4, ql_chunk = (lane % 4) ^ ((lane / 8) & 3);  // chunk c of row r sits at position c ^ ((r >> 1) & 3)
+            const uint32_t qh_row = lane / 2, qh_chunk = lane % 2;
+            u32x4 wstage[6];
+            auto clamp_row = [&](uint32_t r) { return r < a.n ? r : a.n - 1; };
+            auto fetch_w = [&](uint32_t section) {
+                section = section < sections ? section : sections - 1;
+                const uint8_t* ql = wbase[0] + a.spec.qs_offset + uint64_t(section / 2) * 128 + (section % 2) * 64;
+                const uint8_t* qh = wbase[0] + a.spec.qh_offset + uint64_t(section / 2) * 64 + (section % 2) * 32;
     #pragma unroll
-            for (int j = 0; j < 2; ++j) load_raw_q6k(wbase[j], a.spec, wrow[j], bpr, 0, khalf, cur[j]);
-            // K step H of a super-block: section H/2 (128 columns, one set of weight bytes), quarters 2*(H%2) and +1
+                for (int q = 0; q < 4; ++q) wstage[q] = *reinterpret_cast<const u32x4*>(ql + (clamp_row(wave_row0 + q * 16 + ql_row) * row_ql + ql_chunk * 16));
+    #pragma unroll
+                for (int q = 0; q < 2; ++q) wstage[4 + q] = *reinterpret_cast<const u32x4*>(qh + (clamp_row(wave_row0 + q * 32 + qh_row) * row_qh + qh_chunk * 16));
+            };
+            auto store_w = [&](int wbuf) {
+    #pragma unroll
+                for (int q = 0; q < 6; ++q) *reinterpret_cast<u32x4*>(my_w + wbuf * 6144 + (q * 64 + lane) * 16) = wstage[q];
+            };
+            struct Scales { uint32_t sc[4]; float d; };
+            auto load_scales = [&](uint32_t b, int j) {
+                b = b < bpr ? b : bpr - 1;
+                const uint64_t blk_at = wrow[j] * bpr + b;
+                const uint4 sc16 = *reinterpret_cast<const uint4*>(wbase[j] + a.spec.sm_offset + blk_at * 16);
+                Scales r;
+                r.sc[0] = sc16.x; r.sc[1] = sc16.y; r.sc[2] = sc16.z; r.sc[3] = sc16.w;
+                r.d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(wbase[j] + a.spec.dm_offset + blk_at * 2));
+                return r;
+            };
+            Scales scl[2] = {load_scales(0, 0), load_scales(0, 1)}, scl_next[2] = {scl[0], scl[1]};
+            fetch_w(0);
+            store_w(0);
+            RawQ6 raw[2];
+            // K step H of a super-block: section H/2 (128 columns), quarters 2*(H%2) and 2*(H%2)+1 of that section
             auto half_step = [&](uint32_t step, auto h_tag) {
                 constexpr int H = decltype(h_tag)::value;
-                const int buf = H & 1;
-                const bool more = step + 1 < ksteps;
-                if (more) {
-                    fetch_a(step + 1, Slot0{});
-                    if (H & 1) {
+                constexpr int buf = H & 1, wbuf = H / 2;
+                const uint32_t b = step / 4;
+                fetch_a(step + 1 < ksteps ? step + 1 : step, Slot0{});
+                if (H % 2 == 0) fetch_w(step / 2 + 1);
+                if (H == 2) { scl_next[0] = load_scales(b + 1, 0); scl_next[1] = load_scales(b + 1, 1); }
+                lds_barrier();  // lds_a[buf] and this wave's section bytes are complete; every wave has left the other buffers
+                if (H % 2 == 0) {
     #pragma unroll
-                        for (int j = 0; j < 2; ++j) load_raw_q6k(wbase[j], a.spec, wrow[j], bpr, (step + 1) / 2, khalf, nxt[j]);
+                    for (int j = 0; j < 2; ++j) {
+                        const uint8_t* lo = my_w + wbuf * 6144 + (j * 32 + col) * 64;
+                        const uint32_t swz = (col >> 1) & 3;
+                        raw[j].la = *reinterpret_cast<const u32x4*>(lo + ((khalf ^ swz) * 16));
+                        raw[j].lb = *reinterpret_cast<const u32x4*>(lo + (((2 + khalf) ^ swz) * 16));
+                        raw[j].qh = *reinterpret_cast<const u32x4*>(my_w + wbuf * 6144 + 4096 + ((j * 32 + col) * 2 + khalf) * 16);
+                        raw[j].sc[0] = scl[j].sc[(H / 2) * 2]; raw[j].sc[1] = scl[j].sc[(H / 2) * 2 + 1];
                     }
                 }
                 auto quarter = [&](auto q_tag) {
                     constexpr int Q = decltype(q_tag)::value;
                     f16x8 f0[2], f1[2];
-                    frags_q6k<Q>(cur[0], khalf, f0);
-                    frags_q6k<Q>(cur[1], khalf, f1);
-                    if (Q % 2 == 0) lds_barrier();  // lds_a[buf] is complete; every wave has left lds_a[buf ^ 1]
+                    frags_q6k<Q>(raw[0], khalf, f0);
+                    frags_q6k<Q>(raw[1], khalf, f1);
                     mfma(buf, (Q % 2) * 32 + khalf * 16, f0[0], f1[0], H == 0 && Q == 0);
                     mfma(buf, (Q % 2) * 32 + khalf * 16 + 8, f0[1], f1[1], false);
                 };
                 quarter(std::integral_constant<int, 2 * (H % 2)>{});
                 quarter(std::integral_constant<int, 2 * (H % 2) + 1>{});
-                if (H == 3) fold(cur[0].d, cur[1].d);
-                if (more) {
-                    store_a(buf ^ 1, Slot0{});
-                    if (H & 1) { cur[0] = nxt[0]; cur[1] = nxt[1]; }
-                }
+                if (H == 3) fold(scl[0].d, scl[1].d);
+                store_a(buf ^ 1, Slot0{});
+                if (H % 2 == 1) store_w(wbuf ^ 1);
+                if (H == 3) { scl[0] = scl_next[0]; scl[1] = scl_next[1]; }
             };
             for (uint32_t b = 0; b < bpr; ++b) {
                 half_step(b * 4 + 0, std::integral_constant<int, 0>{});
