@@ -296,3 +296,48 @@ def test_moe_routed_reference_brute_force(orc, synth):
         assert np.allclose(h[rid], hh.astype(np.float64), rtol=3e-7, atol=1e-30)
         yy = np.array([sum(d[e, r] * h[rid]) for r in range(channels)])
         assert np.allclose(y[rid], yy, rtol=1e-13, atol=1e-13)
+
+
+def q6k_fields(blocks):
+    """Independent numpy decode of Q6_K blocks -> (integer codes [nb, 256], int8 sub-scales [nb, 16], d [nb])."""
+    blk = np.frombuffer(blocks, dtype=np.uint8).reshape(-1, 210)
+    ql, qh = blk[:, :128].astype(np.int32), blk[:, 128:192].astype(np.int32)
+    q = np.empty((blk.shape[0], 256), dtype=np.int32)
+    for sec in range(2):
+        for l in range(32):
+            a, b, h = ql[:, sec * 64 + l], ql[:, sec * 64 + 32 + l], qh[:, sec * 32 + l]
+            q[:, sec * 128 + l] = (a & 15) | ((h & 3) << 4)
+            q[:, sec * 128 + 32 + l] = (b & 15) | (((h >> 2) & 3) << 4)
+            q[:, sec * 128 + 64 + l] = (a >> 4) | (((h >> 4) & 3) << 4)
+            q[:, sec * 128 + 96 + l] = (b >> 4) | (((h >> 6) & 3) << 4)
+    return q, blk[:, 192:208].view(np.int8).astype(np.int32), blk[:, 208:210].copy().view(np.float16).astype(np.float64)[:, 0]
+
+
+def test_matrix_core_staging_models(orc, synth):
+    """stage_f16 = 2 (Q6_K rows as d * half(sc * (q - 32))) and the h = 256 * half(h / 256) carry restate the HIP
+    kernels' staging; they have no counterpart in the reference, so they are checked against numpy's own half."""
+    rows, cols, tokens = 24, 512, 5
+    w = synth.matrix(14, 9100, rows, cols)
+    x = synth.round_bf16(synth.activations_f32(9101, (tokens, cols)))
+    q, sc, d = q6k_fields(w)
+    prod = (q - 32) * np.repeat(sc, 16, axis=1)
+    assert (np.abs(prod) > 2048).any()  # the case that rounds is present
+    for stage, weights in ((0, prod.astype(np.float64)), (2, prod.astype(np.float16).astype(np.float64))):
+        want = x.astype(np.float64) @ (weights * d[:, None]).reshape(rows, cols).T
+        got = orc.staged_gemm(14, w, cols, x, nrows=rows, stage_f16=stage)
+        assert np.allclose(got, want, rtol=1e-12, atol=1e-9)
+    # h carry: stage 4 rounds h to the half nearest h / 256, stage 0 does not; the down product is then exact
+    channels, hidden, experts = 256, 256, 2
+    gate = synth.matrix(12, 9102, hidden * experts, channels)
+    up = synth.matrix(12, 9103, hidden * experts, channels)
+    down = synth.matrix(14, 9104, channels * experts, hidden)
+    ids = np.array([1, 0, 1], dtype=np.uint32)
+    xs = synth.round_bf16(synth.activations_f32(9105, (3, channels)))
+    h0, _ = orc.moe_routed_reference(12, 14, gate, up, down, channels, hidden, experts, ids, 3, 1, xs, stage=0)
+    h4, y4 = orc.moe_routed_reference(12, 14, gate, up, down, channels, hidden, experts, ids, 3, 1, xs, stage=4)
+    carried = (h0.astype(np.float32) * np.float32(1 / 256)).astype(np.float16).astype(np.float64) * 256.0
+    assert np.array_equal(h4, carried)
+    qd, scd, dd = q6k_fields(down)
+    wd = ((qd - 32) * np.repeat(scd, 16, axis=1) * dd[:, None]).reshape(experts, channels, hidden)
+    want_y = np.stack([wd[ids[r]] @ carried[r] for r in range(3)])
+    assert np.allclose(y4, want_y, rtol=1e-12, atol=1e-6)
