@@ -296,8 +296,29 @@ typedef struct tsp_grouped_moe {
 uint64_t tsp_planar_nax_workspace_bytes(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t channels, uint32_t hidden);
 /* include/tokspur/graph.hpp:478 `planar_nax_grouped_moe` (kernels/planar_moe_v3.metal:2406-2621): expert
  * permutation -> prefix-sum tasks -> gather -> ragged grouped gate/up GEMM with fused SwiGLU (h carried as
- * bf16) -> grouped down GEMM -> scatter of f32 rows to y[rid]. */
+ * the half nearest h / 256) -> grouped down GEMM -> scatter of f32 rows to y[rid]. */
 int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* moe, void* stream);
+
+/* ------------------------------------------------------------------ row top-k of the logits */
+
+/* include/tokspur/sampling.hpp:21-29 `GpuLogitTopKRow` == kernels/logit_topk.metal:17-25 `LogitTopKRowOut`, 528 bytes. */
+typedef struct tsp_logit_topk_row {
+    uint32_t vocabulary;
+    uint32_t count;
+    uint32_t first_nonfinite_col;
+    uint32_t first_subnormal_col;
+    uint32_t ids[64];
+    float logits[64];
+} tsp_logit_topk_row;
+/* include/tokspur/graph.hpp:1030-1031, src/graph.mm:9422-9433: bytes of the partial-row scratch and of the output
+ * rows; 0 (and tsp_last_error) when the bounds are refused. */
+uint64_t tsp_logit_topk_scratch_bytes(uint32_t max_rows, uint32_t max_vocabulary);
+uint64_t tsp_logit_topk_output_bytes(uint32_t max_rows);
+/* include/tokspur/graph.hpp:1033 `logit_topk`, src/graph.mm:9443-9478, kernels/logit_topk.metal:93-365; ordering of
+ * src/sampling.cpp:473-513 `cpu_logit_topk_row`: value descending, column ascending, -0 == +0, non-finite logits
+ * skipped and reported, unused slots id 0 / -inf. logits: rows of `vocabulary` floats, stride_bytes apart. */
+int tsp_logit_topk(const float* logits, uint64_t stride_bytes, uint32_t rows, uint32_t vocabulary, void* partial_scratch,
+                   uint64_t scratch_bytes, void* out_rows, uint64_t out_bytes, void* stream);
 
 #ifdef __cplusplus
 }

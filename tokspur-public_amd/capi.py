@@ -455,6 +455,38 @@ def profile_end():
     return {rows[i].name.decode(): (rows[i].launches, rows[i].total_ms, rows[i].min_ms) for i in range(min(n.value, 64))}
 
 
+TOPK_ROW_DTYPE = np.dtype([("vocabulary", "<u4"), ("count", "<u4"), ("first_nonfinite_col", "<u4"), ("first_subnormal_col", "<u4"),
+                           ("ids", "<u4", 64), ("logits", "<f4", 64)])
+
+
+def logit_topk_scratch_bytes(max_rows, max_vocabulary=1 << 20):
+    f = dll().tsp_logit_topk_scratch_bytes
+    f.restype = C.c_uint64
+    n = f(C.c_uint32(max_rows), C.c_uint32(max_vocabulary))
+    if n == 0:
+        raise FormatError(dll().tsp_last_error().decode())
+    return n
+
+
+def logit_topk_output_bytes(max_rows):
+    f = dll().tsp_logit_topk_output_bytes
+    f.restype = C.c_uint64
+    n = f(C.c_uint32(max_rows))
+    if n == 0:
+        raise FormatError(dll().tsp_last_error().decode())
+    return n
+
+
+def logit_topk(dev, logits, rows, vocabulary, stride_bytes=None, scratch=None, out=None):
+    """Row top-64 (`logit_topk`): returns the device buffer of 528-byte rows; view it with TOPK_ROW_DTYPE on the host."""
+    stride_bytes = vocabulary * 4 if stride_bytes is None else stride_bytes
+    scratch = dev.empty(logit_topk_scratch_bytes(rows, vocabulary), "uint8") if scratch is None else scratch
+    out = dev.empty(logit_topk_output_bytes(rows), "uint8") if out is None else out
+    check(dll().tsp_logit_topk(dev.ptr(logits), C.c_uint64(stride_bytes), C.c_uint32(rows), C.c_uint32(vocabulary), dev.ptr(scratch),
+                               C.c_uint64(dev.nbytes(scratch)), dev.ptr(out), C.c_uint64(dev.nbytes(out)), dev.stream()))
+    return out
+
+
 def calibration_copy(dev, dst, src):
     """Plain copy kernel of a known size (scales a profiler's HBM byte counters)."""
     check(dll().tsp_calibration_copy(dev.ptr(dst), dev.ptr(src), C.c_uint64(dev.nbytes(src)), dev.stream()))
