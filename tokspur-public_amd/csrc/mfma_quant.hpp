@@ -1,0 +1,118 @@
+// Shared pieces of the matrix-core kernels: vector types, the LDS-only barrier, and the unpacking of K-quant blocks
+// into MFMA B fragments of exact integer products (sc * q for Q4_K, sc * (q - 32) for Q6_K) as packed halves.
+#pragma once
+#include "decode.hpp"
+
+namespace tsp {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+enum BKind : int { B_Q4K_RAW = 0, B_Q4K_PLANAR = 1, B_Q6K_PLANAR = 2 };
+
+// Workgroup barrier that waits for this wave's LDS traffic only. __syncthreads() also drains every outstanding
+// global load, which would serialise the prefetch of the next K step behind the barrier.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+__device__ __forceinline__ f16x2 as_h2(uint32_t bits) { return __builtin_bit_cast(f16x2, bits); }
+__device__ __forceinline__ uint32_t as_u32(f16x2 v) { return __builtin_bit_cast(uint32_t, v); }
+__device__ __forceinline__ f16x2 splat(float v) { const _Float16 h = _Float16(v); return f16x2{h, h}; }
+// one rounding per lane: the products below are only exact as fused multiply-adds
+__device__ __forceinline__ f16x2 fma2(f16x2 a, f16x2 b, f16x2 c) { return __builtin_elementwise_fma(a, b, c); }
+
+// Bytes (b0, b1) resp. (b2, b3) of `codes` into the low bytes of two f16 lanes whose high bytes are `hi`.
+__device__ __forceinline__ uint32_t spread01(uint32_t codes, uint32_t hi) { return __builtin_amdgcn_perm(hi, codes, 0x04010400u); }
+__device__ __forceinline__ uint32_t spread23(uint32_t codes, uint32_t hi) { return __builtin_amdgcn_perm(hi, codes, 0x04030402u); }
+
+// Eight codes 0..15 (one per byte of c0, c1) times the integer scale: (1024 + q) * sc - 1024 * sc, exact in f16.
+__device__ __forceinline__ f16x8 scaled8_q4(uint32_t c0, uint32_t c1, f16x2 sc, f16x2 bias) {
+    constexpr uint32_t K = 0x64646464u;  // 0x64xx = 1024 + xx
+    const f16x2 p0 = fma2(as_h2(spread01(c0, K)), sc, bias), p1 = fma2(as_h2(spread23(c0, K)), sc, bias);
+    const f16x2 p2 = fma2(as_h2(spread01(c1, K)), sc, bias), p3 = fma2(as_h2(spread23(c1, K)), sc, bias);
+    return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
+
+// Eight codes 0..63: 0x5400 | (c << 4) = 64 + c, so (64 + c) * sc - 96 * sc = (c - 32) * sc.
+__device__ __forceinline__ f16x8 scaled8_q6(uint32_t c0, uint32_t c1, f16x2 sc, f16x2 bias) {
+    constexpr uint32_t K = 0x54005400u;
+    const f16x2 p0 = fma2(as_h2((spread01(c0, 0) << 4) | K), sc, bias), p1 = fma2(as_h2((spread23(c0, 0) << 4) | K), sc, bias);
+    const f16x2 p2 = fma2(as_h2((spread01(c1, 0) << 4) | K), sc, bias), p3 = fma2(as_h2((spread23(c1, 0) << 4) | K), sc, bias);
+    return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
+
+// ---------------------------------------------------------------- Q4_K operands
+struct HdrQ4 { uint32_t sc[2], mn[2]; float d, dmin; };  // eight 6-bit scales and minima, one per byte
+
+template <int BKIND>
+__device__ __forceinline__ HdrQ4 load_hdr_q4k(const uint8_t* base, const tsp_planar_spec& s, uint64_t row, uint32_t bpr, uint32_t b) {
+    const uint64_t blk = row * bpr + b;
+    HdrQ4 h;
+    if constexpr (BKIND == B_Q4K_PLANAR) {
+        const uint4 sm = *reinterpret_cast<const uint4*>(base + s.sm_offset + blk * 16);
+        const uint32_t dm = *reinterpret_cast<const uint32_t*>(base + s.dm_offset + blk * 4);
+        h.sc[0] = sm.x; h.sc[1] = sm.y; h.mn[0] = sm.z; h.mn[1] = sm.w;
+        h.d = half_bits_to_float(dm & 0xffffu); h.dmin = half_bits_to_float(dm >> 16);
+    } else {
+        const uint4 g = *reinterpret_cast<const uint4*>(base + blk * 144);
+        h.d = half_bits_to_float(g.x & 0xffffu); h.dmin = half_bits_to_float(g.x >> 16);
+        // 12 packed bytes -> one byte per value: sub-blocks 0..3 are the low six bits of bytes 0..7, sub-blocks
+        // 4..7 take four bits from bytes 8..11 and two from the top of bytes 0..7
+        h.sc[0] = g.y & 0x3f3f3f3fu;
+        h.mn[0] = g.z & 0x3f3f3f3fu;
+        h.sc[1] = (g.w & 0x0f0f0f0fu) | ((g.y >> 2) & 0x30303030u);
+        h.mn[1] = ((g.w >> 4) & 0x0f0f0f0fu) | ((g.z >> 2) & 0x30303030u);
+    }
+    return h;
+}
+
+// Fragments of pair P: bytes 16h..16h+15 of the 32-byte pair; low nibbles (HI = 0) are sub-block 2P, high nibbles
+// sub-block 2P+1. Fragment f of a half covers activation columns HI*32 + 16h + f*8 .. +8 of the 64-column slab.
+template <int P, int HI>
+__device__ __forceinline__ void frags_q4k(const u32x4& raw, const HdrQ4& h, f16x8 frag[2]) {
+    constexpr uint32_t M4 = 0x0f0f0f0fu;
+    const uint32_t sc = (h.sc[P >> 1] >> ((P & 1) * 16 + HI * 8)) & 0xffu;
+    const f16x2 s2 = splat(float(sc)), bias = s2 * splat(-1024.0f);
+    frag[0] = scaled8_q4((raw[0] >> (4 * HI)) & M4, (raw[1] >> (4 * HI)) & M4, s2, bias);
+    frag[1] = scaled8_q4((raw[2] >> (4 * HI)) & M4, (raw[3] >> (4 * HI)) & M4, s2, bias);
+}
+
+// B operand of the minima term: the eight integer minima, the same in both k-halves (hi and lo sums).
+__device__ __forceinline__ f16x8 minima_frag(const HdrQ4& h) {
+    constexpr uint32_t K = 0x64646464u;
+    const f16x2 one = splat(1.0f), off = splat(-1024.0f);
+    const f16x2 p0 = fma2(as_h2(spread01(h.mn[0], K)), one, off), p1 = fma2(as_h2(spread23(h.mn[0], K)), one, off);
+    const f16x2 p2 = fma2(as_h2(spread01(h.mn[1], K)), one, off), p3 = fma2(as_h2(spread23(h.mn[1], K)), one, off);
+    return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
+
+// ---------------------------------------------------------------- Q6_K operands (planes ql / qh / sc / d)
+struct RawQ6 { u32x4 la, lb, qh; uint32_t sc[2]; };  // one section: low nibbles of quarters 0/2 and 1/3, high bit pairs, 8 sub-scales
+
+// Quarter Q of the section (elements Q*32 .. Q*32+31): this lane's 16 bytes are elements Q*32 + 16h + 0..15, all in
+// the 16-weight group 2Q + h. Fragment f covers activation columns Q*32 + 16h + f*8 .. +8 of the section.
+template <int Q>
+__device__ __forceinline__ void frags_q6k(const RawQ6& r, uint32_t khalf, f16x8 frag[2]) {
+    constexpr uint32_t M4 = 0x0f0f0f0fu, M2 = 0x30303030u;
+    const u32x4& l = (Q & 1) ? r.lb : r.la;
+    const uint32_t g = 2 * Q + khalf;
+    const int sc = int(int8_t((r.sc[g >> 2] >> ((g & 3) * 8)) & 0xffu));
+    const f16x2 s2 = splat(float(sc)), bias = s2 * splat(-96.0f);
+    uint32_t c[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t low = Q < 2 ? l[i] & M4 : (l[i] >> 4) & M4;
+        uint32_t high;  // bits 2Q..2Q+1 of qh move to bits 4..5 of the code
+        if constexpr (Q == 0) high = r.qh[i] << 4;
+        else if constexpr (Q == 1) high = r.qh[i] << 2;
+        else if constexpr (Q == 2) high = r.qh[i];
+        else high = r.qh[i] >> 2;
+        c[i] = low | (high & M2);
+    }
+    frag[0] = scaled8_q6(c[0], c[1], s2, bias);
+    frag[1] = scaled8_q6(c[2], c[3], s2, bias);
+}
+
+
+}  // namespace tsp

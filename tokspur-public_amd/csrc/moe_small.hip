@@ -10,6 +10,7 @@
 // and the up row of the same hidden unit, so SwiGLU needs one cross-lane move), and Q6_K planes
 // for the down projection. Every other planar encoding goes through the generic arm.
 #include "decode.hpp"
+#include "skinny.hpp"
 
 using namespace tsp;
 
@@ -407,8 +408,15 @@ uint32_t record_slots(const SmallMoeArgs& a) {
     return routes < 128 ? routes : 128;
 }
 
+SkinnyMoe skinny_view(const SmallMoeArgs& a) {
+    return SkinnyMoe{a.pair_lo, a.pair_hi, a.down, a.ids, a.meta, a.x, a.h, a.y, a.x_stride, a.h_stride, a.y_stride,
+                     a.channels, a.hidden, a.experts, a.selected, a.tokens, record_slots(a), a.gu, a.dn, a.error_word};
+}
+
 int launch_gate_up(const SmallMoeArgs& a, hipStream_t s) {
     const uint32_t records = record_slots(a);
+    if (skinny_moe_supported(a.gu.source_type, a.dn.source_type, a.channels, a.hidden, a.x, a.x_stride, a.h, a.h_stride, false))
+        return skinny_moe_gate_up(skinny_view(a), s);
     const bool x_aligned = reinterpret_cast<uintptr_t>(a.x) % 16 == 0 && a.x_stride % 16 == 0;
     if (a.gu.source_type == 12 && x_aligned && (a.channels == 512 || a.channels == 1024 || a.channels == 2048)) {
         const uint32_t bpr = a.channels / 256;
@@ -436,6 +444,8 @@ int launch_gate_up(const SmallMoeArgs& a, hipStream_t s) {
 
 int launch_down(const SmallMoeArgs& a, hipStream_t s) {
     const uint32_t records = record_slots(a);
+    if (a.dn.source_type == 14 && a.hidden % 256 == 0 && a.hidden <= 2048 && reinterpret_cast<uintptr_t>(a.h) % 16 == 0 && a.h_stride % 16 == 0)
+        return skinny_moe_down(skinny_view(a), s);
     const bool h_aligned = reinterpret_cast<uintptr_t>(a.h) % 16 == 0 && a.h_stride % 16 == 0;
     if (a.dn.source_type == 14 && h_aligned && (a.hidden == 256 || a.hidden == 512 || a.hidden == 1024)) {
         const uint32_t bpr = a.hidden / 256;

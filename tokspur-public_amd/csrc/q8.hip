@@ -12,6 +12,7 @@
 //
 // so the four bytes convert with v_cvt_f32_ubyte0..3 and a masked byte (u = 0x80) contributes 0.
 #include "decode.hpp"
+#include "q8_mfma.hpp"
 
 using namespace tsp;
 
@@ -180,6 +181,7 @@ extern "C" int tsp_q8_matvec_many(uint32_t layout, const void* matrix, uint64_t 
     TSP_REQUIRE(!ranges_overlap(y, y_span, matrix, matrix_bytes) && !ranges_overlap(y, y_span, x, x_span), "Q8-many output overlaps an input");
     const Q8Args a{static_cast<const uint8_t*>(matrix), x, y, columns, rows, error_word};
     const auto s = static_cast<hipStream_t>(stream);
+    if (layout == TSP_LAYOUT_GGUF && q8_mfma_supported(matrix, x, columns, rows)) return q8_mfma(matrix, x, y, columns, rows, width, error_word, s);
     switch (width) {
     case 1: return launch<1>(layout, a, s);
     case 2: return launch<2>(layout, a, s);

@@ -1,0 +1,229 @@
+// Q8_0 GEMV for up to eight token rows on the matrix cores (LM head, verify): y[m, r] = sum_k d[r, k/32] * q[r, k] * x[m, k].
+//
+// A Q8_0 row is a run of 34-byte blocks (f16 scale + 32 int8). The int8 quants are exact halves, so a block is two
+// 32x32x16 MFMA steps of the integer quants against the activations; the block's scale multiplies the f32 result
+// once (4 fused multiply-adds per lane for the eight live rows). The activations are scaled by a power of two and
+// split into hi + lo halves, staged once in LDS for all of K, so the result carries 22 significant bits of x: this
+// is the f32 GEMV of the engine to within f32 accumulation error, at ~1.3 VALU operations per weight byte whatever the
+// number of token rows.
+//
+// Raw rows are only 2-byte aligned inside, so the bytes travel global -> registers -> LDS -> registers: a wave reads
+// its 32 weight rows x 8 blocks (272 contiguous bytes per row, 16-byte aligned because 8 blocks = 17 x 16 bytes) with
+// whole-chunk loads by consecutive lanes, parks them in a wave-private LDS tile whose row stride (280 bytes) spreads
+// the rows over all banks, and each lane then picks its 16 quants of a block with aligned dword reads and a byte
+// funnel shift. The next group of 8 blocks is in flight while the current one is multiplied.
+//
+// Workgroups are persistent (one per compute unit, 8 waves): the activations are staged once per workgroup and each
+// wave then walks the 32-row tiles of the matrix with stride (workgroups x 8).
+#include "q8_mfma.hpp"
+
+#include <type_traits>
+
+#include "mfma_quant.hpp"
+
+using namespace tsp;
+
+namespace {
+
+constexpr int kRows = 8;
+constexpr uint32_t kWaves = 8, kThreads = kWaves * kWave;
+constexpr uint32_t kGroupBlocks = 8, kGroupBytes = kGroupBlocks * 34, kGroupChunks = kGroupBytes / 16;  // 272 B = 17 chunks
+constexpr uint32_t kTileStride = 280;                     // bytes between rows of the LDS weight tile
+constexpr uint32_t kTileBytes = 32 * kTileStride;         // 8 960 B per wave
+constexpr uint32_t kStageLoads = (32 * kGroupChunks + kWave - 1) / kWave;  // 9 chunk loads per lane and group (the last half used)
+
+struct Q8MfmaArgs {
+    const uint8_t* matrix;
+    const float* x;   // token-major [M, columns]
+    float* y;         // token-major [M, rows]
+    uint32_t columns, rows, m;
+    uint32_t* error_word;
+};
+
+// Eight int8 quants (two dwords) as exact halves: q ^ 0x80 = q + 128 in 0..255, 0x6400 | u = 1024 + u, minus 1152.
+__device__ __forceinline__ f16x8 quants8(uint32_t w0, uint32_t w1) {
+    constexpr uint32_t K = 0x64646464u;
+    const uint32_t u0 = w0 ^ 0x80808080u, u1 = w1 ^ 0x80808080u;
+    const f16x2 off = splat(-1152.0f);
+    const f16x2 p0 = as_h2(spread01(u0, K)) + off, p1 = as_h2(spread23(u0, K)) + off;
+    const f16x2 p2 = as_h2(spread01(u1, K)) + off, p3 = as_h2(spread23(u1, K)) + off;
+    return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
+
+__global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [hi plane][lo plane][8 weight tiles]
+    __shared__ float wave_max[kWaves];
+
+    const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const uint32_t col = lane % 32, khalf = lane / 32;
+    const uint32_t K = a.columns, chunks = K / 8, groups = K / 256, row_bytes = K / 32 * 34;
+    _Float16* const a_hi = reinterpret_cast<_Float16*>(lds);
+    _Float16* const a_lo = a_hi + kRows * K;
+    uint8_t* const tile = lds + 2 * kRows * K * 2 + wave * kTileBytes;
+
+    // ---- stage the token rows: largest magnitude -> power-of-two scale -> hi/lo halves, 16-byte chunks swizzled by row
+    uint32_t bad = 0;
+    float biggest = 0;
+    for (uint32_t i = tid; i < a.m * (K / 4); i += kThreads) {
+        const float4 v = reinterpret_cast<const float4*>(a.x)[i];
+        if (nonfinite(v.x) || nonfinite(v.y) || nonfinite(v.z) || nonfinite(v.w)) bad = TSP_ERRBIT_NONFINITE;
+        biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    }
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1) biggest = fmaxf(biggest, __shfl_xor(biggest, step, kWave));
+    if (lane == 0) wave_max[wave] = biggest;
+    __syncthreads();
+    biggest = wave_max[0];
+#pragma unroll
+    for (uint32_t w = 1; w < kWaves; ++w) biggest = fmaxf(biggest, wave_max[w]);
+    float scale = 1.0f, inv_scale = 1.0f;
+    if (biggest > 0 && !nonfinite(biggest)) {
+        const int e = int((__float_as_uint(biggest) >> 23) & 0xffu) - 127;
+        int shift = 13 - e;
+        shift = shift > 100 ? 100 : shift < -100 ? -100 : shift;
+        scale = __uint_as_float(uint32_t(127 + shift) << 23);
+        inv_scale = __uint_as_float(uint32_t(127 - shift) << 23);
+    }
+    for (uint32_t i = tid; i < kRows * chunks; i += kThreads) {
+        const uint32_t r = i / chunks, c = i % chunks;
+        f16x8 hi{}, lo{};
+        if (r < a.m) {
+            const float4* src = reinterpret_cast<const float4*>(a.x + uint64_t(r) * K + c * 8);
+            const float4 v0 = src[0], v1 = src[1];
+            const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float s = v[e] * scale;
+                hi[e] = _Float16(s);
+                lo[e] = _Float16(s - float(hi[e]));
+            }
+        }
+        const uint32_t at = (r * chunks + (c ^ r)) * 8;
+        *reinterpret_cast<f16x8*>(a_hi + at) = hi;
+        *reinterpret_cast<f16x8*>(a_lo + at) = lo;
+    }
+    __syncthreads();
+
+    const uint32_t arow = col & 7;
+    auto a_frag = [&](const _Float16* plane, uint32_t chunk) {
+        return *reinterpret_cast<const f16x8*>(plane + (arow * chunks + (chunk ^ arow)) * 8);
+    };
+    // chunk `id` of a group tile: row id / 17 of the wave's 32, bytes (id % 17) * 16 of that row's 272
+    uint2 stage[kStageLoads][2];
+    auto fetch_group = [&](uint32_t row0, uint32_t group) {
+#pragma unroll
+        for (uint32_t t = 0; t < kStageLoads; ++t) {
+            uint32_t id = t * kWave + lane;
+            id = id < 32 * kGroupChunks ? id : 32 * kGroupChunks - 1;  // the tail lanes repeat the last chunk
+            uint32_t row = row0 + id / kGroupChunks;
+            row = row < a.rows ? row : a.rows - 1;
+            const uint4 v = *reinterpret_cast<const uint4*>(a.matrix + uint64_t(row) * row_bytes + group * kGroupBytes + (id % kGroupChunks) * 16);
+            stage[t][0] = uint2{v.x, v.y};
+            stage[t][1] = uint2{v.z, v.w};
+        }
+    };
+    auto store_group = [&]() {
+#pragma unroll
+        for (uint32_t t = 0; t < kStageLoads; ++t) {
+            uint32_t id = t * kWave + lane;
+            id = id < 32 * kGroupChunks ? id : 32 * kGroupChunks - 1;
+            uint8_t* at = tile + (id / kGroupChunks) * kTileStride + (id % kGroupChunks) * 16;  // 8-byte aligned
+            *reinterpret_cast<uint2*>(at) = stage[t][0];
+            *reinterpret_cast<uint2*>(at + 8) = stage[t][1];
+        }
+    };
+
+    // (tile, group) items of this wave in order; the next item's bytes are requested before the current one is multiplied
+    const uint32_t tiles = (a.rows + 31) / 32, walkers = gridDim.x * kWaves, first = blockIdx.x * kWaves + wave;
+    if (first < tiles) fetch_group(first * 32, 0);
+    for (uint32_t t = first; t < tiles; t += walkers) {
+        const uint32_t row0 = t * 32;
+        f32x16 acc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+        for (uint32_t g = 0; g < groups; ++g) {
+            store_group();  // the previous item's reads were issued before this point; LDS serves a wave in order
+            const bool last = g + 1 == groups;
+            const uint32_t next_tile = last ? (t + walkers < tiles ? t + walkers : t) : t;
+            fetch_group(next_tile * 32, last ? 0 : g + 1);  // past the end: a harmless repeat of this tile's first group
+            const uint8_t* mine = tile + col * kTileStride + khalf * 16;
+            auto block = [&](auto b_tag) {
+                constexpr int B = decltype(b_tag)::value;
+                // quants at byte 34 B + 2 + 16 h of the row: dword aligned for odd B, 2 bytes past a dword for even B
+                constexpr uint32_t Q_AT = 34 * B + 2, ALIGNED = Q_AT & ~3u;
+                uint32_t w[4];
+                if constexpr (Q_AT % 4 == 0) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) w[i] = *reinterpret_cast<const uint32_t*>(mine + ALIGNED + 4 * i);
+                } else {
+                    uint32_t d[5];
+#pragma unroll
+                    for (int i = 0; i < 5; ++i) d[i] = *reinterpret_cast<const uint32_t*>(mine + ALIGNED + 4 * i);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) w[i] = __builtin_amdgcn_alignbyte(d[i + 1], d[i], 2);
+                }
+                const float scale_d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(tile + col * kTileStride + 34 * B));
+                const f16x8 b0 = quants8(w[0], w[1]), b1 = quants8(w[2], w[3]);
+                const uint32_t chunk = g * 32 + B * 4 + khalf * 2;  // columns g*256 + B*32 + 16h
+                const f32x16 zero{};
+                // two independent accumulation chains (hi and lo halves of the rows) per block
+                f32x16 part_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag(a_hi, chunk), b0, zero, 0, 0, 0);
+                f32x16 part_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag(a_lo, chunk), b0, zero, 0, 0, 0);
+                part_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag(a_hi, chunk + 1), b1, part_hi, 0, 0, 0);
+                part_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag(a_lo, chunk + 1), b1, part_lo, 0, 0, 0);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[v] = __builtin_fmaf(scale_d, part_hi[v] + part_lo[v], acc[v]);  // rows 4 * khalf + v
+            };
+            block(std::integral_constant<int, 0>{});
+            block(std::integral_constant<int, 1>{});
+            block(std::integral_constant<int, 2>{});
+            block(std::integral_constant<int, 3>{});
+            block(std::integral_constant<int, 4>{});
+            block(std::integral_constant<int, 5>{});
+            block(std::integral_constant<int, 6>{});
+            block(std::integral_constant<int, 7>{});
+        }
+        const uint32_t r = row0 + col;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const uint32_t m = 4 * khalf + v;
+            if (m < a.m && r < a.rows) {
+                const float val = acc[v] * inv_scale;
+                if (nonfinite(val)) bad = TSP_ERRBIT_NONFINITE;
+                a.y[uint64_t(m) * a.rows + r] = val;
+            }
+        }
+    }
+    publish_error(bad, a.error_word);
+}
+
+}  // namespace
+
+namespace tsp {
+
+bool q8_mfma_supported(const void* matrix, const float* x, uint32_t columns, uint32_t rows) {
+    return columns % 256 == 0 && columns <= 2048 && rows >= 32 && reinterpret_cast<uintptr_t>(matrix) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(x) % 16 == 0;
+}
+
+int q8_mfma(const void* matrix, const float* x, float* y, uint32_t columns, uint32_t rows, uint32_t width, uint32_t* error_word, hipStream_t s) {
+    const Q8MfmaArgs a{static_cast<const uint8_t*>(matrix), x, y, columns, rows, width, error_word};
+    const uint32_t lds_bytes = 2 * kRows * columns * 2 + kWaves * kTileBytes;
+    static bool raised = false;
+    static int compute_units = 0;
+    if (!raised) {
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    int(2 * kRows * 2048 * 2 + kWaves * kTileBytes)));
+        int device = 0;
+        TSP_HIP(hipGetDevice(&device));
+        TSP_HIP(hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device));
+        raised = true;
+    }
+    const uint32_t tiles = (rows + 31) / 32;
+    uint32_t grid = uint32_t(compute_units > 0 ? compute_units : 256);
+    if (grid * kWaves > tiles) grid = (tiles + kWaves - 1) / kWaves;
+    TSP_LAUNCH("q8_mfma", s, q8_mfma_kernel<<<grid, kThreads, lds_bytes, s>>>(a));
+    return launch_status("q8_mfma");
+}
+
+}  // namespace tsp

@@ -1,0 +1,412 @@
+// Matrix products with at most eight activation rows per weight matrix (decode, verify, the T <= 8 routed MoE):
+// out[m, n] = sum_k x[m, k] * dec(W[n, k]),  m < 8, on the matrix cores, every weight byte read once.
+//
+// These products are bound by HBM and, with scalar code, by the dequantisation arithmetic: converting and
+// multiplying each weight for each row costs 3+ VALU operations per weight and row. Here the weights go to
+// v_mfma_f32_32x32x16_f16 as exact integer factors (see mfma_quant.hpp: ~1.4 operations per weight, independent
+// of the number of rows), the block scales are applied in f32 once per 256-column super-block, and the eight
+// activation rows occupy 8 of the 32 rows of the MFMA A operand (the matrix cores have capacity to spare).
+//
+// f32 accuracy with f16 operands: the rows are scaled by a power of two so that their largest magnitude lands
+// near 2^14 and split as hi + lo halves (22 significant bits); both halves multiply the same integer weight
+// fragment and accumulate into the same f32 accumulator. Nothing else is rounded before the f32 scaling.
+//
+// One workgroup = one task (a weight matrix and up to 8 rows) x 256 weight rows (128 hidden units for gate/up).
+// The rows are staged once, for all of K, in LDS (hi and lo planes, 16-byte chunks XOR-swizzled by row so the
+// eight rows of a fragment read fall in different banks); after that the four waves run independently, with no
+// barrier in the K loop, each streaming its own 64 weight rows with one super-block of loads in flight.
+#include "skinny.hpp"
+
+#include <type_traits>
+
+#include "mfma_quant.hpp"
+
+using namespace tsp;
+
+namespace {
+
+constexpr int kRows = 8;
+constexpr uint32_t kMaxColumns = 2048;  // 2 planes x 8 rows x 2048 halfs = 64 KB of LDS
+
+enum Source : int { SRC_DENSE = 0, SRC_RECORD_TOKENS = 1, SRC_RECORD_ROUTES = 2 };
+enum Output : int { OUT_ROWS = 0, OUT_SWIGLU = 1 };
+
+struct SkinnyArgs {
+    const float* x;        // activation rows, x_stride bytes apart
+    uint64_t x_stride;
+    const uint8_t* w0;     // dense matrix / pair_lo / down experts
+    const uint8_t* w1;     // pair_hi
+    tsp_planar_spec spec;
+    uint32_t experts, selected, tokens;
+    const uint32_t* ids;   // routes when there is no union block
+    const uint32_t* meta;  // union records
+    uint32_t m, n, k;      // dense: rows of x; weight rows (hidden units for SwiGLU); columns
+    float* out;            // rows out_stride bytes apart
+    uint64_t out_stride;
+    uint32_t* error_word;
+};
+
+struct Task { uint32_t expert, count, src[kRows], dst[kRows]; };
+
+// Task `index`: the dense rows, a union record, or a single route when there is no union block.
+template <int SRC>
+__device__ __forceinline__ bool load_task(const SkinnyArgs& a, uint32_t index, Task& t) {
+    if constexpr (SRC == SRC_DENSE) {
+        t.expert = 0; t.count = a.m;
+#pragma unroll
+        for (int k = 0; k < kRows; ++k) t.src[k] = t.dst[k] = k;
+        return index == 0;
+    } else if (a.meta) {
+        if (index >= a.meta[6]) return false;
+        t.expert = a.meta[8 + index];
+        t.count = a.meta[136 + index];
+#pragma unroll
+        for (int k = 0; k < kRows; ++k) {
+            const uint32_t token = a.meta[264 + index * 8 + k], route = a.meta[1288 + index * 8 + k];
+            t.src[k] = SRC == SRC_RECORD_TOKENS ? token : route;
+            t.dst[k] = route;
+        }
+        return true;
+    } else {
+        if (index >= a.tokens * a.selected) return false;
+        t.expert = a.ids[index];
+        t.count = 1;
+#pragma unroll
+        for (int k = 0; k < kRows; ++k) { t.src[k] = SRC == SRC_RECORD_TOKENS ? index / a.selected : index; t.dst[k] = index; }
+        return true;
+    }
+}
+
+// KS = number of K slices: a workgroup has 4 * KS waves, wave w owns weight-row group w % 4 and K slice w / 4; the
+// slices' partial sums meet in LDS at the end (fixed order, so results do not depend on timing). With about one task
+// tile per compute unit, slicing K is what puts more than one wave on each SIMD.
+template <int BKIND, int OUT, int SRC, int KS>
+__global__ __launch_bounds__(256 * KS, 2) void skinny_kernel(SkinnyArgs a) {
+    constexpr bool Q6 = BKIND == B_Q6K_PLANAR;
+    constexpr uint32_t THREADS = 256 * KS;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [hi plane][lo plane][activation sums]
+    __shared__ float wave_max[4 * KS];
+
+    const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = (tid / kWave) % 4, slice = tid / (4 * kWave);
+    const uint32_t col = lane % 32, khalf = lane / 32;
+    Task task;
+    if (!load_task<SRC>(a, blockIdx.y, task)) return;
+    if (task.expert >= a.experts || task.count == 0 || task.count > kRows) {
+        if (tid == 0 && blockIdx.x == 0 && (task.expert >= a.experts || task.count > kRows)) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+        return;
+    }
+    const uint32_t K = a.k, bpr = K / 256, chunks = K / 8;  // 16-byte chunks per row and plane
+    _Float16* const a_hi = reinterpret_cast<_Float16*>(lds);
+    _Float16* const a_lo = a_hi + kRows * K;
+    _Float16* const sums = a_lo + kRows * K;  // [row][super-block][8 hi, 8 lo] of (sub-block sum / 32), Q4_K only
+
+    // ---- stage the rows: largest magnitude -> power-of-two scale -> hi/lo halves (+ sub-block sums)
+    uint32_t bad = 0;
+    float biggest = 0;
+    for (uint32_t i = tid; i < kRows * K / 4; i += THREADS) {
+        const uint32_t r = i / (K / 4), c4 = i % (K / 4);
+        if (r < task.count) {
+            const float4 v = *reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.x) + uint64_t(task.src[r]) * a.x_stride + c4 * 16);
+            if (nonfinite(v.x) || nonfinite(v.y) || nonfinite(v.z) || nonfinite(v.w)) bad = TSP_ERRBIT_NONFINITE;
+            biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        }
+    }
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1) biggest = fmaxf(biggest, __shfl_xor(biggest, step, kWave));
+    if (lane == 0) wave_max[tid / kWave] = biggest;
+    __syncthreads();
+    biggest = wave_max[0];
+#pragma unroll
+    for (int w = 1; w < 4 * KS; ++w) biggest = fmaxf(biggest, wave_max[w]);
+    // scale = 2^(13 - exponent(biggest)): the largest |x * scale| is below 2^15, the sub-block sums / 32 below 2^15 too
+    float scale = 1.0f, inv_scale = 1.0f;
+    if (biggest > 0 && !nonfinite(biggest)) {
+        const int e = int((__float_as_uint(biggest) >> 23) & 0xffu) - 127;
+        int shift = 13 - e;
+        shift = shift > 100 ? 100 : shift < -100 ? -100 : shift;
+        scale = __uint_as_float(uint32_t(127 + shift) << 23);
+        inv_scale = __uint_as_float(uint32_t(127 - shift) << 23);
+    }
+    for (uint32_t i = tid; i < kRows * chunks; i += THREADS) {
+        const uint32_t r = i / chunks, c = i % chunks;
+        f16x8 hi{}, lo{};
+        float sum = 0;
+        if (r < task.count) {
+            const float4* src = reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.x) + uint64_t(task.src[r]) * a.x_stride + c * 32);
+            const float4 v0 = src[0], v1 = src[1];
+            const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float s = v[e] * scale;
+                hi[e] = _Float16(s);
+                lo[e] = _Float16(s - float(hi[e]));
+                sum += s;
+            }
+        }
+        const uint32_t at = (r * chunks + (c ^ r)) * 8;
+        *reinterpret_cast<f16x8*>(a_hi + at) = hi;
+        *reinterpret_cast<f16x8*>(a_lo + at) = lo;
+        if constexpr (!Q6) {
+            // four neighbouring lanes hold the four chunks of one 32-column sub-block (chunks is a multiple of 32)
+            sum += __shfl_xor(sum, 1, kWave);
+            sum += __shfl_xor(sum, 2, kWave);
+            if ((c & 3) == 0) {
+                const float s32 = sum * 0.03125f;
+                const _Float16 h = _Float16(s32);
+                const uint32_t sub = c / 4;
+                _Float16* o = sums + (r * bpr + sub / 8) * 16 + sub % 8;
+                o[0] = h;
+                o[8] = _Float16(s32 - float(h));
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- weight rows of this wave
+    const uint8_t* wbase[2];
+    uint32_t wrow[2], out_col[2];
+    bool col_live[2];
+    if constexpr (OUT == OUT_SWIGLU) {
+        const uint32_t unit = blockIdx.x * 128 + wave * 32 + col;
+        const uint32_t half_e = a.experts / 2;
+        const uint8_t* pair = (task.expert < half_e ? a.w0 : a.w1) + uint64_t(task.expert < half_e ? task.expert : task.expert - half_e) * 2 * a.spec.planar_expert_bytes;
+        wbase[0] = pair; wbase[1] = pair + a.spec.planar_expert_bytes;
+        col_live[0] = col_live[1] = unit < a.n;
+        wrow[0] = wrow[1] = col_live[0] ? unit : a.n - 1;
+        out_col[0] = out_col[1] = unit;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t n = blockIdx.x * 256 + wave * 64 + j * 32 + col;
+            col_live[j] = n < a.n;
+            wrow[j] = col_live[j] ? n : a.n - 1;
+            out_col[j] = n;
+            wbase[j] = BKIND == B_Q4K_RAW ? a.w0 : a.w0 + uint64_t(task.expert) * a.spec.planar_expert_bytes;
+        }
+    }
+
+    const uint32_t b_begin = slice * (bpr / KS), b_end = b_begin + bpr / KS;  // the host picks KS so that it divides bpr
+    f32x16 acc[2], blk[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.0f;
+
+    // A fragment of the 16-column step whose first column is 8 * chunk: rows 8..31 of the operand repeat rows 0..7
+    const uint32_t arow = col & 7;
+    auto a_frag = [&](const _Float16* plane, uint32_t chunk) {
+        return *reinterpret_cast<const f16x8*>(plane + (arow * chunks + (chunk ^ arow)) * 8);
+    };
+    // both halves of the rows against the same weight fragments; `first` starts the super-block accumulator from zero
+    auto mfma = [&](uint32_t chunk, const f16x8& b0, const f16x8& b1, bool first) {
+        const f16x8 ah = a_frag(a_hi, chunk), al = a_frag(a_lo, chunk);
+        if (first) {
+            const f32x16 zero{};
+            blk[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b0, zero, 0, 0, 0);
+            blk[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b1, zero, 0, 0, 0);
+        } else {
+            blk[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b0, blk[0], 0, 0, 0);
+            blk[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b1, blk[1], 0, 0, 0);
+        }
+        blk[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b0, blk[0], 0, 0, 0);
+        blk[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b1, blk[1], 0, 0, 0);
+    };
+    // only accumulator registers 0..3 hold rows 0..7 (row = 4 * khalf + v)
+    auto fold = [&](float d0, float d1) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            acc[0][v] = __builtin_fmaf(d0, blk[0][v], acc[0][v]);
+            acc[1][v] = __builtin_fmaf(d1, blk[1][v], acc[1][v]);
+        }
+    };
+
+    if constexpr (Q6) {
+        struct BlockQ6 { u32x4 la[2], lb[2], qh[2]; uint32_t sc[4]; float d; };
+        auto load_block = [&](uint32_t b, int j) {
+            b = b < bpr ? b : bpr - 1;
+            const uint64_t at = uint64_t(wrow[j]) * bpr + b;
+            const uint8_t* ql = wbase[j] + a.spec.qs_offset + at * 128 + khalf * 16;
+            const uint8_t* qh = wbase[j] + a.spec.qh_offset + at * 64 + khalf * 16;
+            BlockQ6 r;
+#pragma unroll
+            for (int sec = 0; sec < 2; ++sec) {
+                r.la[sec] = *reinterpret_cast<const u32x4*>(ql + sec * 64);
+                r.lb[sec] = *reinterpret_cast<const u32x4*>(ql + sec * 64 + 32);
+                r.qh[sec] = *reinterpret_cast<const u32x4*>(qh + sec * 32);
+            }
+            const uint4 sc16 = *reinterpret_cast<const uint4*>(wbase[j] + a.spec.sm_offset + at * 16);
+            r.sc[0] = sc16.x; r.sc[1] = sc16.y; r.sc[2] = sc16.z; r.sc[3] = sc16.w;
+            r.d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(wbase[j] + a.spec.dm_offset + at * 2));
+            return r;
+        };
+        BlockQ6 cur[2] = {load_block(b_begin, 0), load_block(b_begin, 1)};
+        for (uint32_t b = b_begin; b < b_end; ++b) {
+            const BlockQ6 nxt[2] = {load_block(b + 1, 0), load_block(b + 1, 1)};
+            auto section = [&](auto sec_tag) {
+                constexpr int SEC = decltype(sec_tag)::value;
+                RawQ6 raw[2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    raw[j].la = cur[j].la[SEC]; raw[j].lb = cur[j].lb[SEC]; raw[j].qh = cur[j].qh[SEC];
+                    raw[j].sc[0] = cur[j].sc[SEC * 2]; raw[j].sc[1] = cur[j].sc[SEC * 2 + 1];
+                }
+                auto quarter = [&](auto q_tag) {
+                    constexpr int Q = decltype(q_tag)::value;
+                    f16x8 f0[2], f1[2];
+                    frags_q6k<Q>(raw[0], khalf, f0);
+                    frags_q6k<Q>(raw[1], khalf, f1);
+                    const uint32_t chunk = b * 32 + SEC * 16 + Q * 4 + khalf * 2;  // columns b*256 + SEC*128 + Q*32 + 16h
+                    mfma(chunk, f0[0], f1[0], SEC == 0 && Q == 0);
+                    mfma(chunk + 1, f0[1], f1[1], false);
+                };
+                quarter(std::integral_constant<int, 0>{});
+                quarter(std::integral_constant<int, 1>{});
+                quarter(std::integral_constant<int, 2>{});
+                quarter(std::integral_constant<int, 3>{});
+            };
+            section(std::integral_constant<int, 0>{});
+            section(std::integral_constant<int, 1>{});
+            fold(cur[0].d, cur[1].d);
+            cur[0] = nxt[0]; cur[1] = nxt[1];
+        }
+    } else {
+        constexpr uint32_t BLK = BKIND == B_Q4K_PLANAR ? 128 : 144, QS_AT = BKIND == B_Q4K_PLANAR ? 0 : 16;
+        struct BlockQ4 { u32x4 pair[4]; HdrQ4 hdr; };
+        auto load_block = [&](uint32_t b, int j) {
+            b = b < bpr ? b : bpr - 1;
+            const uint8_t* qs = wbase[j] + (BKIND == B_Q4K_PLANAR ? a.spec.qs_offset : 0) + (uint64_t(wrow[j]) * bpr + b) * BLK + QS_AT + khalf * 16;
+            BlockQ4 r;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) r.pair[p] = *reinterpret_cast<const u32x4*>(qs + p * 32);
+            r.hdr = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, b);
+            return r;
+        };
+        BlockQ4 cur[2] = {load_block(b_begin, 0), load_block(b_begin, 1)};
+        for (uint32_t b = b_begin; b < b_end; ++b) {
+            const BlockQ4 nxt[2] = {load_block(b + 1, 0), load_block(b + 1, 1)};
+            auto pair_step = [&](auto p_tag) {
+                constexpr int P = decltype(p_tag)::value;
+                f16x8 f0[2], f1[2];
+                const uint32_t chunk = b * 32 + P * 8 + khalf * 2;  // columns b*256 + P*64 + 16h
+                frags_q4k<P, 0>(cur[0].pair[P], cur[0].hdr, f0);
+                frags_q4k<P, 0>(cur[1].pair[P], cur[1].hdr, f1);
+                mfma(chunk, f0[0], f1[0], P == 0);
+                mfma(chunk + 1, f0[1], f1[1], false);
+                frags_q4k<P, 1>(cur[0].pair[P], cur[0].hdr, f0);
+                frags_q4k<P, 1>(cur[1].pair[P], cur[1].hdr, f1);
+                mfma(chunk + 4, f0[0], f1[0], false);
+                mfma(chunk + 5, f0[1], f1[1], false);
+            };
+            pair_step(std::integral_constant<int, 0>{});
+            pair_step(std::integral_constant<int, 1>{});
+            pair_step(std::integral_constant<int, 2>{});
+            pair_step(std::integral_constant<int, 3>{});
+            fold(cur[0].hdr.d, cur[1].hdr.d);
+            // minima: acc -= 32 * dmin * sum_s (Sx / 32)(hi + lo)[m, s] * mn[n, s]
+            const f16x8 m0 = minima_frag(cur[0].hdr), m1 = minima_frag(cur[1].hdr);
+            const f16x8 sf = *reinterpret_cast<const f16x8*>(sums + (arow * bpr + b) * 16 + khalf * 8);
+            const f32x16 zero{};
+            blk[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m0, zero, 0, 0, 0);
+            blk[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m1, zero, 0, 0, 0);
+            fold(-32.0f * cur[0].hdr.dmin, -32.0f * cur[1].hdr.dmin);
+            cur[0] = nxt[0]; cur[1] = nxt[1];
+        }
+    }
+
+    // ---- partial sums of slices 1.. are added into slice 0 in slice order; the activation planes are free by then
+    if constexpr (KS > 1) {
+        float* const partial = reinterpret_cast<float*>(lds);  // [slice - 1][wave][tile][v][lane]
+        __syncthreads();
+        if (slice > 0) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) partial[((((slice - 1) * 4 + wave) * 2 + j) * 4 + v) * kWave + lane] = acc[j][v];
+        }
+        __syncthreads();
+        if (slice > 0) { publish_error(bad, a.error_word); return; }
+#pragma unroll
+        for (int s = 1; s < KS; ++s)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[j][v] += partial[((((s - 1) * 4 + wave) * 2 + j) * 4 + v) * kWave + lane];
+    }
+    // ---- epilogue: accumulator v of tile j is row 4 * khalf + v, weight row `col`
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const uint32_t r = 4 * khalf + v;
+        if (r >= task.count) continue;
+        uint8_t* orow = reinterpret_cast<uint8_t*>(a.out) + uint64_t(task.dst[r]) * a.out_stride;
+        if constexpr (OUT == OUT_SWIGLU) {
+            if (!col_live[0]) continue;
+            const float g = acc[0][v] * inv_scale, u = acc[1][v] * inv_scale;
+            const float sg = g >= 0 ? 1.0f / (1.0f + expf(-g)) : expf(g) / (1.0f + expf(g));
+            const float h = (g * sg) * u;
+            if (nonfinite(g) || nonfinite(u) || nonfinite(h)) bad = TSP_ERRBIT_NONFINITE;
+            reinterpret_cast<float*>(orow)[out_col[0]] = h;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (!col_live[j]) continue;
+                const float val = acc[j][v] * inv_scale;
+                if (nonfinite(val)) bad = TSP_ERRBIT_NONFINITE;
+                reinterpret_cast<float*>(orow)[out_col[j]] = val;
+            }
+        }
+    }
+    publish_error(bad, a.error_word);
+}
+
+uint32_t lds_bytes(uint32_t columns, bool sums) { return 2 * kRows * columns * 2 + (sums ? kRows * (columns / 256) * 32 : 0); }
+
+template <int BKIND, int OUT, int SRC, int KS>
+int launch_sliced(const char* name, const SkinnyArgs& a, uint32_t col_tiles, uint32_t tasks, hipStream_t s) {
+    const uint32_t bytes = lds_bytes(a.k, BKIND != B_Q6K_PLANAR);
+    static bool raised = false;
+    if (!raised) {
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&skinny_kernel<BKIND, OUT, SRC, KS>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    int(lds_bytes(kMaxColumns, true))));
+        raised = true;
+    }
+    TSP_LAUNCH(name, s, skinny_kernel<BKIND, OUT, SRC, KS><<<dim3(col_tiles, tasks), 256 * KS, bytes, s>>>(a));
+    return launch_status(name);
+}
+
+// Two K slices whenever the super-blocks split evenly: the task tiles of these products number about one per compute unit.
+template <int BKIND, int OUT, int SRC>
+int launch(const char* name, const SkinnyArgs& a, uint32_t col_tiles, uint32_t tasks, hipStream_t s) {
+    if ((a.k / 256) % 2 == 0) return launch_sliced<BKIND, OUT, SRC, 2>(name, a, col_tiles, tasks, s);
+    return launch_sliced<BKIND, OUT, SRC, 1>(name, a, col_tiles, tasks, s);
+}
+
+bool aligned16(const void* p, uint64_t stride) { return reinterpret_cast<uintptr_t>(p) % 16 == 0 && stride % 16 == 0; }
+
+}  // namespace
+
+namespace tsp {
+
+bool skinny_moe_supported(uint32_t gate_up_type, uint32_t down_type, uint32_t channels, uint32_t hidden, const void* x, uint64_t x_stride,
+                          const void* h, uint64_t h_stride, bool with_down) {
+    if (gate_up_type != 12 || channels % 256 || channels > kMaxColumns || !aligned16(x, x_stride)) return false;
+    if (with_down && (down_type != 14 || hidden % 256 || hidden > kMaxColumns || !aligned16(h, h_stride))) return false;
+    return true;
+}
+
+int skinny_moe_gate_up(const SkinnyMoe& m, hipStream_t s) {
+    SkinnyArgs a{};
+    a.x = m.x; a.x_stride = m.x_stride; a.w0 = m.pair_lo; a.w1 = m.pair_hi; a.spec = m.gu; a.experts = m.experts; a.selected = m.selected;
+    a.tokens = m.tokens; a.ids = m.ids; a.meta = m.meta; a.n = m.hidden; a.k = m.channels; a.out = m.h; a.out_stride = m.h_stride;
+    a.error_word = m.error_word;
+    return launch<B_Q4K_PLANAR, OUT_SWIGLU, SRC_RECORD_TOKENS>("skinny_gate_up_swiglu", a, (m.hidden + 127) / 128, m.records, s);
+}
+
+int skinny_moe_down(const SkinnyMoe& m, hipStream_t s) {
+    SkinnyArgs a{};
+    a.x = m.h; a.x_stride = m.h_stride; a.w0 = m.down; a.spec = m.dn; a.experts = m.experts; a.selected = m.selected;
+    a.tokens = m.tokens; a.ids = m.ids; a.meta = m.meta; a.n = m.channels; a.k = m.hidden; a.out = m.y; a.out_stride = m.y_stride;
+    a.error_word = m.error_word;
+    return launch<B_Q6K_PLANAR, OUT_ROWS, SRC_RECORD_ROUTES>("skinny_down", a, (m.channels + 255) / 256, m.records, s);
+}
+
+}  // namespace tsp
