@@ -13,8 +13,8 @@
 // the rows over all banks, and each lane then picks its 16 quants of a block with aligned dword reads and a byte
 // funnel shift. The next group of 8 blocks is in flight while the current one is multiplied.
 //
-// Workgroups are persistent (one per compute unit, 8 waves): the activations are staged once per workgroup and each
-// wave then walks the 32-row tiles of the matrix with stride (workgroups x 8).
+// Workgroups are persistent (one per compute unit, 8 waves): the activations are staged once per workgroup, which owns
+// a contiguous share of the matrix's 32-row tiles; its waves take tiles from that share through a counter in LDS.
 #include "q8_mfma.hpp"
 
 #include <type_traits>
@@ -53,10 +53,12 @@ __device__ __forceinline__ f16x8 quants8(uint32_t w0, uint32_t w1) {
 __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [hi plane][lo plane][8 weight tiles]
     __shared__ float wave_max[kWaves];
+    __shared__ uint32_t next_tile;
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const uint32_t col = lane % 32, khalf = lane / 32;
     const uint32_t K = a.columns, chunks = K / 8, groups = K / 256, row_bytes = K / 32 * 34;
+    if (tid == 0) next_tile = uint32_t(uint64_t((a.rows + 31) / 32) * blockIdx.x / gridDim.x);
     _Float16* const a_hi = reinterpret_cast<_Float16*>(lds);
     _Float16* const a_lo = a_hi + kRows * K;
     uint8_t* const tile = lds + 2 * kRows * K * 2 + wave * kTileBytes;
@@ -133,10 +135,19 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
         }
     };
 
-    // (tile, group) items of this wave in order; the next item's bytes are requested before the current one is multiplied
-    const uint32_t tiles = (a.rows + 31) / 32, walkers = gridDim.x * kWaves, first = blockIdx.x * kWaves + wave;
-    if (first < tiles) fetch_group(first * 32, 0);
-    for (uint32_t t = first; t < tiles; t += walkers) {
+    // Each workgroup owns a contiguous share of the 32-row tiles and its waves take the next free tile of that share from
+    // a counter in LDS (which wave computes a tile does not change the result). The bytes of the next (tile, group) item
+    // are requested before the current one is multiplied, so a wave always holds its next tile index one step ahead.
+    const uint32_t tiles = (a.rows + 31) / 32;
+    const uint32_t share_end = uint32_t(uint64_t(tiles) * (blockIdx.x + 1) / gridDim.x);
+    auto take_tile = [&]() {
+        uint32_t t = 0;
+        if (lane == 0) t = atomicAdd(&next_tile, 1u);
+        return uint32_t(__builtin_amdgcn_readfirstlane(int(t)));
+    };
+    uint32_t t = take_tile(), t_next = take_tile();
+    if (t < share_end) fetch_group(t * 32, 0);
+    for (; t < share_end; t = t_next, t_next = take_tile()) {
         const uint32_t row0 = t * 32;
         f32x16 acc;
 #pragma unroll
@@ -144,8 +155,8 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
         for (uint32_t g = 0; g < groups; ++g) {
             store_group();  // the previous item's reads were issued before this point; LDS serves a wave in order
             const bool last = g + 1 == groups;
-            const uint32_t next_tile = last ? (t + walkers < tiles ? t + walkers : t) : t;
-            fetch_group(next_tile * 32, last ? 0 : g + 1);  // past the end: a harmless repeat of this tile's first group
+            const uint32_t following = last ? (t_next < share_end ? t_next : t) : t;
+            fetch_group(following * 32, last ? 0 : g + 1);  // past the end: a harmless repeat of this tile's first group
             const uint8_t* mine = tile + col * kTileStride + khalf * 16;
             auto block = [&](auto b_tag) {
                 constexpr int B = decltype(b_tag)::value;
