@@ -1,0 +1,331 @@
+// Tests of tokspur::HipGraph on a GPU, written the way the engine's own graph tests are (tests/test_moe.cpp,
+// tests/test_planar_pack_v3.cpp): build weights with the tests' LCG fixture, run the operators through the graph
+// class, compare with the CPU reference, and check the lifecycle and error contract (idle / encoding phases,
+// ledger, budget, sticky error word, no allocation while encoding, canaries).
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <cstdlib>
+#include <functional>
+#include <string>
+#include <vector>
+
+#include "hip_graph.hpp"
+#include "tokspur_hip.h"
+#include "tokspur_oracle.h"
+
+using namespace tokspur;
+
+namespace {
+int checks = 0, failures = 0;
+void expect(bool ok, const char* what, int line) {
+    ++checks;
+    if (!ok) { ++failures; std::printf("FAILED line %d: %s\n", line, what); std::fflush(stdout); }
+}
+#define EXPECT(cond) expect((cond), #cond, __LINE__)
+bool throws_format(const std::function<void()>& f) {
+    try { f(); } catch (const FormatError&) { return true; } catch (...) { return false; }
+    return false;
+}
+template <class T> std::span<const std::byte> bytes_of(const std::vector<T>& v) { return std::as_bytes(std::span<const T>(v)); }
+template <class T> std::vector<T> read_as(HipGraph& g, GpuView v) {
+    std::vector<T> out(v.bytes / sizeof(T));
+    g.read(v, std::as_writable_bytes(std::span<T>(out)));
+    return out;
+}
+std::vector<float> lcg_floats(uint32_t seed, size_t n) {  // tests/test_planar_pack_v3.cpp input generator
+    std::vector<float> out(n);
+    uint32_t rng = seed;
+    for (auto& v : out) { rng = rng * 1664525u + 1013904223u; v = float(int(rng % 1993u) - 996) / 997.0f; }
+    return out;
+}
+std::vector<uint8_t> fixture(uint32_t type, uint32_t k, uint32_t r, uint32_t e) {
+    uint32_t epb = 0, bpb = 0;
+    orc_encoding(type, &epb, &bpb);
+    std::vector<uint8_t> w(size_t(k / epb) * bpb * r * e);
+    if (type == 14) {  // the LCG fixture leaves Q6_K's scale (bytes 208..209) random: give it a small finite half
+        uint32_t rng = 77;
+        for (auto& b : w) { rng = rng * 1664525u + 1013904223u; b = uint8_t(rng >> 24); }
+        for (size_t at = 0; at < w.size(); at += 210) { w[at + 208] = uint8_t(at / 210 % 7); w[at + 209] = 0x1c; }
+    } else {
+        orc_fixture_weights(type, k, r, e, w.data(), w.size());
+    }
+    return w;
+}
+// error in units of the row's largest magnitude: the LCG fixture's scales give outputs of ~1e5 with heavy cancellation, where
+// |a - e| / max(1, |e|) per element would measure the cancellation and not the kernel
+double row_error(const std::vector<float>& got, const std::vector<double>& want) {
+    double worst = 0, scale = 1;
+    for (double v : want) scale = std::max(scale, std::fabs(v));
+    for (size_t i = 0; i < got.size(); ++i) worst = std::max(worst, std::fabs(double(got[i]) - want[i]) / scale);
+    return worst;
+}
+double scaled_error(const std::vector<float>& got, const std::vector<double>& want) {  // src/ffn_check.cpp:48-56
+    double worst = 0;
+    for (size_t i = 0; i < got.size(); ++i) worst = std::max(worst, std::fabs(double(got[i]) - want[i]) / std::max(1.0, std::fabs(want[i])));
+    return worst;
+}
+std::vector<uint8_t> coloc_half(const tsp_planar_spec& spec, const std::vector<uint8_t>& gate, const std::vector<uint8_t>& up, uint32_t experts, uint32_t half) {
+    std::vector<uint8_t> out(size_t(experts / 2) * 2 * spec.planar_expert_bytes);
+    if (tsp_pack_coloc_half(&spec, gate.data(), up.data(), experts, half, out.data(), out.size()) != TSP_OK) std::printf("pack failed: %s\n", tsp_last_error());
+    return out;
+}
+std::vector<uint8_t> planar_stack(const tsp_planar_spec& spec, const std::vector<uint8_t>& gguf, uint32_t experts) {
+    std::vector<uint8_t> out(size_t(experts) * spec.planar_expert_bytes);
+    for (uint32_t e = 0; e < experts; ++e)
+        tsp_pack_expert_planar_v3(&spec, gguf.data() + size_t(e) * spec.source_expert_bytes, spec.source_expert_bytes,
+                                  out.data() + size_t(e) * spec.planar_expert_bytes, spec.planar_expert_bytes);
+    return out;
+}
+
+void test_ledger_and_phases() {
+    HipGraph g(1 << 20);
+    const GpuView a = g.zeros(4096, "a");
+    EXPECT(g.memory().live_bytes == 4096 && g.memory().allocations == 1 && g.memory().budget == (1u << 20));
+    EXPECT(throws_format([&] { (void)g.zeros(2u << 20, "too big"); }));  // budget
+    std::vector<float> host(1024, 1.5f);
+    g.write(a, bytes_of(host));
+    EXPECT(read_as<float>(g, g.slice(a, 16, 8))[1] == 1.5f);
+    EXPECT(throws_format([&] { (void)g.slice(a, 4090, 16); }));
+    const GpuView w = g.upload(bytes_of(host), "weights");
+    EXPECT(throws_format([&] { g.write(w, bytes_of(host)); }));  // immutable
+    EXPECT(throws_format([&] { g.swiglu(a, a, a); }));           // operator while idle
+    HipGraph other(1 << 20);
+    EXPECT(throws_format([&] { (void)other.read(a); }));          // foreign view
+    g.begin();
+    EXPECT(throws_format([&] { (void)g.zeros(16, "while encoding"); }));
+    EXPECT(throws_format([&] { (void)g.read(a); }));
+    g.abort();
+    g.release(a);
+    EXPECT(throws_format([&] { (void)g.read(a); }));              // released view is never rebound
+    EXPECT(g.memory().live_bytes == 4096 && g.memory().peak_bytes == 8192);
+    EXPECT(!g.device_name().empty());
+}
+
+void test_gemv_route_mixture_topk() {
+    const uint32_t K = 512, R = 96, E = 64, S = 6;
+    HipGraph g(64u << 20);
+    const auto w = fixture(12, K, R, 1);
+    const auto x = lcg_floats(5, K);
+    const GpuView dw = g.upload(bytes_of(w), "w"), dx = g.upload(bytes_of(x), "x", false), dy = g.zeros(R * 4, "y");
+    const auto logits = lcg_floats(9, E);
+    const GpuView dl = g.upload(bytes_of(logits), "logits", false), di = g.zeros(S * 4, "ids"), dwt = g.zeros(S * 4, "weights");
+    const GpuView topk_scratch = g.zeros(HipGraph::logit_topk_scratch_bytes(1, E), "scratch"), topk_out = g.zeros(HipGraph::logit_topk_output_bytes(1), "rows");
+    g.prepare_logit_topk();
+    const uint64_t allocations = g.memory().allocations;
+    g.begin();
+    g.gemv(12, dw, dx, dy, K, R);
+    g.route(dl, di, dwt, S, RouterMode::softmax, true);
+    g.logit_topk({dl, 1, E, uint64_t(E) * 4}, topk_scratch, topk_out);
+    const BatchResult r = g.submit();
+    EXPECT(r.dispatches == 3 && r.gpu_ms > 0 && g.memory().allocations == allocations);  // nothing allocated while encoding
+    std::vector<double> want(R);
+    orc_reference_gemv(12, w.data(), w.size(), K, R, x.data(), K, want.data());
+    EXPECT(scaled_error(read_as<float>(g, dy), want) <= 5e-5);
+    std::vector<double> dlogits(logits.begin(), logits.end()), wweights(S);
+    std::vector<uint32_t> wids(S);
+    orc_route_reference(dlogits.data(), E, S, 0, 1, wids.data(), wweights.data());
+    EXPECT(read_as<uint32_t>(g, di) == wids);
+    EXPECT(scaled_error(read_as<float>(g, dwt), wweights) <= 1e-6);
+    orc_logit_topk_row row{};
+    orc_logit_topk_row_cpu(logits.data(), E, &row);
+    const auto got = read_as<GpuLogitTopKRow>(g, topk_out);
+    EXPECT(got[0].count == row.count && std::memcmp(got[0].ids.data(), row.ids, 256) == 0 && std::memcmp(got[0].logits.data(), row.logits, 256) == 0);
+    EXPECT(got[0].ids[0] == wids[0]);  // arg-max agrees with the router's first choice
+    // aliasing is refused before anything is encoded
+    g.begin();
+    EXPECT(throws_format([&] { g.gemv(12, dw, dx, dx, K, K); }));
+    g.abort();
+}
+
+struct MoeFixture {
+    MoeShape shape;
+    std::vector<uint8_t> gate, up, down, sgate, sup, sdown;
+    std::vector<float> router, shared_router;
+};
+
+MoeFixture make_moe(uint32_t channels, uint32_t hidden, uint32_t experts, uint32_t selected) {
+    MoeFixture f{{channels, hidden, experts, selected}};
+    f.gate = fixture(12, channels, hidden, experts);
+    f.up = fixture(12, channels, hidden, experts);
+    for (auto& b : f.up) b = uint8_t(b * 3 + 1);
+    for (size_t at = 0; at < f.up.size(); at += 144) { std::memcpy(&f.up[at], &f.gate[at], 4); }
+    f.down = fixture(14, hidden, channels, experts);
+    f.sgate = fixture(12, channels, hidden, 2);
+    f.sup = f.sgate;
+    f.sdown = fixture(14, hidden, channels, 2);
+    f.router = lcg_floats(31, size_t(experts) * channels);
+    f.shared_router = lcg_floats(37, channels);
+    for (auto& v : f.shared_router) v *= 0.05f;
+    return f;
+}
+
+struct MoeOnGraph { MoeWeights w; };
+
+MoeOnGraph upload_moe(HipGraph& g, const MoeFixture& f) {
+    tsp_planar_spec gu{}, dn{};
+    tsp_make_expert_spec(12, f.shape.channels, f.shape.hidden, &gu);
+    tsp_make_expert_spec(14, f.shape.hidden, f.shape.channels, &dn);
+    const uint32_t E = f.shape.experts;
+    MoeOnGraph m{};
+    m.w.router = {g.upload(bytes_of(f.router), "router"), 0};
+    m.w.gate = {g.upload(bytes_of(coloc_half(gu, f.gate, f.up, E, 0)), "pair_lo"), 12};
+    m.w.up = {g.upload(bytes_of(coloc_half(gu, f.gate, f.up, E, 1)), "pair_hi"), 12};
+    m.w.down = {g.upload(bytes_of(planar_stack(dn, f.down, E)), "down"), 14};
+    g.register_planar_matrix(m.w.gate.view, {12, 2, f.shape.channels, f.shape.hidden, E});
+    g.register_planar_matrix(m.w.up.view, {12, 3, f.shape.channels, f.shape.hidden, E});
+    g.register_planar_matrix(m.w.down.view, {14, 10, f.shape.hidden, f.shape.channels, E});
+    m.w.shared_router = {g.upload(bytes_of(f.shared_router), "shared router"), 0};
+    return m;
+}
+
+// CPU composition: src/moe.cpp:37-83 order, double accumulation (tests/test_moe.cpp:131-163)
+std::vector<double> cpu_moe_token(const MoeFixture& f, const float* x, bool shared_planar_pair) {
+    const MoeShape s = f.shape;
+    std::vector<double> logits(s.experts), weights(s.selected), out(s.channels);
+    orc_reference_gemv(0, reinterpret_cast<const uint8_t*>(f.router.data()), f.router.size() * 4, s.channels, s.experts, x, s.channels, logits.data());
+    std::vector<double> flogits(s.experts);
+    for (uint32_t e = 0; e < s.experts; ++e) flogits[e] = double(float(logits[e]));
+    std::vector<uint32_t> ids(s.selected);
+    orc_route_reference(flogits.data(), s.experts, s.selected, 0, 1, ids.data(), weights.data());
+    std::vector<double> h(size_t(s.selected) * s.hidden), y(size_t(s.selected) * s.channels);
+    std::vector<float> xs(size_t(s.selected) * s.channels);
+    orc_moe_routed_reference(12, 14, f.gate.data(), f.up.data(), f.down.data(), s.channels, s.hidden, s.experts, ids.data(), 1, s.selected, x, s.channels, 1, 0,
+                             h.data(), y.data(), 1);
+    std::vector<double> sh(s.hidden), sy(s.channels);
+    const uint32_t zero = 0;
+    orc_moe_routed_reference(12, 14, f.sgate.data(), f.sup.data(), f.sdown.data(), s.channels, s.hidden, 2, &zero, 1, 1, x, s.channels, 1, 0, sh.data(), sy.data(), 1);
+    double shared_logit = 0;
+    orc_reference_gemv(0, reinterpret_cast<const uint8_t*>(f.shared_router.data()), f.shared_router.size() * 4, s.channels, 1, x, s.channels, &shared_logit);
+    if (shared_planar_pair == false && std::getenv("TSP_TEST_VERBOSE"))
+        std::printf("  cpu ids %u %u %u logits %g %g %g shared_logit %g shared_down[0..1] %g %g down[0] %g\n", ids[0], ids[1], ids[2], logits[0], logits[1],
+                    logits[2], shared_logit, sy[0], sy[1], y[0]);
+    orc_mixture_reference(y.data(), weights.data(), s.selected, sy.data(), s.channels, double(float(shared_logit)), out.data());
+    return out;
+}
+
+void test_encode_moe_single_token() {
+    const MoeFixture f = make_moe(256, 256, 8, 3);
+    HipGraph g(256u << 20);
+    MoeOnGraph m = upload_moe(g, f);
+    // the single-token composition runs the shared expert as three raw-GGUF GEMVs (src/moe.cpp:71-78)
+    const size_t gu_bytes = size_t(f.shape.channels / 256) * 144 * f.shape.hidden, dn_bytes = size_t(f.shape.hidden / 256) * 210 * f.shape.channels;
+    m.w.shared_gate = {g.upload(std::as_bytes(std::span(f.sgate.data(), gu_bytes)), "shared gate"), 12};
+    m.w.shared_up = {g.upload(std::as_bytes(std::span(f.sup.data(), gu_bytes)), "shared up"), 12};
+    m.w.shared_down = {g.upload(std::as_bytes(std::span(f.sdown.data(), dn_bytes)), "shared down"), 14};
+    g.prepare_planar_moe_v3(12, 14, false);
+    const MoeScratch scratch = allocate_moe_scratch(g, f.shape);
+    const auto x = lcg_floats(101, f.shape.channels);
+    const GpuView dx = g.upload(bytes_of(x), "x", false), dy = g.zeros(uint64_t(f.shape.channels) * 4, "y");
+    EXPECT(is_planar_moe(g, m.w, f.shape) && g.planar_matrix_count() == 3);
+    const uint64_t allocations = g.memory().allocations;
+    g.begin();
+    encode_moe(g, m.w, scratch, dx, dy, f.shape, RouterMode::softmax, true);
+    const BatchResult r = g.submit();
+    EXPECT(r.dispatches == 9 && g.memory().allocations == allocations);
+    // Q6_K integer products above 2048 lose their lowest bit on the matrix cores: a few 1e-5 of the row scale
+    const double err = row_error(read_as<float>(g, dy), cpu_moe_token(f, x.data(), false));
+    std::printf("encode_moe single token: error / row max %.3e\n", err);
+    if (err > 2e-4) {  // say which stage differs
+        const auto ids = read_as<uint32_t>(g, scratch.indices);
+        const auto lg = read_as<float>(g, scratch.logits);
+        const auto sl = read_as<float>(g, scratch.shared_logit);
+        const auto sd = read_as<float>(g, scratch.shared_down);
+        const auto dn = read_as<float>(g, scratch.down);
+        std::printf("  ids %u %u %u logits %g %g %g shared_logit %g shared_down[0..1] %g %g down[0] %g\n", ids[0], ids[1], ids[2], lg[0], lg[1], lg[2], sl[0], sd[0], sd[1], dn[0]);
+    }
+    EXPECT(err <= 2e-4);
+    // a non-finite input poisons only its own batch (tests/test_moe.cpp:175-185)
+    std::vector<float> bad = x;
+    bad[7] = NAN;
+    g.write(dx, bytes_of(bad));
+    g.begin();
+    encode_moe(g, m.w, scratch, dx, dy, f.shape, RouterMode::softmax, true);
+    EXPECT(throws_format([&] { (void)g.submit(); }));
+    g.write(dx, bytes_of(x));
+    g.begin();
+    encode_moe(g, m.w, scratch, dx, dy, f.shape, RouterMode::softmax, true);
+    (void)g.submit();
+    EXPECT(row_error(read_as<float>(g, dy), cpu_moe_token(f, x.data(), false)) <= 2e-4);
+    // registration is closed once a batch has begun; registered matrices stay resident
+    EXPECT(throws_format([&] { g.register_planar_matrix(m.w.down.view, {14, 10, f.shape.hidden, f.shape.channels, f.shape.experts}); }));
+    EXPECT(throws_format([&] { g.release(m.w.down.view); }));
+    release_moe_scratch(g, scratch);
+}
+
+void test_encode_moe_batch() {
+    const uint32_t T = 70;
+    const MoeFixture f = make_moe(256, 256, 8, 3);
+    HipGraph g(512u << 20);
+    MoeOnGraph m = upload_moe(g, f);
+    tsp_planar_spec gu{}, dn{};
+    tsp_make_expert_spec(12, f.shape.channels, f.shape.hidden, &gu);
+    tsp_make_expert_spec(14, f.shape.hidden, f.shape.channels, &dn);
+    m.w.shared_gate = {g.upload(bytes_of(coloc_half(gu, f.sgate, f.sup, 2, 0)), "shared pair_lo"), 12};
+    m.w.shared_up = {g.upload(bytes_of(coloc_half(gu, f.sgate, f.sup, 2, 1)), "shared pair_hi"), 12};
+    m.w.shared_down = {g.upload(bytes_of(planar_stack(dn, f.sdown, 2)), "shared down"), 14};
+    g.register_planar_matrix(m.w.shared_gate.view, {12, 2, f.shape.channels, f.shape.hidden, 2});
+    g.register_planar_matrix(m.w.shared_up.view, {12, 3, f.shape.channels, f.shape.hidden, 2});
+    g.register_planar_matrix(m.w.shared_down.view, {14, 10, f.shape.hidden, f.shape.channels, 2});
+    g.prepare_planar_moe_v3(12, 14, true, T, f.shape.experts, f.shape.selected, f.shape.channels, f.shape.hidden);
+    const MoeBatchScratch scratch = allocate_moe_batch_scratch(g, f.shape, T);
+    // inputs are bf16-valued (the prefill path carries activations as bf16) with a two-float pad per row that must stay untouched
+    const uint32_t stride = f.shape.channels + 2;
+    std::vector<float> x = lcg_floats(303, size_t(T) * stride), logits(size_t(T) * f.shape.experts);
+    for (auto& v : x) { uint32_t bad = 0; v = orc_bf16_to_f32(orc_round_bf16_bits(v, &bad)); }
+    for (uint32_t t = 0; t < T; ++t) {
+        std::vector<double> l(f.shape.experts);
+        orc_reference_gemv(0, reinterpret_cast<const uint8_t*>(f.router.data()), f.router.size() * 4, f.shape.channels, f.shape.experts, &x[size_t(t) * stride],
+                           f.shape.channels, l.data());
+        for (uint32_t e = 0; e < f.shape.experts; ++e) logits[size_t(t) * f.shape.experts + e] = float(l[e]);
+    }
+    const GpuView dx = g.upload(bytes_of(x), "x", false), dl = g.upload(bytes_of(logits), "logits", false);
+    std::vector<float> canary(size_t(T) * stride, -9.0f);
+    const GpuView dy = g.upload(bytes_of(canary), "y", false);
+    const uint64_t allocations = g.memory().allocations;
+    g.begin();
+    encode_moe_batch(g, m.w, scratch, dl, {dx, T, f.shape.channels, uint64_t(stride) * 4}, {dy, T, f.shape.channels, uint64_t(stride) * 4}, f.shape,
+                     RouterMode::softmax, true);
+    const BatchResult r = g.submit();
+    EXPECT(r.dispatches == 5 && g.memory().allocations == allocations);
+    const auto y = read_as<float>(g, dy);
+    double worst = 0;
+    bool pads = true;
+    for (uint32_t t = 0; t < T; ++t) {
+        const auto want = cpu_moe_token(f, &x[size_t(t) * stride], true);
+        double scale = 1;
+        for (double v : want) scale = std::max(scale, std::fabs(v));
+        for (uint32_t c = 0; c < f.shape.channels; ++c) worst = std::max(worst, std::fabs(double(y[size_t(t) * stride + c]) - want[c]) / scale);
+        pads = pads && y[size_t(t) * stride + f.shape.channels] == -9.0f && y[size_t(t) * stride + f.shape.channels + 1] == -9.0f;
+    }
+    std::printf("encode_moe_batch T=%u: max error / row max %.3e\n", T, worst);
+    EXPECT(worst <= 2e-3 && pads);
+    // a token that selects one expert twice is a device-side refusal
+    std::vector<uint32_t> ids = read_as<uint32_t>(g, scratch.indices);
+    g.begin();
+    g.prefill_route_batch(dl, scratch.indices, scratch.weights, f.shape.experts, f.shape.selected, T, RouterMode::softmax, true);
+    (void)g.submit();
+    ids[1] = ids[0];
+    g.write(scratch.indices, bytes_of(ids));
+    g.begin();
+    g.planar_nax_grouped_moe(m.w.gate.view, m.w.up.view, m.w.down.view, scratch.indices, {dx, T, f.shape.channels, uint64_t(stride) * 4},
+                             {scratch.expert_down, T * f.shape.selected, f.shape.channels, uint64_t(f.shape.channels) * 4}, scratch.token_map, scratch.counts,
+                             scratch.tasks, f.shape.experts, f.shape.selected);
+    EXPECT(throws_format([&] { (void)g.submit(); }));
+    release_moe_batch_scratch(g, scratch);
+}
+}  // namespace
+
+int main() {
+    const std::pair<const char*, void (*)()> tests[] = {{"ledger and phases", test_ledger_and_phases},
+                                                         {"gemv, route, mixture, top-k", test_gemv_route_mixture_topk},
+                                                         {"encode_moe single token", test_encode_moe_single_token},
+                                                         {"encode_moe_batch", test_encode_moe_batch}};
+    for (const auto& [name, fn] : tests) {
+        std::printf("== %s\n", name);
+        std::fflush(stdout);
+        try { fn(); } catch (const std::exception& e) { ++failures; std::printf("FAILED: unexpected exception in %s: %s\n", name, e.what()); }
+    }
+    std::printf("%d checks, %d failures\n", checks, failures);
+    return failures ? 1 : 0;
+}

@@ -144,3 +144,17 @@ def test_missing_library_fails_loudly(tsp, monkeypatch, tmp_path):
     monkeypatch.setattr(tsp, "LIB_PATH", str(tmp_path / "absent.so"))
     with pytest.raises(RuntimeError, match="no fallback"):
         tsp.dll()
+
+
+def test_host_class_library_exports_graph_operators():
+    """libtokspur_graph.so (tokspur::HipGraph, the C++ mirror of the engine's graph class) carries every operator of the path."""
+    import subprocess
+    lib = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tokspur-public_amd", "libtokspur_graph.so")
+    assert os.path.exists(lib), "run __graft_entry__.build()"
+    names = subprocess.run(["nm", "-D", "--demangle", lib], stdout=subprocess.PIPE, text=True, check=True).stdout
+    for op in ("gemv", "gemv_rows", "q8_matvec_many", "route", "prefill_route_batch", "routed_gemv", "swiglu", "mixture", "prefill_mixture_batch",
+               "register_planar_matrix", "planar_matrix_shape", "prepare_planar_moe_v3", "planar_moe_gate_up_swiglu_m8", "planar_moe_routed_m8",
+               "planar_nax_grouped_moe", "dense_mm", "logit_topk", "validate_disjoint", "begin", "submit", "abort", "zeros", "upload", "release"):
+        assert f"tokspur::HipGraph::{op}(" in names, op
+    for fn in ("tokspur::encode_moe(", "tokspur::encode_moe_batch(", "tokspur::allocate_moe_scratch(", "tokspur::is_planar_moe("):
+        assert fn in names, fn

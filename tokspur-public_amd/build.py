@@ -52,5 +52,35 @@ def build(verbose=False, jobs=8):
     return LIB
 
 
+def build_host():
+    """The C++ host class (tokspur::HipGraph) over the C ABI: host/hip_graph.cpp -> libtokspur_graph.so."""
+    root = os.path.dirname(HERE)
+    cmd = ["hipcc", "-std=c++20", "-O2", "-fPIC", "-shared", "-Wall", os.path.join(HERE, "host", "hip_graph.cpp"),
+           "-I", os.path.join(root, "include"), "-L", HERE, "-ltokspur_hip", "-Wl,-rpath,$ORIGIN", "-o", HOST_LIB]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode:
+        raise RuntimeError(f"host library build failed:\n{proc.stdout}")
+    return HOST_LIB
+
+
+def build_native_tests():
+    """tests/native/*.cpp -> tests/native/bin/ (they link the host library, the C ABI and the CPU oracle as checker)."""
+    root = os.path.dirname(HERE)
+    src_dir, out_dir = os.path.join(root, "tests", "native"), os.path.join(root, "tests", "native", "bin")
+    os.makedirs(out_dir, exist_ok=True)
+    built = []
+    for name in sorted(f for f in os.listdir(src_dir) if f.endswith(".cpp")):
+        out = os.path.join(out_dir, name[:-4])
+        cmd = ["hipcc", "-std=c++20", "-O2", "-Wall", os.path.join(src_dir, name), "-I", os.path.join(HERE, "host"), "-I", os.path.join(root, "include"),
+               "-I", os.path.join(root, "oracle"), "-L", HERE, "-ltokspur_graph", "-ltokspur_hip", "-L", os.path.join(root, "oracle"), "-loracle",
+               "-Wl,-rpath," + HERE, "-Wl,-rpath," + os.path.join(root, "oracle"), "-o", out]
+        proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode:
+            raise RuntimeError(f"native test build failed for {name}:\n{proc.stdout}")
+        built.append(out)
+    return built
+
+
 if __name__ == "__main__":
     print(build(verbose="-v" in sys.argv))
+    print(build_host())

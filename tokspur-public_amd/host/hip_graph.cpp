@@ -1,0 +1,660 @@
+// tokspur::HipGraph over the C ABI of include/tokspur_hip.h. See hip_graph.hpp for the contract.
+#include "hip_graph.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <chrono>
+#include <cstring>
+#include <thread>
+
+#include "tokspur_hip.h"
+
+namespace tokspur {
+namespace {
+
+void require(bool condition, const char* message) {
+    if (!condition) throw FormatError(message);
+}
+void hip(hipError_t status, const char* what) {
+    if (status != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(status));
+}
+// host-side refusals of the C ABI keep the engine's exception type
+void check(int status) {
+    if (status == TSP_OK) return;
+    if (status == TSP_ERR_FORMAT) throw FormatError(tsp_last_error());
+    throw std::runtime_error(tsp_last_error());
+}
+uint64_t checked_mul(uint64_t a, uint64_t b) {
+    require(b == 0 || a <= UINT64_MAX / b, "size overflow");
+    return a * b;
+}
+uint64_t next_owner() {
+    static uint64_t counter = 0x746f6b73;
+    return ++counter;
+}
+
+struct Allocation {
+    void* device = nullptr;
+    uint64_t bytes = 0;
+    bool live = false, immutable = false;
+    std::string label;
+};
+struct PlanarEntry {
+    size_t slot;
+    uint64_t offset, bytes;
+    PlanarMatrixShape shape;
+};
+
+}  // namespace
+
+struct HipGraph::Impl {
+    uint64_t owner = next_owner();
+    uint64_t budget = 0, live_bytes = 0, peak_bytes = 0, allocations = 0;
+    std::vector<Allocation> slots;  // never recycled
+    std::vector<PlanarEntry> planar;
+    std::thread::id thread = std::this_thread::get_id();
+    hipStream_t stream = nullptr;
+    hipEvent_t started = nullptr, finished = nullptr;
+    uint32_t* error_word = nullptr;
+    bool encoding = false, locked = false, topk_prepared = false;
+    uint64_t dispatches = 0;
+    std::chrono::steady_clock::time_point wall_start;
+    // scratch sized while idle by the prepare_* calls
+    void* union_meta = nullptr;
+    void* nax_workspace = nullptr;
+    uint64_t nax_workspace_bytes = 0;
+    void* dense_workspace = nullptr;
+    uint64_t dense_workspace_bytes = 0;
+    uint32_t prepared_gate_up = 0, prepared_down = 0;
+
+    void same_thread() const { require(std::this_thread::get_id() == thread, "GPU graph used from another thread"); }
+    void idle() const {
+        same_thread();
+        require(!encoding, "GPU graph operation requires an idle graph");
+    }
+    void active() {
+        same_thread();
+        require(encoding, "GPU graph operator outside begin/submit");
+        ++dispatches;
+    }
+    const Allocation& allocation(const GpuView& v, bool writable = false) const {
+        require(v.owner == owner && v.slot < slots.size() && slots[v.slot].live, "released or foreign GPU view");
+        const Allocation& a = slots[v.slot];
+        require(v.offset <= a.bytes && v.bytes <= a.bytes - v.offset, "GPU view out of bounds");
+        require(!writable || !a.immutable, "immutable GPU view used as a destination");
+        return a;
+    }
+    uint8_t* device(const GpuView& v, bool writable = false) const { return static_cast<uint8_t*>(allocation(v, writable).device) + v.offset; }
+    void charge(uint64_t bytes) {
+        require(bytes > 0 && bytes <= budget - std::min(budget, live_bytes), "GPU graph byte budget exceeded");
+        live_bytes += bytes;
+        peak_bytes = std::max(peak_bytes, live_bytes);
+    }
+    GpuView make(uint64_t bytes, std::string label, bool immutable) {
+        charge(bytes);
+        void* p = nullptr;
+        const hipError_t status = hipMalloc(&p, bytes);
+        if (status != hipSuccess) { live_bytes -= bytes; hip(status, "hipMalloc"); }
+        slots.push_back({p, bytes, true, immutable, std::move(label)});
+        ++allocations;
+        return {owner, slots.size() - 1, 0, bytes};
+    }
+    void* raw(uint64_t bytes) {  // internal scratch: charged like any other allocation
+        charge(bytes);
+        void* p = nullptr;
+        const hipError_t status = hipMalloc(&p, bytes);
+        if (status != hipSuccess) { live_bytes -= bytes; hip(status, "hipMalloc"); }
+        ++allocations;
+        return p;
+    }
+    static bool overlaps(const GpuView& a, const GpuView& b) {
+        return a.slot == b.slot && a.offset < b.offset + b.bytes && b.offset < a.offset + a.bytes;
+    }
+    const PlanarEntry* planar_of(const GpuView& v) const {
+        for (const auto& e : planar)
+            if (e.slot == v.slot && e.offset == v.offset && e.bytes == v.bytes) return &e;
+        return nullptr;
+    }
+    // rows of `columns` floats, `stride` bytes apart, inside the view
+    void rows_fit(const GpuRowsF32& r, const char* message) const {
+        require(r.rows >= 1 && r.columns >= 1 && r.stride_bytes >= uint64_t(r.columns) * 4 && r.stride_bytes % 4 == 0 &&
+                    r.view.bytes >= uint64_t(r.rows - 1) * r.stride_bytes + uint64_t(r.columns) * 4,
+                message);
+    }
+};
+
+HipGraph::HipGraph(uint64_t byte_budget) : impl_(std::make_unique<Impl>()) {
+    require(byte_budget > 0, "GPU graph byte budget must be positive");
+    require(tsp_abi_version() >= 1, "tokspur HIP library too old");
+    impl_->budget = byte_budget;
+    hip(hipStreamCreate(&impl_->stream), "hipStreamCreate");
+    hip(hipEventCreate(&impl_->started), "hipEventCreate");
+    hip(hipEventCreate(&impl_->finished), "hipEventCreate");
+    hip(hipMalloc(reinterpret_cast<void**>(&impl_->error_word), 256), "hipMalloc");
+    hip(hipMemset(impl_->error_word, 0, 256), "hipMemset");
+}
+
+HipGraph::~HipGraph() {
+    if (!impl_) return;
+    (void)hipStreamSynchronize(impl_->stream);
+    for (auto& a : impl_->slots)
+        if (a.live) (void)hipFree(a.device);
+    for (void* p : {impl_->union_meta, impl_->nax_workspace, impl_->dense_workspace, static_cast<void*>(impl_->error_word)})
+        if (p) (void)hipFree(p);
+    (void)hipEventDestroy(impl_->started);
+    (void)hipEventDestroy(impl_->finished);
+    (void)hipStreamDestroy(impl_->stream);
+}
+
+// ------------------------------------------------------------------ storage
+GpuView HipGraph::zeros(uint64_t bytes, std::string label) {
+    impl_->idle();
+    const GpuView v = impl_->make(bytes, std::move(label), false);
+    hip(hipMemset(impl_->device(v), 0, bytes), "hipMemset");
+    return v;
+}
+
+GpuView HipGraph::upload(std::span<const std::byte> data, std::string label, bool immutable) {
+    impl_->idle();
+    require(!data.empty(), "empty GPU upload");
+    const GpuView v = impl_->make(data.size(), std::move(label), immutable);
+    hip(hipMemcpy(impl_->slots[v.slot].device, data.data(), data.size(), hipMemcpyHostToDevice), "hipMemcpy");
+    return v;
+}
+
+GpuView HipGraph::slice(GpuView buffer, uint64_t offset, uint64_t bytes) const {
+    (void)impl_->allocation(buffer);
+    require(bytes > 0 && offset <= buffer.bytes && bytes <= buffer.bytes - offset, "GPU slice out of bounds");
+    return {buffer.owner, buffer.slot, buffer.offset + offset, bytes};
+}
+
+void HipGraph::write(GpuView destination, std::span<const std::byte> data) {
+    impl_->idle();
+    require(data.size() == destination.bytes, "GPU write size mismatch");
+    hip(hipMemcpy(impl_->device(destination, true), data.data(), data.size(), hipMemcpyHostToDevice), "hipMemcpy");
+}
+
+std::vector<std::byte> HipGraph::read(GpuView source) const {
+    std::vector<std::byte> out(source.bytes);
+    read(source, out);
+    return out;
+}
+
+void HipGraph::read(GpuView source, std::span<std::byte> destination) const {
+    impl_->idle();
+    require(destination.size() == source.bytes, "GPU read size mismatch");
+    hip(hipMemcpy(destination.data(), impl_->device(source), source.bytes, hipMemcpyDeviceToHost), "hipMemcpy");
+}
+
+void HipGraph::release(GpuView full_buffer) {
+    impl_->idle();
+    const Allocation& a = impl_->allocation(full_buffer);
+    require(full_buffer.offset == 0 && full_buffer.bytes == a.bytes, "release requires the full buffer view");
+    for (const auto& e : impl_->planar) require(e.slot != full_buffer.slot, "registered planar matrices stay resident");
+    hip(hipFree(a.device), "hipFree");
+    Allocation& slot = impl_->slots[full_buffer.slot];
+    impl_->live_bytes -= slot.bytes;
+    slot.live = false;
+    slot.device = nullptr;
+}
+
+GraphMemory HipGraph::memory() const { return {impl_->budget, impl_->live_bytes, impl_->peak_bytes, impl_->allocations}; }
+
+std::string HipGraph::device_name() const {
+    int device = 0;
+    hip(hipGetDevice(&device), "hipGetDevice");
+    hipDeviceProp_t props{};
+    hip(hipGetDeviceProperties(&props, device), "hipGetDeviceProperties");
+    return props.name[0] ? std::string(props.name) : std::string(props.gcnArchName);
+}
+
+void HipGraph::validate_disjoint(std::span<const GpuView> inputs, std::span<const GpuView> destinations) const {
+    for (const auto& d : destinations) {
+        (void)impl_->allocation(d, true);
+        for (const auto& i : inputs) {
+            (void)impl_->allocation(i);
+            require(!Impl::overlaps(d, i), "unsupported GPU buffer alias");
+        }
+    }
+    for (size_t a = 0; a < destinations.size(); ++a)
+        for (size_t b = a + 1; b < destinations.size(); ++b) require(!Impl::overlaps(destinations[a], destinations[b]), "unsupported GPU buffer alias");
+}
+
+// ------------------------------------------------------------------ Pack v3 registration
+void HipGraph::register_planar_matrix(GpuView matrix, PlanarMatrixShape shape) {
+    impl_->idle();
+    require(!impl_->locked, "planar matrices are registered before the first batch");
+    const Allocation& a = impl_->allocation(matrix);
+    require(a.immutable, "planar matrix must be an immutable view");
+    require(reinterpret_cast<uintptr_t>(impl_->device(matrix)) % 16 == 0, "planar matrix requires 16-byte alignment");
+    require(shape.experts >= 1 && shape.experts <= 4096 && shape.kind >= 2 && shape.kind <= TSP_KIND_Q6K_PLANAR_X, "planar matrix kind mismatch");
+    const bool coloc = shape.kind >= 2 && shape.kind <= 7;
+    const uint32_t expected = shape.kind <= 3 ? 12u : shape.kind <= 5 ? 13u : shape.kind <= 7 ? 8u : shape.kind == 8 ? 7u : shape.kind == 9 ? 8u : 14u;
+    require(shape.source_type == expected, "planar matrix kind does not match its source type");
+    tsp_planar_spec spec{};
+    check(tsp_make_expert_spec(shape.source_type, shape.columns, shape.rows, &spec));
+    // a co-located tensor holds half of the experts as [gate_e, up_e] pairs
+    require(!coloc || shape.experts % 2 == 0, "co-located gate/up tensors hold an even number of experts");
+    const uint64_t want = coloc ? checked_mul(checked_mul(shape.experts / 2, 2), spec.planar_expert_bytes) : checked_mul(shape.experts, spec.planar_expert_bytes);
+    require(matrix.bytes == want, "planar matrix byte span mismatch");
+    for (const auto& e : impl_->planar)
+        require(!Impl::overlaps(matrix, {impl_->owner, e.slot, e.offset, e.bytes}), "planar matrix overlaps a registered matrix");
+    impl_->planar.push_back({matrix.slot, matrix.offset, matrix.bytes, shape});
+}
+
+uint64_t HipGraph::planar_matrix_count() const { return impl_->planar.size(); }
+
+std::optional<PlanarMatrixShape> HipGraph::planar_matrix_shape(GpuView matrix) const {
+    const PlanarEntry* e = impl_->planar_of(matrix);
+    return e ? std::optional<PlanarMatrixShape>(e->shape) : std::nullopt;
+}
+
+void HipGraph::prepare_planar_moe_v3(uint32_t gate_up_encoding, uint32_t down_encoding, bool prepare_nax, uint32_t max_nax_tokens,
+                                     uint32_t max_experts, uint32_t max_selected, uint32_t max_channels, uint32_t max_hidden) {
+    impl_->idle();
+    require((gate_up_encoding == 12 || gate_up_encoding == 13 || gate_up_encoding == 8) && (down_encoding == 7 || down_encoding == 8 || down_encoding == 14),
+            "unsupported planar v3 MoE encodings");
+    require(max_nax_tokens >= 1 && max_nax_tokens <= 2048 && max_experts >= 2 && max_experts <= 512 && max_selected >= 1 && max_selected <= 16 &&
+                max_channels >= 256 && max_hidden >= 256,
+            "planar v3 MoE preparation bounds mismatch");
+    if (!impl_->union_meta) impl_->union_meta = impl_->raw(9280);
+    if (prepare_nax) {
+        const uint32_t channels = (max_channels + 255) / 256 * 256, hidden = (max_hidden + 255) / 256 * 256;
+        const uint64_t bytes = tsp_planar_nax_workspace_bytes(max_nax_tokens, max_selected, max_experts, channels, hidden);
+        if (bytes > impl_->nax_workspace_bytes) {
+            require(impl_->nax_workspace == nullptr, "planar v3 NAX scratch is sized once");
+            impl_->nax_workspace = impl_->raw(bytes);
+            impl_->nax_workspace_bytes = bytes;
+        }
+    }
+    impl_->prepared_gate_up = gate_up_encoding;
+    impl_->prepared_down = down_encoding;
+}
+
+void HipGraph::prepare_dense_mm(uint32_t max_tokens, uint32_t max_columns) {
+    impl_->idle();
+    require(max_tokens >= 1 && max_tokens <= 65536 && max_columns >= 256 && max_columns <= 65536, "dense dequant-GEMM preparation bounds mismatch");
+    const uint64_t bytes = tsp_dense_mm_workspace_bytes(max_tokens, (max_columns + 255) / 256 * 256);
+    require(impl_->dense_workspace == nullptr, "dense dequant-GEMM scratch is sized once");
+    impl_->dense_workspace = impl_->raw(bytes);
+    impl_->dense_workspace_bytes = bytes;
+}
+
+// ------------------------------------------------------------------ batches
+void HipGraph::begin() {
+    impl_->idle();
+    impl_->locked = true;
+    impl_->encoding = true;
+    impl_->dispatches = 0;
+    impl_->wall_start = std::chrono::steady_clock::now();
+    hip(hipEventRecord(impl_->started, impl_->stream), "hipEventRecord");
+}
+
+void HipGraph::abort() {
+    impl_->same_thread();
+    require(impl_->encoding, "no GPU batch to abort");
+    // launches already enqueued cannot be recalled: drain them, then drop whatever they flagged
+    hip(hipStreamSynchronize(impl_->stream), "hipStreamSynchronize");
+    hip(hipMemset(impl_->error_word, 0, 4), "hipMemset");
+    impl_->encoding = false;
+}
+
+BatchResult HipGraph::submit() {
+    impl_->same_thread();
+    require(impl_->encoding, "no GPU batch to submit");
+    hip(hipEventRecord(impl_->finished, impl_->stream), "hipEventRecord");
+    hip(hipStreamSynchronize(impl_->stream), "hipStreamSynchronize");
+    impl_->encoding = false;
+    uint32_t word = 0;
+    hip(hipMemcpy(&word, impl_->error_word, 4, hipMemcpyDeviceToHost), "hipMemcpy");
+    if (word) {
+        hip(hipMemset(impl_->error_word, 0, 4), "hipMemset");  // later batches are unaffected
+        throw FormatError("GPU graph produced nonfinite values or invalid gates");
+    }
+    float gpu_ms = 0;
+    hip(hipEventElapsedTime(&gpu_ms, impl_->started, impl_->finished), "hipEventElapsedTime");
+    const double wall_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - impl_->wall_start).count();
+    return {impl_->dispatches, wall_ms, gpu_ms};
+}
+
+// ------------------------------------------------------------------ operators
+void HipGraph::gemv(uint32_t encoding, GpuView matrix, GpuView input, GpuView output, uint32_t columns, uint32_t rows) {
+    auto& p = *impl_; p.active();
+    require(input.bytes == uint64_t(columns) * 4 && output.bytes == uint64_t(rows) * 4, "GEMV vector byte span mismatch");
+    const std::array in{matrix, input};
+    validate_disjoint(in, std::array{output});
+    const PlanarEntry* planar = p.planar_of(matrix);
+    check(tsp_gemv(encoding, planar ? TSP_LAYOUT_PLANAR_V3 : TSP_LAYOUT_GGUF, p.device(matrix), matrix.bytes, reinterpret_cast<const float*>(p.device(input)),
+                   reinterpret_cast<float*>(p.device(output, true)), columns, rows, p.error_word, p.stream));
+}
+
+void HipGraph::gemv_rows(uint32_t encoding, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output) {
+    auto& p = *impl_; p.active();
+    p.rows_fit(input, "GEMV rows geometry mismatch");
+    p.rows_fit(output, "GEMV rows geometry mismatch");
+    require(input.rows == output.rows, "GEMV rows geometry mismatch");
+    validate_disjoint(std::array{matrix, input.view}, std::array{output.view});
+    check(tsp_gemv_rows(encoding, TSP_LAYOUT_GGUF, p.device(matrix), matrix.bytes, reinterpret_cast<const float*>(p.device(input.view)), input.stride_bytes,
+                        reinterpret_cast<float*>(p.device(output.view, true)), output.stride_bytes, input.rows, input.columns, output.columns,
+                        p.error_word, p.stream));
+}
+
+void HipGraph::prepare_q8_matvec_many(uint32_t width) {
+    impl_->idle();
+    require(width == 1 || width == 2 || width == 4 || width == 8, "unsupported Q8-many pipeline width");
+}
+
+void HipGraph::q8_matvec_many(GpuView matrix, GpuView input, GpuView output, uint32_t columns, uint32_t rows, uint32_t width) {
+    auto& p = *impl_; p.active();
+    require(input.bytes == uint64_t(columns) * width * 4 && output.bytes == uint64_t(rows) * width * 4, "Q8-many vector byte span mismatch");
+    validate_disjoint(std::array{matrix, input}, std::array{output});
+    check(tsp_q8_matvec_many(TSP_LAYOUT_GGUF, p.device(matrix), matrix.bytes, reinterpret_cast<const float*>(p.device(input)),
+                             reinterpret_cast<float*>(p.device(output, true)), columns, rows, width, p.error_word, p.stream));
+}
+
+void HipGraph::route(GpuView logits, GpuView indices, GpuView weights, uint32_t selected, RouterMode mode, bool normalize_selected) {
+    auto& p = *impl_; p.active();
+    require(logits.bytes % 4 == 0 && logits.bytes / 4 <= 4096 && indices.bytes == uint64_t(selected) * 4 && weights.bytes == uint64_t(selected) * 4,
+            "graph router shape/mode mismatch");
+    validate_disjoint(std::array{logits}, std::array{indices, weights});
+    check(tsp_route(reinterpret_cast<const float*>(p.device(logits)), reinterpret_cast<uint32_t*>(p.device(indices, true)),
+                    reinterpret_cast<float*>(p.device(weights, true)), uint32_t(logits.bytes / 4), selected, uint32_t(mode), normalize_selected,
+                    p.error_word, p.stream));
+}
+
+void HipGraph::prefill_route_batch(GpuView logits, GpuView indices, GpuView weights, uint32_t experts, uint32_t selected, uint32_t tokens,
+                                   RouterMode mode, bool normalize_selected) {
+    auto& p = *impl_; p.active();
+    require(logits.bytes == checked_mul(checked_mul(tokens, experts), 4) && indices.bytes == checked_mul(checked_mul(tokens, selected), 4) &&
+                weights.bytes == indices.bytes,
+            "prefill route batch geometry/mode mismatch");
+    validate_disjoint(std::array{logits}, std::array{indices, weights});
+    check(tsp_route_batch(reinterpret_cast<const float*>(p.device(logits)), reinterpret_cast<uint32_t*>(p.device(indices, true)),
+                          reinterpret_cast<float*>(p.device(weights, true)), experts, selected, tokens, uint32_t(mode), normalize_selected,
+                          p.error_word, p.stream));
+}
+
+void HipGraph::routed_gemv(uint32_t encoding, GpuView matrices, GpuView indices, GpuView input, GpuView output, uint32_t columns, uint32_t rows,
+                           uint32_t experts, bool broadcast_input) {
+    auto& p = *impl_; p.active();
+    require(indices.bytes % 4 == 0 && indices.bytes >= 4, "routed GEMV index span mismatch");
+    const uint32_t selected = uint32_t(indices.bytes / 4);
+    require(input.bytes == uint64_t(columns) * 4 * (broadcast_input ? 1 : selected) && output.bytes == uint64_t(rows) * 4 * selected,
+            "routed GEMV vector byte span mismatch");
+    validate_disjoint(std::array{matrices, indices, input}, std::array{output});
+    check(tsp_routed_gemv(encoding, p.device(matrices), matrices.bytes, reinterpret_cast<const uint32_t*>(p.device(indices)),
+                          reinterpret_cast<const float*>(p.device(input)), reinterpret_cast<float*>(p.device(output, true)), columns, rows, experts,
+                          selected, broadcast_input, p.error_word, p.stream));
+}
+
+void HipGraph::swiglu(GpuView gate, GpuView up, GpuView output, float scale) {
+    auto& p = *impl_; p.active();
+    require(gate.bytes == up.bytes && gate.bytes == output.bytes && gate.bytes % 4 == 0 && gate.bytes > 0, "graph SwiGLU shape/scale mismatch");
+    (void)p.allocation(gate); (void)p.allocation(up);
+    check(tsp_swiglu(reinterpret_cast<const float*>(p.device(gate)), reinterpret_cast<const float*>(p.device(up)),
+                     reinterpret_cast<float*>(p.device(output, true)), gate.bytes / 4, scale, p.error_word, p.stream));
+}
+
+void HipGraph::mixture(GpuView expert_outputs, GpuView weights, GpuView shared_output, GpuView shared_logit, GpuView output) {
+    auto& p = *impl_; p.active();
+    require(output.bytes % 4 == 0 && output.bytes > 0 && weights.bytes % 4 == 0 && weights.bytes > 0 && shared_output.bytes == output.bytes &&
+                shared_logit.bytes == 4 && expert_outputs.bytes == checked_mul(output.bytes, weights.bytes / 4),
+            "mixture shape mismatch");
+    validate_disjoint(std::array{expert_outputs, weights, shared_output, shared_logit}, std::array{output});
+    check(tsp_mixture(reinterpret_cast<const float*>(p.device(expert_outputs)), reinterpret_cast<const float*>(p.device(weights)),
+                      reinterpret_cast<const float*>(p.device(shared_output)), reinterpret_cast<const float*>(p.device(shared_logit)),
+                      reinterpret_cast<float*>(p.device(output, true)), uint32_t(output.bytes / 4), uint32_t(weights.bytes / 4), p.error_word, p.stream));
+}
+
+void HipGraph::prefill_mixture_batch(GpuView experts, GpuView weights, GpuView shared, GpuView shared_logit, GpuRowsF32 output, uint32_t selected) {
+    auto& p = *impl_; p.active();
+    p.rows_fit(output, "mixture shape mismatch");
+    const uint64_t tokens = output.rows, channels = output.columns;
+    require(selected >= 1 && experts.bytes == checked_mul(checked_mul(tokens * selected, channels), 4) && weights.bytes == tokens * selected * 4 &&
+                shared.bytes == tokens * channels * 4 && shared_logit.bytes == tokens * 4,
+            "mixture shape mismatch");
+    validate_disjoint(std::array{experts, weights, shared, shared_logit}, std::array{output.view});
+    check(tsp_mixture_batch(reinterpret_cast<const float*>(p.device(experts)), reinterpret_cast<const float*>(p.device(weights)),
+                            reinterpret_cast<const float*>(p.device(shared)), reinterpret_cast<const float*>(p.device(shared_logit)),
+                            reinterpret_cast<float*>(p.device(output.view, true)), output.stride_bytes, output.columns, selected, output.rows,
+                            p.error_word, p.stream));
+}
+
+namespace {
+struct PlanarTriple { PlanarMatrixShape lo, hi, dn; };
+}
+
+void HipGraph::planar_moe_gate_up_swiglu_m8(GpuView pair_lo, GpuView pair_hi, GpuView indices, GpuRowsF32 input, GpuRowsF32 expert_hidden,
+                                            uint32_t experts, uint32_t selected) {
+    auto& p = *impl_; p.active();
+    const PlanarEntry* lo = p.planar_of(pair_lo);
+    const PlanarEntry* hi = p.planar_of(pair_hi);
+    require(lo && hi && p.union_meta, "planar v3 MoE requires registered matrices and prepare_planar_moe_v3");
+    p.rows_fit(input, "planar v3 MoE shape or stride mismatch");
+    p.rows_fit(expert_hidden, "planar v3 MoE shape or stride mismatch");
+    require(lo->shape.experts == experts && hi->shape.experts == experts && input.rows >= 1 && input.rows <= 8 &&
+                expert_hidden.rows == input.rows * selected && indices.bytes == uint64_t(expert_hidden.rows) * 4 &&
+                input.columns == lo->shape.columns && expert_hidden.columns == lo->shape.rows,
+            "planar v3 MoE shape or stride mismatch");
+    validate_disjoint(std::array{pair_lo, pair_hi, indices, input.view}, std::array{expert_hidden.view});
+    tsp_small_moe m{};
+    m.pair_lo = p.device(pair_lo); m.pair_hi = p.device(pair_hi);
+    m.gate_kind = lo->shape.kind; m.up_kind = hi->shape.kind; m.down_kind = TSP_KIND_Q8_PLANAR;
+    m.channels = input.columns; m.hidden = expert_hidden.columns; m.experts = experts; m.selected = selected; m.tokens = input.rows;
+    m.ids = reinterpret_cast<const uint32_t*>(p.device(indices));
+    m.x = reinterpret_cast<const float*>(p.device(input.view)); m.x_stride_bytes = input.stride_bytes;
+    m.h = reinterpret_cast<float*>(p.device(expert_hidden.view, true)); m.h_stride_bytes = expert_hidden.stride_bytes;
+    m.union_meta = static_cast<uint32_t*>(p.union_meta); m.error_word = p.error_word;
+    check(tsp_planar_moe_gate_up_swiglu_m8(&m, p.stream));
+}
+
+void HipGraph::planar_moe_routed_m8(GpuView pair_lo, GpuView pair_hi, GpuView down_weights, GpuView indices, GpuRowsF32 input,
+                                    GpuRowsF32 expert_hidden, GpuRowsF32 expert_down, uint32_t experts, uint32_t selected) {
+    auto& p = *impl_; p.active();
+    const PlanarEntry* lo = p.planar_of(pair_lo);
+    const PlanarEntry* hi = p.planar_of(pair_hi);
+    const PlanarEntry* dn = p.planar_of(down_weights);
+    require(lo && hi && dn && p.union_meta, "planar v3 MoE requires registered matrices and prepare_planar_moe_v3");
+    p.rows_fit(input, "planar v3 MoE shape or stride mismatch");
+    p.rows_fit(expert_hidden, "planar v3 MoE shape or stride mismatch");
+    p.rows_fit(expert_down, "planar v3 MoE shape or stride mismatch");
+    require(lo->shape.experts == experts && hi->shape.experts == experts && dn->shape.experts == experts && input.rows >= 1 && input.rows <= 8 &&
+                expert_hidden.rows == input.rows * selected && expert_down.rows == expert_hidden.rows &&
+                indices.bytes == uint64_t(expert_hidden.rows) * 4 && input.columns == lo->shape.columns &&
+                expert_hidden.columns == lo->shape.rows && dn->shape.columns == expert_hidden.columns && dn->shape.rows == expert_down.columns &&
+                expert_down.columns == input.columns,
+            "planar v3 MoE shape or stride mismatch");
+    validate_disjoint(std::array{pair_lo, pair_hi, down_weights, indices, input.view}, std::array{expert_hidden.view, expert_down.view});
+    tsp_small_moe m{};
+    m.pair_lo = p.device(pair_lo); m.pair_hi = p.device(pair_hi); m.down = p.device(down_weights);
+    m.gate_kind = lo->shape.kind; m.up_kind = hi->shape.kind; m.down_kind = dn->shape.kind;
+    m.channels = input.columns; m.hidden = expert_hidden.columns; m.experts = experts; m.selected = selected; m.tokens = input.rows;
+    m.ids = reinterpret_cast<const uint32_t*>(p.device(indices));
+    m.x = reinterpret_cast<const float*>(p.device(input.view)); m.x_stride_bytes = input.stride_bytes;
+    m.h = reinterpret_cast<float*>(p.device(expert_hidden.view, true)); m.h_stride_bytes = expert_hidden.stride_bytes;
+    m.y = reinterpret_cast<float*>(p.device(expert_down.view, true)); m.y_stride_bytes = expert_down.stride_bytes;
+    m.union_meta = static_cast<uint32_t*>(p.union_meta); m.error_word = p.error_word;
+    check(tsp_planar_moe_routed_m8(&m, p.stream));
+}
+
+void HipGraph::planar_nax_grouped_moe(GpuView pair_lo, GpuView pair_hi, GpuView down_weights, GpuView indices, GpuRowsF32 input,
+                                      GpuRowsF32 expert_down, GpuView token_map, GpuView counts, GpuView tasks, uint32_t experts,
+                                      uint32_t selected) {
+    auto& p = *impl_; p.active();
+    const PlanarEntry* lo = p.planar_of(pair_lo);
+    const PlanarEntry* hi = p.planar_of(pair_hi);
+    const PlanarEntry* dn = p.planar_of(down_weights);
+    require(lo && hi && dn && p.nax_workspace, "planar v3 NAX grouped MoE requires registered matrices and prepared scratch");
+    p.rows_fit(input, "planar v3 NAX grouped MoE shape or stride mismatch");
+    p.rows_fit(expert_down, "planar v3 NAX grouped MoE shape or stride mismatch");
+    const uint32_t tokens = input.rows;
+    require(lo->shape.experts == experts && hi->shape.experts == experts && dn->shape.experts == experts && expert_down.rows == tokens * selected &&
+                indices.bytes == uint64_t(tokens) * selected * 4 && input.columns == lo->shape.columns && expert_down.columns == input.columns &&
+                dn->shape.columns == lo->shape.rows && dn->shape.rows == input.columns,
+            "planar v3 NAX grouped MoE shape or stride mismatch");
+    require(token_map.bytes >= checked_mul(checked_mul(experts, tokens), 4) && counts.bytes >= uint64_t(experts) * 4 &&
+                tasks.bytes >= (2 + 2 * (uint64_t(tokens) * selected / 32 + experts)) * 4,
+            "planar v3 NAX grouped MoE routing scratch too small");
+    const uint64_t need = tsp_planar_nax_workspace_bytes(tokens, selected, experts, input.columns, lo->shape.rows);
+    require(need <= p.nax_workspace_bytes, "planar v3 NAX scratch too small for requested batch");
+    validate_disjoint(std::array{pair_lo, pair_hi, down_weights, indices, input.view}, std::array{expert_down.view, token_map, counts, tasks});
+    tsp_grouped_moe m{};
+    m.pair_lo = p.device(pair_lo); m.pair_hi = p.device(pair_hi); m.down = p.device(down_weights);
+    m.gate_kind = lo->shape.kind; m.up_kind = hi->shape.kind; m.down_kind = dn->shape.kind;
+    m.channels = input.columns; m.hidden = lo->shape.rows; m.experts = experts; m.selected = selected; m.tokens = tokens;
+    m.ids = reinterpret_cast<const uint32_t*>(p.device(indices));
+    m.x = reinterpret_cast<const float*>(p.device(input.view)); m.x_stride_bytes = input.stride_bytes;
+    m.y = reinterpret_cast<float*>(p.device(expert_down.view, true)); m.y_stride_bytes = expert_down.stride_bytes;
+    m.token_map = reinterpret_cast<uint32_t*>(p.device(token_map, true));
+    m.counts = reinterpret_cast<uint32_t*>(p.device(counts, true));
+    m.tasks = reinterpret_cast<uint32_t*>(p.device(tasks, true));
+    m.workspace = p.nax_workspace; m.workspace_bytes = p.nax_workspace_bytes; m.error_word = p.error_word;
+    check(tsp_planar_nax_grouped_moe(&m, p.stream));
+}
+
+void HipGraph::dense_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output) {
+    auto& p = *impl_; p.active();
+    require(p.dense_workspace, "dense dequant-GEMM requires prepare_dense_mm");
+    p.rows_fit(input, "dense dequant-GEMM geometry");
+    p.rows_fit(output, "dense dequant-GEMM geometry");
+    require(input.rows == output.rows, "dense dequant-GEMM geometry");
+    require(tsp_dense_mm_workspace_bytes(input.rows, input.columns) <= p.dense_workspace_bytes, "dense dequant-GEMM workspace too small");
+    validate_disjoint(std::array{matrix, input.view}, std::array{output.view});
+    check(tsp_dense_mm(encoding, uint32_t(layout), p.device(matrix), matrix.bytes, p.device(input.view), input.stride_bytes, 0,
+                       p.device(output.view, true), output.stride_bytes, 0, input.rows, input.columns, output.columns, p.dense_workspace,
+                       p.dense_workspace_bytes, p.error_word, p.stream));
+}
+
+uint64_t HipGraph::logit_topk_scratch_bytes(uint32_t max_rows, uint32_t max_vocabulary) {
+    const uint64_t bytes = tsp_logit_topk_scratch_bytes(max_rows, max_vocabulary);
+    require(bytes > 0, "GPU logit top-k scratch bounds mismatch");
+    return bytes;
+}
+
+uint64_t HipGraph::logit_topk_output_bytes(uint32_t max_rows) {
+    const uint64_t bytes = tsp_logit_topk_output_bytes(max_rows);
+    require(bytes > 0, "GPU logit top-k output row count out of bounds");
+    return bytes;
+}
+
+void HipGraph::prepare_logit_topk() {
+    impl_->idle();
+    impl_->topk_prepared = true;
+}
+
+void HipGraph::logit_topk(GpuRowsF32 logits, GpuView partial_scratch, GpuView out_rows) {
+    auto& p = *impl_; p.active();
+    require(p.topk_prepared, "GPU logit top-k requires prepared direct batches");
+    p.rows_fit(logits, "GPU logit top-k geometry mismatch");
+    validate_disjoint(std::array{logits.view}, std::array{partial_scratch, out_rows});
+    check(tsp_logit_topk(reinterpret_cast<const float*>(p.device(logits.view)), logits.stride_bytes, logits.rows, logits.columns,
+                         p.device(partial_scratch, true), partial_scratch.bytes, p.device(out_rows, true), out_rows.bytes, p.stream));
+}
+
+// ------------------------------------------------------------------ MoE compositions
+namespace {
+void shape_check(MoeShape s) {  // src/moe.cpp:9-12
+    require(s.channels >= 1 && s.hidden >= 1 && s.experts >= 1 && s.selected >= 1 && s.selected <= s.experts && s.selected <= 64,
+            "mixture sublayer shape mismatch");
+}
+}  // namespace
+
+MoeScratch allocate_moe_scratch(HipGraph& graph, MoeShape shape) {
+    shape_check(shape);
+    const std::array<uint64_t, 10> counts{shape.experts, shape.selected, shape.selected, checked_mul(shape.hidden, shape.selected),
+                                          checked_mul(shape.hidden, shape.selected), checked_mul(shape.channels, shape.selected), shape.hidden,
+                                          shape.hidden, shape.channels, 1};
+    std::array<GpuView, 10> views{};
+    size_t made = 0;
+    try {
+        for (; made < counts.size(); ++made) views[made] = graph.zeros(checked_mul(counts[made], 4), "mixture scratch");
+    } catch (...) {
+        for (size_t i = 0; i < made; ++i) graph.release(views[i]);
+        throw;
+    }
+    return {views[0], views[1], views[2], views[3], views[4], views[5], views[6], views[7], views[8], views[9]};
+}
+
+void release_moe_scratch(HipGraph& graph, const MoeScratch& scratch) {
+    for (const auto view : scratch.views()) graph.release(view);
+}
+
+bool is_planar_moe(const HipGraph& g, const MoeWeights& w, MoeShape s) {
+    const auto lo = g.planar_matrix_shape(w.gate.view);
+    const auto hi = g.planar_matrix_shape(w.up.view);
+    const auto dn = g.planar_matrix_shape(w.down.view);
+    if (!lo || !hi || !dn) return false;
+    return (lo->kind == 2u || lo->kind == 4u || lo->kind == 6u) && (hi->kind == 3u || hi->kind == 5u || hi->kind == 7u) &&
+           (dn->kind == 8u || dn->kind == 9u || dn->kind == 10u) && lo->source_type == w.gate.encoding && hi->source_type == w.up.encoding &&
+           dn->source_type == w.down.encoding && lo->source_type == hi->source_type && lo->columns == s.channels && lo->rows == s.hidden &&
+           lo->experts == s.experts && hi->columns == s.channels && hi->rows == s.hidden && hi->experts == s.experts && dn->columns == s.hidden &&
+           dn->rows == s.channels && dn->experts == s.experts;
+}
+
+void encode_moe(HipGraph& graph, const MoeWeights& w, const MoeScratch& s, GpuView input, GpuView output, MoeShape shape, RouterMode mode,
+                bool normalize_selected) {
+    shape_check(shape);
+    graph.gemv(w.router.encoding, w.router.view, input, s.logits, shape.channels, shape.experts);
+    graph.route(s.logits, s.indices, s.weights, shape.selected, mode, normalize_selected);
+    if (is_planar_moe(graph, w, shape)) {
+        graph.planar_moe_routed_m8(w.gate.view, w.up.view, w.down.view, s.indices, {input, 1, shape.channels, uint64_t(shape.channels) * 4},
+                                   {s.gate, shape.selected, shape.hidden, uint64_t(shape.hidden) * 4},
+                                   {s.down, shape.selected, shape.channels, uint64_t(shape.channels) * 4}, shape.experts, shape.selected);
+    } else {
+        graph.routed_gemv(w.gate.encoding, w.gate.view, s.indices, input, s.gate, shape.channels, shape.hidden, shape.experts, true);
+        graph.routed_gemv(w.up.encoding, w.up.view, s.indices, input, s.up, shape.channels, shape.hidden, shape.experts, true);
+        graph.swiglu(s.gate, s.up, s.gate);
+        graph.routed_gemv(w.down.encoding, w.down.view, s.indices, s.gate, s.down, shape.hidden, shape.channels, shape.experts, false);
+    }
+    graph.gemv(w.shared_gate.encoding, w.shared_gate.view, input, s.shared_gate, shape.channels, shape.hidden);
+    graph.gemv(w.shared_up.encoding, w.shared_up.view, input, s.shared_up, shape.channels, shape.hidden);
+    graph.swiglu(s.shared_gate, s.shared_up, s.shared_gate);
+    graph.gemv(w.shared_down.encoding, w.shared_down.view, s.shared_gate, s.shared_down, shape.hidden, shape.channels);
+    graph.gemv(w.shared_router.encoding, w.shared_router.view, input, s.shared_logit, shape.channels, 1);
+    graph.mixture(s.down, s.weights, s.shared_down, s.shared_logit, output);
+}
+
+MoeBatchScratch allocate_moe_batch_scratch(HipGraph& graph, MoeShape shape, uint32_t tokens) {
+    shape_check(shape);
+    require(tokens >= 1 && tokens <= 2048, "prefill MoE token count out of bounds");
+    const uint64_t routes = uint64_t(tokens) * shape.selected;
+    const auto tasks_bytes = [&](uint64_t r, uint64_t experts) { return (2 + 2 * (r / 32 + experts)) * 4; };
+    const std::array<uint64_t, 12> bytes{routes * 4, routes * 4, checked_mul(routes * shape.channels, 4), checked_mul(uint64_t(shape.experts) * tokens, 4),
+                                         uint64_t(shape.experts) * 4, tasks_bytes(routes, shape.experts), uint64_t(tokens) * 4,
+                                         checked_mul(uint64_t(tokens) * shape.channels, 4), uint64_t(2) * tokens * 4, 2 * 4, tasks_bytes(tokens, 2),
+                                         uint64_t(tokens) * 4};
+    std::array<GpuView, 12> v{};
+    size_t made = 0;
+    try {
+        for (; made < bytes.size(); ++made) v[made] = graph.zeros(bytes[made], "prefill mixture scratch");
+    } catch (...) {
+        for (size_t i = 0; i < made; ++i) graph.release(v[i]);
+        throw;
+    }
+    return {v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], v[9], v[10], v[11]};
+}
+
+void release_moe_batch_scratch(HipGraph& graph, const MoeBatchScratch& s) {
+    for (const auto view : {s.indices, s.weights, s.expert_down, s.token_map, s.counts, s.tasks, s.shared_indices, s.shared_down, s.shared_token_map,
+                            s.shared_counts, s.shared_tasks, s.shared_logit})
+        graph.release(view);
+}
+
+void encode_moe_batch(HipGraph& graph, const MoeWeights& w, const MoeBatchScratch& s, GpuView logits, GpuRowsF32 input, GpuRowsF32 output,
+                      MoeShape shape, RouterMode mode, bool normalize_selected) {
+    shape_check(shape);
+    const uint32_t tokens = input.rows;
+    graph.prefill_route_batch(logits, s.indices, s.weights, shape.experts, shape.selected, tokens, mode, normalize_selected);
+    graph.planar_nax_grouped_moe(w.gate.view, w.up.view, w.down.view, s.indices, input,
+                                 {s.expert_down, tokens * shape.selected, shape.channels, uint64_t(shape.channels) * 4}, s.token_map, s.counts, s.tasks,
+                                 shape.experts, shape.selected);
+    // the shared expert is a two-expert planar stack of which every token selects expert 0 (shared_indices stay zero)
+    graph.planar_nax_grouped_moe(w.shared_gate.view, w.shared_up.view, w.shared_down.view, s.shared_indices, input,
+                                 {s.shared_down, tokens, shape.channels, uint64_t(shape.channels) * 4}, s.shared_token_map, s.shared_counts,
+                                 s.shared_tasks, 2, 1);
+    graph.gemv_rows(w.shared_router.encoding, w.shared_router.view, input, {s.shared_logit, tokens, 1, 4});
+    graph.prefill_mixture_batch(s.expert_down, s.weights, s.shared_down, s.shared_logit, output, shape.selected);
+}
+
+}  // namespace tokspur

@@ -1,0 +1,178 @@
+// tokspur::HipGraph — the host side of the quantized-matmul / MoE path on one MI355X, with the operator
+// interface of the engine's graph class (include/tokspur/graph.hpp:431-1168 `MetalGraph`) for this path:
+// same handle types, same operator names and argument meaning, same lifecycle and error behaviour.
+//
+//   * buffers are `GpuView` capabilities issued by this graph (zeros / upload / slice), charged to a byte
+//     budget and checked on every use; a released or foreign view is refused, never rebound
+//     (graph.hpp:94-101, ledger graph.mm:1866-1893);
+//   * allocation, upload, read-back and registration are legal only while the graph is idle; operators are
+//     legal only between begin() and submit() / abort() (graph.mm:991-992); nothing is allocated while encoding;
+//   * host-side refusals throw FormatError before anything is enqueued; device-side conditions (non-finite
+//     values, bad expert ids) set a sticky word that submit() reads and turns into
+//     FormatError("GPU graph produced nonfinite values or invalid gates") (graph.mm:3977-3978);
+//   * one host thread and one in-order HIP stream per graph.
+//
+// Every operator forwards to one entry point of the C ABI in include/tokspur_hip.h.
+#pragma once
+
+#include <array>
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <optional>
+#include <span>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace tokspur {
+
+// include/tokspur/gguf.hpp:16-19
+class FormatError : public std::runtime_error {
+public:
+    using std::runtime_error::runtime_error;
+};
+
+// include/tokspur/graph.hpp:96-108
+struct GpuView {
+    uint64_t owner = 0;
+    size_t slot = 0;
+    uint64_t offset = 0;
+    uint64_t bytes = 0;
+};
+struct GpuRowsF32 {
+    GpuView view;
+    uint32_t rows = 0;
+    uint32_t columns = 0;
+    uint64_t stride_bytes = 0;
+};
+// include/tokspur/graph.hpp:123-129; kind 10 (Q6_K planes) is this library's extension
+struct PlanarMatrixShape {
+    uint32_t source_type = 0;
+    uint32_t kind = 0;
+    uint32_t columns = 0;
+    uint32_t rows = 0;
+    uint32_t experts = 0;
+};
+// include/tokspur/graph.hpp:140-146 (the fields that exist without Metal)
+struct GraphMemory {
+    uint64_t budget = 0;
+    uint64_t live_bytes = 0;
+    uint64_t peak_bytes = 0;
+    uint64_t allocations = 0;
+};
+// include/tokspur/graph.hpp:270-275
+struct BatchResult {
+    uint64_t dispatches = 0;
+    double wall_ms = 0;
+    double gpu_ms = 0;
+};
+// include/tokspur/routing.hpp:10, include/tokspur/grouped_mm.hpp:6 (+ the Pack v3 planes as layout 3)
+enum class RouterMode : uint32_t { softmax, sigmoid };
+enum class PrefillWeightLayout : uint32_t { gguf = 0, q8_lanes_v1 = 1, q51_lanes_v1 = 2, planar_v3 = 3 };
+// include/tokspur/sampling.hpp:21-29
+struct GpuLogitTopKRow {
+    uint32_t vocabulary = 0;
+    uint32_t count = 0;
+    uint32_t first_nonfinite_col = 0xffffffffu;
+    uint32_t first_subnormal_col = 0xffffffffu;
+    std::array<uint32_t, 64> ids{};
+    std::array<float, 64> logits{};
+};
+static_assert(sizeof(GpuLogitTopKRow) == 528, "GpuLogitTopKRow ABI");
+
+class HipGraph {
+public:
+    explicit HipGraph(uint64_t byte_budget);
+    ~HipGraph();
+    HipGraph(const HipGraph&) = delete;
+    HipGraph& operator=(const HipGraph&) = delete;
+
+    // ---- storage (idle only), graph.hpp:438-496
+    [[nodiscard]] GpuView zeros(uint64_t bytes, std::string label);
+    [[nodiscard]] GpuView upload(std::span<const std::byte> data, std::string label, bool immutable = true);
+    [[nodiscard]] GpuView slice(GpuView buffer, uint64_t offset, uint64_t bytes) const;
+    void write(GpuView destination, std::span<const std::byte> data);
+    [[nodiscard]] std::vector<std::byte> read(GpuView source) const;
+    void read(GpuView source, std::span<std::byte> destination) const;
+    void release(GpuView full_buffer);
+    [[nodiscard]] GraphMemory memory() const;
+    [[nodiscard]] std::string device_name() const;
+    void validate_disjoint(std::span<const GpuView> inputs, std::span<const GpuView> destinations) const;  // graph.hpp:671
+
+    // ---- Pack v3 registration (idle only, before the first batch), graph.hpp:465-471
+    void register_planar_matrix(GpuView matrix, PlanarMatrixShape shape);
+    [[nodiscard]] uint64_t planar_matrix_count() const;
+    [[nodiscard]] std::optional<PlanarMatrixShape> planar_matrix_shape(GpuView matrix) const;
+    void prepare_planar_moe_v3(uint32_t gate_up_encoding, uint32_t down_encoding, bool prepare_nax = true,
+                               uint32_t max_nax_tokens = 2048, uint32_t max_experts = 512, uint32_t max_selected = 10,
+                               uint32_t max_channels = 2560, uint32_t max_hidden = 640);
+    void prepare_dense_mm(uint32_t max_tokens, uint32_t max_columns);  // workspace of dense_mm, sized while idle
+
+    // ---- batches, graph.hpp:709-714
+    void begin();
+    void abort();
+    [[nodiscard]] BatchResult submit();
+
+    // ---- operators (between begin and submit)
+    void gemv(uint32_t encoding, GpuView matrix, GpuView input, GpuView output, uint32_t columns, uint32_t rows);  // graph.hpp:730
+    void gemv_rows(uint32_t encoding, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output);                         // graph.hpp:733
+    void prepare_q8_matvec_many(uint32_t width);                                                                    // graph.hpp:744
+    void q8_matvec_many(GpuView matrix, GpuView input, GpuView output, uint32_t columns, uint32_t rows, uint32_t width);
+    void route(GpuView logits, GpuView indices, GpuView weights, uint32_t selected, RouterMode mode, bool normalize_selected);  // 1091
+    void prefill_route_batch(GpuView logits, GpuView indices, GpuView weights, uint32_t experts, uint32_t selected,
+                             uint32_t tokens, RouterMode mode, bool normalize_selected);                             // graph.hpp:852
+    void routed_gemv(uint32_t encoding, GpuView matrices, GpuView indices, GpuView input, GpuView output, uint32_t columns,
+                     uint32_t rows, uint32_t experts, bool broadcast_input);                                         // graph.hpp:1093
+    void swiglu(GpuView gate, GpuView up, GpuView output, float scale = 1);                                          // graph.hpp:990
+    void mixture(GpuView expert_outputs, GpuView weights, GpuView shared_output, GpuView shared_logit, GpuView output);  // 1102
+    void prefill_mixture_batch(GpuView experts, GpuView weights, GpuView shared, GpuView shared_logit, GpuRowsF32 output,
+                               uint32_t selected);                                                                  // graph.hpp:853
+    void planar_moe_gate_up_swiglu_m8(GpuView pair_lo, GpuView pair_hi, GpuView indices, GpuRowsF32 input,
+                                      GpuRowsF32 expert_hidden, uint32_t experts, uint32_t selected);               // graph.hpp:472
+    void planar_moe_routed_m8(GpuView pair_lo, GpuView pair_hi, GpuView down_weights, GpuView indices, GpuRowsF32 input,
+                              GpuRowsF32 expert_hidden, GpuRowsF32 expert_down, uint32_t experts, uint32_t selected);  // 475
+    void planar_nax_grouped_moe(GpuView pair_lo, GpuView pair_hi, GpuView down_weights, GpuView indices, GpuRowsF32 input,
+                                GpuRowsF32 expert_down, GpuView token_map, GpuView counts, GpuView tasks, uint32_t experts,
+                                uint32_t selected);                                                                  // graph.hpp:478
+    // graph.hpp:750-753 `grouped_mm` with experts = 1, selected = 1, broadcast: the dense dequant-GEMM (Q4_K rows or planes)
+    void dense_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output);
+    static uint64_t logit_topk_scratch_bytes(uint32_t max_rows, uint32_t max_vocabulary = 1u << 20);                 // graph.hpp:1030
+    static uint64_t logit_topk_output_bytes(uint32_t max_rows);
+    void prepare_logit_topk();
+    void logit_topk(GpuRowsF32 logits, GpuView partial_scratch, GpuView out_rows);                                    // graph.hpp:1033
+
+private:
+    struct Impl;
+    std::unique_ptr<Impl> impl_;
+};
+
+// ---- the MoE sublayer for one token, include/tokspur/moe.hpp:9-45, src/moe.cpp:13-83
+struct GpuMatrix { GpuView view; uint32_t encoding; };
+struct MoeShape { uint32_t channels, hidden, experts, selected; };
+struct MoeWeights { GpuMatrix router, gate, up, down, shared_gate, shared_up, shared_down, shared_router; };
+struct MoeScratch {
+    GpuView logits, indices, weights, gate, up, down, shared_gate, shared_up, shared_down, shared_logit;
+    [[nodiscard]] std::array<GpuView, 10> views() const { return {logits, indices, weights, gate, up, down, shared_gate, shared_up, shared_down, shared_logit}; }
+};
+MoeScratch allocate_moe_scratch(HipGraph& graph, MoeShape shape);
+void release_moe_scratch(HipGraph& graph, const MoeScratch& scratch);
+[[nodiscard]] bool is_planar_moe(const HipGraph& graph, const MoeWeights& weights, MoeShape shape);
+// Encodes router GEMV -> top-k -> routed experts -> shared expert -> mixture into the caller's current batch; allocates,
+// reads and commits nothing.
+void encode_moe(HipGraph& graph, const MoeWeights& weights, const MoeScratch& scratch, GpuView input, GpuView output,
+                MoeShape shape, RouterMode mode, bool normalize_selected);
+
+// ---- the prefill MoE sublayer for a batch of tokens (the routed half of src/moe_mm_many.cpp:126-283): batch router top-k ->
+// grouped planar MoE -> shared expert through the same grouped path -> batch mixture. Logits are an input (the router
+// projection is outside this path).
+struct MoeBatchScratch {
+    GpuView indices, weights, expert_down, token_map, counts, tasks, shared_indices, shared_down, shared_token_map, shared_counts,
+        shared_tasks, shared_logit;
+};
+MoeBatchScratch allocate_moe_batch_scratch(HipGraph& graph, MoeShape shape, uint32_t tokens);
+void release_moe_batch_scratch(HipGraph& graph, const MoeBatchScratch& scratch);
+void encode_moe_batch(HipGraph& graph, const MoeWeights& weights, const MoeBatchScratch& scratch, GpuView logits, GpuRowsF32 input,
+                      GpuRowsF32 output, MoeShape shape, RouterMode mode, bool normalize_selected);
+
+}  // namespace tokspur
