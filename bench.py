@@ -101,10 +101,16 @@ def main():
     def routed_only():
         capi.planar_nax_grouped_moe(gpu, w, ids, d_x, T, S, scratch, y=y)
 
+    side = torch.cuda.Stream()  # default priority: the shared expert only needs x, so it runs beside the routed experts
+
     def step_c3():
+        main = torch.cuda.current_stream()
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            capi.planar_nax_grouped_moe(gpu, ws, ids_shared, d_x, T, 1, scratch_s, y=ys)
         gpu.route(d_logits, S, 0, True, tokens=T, out=(ids, wts))
         routed_only()
-        capi.planar_nax_grouped_moe(gpu, ws, ids_shared, d_x, T, 1, scratch_s, y=ys)
+        main.wait_stream(side)
         gpu.mixture(y, wts, ys, shared_logit, C, S, tokens=T, out=out)
 
     ms_step = timed(torch, step_c3, args.steps, args.warmup)
@@ -209,9 +215,13 @@ def main():
         def step_c2():
             lg, xx = sets[state["i"] % len(sets)]
             state["i"] += 1
+            main = torch.cuda.current_stream()
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                capi.planar_moe_routed_m8(gpu, ws, ids_s2, xx, T2, 1, h=hs2, y=ys2)
             gpu.route(lg, S, 0, True, tokens=T2, out=(ids2, wts2))
             capi.planar_moe_routed_m8(gpu, w, ids2, xx, T2, S, h=h2, y=y2)
-            capi.planar_moe_routed_m8(gpu, ws, ids_s2, xx, T2, 1, h=hs2, y=ys2)
+            main.wait_stream(side)
             gpu.mixture(y2, wts2, ys2, sl2, C, S, tokens=T2, out=out2)
 
         ms = timed(torch, step_c2, 48, 16)

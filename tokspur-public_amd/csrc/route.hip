@@ -25,13 +25,40 @@ __device__ __forceinline__ float route_activation(float logit, float maximum, ui
     return sigmoid_f(logit);
 }
 
-__device__ __forceinline__ float wave_max(float v) {
-    for (int m = 1; m < kWave; m <<= 1) v = fmaxf(v, __shfl_xor(v, m, kWave));
-    return v;
+// A candidate as one 64-bit key: high word = the logit mapped to an unsigned integer of the same order (-0 as +0), low
+// word = ~expert, so the largest key is the largest logit and, among equal logits, the lowest expert id. 0 = no candidate.
+__device__ __forceinline__ uint64_t route_key(float logit, uint32_t expert) {
+    uint32_t bits = __float_as_uint(logit);
+    if ((bits & 0x7fffffffu) == 0) bits = 0;
+    const uint32_t ordered = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+    return (uint64_t(ordered) << 32) | uint32_t(~expert);
 }
-__device__ __forceinline__ uint32_t wave_min(uint32_t v) {
-    for (int m = 1; m < kWave; m <<= 1) { const uint32_t o = __shfl_xor(v, m, kWave); v = o < v ? o : v; }
-    return v;
+__device__ __forceinline__ float route_key_logit(uint64_t key) {
+    const uint32_t ordered = uint32_t(key >> 32);
+    return __uint_as_float((ordered & 0x80000000u) ? (ordered & 0x7fffffffu) : ~ordered);
+}
+template <int Ctrl>
+__device__ __forceinline__ uint64_t dpp_max_u64(uint64_t v) {
+    const uint32_t lo = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v)), Ctrl, 0xf, 0xf, true));
+    const uint32_t hi = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v >> 32)), Ctrl, 0xf, 0xf, true));
+    const uint64_t other = (uint64_t(hi) << 32) | lo;
+    return other > v ? other : v;
+}
+// Largest key of the wave, uniform: four cross-lane steps inside each row of 16 lanes, then the four rows by scalar reads.
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
+    v = dpp_max_u64<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_max_u64<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_max_u64<0x141>(v);  // row_half_mirror
+    v = dpp_max_u64<0x140>(v);  // row_mirror
+    uint64_t best = 0;
+#pragma unroll
+    for (int row = 0; row < 4; ++row) {
+        const uint32_t lo = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(v)), row * 16));
+        const uint32_t hi = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(v >> 32)), row * 16));
+        const uint64_t k = (uint64_t(hi) << 32) | lo;
+        best = k > best ? k : best;
+    }
+    return best;
 }
 __device__ __forceinline__ float wave_sum_shfl(float v) {
     for (int m = 1; m < kWave; m <<= 1) v += __shfl_xor(v, m, kWave);
@@ -46,37 +73,34 @@ __global__ __launch_bounds__(64) void route_rows(const float* __restrict__ logit
     const uint32_t row = blockIdx.x, lane = threadIdx.x;
     if (row >= tokens) return;
     const float* row_logits = logits + uint64_t(row) * experts;
-    float cand[CAND];
+    uint64_t cand[CAND];
     uint32_t bad = 0;
 #pragma unroll
     for (int k = 0; k < CAND; ++k) {
         const uint32_t i = lane + k * kWave;
-        float v = -INFINITY;
+        uint64_t key = 0;
         if (i < experts) {
-            v = row_logits[i];
+            float v = row_logits[i];
             if (nonfinite(v)) { bad |= TSP_ERRBIT_NONFINITE; v = -INFINITY; }
+            key = route_key(v, i);
         }
-        cand[k] = v;
+        cand[k] = key;
     }
     // chosen logit j is kept by lane j (selected <= 64)
     float chosen_mine = 0, chosen_first = 0;
     for (uint32_t s = 0; s < selected; ++s) {
-        float best = -INFINITY;
-        uint32_t expert = 0xffffffffu;
+        uint64_t best = 0;
 #pragma unroll
-        for (int k = 0; k < CAND; ++k) {
-            const uint32_t i = lane + k * kWave;
-            if (i < experts && (cand[k] > best || (cand[k] == best && i < expert))) { best = cand[k]; expert = i; }
-        }
-        const float score = wave_max(best);
-        uint32_t chosen = wave_min(best == score ? expert : 0xffffffffu);
-        if (chosen >= experts) { bad |= TSP_ERRBIT_INDEX; chosen = 0; }
+        for (int k = 0; k < CAND; ++k) best = cand[k] > best ? cand[k] : best;
+        best = wave_max_u64(best);
+        uint32_t chosen = ~uint32_t(best);
+        if (best == 0 || chosen >= experts) { bad |= TSP_ERRBIT_INDEX; chosen = 0; }
         if (lane == 0) indices[uint64_t(row) * selected + s] = chosen;
-        const float value = nonfinite(score) ? row_logits[chosen] : score;
+        const float value = best == 0 ? row_logits[chosen] : route_key_logit(best);
         if (s == 0) chosen_first = value;
         if (s == lane) chosen_mine = value;
 #pragma unroll
-        for (int k = 0; k < CAND; ++k) if (chosen == lane + k * kWave) cand[k] = -INFINITY;
+        for (int k = 0; k < CAND; ++k) if (cand[k] == best) cand[k] = 0;
     }
     const float act = lane < selected ? route_activation(chosen_mine, chosen_first, mode, normalize) : 0.0f;
     float sum = mode ? 1.0f : 0.0f;
