@@ -259,8 +259,8 @@ int tsp_planar_moe_routed_m8(const tsp_small_moe* moe, void* stream);
 
 /* include/tokspur/graph.hpp:750-753 `grouped_mm` with experts = selected = 1, broadcast (the dense case,
  * kernels/grouped_mm.metal:159-243) and 859-860 `dense_mm_q8`: out[t, r] = sum_c x[t, c] * dec(W[r, c]) for
- * `tokens` rows. Declared precision as in the engine: weights dequantised in f32 and staged as f16,
- * activations staged as bf16-valued f16, f32 accumulation. Input rows are f32 or bf16, output rows f32 or
+ * `tokens` rows. Activations are used as bf16 values (carried as f16), weights enter the matrix cores as exact integer
+ * factors whose block scales are applied in f32, f32 accumulation. Input rows are f32 or bf16, output rows f32 or
  * bf16 (RNE); strides in bytes. Q4_K raw GGUF rows or planar planes, Q6_K planes. `workspace` is caller
  * owned scratch of tsp_dense_mm_workspace_bytes(tokens, columns) bytes, 16-byte aligned. */
 uint64_t tsp_dense_mm_workspace_bytes(uint32_t tokens, uint32_t columns);
@@ -268,6 +268,17 @@ int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matrix, uint64_
                  uint64_t input_stride_bytes, int input_is_bf16, void* output, uint64_t output_stride_bytes, int output_is_bf16,
                  uint32_t tokens, uint32_t columns, uint32_t rows, void* workspace, uint64_t workspace_bytes,
                  uint32_t* error_word, void* stream);
+
+/* include/tokspur/graph.hpp:750-753 `grouped_mm` (src/graph.mm:4534-4606; kernels/grouped_mm.metal:159-243; route and task
+ * preparation kernels/grouped_mpp.metal:12-64): for every route rid = t*selected + slot, output[rid, :] = W[ids[rid]] * x, with x the
+ * token's row (broadcast) or row rid of the input. `matrices` is a raw GGUF stack [experts][rows][row bytes] (Q4_K here); token_map,
+ * counts and tasks (tile 32) are outputs with the engine's layouts. Activations are used as bf16 values, weights as exact integer
+ * factors with f32 block scales, f32 accumulation. workspace: tsp_grouped_mm_workspace_bytes(...) bytes, 256-byte aligned. */
+uint64_t tsp_grouped_mm_workspace_bytes(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t columns, int broadcast);
+int tsp_grouped_mm(uint32_t encoding, uint32_t layout, const void* matrices, uint64_t matrices_bytes, const uint32_t* ids,
+                   const float* input, uint64_t input_stride_bytes, float* output, uint64_t output_stride_bytes, uint32_t* token_map,
+                   uint32_t* counts, uint32_t* tasks, uint32_t columns, uint32_t rows, uint32_t experts, uint32_t selected,
+                   uint32_t tokens, int broadcast, void* workspace, uint64_t workspace_bytes, uint32_t* error_word, void* stream);
 
 /* The operands of `planar_nax_grouped_moe` (include/tokspur/graph.hpp:478-481; src/graph.mm:9293-9420).
  * x holds `tokens` f32 rows of `channels`; y (the engine's expert_down) holds tokens*selected f32 rows

@@ -124,6 +124,38 @@ def test_config1_dense_q4k_gemm(gpu, tsp, orc, synth, tokens):
     assert np.array_equal(out_p, out_f32[perm])
 
 
+# ---------------------------------------------------------------------------------- grouped GEMM, raw GGUF stacks
+
+@pytest.mark.parametrize("broadcast", [True, False])
+@pytest.mark.parametrize("tokens,selected,experts", [(1, 1, 1), (40, 3, 6), (200, 2, 4)])
+def test_grouped_mm_raw_q4k(gpu, tsp, orc, synth, tokens, selected, experts, broadcast):
+    """`grouped_mm` on raw GGUF Q4_K expert stacks (graph.hpp:750-753): out[rid] = W[ids[rid]] x, x per token (broadcast) or per
+    route; routes, counts and tile-32 tasks are the engine's, rows beyond the matrix and the row padding stay untouched."""
+    cols, rows = 512, 160
+    w = synth.matrix(12, 2500 + experts, rows * experts, cols)
+    rng = np.random.default_rng(tokens * 7 + selected)
+    ids = np.stack([rng.permutation(experts)[:selected] for _ in range(tokens)]).astype(np.uint32).reshape(-1)
+    routes = tokens * selected
+    in_rows = tokens if broadcast else routes
+    x = synth.round_bf16(synth.activations_f32(2501 + tokens, (in_rows, cols + 4)))
+    out = gpu.full((routes, rows + 4), -9.0)
+    got, scratch = tsp.grouped_mm(gpu, 12, gpu.upload(w), gpu.upload(ids), gpu.upload(x), cols, rows, experts, selected, tokens, broadcast,
+                                  out=out, x_stride=(cols + 4) * 4, out_stride=(rows + 4) * 4)
+    got = got.cpu().numpy()
+    assert gpu.error() == 0 and (got[:, rows:] == -9.0).all()
+    per_expert = (cols // 256) * 144 * rows
+    for rid in range(routes):
+        e = int(ids[rid])
+        xr = x[rid // selected if broadcast else rid, :cols]
+        want = orc.staged_gemm(12, w[e * per_expert:(e + 1) * per_expert], cols, xr[None, :], nrows=rows, stage_f16=False)[0]
+        assert max_rel_error(got[rid, :rows], want) <= 2e-5
+    want_map, want_counts, _ = orc.grouped_routes(ids, experts, selected, tokens)
+    assert np.array_equal(scratch["counts"].cpu().numpy().view(np.uint32), want_counts)
+    assert np.array_equal(scratch["tasks"].cpu().numpy().view(np.uint32), orc.grouped_tasks(want_counts, experts, selected, tokens, 32)[0])
+    with pytest.raises(tsp.FormatError):
+        tsp.grouped_mm(gpu, 8, gpu.upload(w), gpu.upload(ids), gpu.upload(x), cols, rows, experts, selected, tokens, broadcast)
+
+
 # ---------------------------------------------------------------------------------- grouped MoE
 
 def reference_ids(n, selected, experts):

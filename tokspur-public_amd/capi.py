@@ -394,6 +394,26 @@ def dense_mm_workspace_bytes(tokens, columns):
     return f(C.c_uint32(tokens), C.c_uint32(columns))
 
 
+def grouped_mm(dev, encoding, matrices, ids, x, columns, rows, experts, selected, tokens, broadcast, out=None, scratch=None,
+               x_stride=None, out_stride=None):
+    """Raw-GGUF grouped dequant-GEMM (`grouped_mm`): out[rid] = W[ids[rid]] x (x per token when broadcast, else per route)."""
+    f = dll().tsp_grouped_mm_workspace_bytes
+    f.restype = C.c_uint64
+    routes = tokens * selected
+    out = dev.empty((routes, rows)) if out is None else out
+    if scratch is None:
+        scratch = {"token_map": dev.zeros(experts * tokens, "int32"), "counts": dev.zeros(experts, "int32"),
+                   "tasks": dev.zeros(2 + 2 * (routes // 32 + experts), "int32"),
+                   "workspace": dev.empty(f(C.c_uint32(tokens), C.c_uint32(selected), C.c_uint32(experts), C.c_uint32(columns), C.c_int(bool(broadcast))), "uint8")}
+    check(dll().tsp_grouped_mm(C.c_uint32(encoding), C.c_uint32(LAYOUT_GGUF), dev.ptr(matrices), C.c_uint64(dev.nbytes(matrices)), dev.ptr(ids),
+                               dev.ptr(x), C.c_uint64(columns * 4 if x_stride is None else x_stride), dev.ptr(out),
+                               C.c_uint64(rows * 4 if out_stride is None else out_stride), dev.ptr(scratch["token_map"]), dev.ptr(scratch["counts"]),
+                               dev.ptr(scratch["tasks"]), C.c_uint32(columns), C.c_uint32(rows), C.c_uint32(experts), C.c_uint32(selected),
+                               C.c_uint32(tokens), C.c_int(bool(broadcast)), dev.ptr(scratch["workspace"]), C.c_uint64(dev.nbytes(scratch["workspace"])),
+                               dev.ptr(dev.err), dev.stream()))
+    return out, scratch
+
+
 def planar_nax_workspace_bytes(tokens, selected, experts, channels, hidden):
     f = dll().tsp_planar_nax_workspace_bytes
     f.restype = C.c_uint64

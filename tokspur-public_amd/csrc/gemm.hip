@@ -33,7 +33,7 @@ using namespace tsp;
 namespace {
 
 enum Epilogue : int { EPI_F32 = 0, EPI_BF16 = 1, EPI_SWIGLU = 2 };
-enum Rows : int { ROWS_DENSE = 0, ROWS_GATHER_TOKENS = 1, ROWS_TASK_SLOTS = 2 };
+enum Rows : int { ROWS_DENSE = 0, ROWS_GATHER_TOKENS = 1, ROWS_TASK_SLOTS = 2, ROWS_ROUTES = 3 };
 
 constexpr int kTaskRows = 64;
 constexpr int kRowTiles = kTaskRows / 32;
@@ -56,6 +56,8 @@ struct GemmArgs {
     uint64_t out_stride;      // bytes
     float out_scale;
     uint32_t* error_word;
+    uint64_t raw_expert_bytes;       // raw GGUF expert stacks: bytes between experts (0 for one dense matrix)
+    uint32_t broadcast;              // ROWS_ROUTES: one input row per token instead of one per route
     uint32_t col_tiles, task_slots;  // logical grid: column tiles x tasks, launched as one linear grid
 };
 
@@ -122,7 +124,12 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
             // rows past the task's end re-read its first row: their accumulators are never stored
             uint32_t rid = a.token_map[uint64_t(expert) * a.tokens + start + (tid < nrows ? tid : 0)];
             if (rid >= a.tokens * a.selected || a.ids[rid] != expert) { rid = 0xffffffffu; task_bad = 1; }
-            row_src[tid] = ROWS == ROWS_GATHER_TOKENS ? (rid == 0xffffffffu ? 0 : rid / a.selected) : task * kTaskRows + (tid < nrows ? tid : 0);
+            // activation row: the route's token (gate/up, broadcast grouped GEMM), the route itself (grouped GEMM with one input
+            // row per route) or the task's slot in the intermediate buffer (down); output row: task slot or route
+            const uint32_t safe = rid == 0xffffffffu ? 0 : rid;
+            row_src[tid] = ROWS == ROWS_GATHER_TOKENS ? safe / a.selected
+                         : ROWS == ROWS_ROUTES       ? (a.broadcast ? safe / a.selected : safe)
+                                                     : task * kTaskRows + (tid < nrows ? tid : 0);
             row_dst[tid] = ROWS == ROWS_GATHER_TOKENS ? task * kTaskRows + tid : rid;
         }
     }
@@ -150,7 +157,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
             col_live[j] = n < a.n;
             wrow[j] = col_live[j] ? n : a.n - 1;
             out_col[j] = n;
-            wbase[j] = BKIND == B_Q4K_RAW ? a.w0 : a.w0 + uint64_t(expert) * a.spec.planar_expert_bytes;
+            wbase[j] = a.w0 + uint64_t(expert) * (BKIND == B_Q4K_RAW ? a.raw_expert_bytes : a.spec.planar_expert_bytes);
         }
     }
     const uint32_t bpr = a.k / 256;
@@ -503,7 +510,7 @@ __global__ __launch_bounds__(256) void to_f16_rows(const void* __restrict__ src,
 
 template <int BKIND, int EPI, int ROWS>
 int launch(const GemmArgs& a, uint32_t col_tiles, uint32_t tasks, hipStream_t s) {
-    constexpr const char* name = EPI == EPI_SWIGLU ? "gemm_gate_up_swiglu" : ROWS == ROWS_TASK_SLOTS ? "gemm_down" : "gemm_dense";
+    constexpr const char* name = EPI == EPI_SWIGLU ? "gemm_gate_up_swiglu" : ROWS == ROWS_TASK_SLOTS ? "gemm_down" : ROWS == ROWS_ROUTES ? "gemm_grouped" : "gemm_dense";
     GemmArgs g = a;
     g.col_tiles = col_tiles;
     g.task_slots = tasks;
@@ -577,6 +584,71 @@ extern "C" int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matr
                                                                : launch<B_Q4K_PLANAR, EPI_F32, ROWS_DENSE>(a, col_tiles, tasks, s);
     return output_is_bf16 ? launch<B_Q4K_RAW, EPI_BF16, ROWS_DENSE>(a, col_tiles, tasks, s)
                           : launch<B_Q4K_RAW, EPI_F32, ROWS_DENSE>(a, col_tiles, tasks, s);
+}
+
+// ---------------------------------------------------------------- grouped GEMM over raw GGUF expert stacks
+namespace {
+struct GroupedLayout { uint64_t xh, sx, tasks, total; uint32_t bound, in_rows; };
+GroupedLayout grouped_layout(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t columns, int broadcast) {
+    GroupedLayout l{};
+    l.in_rows = broadcast ? tokens : tokens * selected;
+    l.bound = tokens * selected / kTaskRows + experts;
+    l.sx = align256(uint64_t(l.in_rows) * columns * 2);
+    l.tasks = l.sx + align256(uint64_t(l.in_rows) * (columns / 256) * 32);
+    l.total = l.tasks + align256((2 + 2 * uint64_t(l.bound)) * 4);
+    return l;
+}
+}  // namespace
+
+extern "C" uint64_t tsp_grouped_mm_workspace_bytes(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t columns, int broadcast) {
+    return grouped_layout(tokens, selected, experts, columns, broadcast).total;
+}
+
+extern "C" int tsp_grouped_mm(uint32_t encoding, uint32_t layout, const void* matrices, uint64_t matrices_bytes, const uint32_t* ids,
+                              const float* input, uint64_t input_stride_bytes, float* output, uint64_t output_stride_bytes,
+                              uint32_t* token_map, uint32_t* counts, uint32_t* tasks, uint32_t columns, uint32_t rows, uint32_t experts,
+                              uint32_t selected, uint32_t tokens, int broadcast, void* workspace, uint64_t workspace_bytes,
+                              uint32_t* error_word, void* stream) {
+    TSP_REQUIRE(encoding == 12 && layout == TSP_LAYOUT_GGUF, "grouped dequant-GEMM on the matrix cores takes raw GGUF Q4_K expert stacks");
+    TSP_REQUIRE(columns && columns <= 65536 && columns % 256 == 0 && rows && rows <= 32768 && experts >= 1 && experts <= 512 &&
+                    selected >= 1 && selected <= 16 && selected <= experts && tokens >= 1 && tokens <= 2048,
+                "grouped prefill geometry mismatch");
+    const uint64_t expert_bytes = uint64_t(columns / 256) * 144 * rows;
+    TSP_REQUIRE(matrices_bytes == expert_bytes * experts && expert_bytes < (1ull << 32), "grouped prefill matrix byte span mismatch");
+    TSP_REQUIRE(input_stride_bytes >= uint64_t(columns) * 4 && input_stride_bytes % 4 == 0 && output_stride_bytes >= uint64_t(rows) * 4 &&
+                    output_stride_bytes % 4 == 0,
+                "grouped prefill row stride");
+    TSP_REQUIRE(matrices && ids && input && output && token_map && counts && tasks && workspace && error_word, "null device pointer");
+    const GroupedLayout l = grouped_layout(tokens, selected, experts, columns, broadcast);
+    TSP_REQUIRE(workspace_bytes >= l.total && reinterpret_cast<uintptr_t>(workspace) % 256 == 0 && reinterpret_cast<uintptr_t>(matrices) % 16 == 0,
+                "grouped prefill buffer span or alignment is invalid");
+    const uint32_t routes = tokens * selected;
+    const uint64_t in_span = uint64_t(l.in_rows - 1) * input_stride_bytes + uint64_t(columns) * 4;
+    const uint64_t out_span = uint64_t(routes - 1) * output_stride_bytes + uint64_t(rows) * 4;
+    const void* ins[] = {matrices, ids, input};
+    const uint64_t in_bytes[] = {matrices_bytes, uint64_t(routes) * 4, in_span};
+    const void* outs[] = {output, token_map, counts, tasks, workspace};
+    const uint64_t out_bytes[] = {out_span, uint64_t(experts) * tokens * 4, uint64_t(experts) * 4, (2 + 2 * (uint64_t(routes) / 32 + experts)) * 4, l.total};
+    for (int o = 0; o < 5; ++o) {
+        for (int i = 0; i < 3; ++i) TSP_REQUIRE(!ranges_overlap(outs[o], out_bytes[o], ins[i], in_bytes[i]), "grouped prefill outputs overlap inputs");
+        for (int q = 0; q < o; ++q) TSP_REQUIRE(!ranges_overlap(outs[o], out_bytes[o], outs[q], out_bytes[q]), "grouped prefill outputs overlap each other");
+    }
+    const auto s = static_cast<hipStream_t>(stream);
+    auto* ws = static_cast<uint8_t*>(workspace);
+    auto* xh = reinterpret_cast<_Float16*>(ws);
+    auto* sx = reinterpret_cast<_Float16*>(ws + l.sx);
+    auto* task_list = reinterpret_cast<uint32_t*>(ws + l.tasks);
+    int rc = tsp_grouped_routes(ids, token_map, counts, experts, selected, tokens, error_word, stream);
+    if (rc == TSP_OK) rc = tsp_grouped_tasks(counts, tasks, experts, selected, tokens, 32, error_word, stream);
+    if (rc == TSP_OK) rc = tsp_grouped_tasks(counts, task_list, experts, selected, tokens, kTaskRows, error_word, stream);
+    if (rc == TSP_OK) rc = convert_rows(input, input_stride_bytes, 0, xh, sx, l.in_rows, columns, error_word, s);
+    if (rc != TSP_OK) return rc;
+    GemmArgs a{};
+    a.a = xh; a.a_stride = columns; a.sx = sx; a.w0 = static_cast<const uint8_t*>(matrices); a.raw_expert_bytes = expert_bytes;
+    a.experts = experts; a.tasks = task_list; a.counts = counts; a.token_map = token_map; a.ids = ids; a.tokens = tokens; a.selected = selected;
+    a.broadcast = broadcast ? 1 : 0; a.n = rows; a.k = columns; a.out = output; a.out_stride = output_stride_bytes; a.out_scale = 1.0f;
+    a.error_word = error_word;
+    return launch<B_Q4K_RAW, EPI_F32, ROWS_ROUTES>(a, (rows + 255) / 256, l.bound, s);
 }
 
 // ---------------------------------------------------------------- grouped MoE

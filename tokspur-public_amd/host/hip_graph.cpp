@@ -66,6 +66,8 @@ struct HipGraph::Impl {
     uint64_t nax_workspace_bytes = 0;
     void* dense_workspace = nullptr;
     uint64_t dense_workspace_bytes = 0;
+    void* grouped_workspace = nullptr;
+    uint64_t grouped_workspace_bytes = 0;
     uint32_t prepared_gate_up = 0, prepared_down = 0;
 
     void same_thread() const { require(std::this_thread::get_id() == thread, "GPU graph used from another thread"); }
@@ -140,7 +142,7 @@ HipGraph::~HipGraph() {
     (void)hipStreamSynchronize(impl_->stream);
     for (auto& a : impl_->slots)
         if (a.live) (void)hipFree(a.device);
-    for (void* p : {impl_->union_meta, impl_->nax_workspace, impl_->dense_workspace, static_cast<void*>(impl_->error_word)})
+    for (void* p : {impl_->union_meta, impl_->nax_workspace, impl_->dense_workspace, impl_->grouped_workspace, static_cast<void*>(impl_->error_word)})
         if (p) (void)hipFree(p);
     (void)hipEventDestroy(impl_->started);
     (void)hipEventDestroy(impl_->finished);
@@ -511,6 +513,38 @@ void HipGraph::planar_nax_grouped_moe(GpuView pair_lo, GpuView pair_hi, GpuView 
     m.tasks = reinterpret_cast<uint32_t*>(p.device(tasks, true));
     m.workspace = p.nax_workspace; m.workspace_bytes = p.nax_workspace_bytes; m.error_word = p.error_word;
     check(tsp_planar_nax_grouped_moe(&m, p.stream));
+}
+
+void HipGraph::prepare_grouped_mm(uint32_t encoding, PrefillWeightLayout layout, uint32_t max_tokens, uint32_t max_selected, uint32_t max_experts,
+                                  uint32_t max_columns) {
+    impl_->idle();
+    require(encoding == 12 && layout == PrefillWeightLayout::gguf, "grouped prefill requires idle preparation and direct batches");
+    require(impl_->grouped_workspace == nullptr, "grouped prefill scratch is sized once");
+    const uint64_t bytes = tsp_grouped_mm_workspace_bytes(max_tokens, max_selected, max_experts, (max_columns + 255) / 256 * 256, 0);
+    impl_->grouped_workspace = impl_->raw(bytes);
+    impl_->grouped_workspace_bytes = bytes;
+}
+
+void HipGraph::grouped_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView matrices, GpuView indices, GpuRowsF32 input, GpuRowsF32 output,
+                          GpuView token_map, GpuView counts, GpuView tasks, uint32_t experts, uint32_t selected, bool broadcast) {
+    auto& p = *impl_; p.active();
+    require(p.grouped_workspace, "grouped prefill requires idle preparation and direct batches");
+    require(selected && output.rows % selected == 0, "grouped prefill route-row count mismatch");
+    const uint32_t tokens = output.rows / selected;
+    require(input.rows == (broadcast ? tokens : output.rows), "grouped prefill input-row count mismatch");
+    p.rows_fit(input, "grouped prefill buffer span or alignment is invalid");
+    p.rows_fit(output, "grouped prefill buffer span or alignment is invalid");
+    require(indices.bytes == uint64_t(output.rows) * 4 && token_map.bytes >= checked_mul(checked_mul(experts, tokens), 4) && counts.bytes >= uint64_t(experts) * 4 &&
+                tasks.bytes >= (2 + 2 * (uint64_t(output.rows) / 32 + experts)) * 4,
+            "grouped prefill buffer span or alignment is invalid");
+    require(tsp_grouped_mm_workspace_bytes(tokens, selected, experts, input.columns, broadcast) <= p.grouped_workspace_bytes,
+            "grouped prefill scratch too small for requested batch");
+    validate_disjoint(std::array{matrices, input.view, indices}, std::array{output.view, token_map, counts, tasks});
+    check(tsp_grouped_mm(encoding, uint32_t(layout), p.device(matrices), matrices.bytes, reinterpret_cast<const uint32_t*>(p.device(indices)),
+                         reinterpret_cast<const float*>(p.device(input.view)), input.stride_bytes, reinterpret_cast<float*>(p.device(output.view, true)),
+                         output.stride_bytes, reinterpret_cast<uint32_t*>(p.device(token_map, true)), reinterpret_cast<uint32_t*>(p.device(counts, true)),
+                         reinterpret_cast<uint32_t*>(p.device(tasks, true)), input.columns, output.columns, experts, selected, tokens, broadcast,
+                         p.grouped_workspace, p.grouped_workspace_bytes, p.error_word, p.stream));
 }
 
 void HipGraph::dense_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output) {

@@ -135,7 +135,12 @@ public:
     void planar_nax_grouped_moe(GpuView pair_lo, GpuView pair_hi, GpuView down_weights, GpuView indices, GpuRowsF32 input,
                                 GpuRowsF32 expert_down, GpuView token_map, GpuView counts, GpuView tasks, uint32_t experts,
                                 uint32_t selected);                                                                  // graph.hpp:478
-    // graph.hpp:750-753 `grouped_mm` with experts = 1, selected = 1, broadcast: the dense dequant-GEMM (Q4_K rows or planes)
+    // graph.hpp:750-753 `prepare_grouped_mm` / `grouped_mm`: raw GGUF Q4_K expert stacks, one output row per route
+    void prepare_grouped_mm(uint32_t encoding, PrefillWeightLayout layout, uint32_t max_tokens = 2048, uint32_t max_selected = 10,
+                            uint32_t max_experts = 512, uint32_t max_columns = 2560);
+    void grouped_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView matrices, GpuView indices, GpuRowsF32 input, GpuRowsF32 output,
+                    GpuView token_map, GpuView counts, GpuView tasks, uint32_t experts, uint32_t selected, bool broadcast);
+    // the same with experts = 1, selected = 1, broadcast: the dense dequant-GEMM (Q4_K rows or planes, Q6_K planes)
     void dense_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output);
     static uint64_t logit_topk_scratch_bytes(uint32_t max_rows, uint32_t max_vocabulary = 1u << 20);                 // graph.hpp:1030
     static uint64_t logit_topk_output_bytes(uint32_t max_rows);
