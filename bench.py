@@ -167,6 +167,22 @@ def main():
         cpu = {"value": T / (per_route * (T * S + T)), "unit": "tok/s", "cores": 1, "kind": kind,
                "sample": f"{done} of {T * S + T} expert routes of configs[3] (dequantize + double-accumulate GEMV for gate, up, down), "
                          f"{per_route * 1e3:.1f} ms per route, extrapolated linearly"}
+        # the same arithmetic, weight rows split over the host cores this process may use (the restated code: the
+        # reference ships its GEMV single-threaded)
+        cores = max(1, min(16, len(os.sched_getaffinity(0))))
+        t0, done = time.perf_counter(), 0
+        while done < 2048 and time.perf_counter() - t0 < 6.0:
+            rid = (done * 397) % (T * S)
+            e, xv = int(id_host[rid]), x[rid // S]
+            g = orc.reference_gemv_mt(12, gate[e * gsz:(e + 1) * gsz], C, H, xv, cores)
+            u = orc.reference_gemv_mt(12, up[e * gsz:(e + 1) * gsz], C, H, xv, cores)
+            gf = g.astype(np.float32)
+            h = (gf / (np.float32(1) + np.exp(-gf))) * u.astype(np.float32)
+            orc.reference_gemv_mt(14, down[e * dsz:(e + 1) * dsz], H, C, h, cores)
+            done += 1
+        per_route_mt = (time.perf_counter() - t0) / done
+        cpu["all_cores"] = {"value": T / (per_route_mt * (T * S + T)), "unit": "tok/s", "cores": cores, "kind": "port",
+                            "sample": f"{done} routes, {per_route_mt * 1e3:.2f} ms per route"}
 
     # ------------------------------------------------------------------ secondary configs
     if not args.skip_secondary:
@@ -196,6 +212,9 @@ def main():
                                   "note": "per-launch time over a 566 MB rotation of weight copies; a 4.7 MB launch is latency bound"}
         ms = timed(torch, lambda: gpu.gemv(12, copies[0], x0, C, 4096, y=y0), 240, 20)
         configs["c0_gemv_q4k"]["cache_resident_us"] = ms * 1e3
+        state["i"] = 0
+        k0 = profiled(capi, torch, gemv_rot, 120)
+        configs["c0_gemv_q4k"]["kernel_us"] = round(min(v["avg_us"] for v in k0.values()), 2)
         del copies
         # config 2: MoE verify T = 8 on the config-3 experts; eight router inputs in rotation so the ~150 MB of
         # selected experts differ from step to step and do not sit in the 256 MB last-level cache
@@ -245,6 +264,13 @@ def main():
             ms = timed(torch, lm_head, k2, 2)
             b4 = 330612736 + 615936 * m
             configs[f"c4_lm_head_q8_m{m}"] = {"us": ms * 1e3, "hbm_gbps": b4 / (ms * 1e-3) / 1e9, "hbm_frac": b4 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+            tk_scratch, tk_rows = gpu.empty(capi.logit_topk_scratch_bytes(m, V), "uint8"), gpu.empty(capi.logit_topk_output_bytes(m), "uint8")
+
+            def lm_head_argmax():
+                lm_head()
+                capi.logit_topk(gpu, y4, m, V, scratch=tk_scratch, out=tk_rows)
+
+            configs[f"c4_lm_head_q8_m{m}"]["us_with_top64"] = timed(torch, lm_head_argmax, k2, 2) * 1e3
         assert gpu.error() == 0, "device error word set during the secondary configurations"
 
     line = {
