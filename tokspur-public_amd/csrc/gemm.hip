@@ -17,11 +17,11 @@
 // One workgroup = 4 waves = one task (<= 64 activation rows of one expert, or one 64-row slab of a dense
 // matrix) x 256 weight rows. Each wave owns 64 weight rows (two 32-wide MFMA column tiles) and all 64
 // activation rows (two row tiles).
-//   * Weights never touch LDS: a lane loads 16 contiguous bytes of ITS weight row per K step straight
-//     into MFMA B-fragment order (lane = (row % 32, k-half)); every weight is unpacked once per task.
-//   * Activations are shared by the four waves: staged global -> LDS (padded rows), double buffered, one
-//     LDS-only barrier per K step; the next step's weight bytes and activation slab are requested before
-//     the current step is unpacked.
+//   * Quant bytes are loaded row-wise (one instruction = sixteen rows x 64 contiguous bytes), half a super-block ahead,
+//     parked in wave-private swizzled LDS and read back in MFMA B-fragment order (lane = (row % 32, k-half)); every
+//     weight is unpacked once per task.
+//   * Activations are shared by the four waves: 64 rows x 128 bytes per K step go global -> LDS directly (no registers),
+//     two and three steps ahead, into a ring of four slabs; one LDS-only barrier per K step.
 //   * For gate/up the two column tiles of a wave are the gate rows and the up rows of the same 32 hidden
 //     units, so SwiGLU is an element-wise epilogue on accumulator registers.
 #include "mfma_quant.hpp"
@@ -66,17 +66,27 @@ template <int BKIND, int EPI, int ROWS>
 __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two workgroups per CU: <= 256 registers per lane
     constexpr bool Q6 = BKIND == B_Q6K_PLANAR;
     constexpr int KSTEP = 64;
-    constexpr int LDA = KSTEP + 8;   // halfs per staged row: 16 bytes of padding spreads 16-byte reads over the banks
+    // LDS, carved by hand so that two workgroups fit one CU's 160 KB:
+    //   [ring of 4 activation slabs, 8 KB each][quant bytes, private to each wave, double buffered][Q4_K: activation sums x 2]
+    // One slab = 64 rows x 128 bytes, written by direct global -> LDS loads: 16-byte chunk c of row r sits at position
+    // r * 8 + (c ^ (r & 7)), so the loads fill LDS linearly by lane and the fragment reads spread over all banks.
+    // Quant bytes, half a super-block at a time: Q4_K [wave][buffer][64 rows][4 chunks of 16 B], Q6_K the same for the low
+    // nibbles plus [64 rows][2 chunks] of high bits; chunks are swizzled so that the row-wise stores and the column-wise
+    // reads both spread over all banks.
+    // The row tables live where no slab is yet (source rows, before the loop: the tail of slab 3) or any more (destination
+    // rows, after the loop: the head of slab 0).
+    constexpr int RING = 4, SLAB = kTaskRows * KSTEP * 2;
     constexpr int LDS_SX = 24;       // halfs per staged row of activation sums (16 used)
-    __shared__ __attribute__((aligned(16))) _Float16 lds_a[2][kTaskRows * LDA];
-    __shared__ __attribute__((aligned(16))) _Float16 lds_sx[2][Q6 ? 8 : kTaskRows * LDS_SX];
-    // Quant bytes, half a super-block at a time, double buffered, private to each wave: Q4_K
-    // [wave][buffer][64 rows][4 chunks of 16 B], Q6_K the same for the low nibbles plus [64 rows][2 chunks] of high bits.
-    // Chunks are swizzled so that the row-wise stores and the column-wise reads both spread over all banks
-    __shared__ __attribute__((aligned(16))) uint8_t lds_w[Q6 ? 4 * 2 * 64 * 96 : 4 * 2 * 64 * 64];
-    __shared__ uint32_t row_src[kTaskRows];
-    __shared__ uint32_t row_dst[kTaskRows];
-    __shared__ uint32_t task_bad;
+    constexpr int W_AT = RING * SLAB, W_BYTES = Q6 ? 4 * 2 * 64 * 96 : 4 * 2 * 64 * 64;
+    constexpr int SX_AT = W_AT + W_BYTES, SX_BYTES = Q6 ? 0 : 2 * kTaskRows * LDS_SX * 2;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[SX_AT + SX_BYTES];
+    static_assert(sizeof(lds_raw) <= 80 * 1024, "two workgroups per CU");
+    uint8_t* const lds_w = lds_raw + W_AT;
+    _Float16* const lds_sx = reinterpret_cast<_Float16*>(lds_raw + SX_AT);  // [2][kTaskRows * LDS_SX]
+    uint32_t* const row_src = reinterpret_cast<uint32_t*>(lds_raw + 3 * SLAB + SLAB - 512);
+    uint32_t* const task_bad_at = row_src + kTaskRows;
+    uint32_t* const row_dst = reinterpret_cast<uint32_t*>(lds_raw);
+#define task_bad (*task_bad_at)
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const uint32_t col = lane % 32, khalf = lane / 32;
@@ -97,13 +107,14 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
 
     // ---- task resolution
     uint32_t expert = 0, nrows = 0;
+    uint32_t my_dst = 0xffffffffu;  // output row of activation row `tid` (threads 0..63), parked in a register during the loop
     if (tid == 0) task_bad = 0;
     __syncthreads();
     if constexpr (ROWS == ROWS_DENSE) {
         const uint32_t row0 = task * kTaskRows;
         if (row0 >= a.m) return;
         nrows = a.m - row0 < kTaskRows ? a.m - row0 : kTaskRows;
-        if (tid < kTaskRows) { row_src[tid] = row0 + (tid < nrows ? tid : 0); row_dst[tid] = row0 + tid; }
+        if (tid < kTaskRows) { row_src[tid] = row0 + (tid < nrows ? tid : 0); my_dst = row0 + tid; }
     } else {
         const uint32_t bound = a.tokens * a.selected / kTaskRows + a.experts;
         const uint32_t live = a.tasks[0];
@@ -130,7 +141,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
             row_src[tid] = ROWS == ROWS_GATHER_TOKENS ? safe / a.selected
                          : ROWS == ROWS_ROUTES       ? (a.broadcast ? safe / a.selected : safe)
                                                      : task * kTaskRows + (tid < nrows ? tid : 0);
-            row_dst[tid] = ROWS == ROWS_GATHER_TOKENS ? task * kTaskRows + tid : rid;
+            my_dst = ROWS == ROWS_GATHER_TOKENS ? task * kTaskRows + tid : rid;
         }
     }
     __syncthreads();
@@ -171,26 +182,31 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    // ---- activation staging, global -> registers -> LDS: per step 64 rows x 128 bytes; instruction i of thread t takes
-    // the 16-byte chunk t % 8 of row t / 8 + 32 i, so one wave instruction reads eight rows' whole 128 bytes
-    const uint32_t st_row = tid / 8, st_chunk = tid % 8;
+    // ---- activation staging, global -> LDS directly, two K steps ahead: per step 64 rows x 128 bytes; instruction i of
+    // thread t fills LDS position t + 256 i (16-byte units) = slot t % 8 of row t / 8 + 32 i with chunk (t % 8) ^ (row % 8)
+    // of that row, so eight neighbouring lanes still read one row's whole 128 bytes
+    const uint32_t st_row = tid / 8, st_chunk = (tid % 8) ^ ((tid / 8) & 7);
     const _Float16* st_src0 = a.a + uint64_t(row_src[st_row]) * a.a_stride + st_chunk * 8;
     const _Float16* st_src1 = a.a + uint64_t(row_src[st_row + 32]) * a.a_stride + st_chunk * 8;
-    u32x4 stage[1][2] = {};
-    using Slot0 = std::integral_constant<int, 0>;
-    using Slot1 = std::integral_constant<int, 1>;  // tags also used as tile / position indices below
+    // fragment reads: lane (col, khalf) takes chunk {2 khalf, 2 khalf + 1, 4 + 2 khalf, 5 + 2 khalf}[q] of row col (+ 32 i)
+    uint32_t a_off[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) a_off[q] = col * 128 + (((q / 2) * 4 + 2 * khalf + (q % 2)) ^ (col & 7)) * 16;
+    // LDS address of this wave's 1 KB share of slab 0, rows 0..31 (uniform over the wave)
+    const uint32_t slab_lds = __builtin_amdgcn_readfirstlane(lds_address(lds_raw) + wave * 1024);
     // activation sums of one super-block: 64 rows x 32 bytes, threads 0..127 copy 16 bytes each
     const uint32_t sx_row = (tid / 2) % kTaskRows, sx_seg = tid % 2;
+    const uint32_t sx_src = row_src[sx_row];  // read now: the table's LDS becomes a slab once the loop runs
     uint4 sx_stage{};
     auto fetch_sx = [&](uint32_t b) {
         if constexpr (!Q6) {
             // 64 rows x 32 bytes; threads 128..255 repeat the work of 0..127 so that no load sits under a branch
-            sx_stage = *reinterpret_cast<const uint4*>(a.sx + (uint64_t(row_src[sx_row]) * bpr + b) * 16 + sx_seg * 8);
+            sx_stage = *reinterpret_cast<const uint4*>(a.sx + (uint64_t(sx_src) * bpr + b) * 16 + sx_seg * 8);
         }
     };
     auto store_sx = [&](int buf) {
         if constexpr (!Q6) {
-            *reinterpret_cast<uint4*>(&lds_sx[buf][sx_row * LDS_SX + sx_seg * 8]) = sx_stage;
+            *reinterpret_cast<uint4*>(&lds_sx[buf * kTaskRows * LDS_SX + sx_row * LDS_SX + sx_seg * 8]) = sx_stage;
         }
     };
     // The whole K loop is instantiated once per number of live 32-row tiles, so that its body is straight-line code:
@@ -198,21 +214,17 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
     // two MFMAs, and nothing could be scheduled across them.
     auto run = [&](auto mt_tag) {
         constexpr int MT = decltype(mt_tag)::value;
-        auto fetch_a = [&](uint32_t step, auto slot_tag) {  // rows 32..63 only when the task has them
-            constexpr int SLOT = decltype(slot_tag)::value;
-            stage[SLOT][0] = *reinterpret_cast<const u32x4*>(st_src0 + uint64_t(step) * KSTEP);
-            if constexpr (MT == 2) stage[SLOT][1] = *reinterpret_cast<const u32x4*>(st_src1 + uint64_t(step) * KSTEP);
-        };
-        auto store_a = [&](int buf, auto slot_tag) {
-            constexpr int SLOT = decltype(slot_tag)::value;
-            *reinterpret_cast<u32x4*>(&lds_a[buf][st_row * LDA + st_chunk * 8]) = stage[SLOT][0];
-            if constexpr (MT == 2) *reinterpret_cast<u32x4*>(&lds_a[buf][(st_row + 32) * LDA + st_chunk * 8]) = stage[SLOT][1];
+        auto dma_a = [&](uint32_t step, int ring) {  // rows 32..63 only when the task has them; steps past the end re-read the last
+            step = step < ksteps ? step : ksteps - 1;
+            const uint32_t dst = slab_lds + ring * SLAB;
+            load_to_lds_16(st_src0 + uint64_t(step) * KSTEP, dst);
+            if constexpr (MT == 2) load_to_lds_16(st_src1 + uint64_t(step) * KSTEP, dst + 4096);
         };
         // one k16 MFMA per (row tile, column tile); `first` starts the super-block accumulator from zero
-        auto mfma = [&](int buf, int k0, const f16x8& b0, const f16x8& b1, bool first) {
+        auto mfma = [&](int ring, int q, const f16x8& b0, const f16x8& b1, bool first) {
     #pragma unroll
             for (int i = 0; i < MT; ++i) {
-                const f16x8 af = *reinterpret_cast<const f16x8*>(&lds_a[buf][(i * 32 + col) * LDA + k0]);
+                const f16x8 af = *reinterpret_cast<const f16x8*>(lds_raw + ring * SLAB + i * 4096 + a_off[q]);
                 if (first) {
                     const f32x16 zero{};
                     blk[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b0, zero, 0, 0, 0);
@@ -234,8 +246,8 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
             }
         };
 
-        fetch_a(0, Slot0{});
-        store_a(0, Slot0{});
+        dma_a(0, 0);
+        dma_a(1, 1);
         if constexpr (Q6) {
             // Q6_K planes. Low nibbles (64 B) and high bit pairs (32 B) of one 128-column section per row travel
             // global -> registers -> LDS -> fragment registers one section (two K steps) ahead, loaded row-wise like
@@ -279,12 +291,16 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
             // K step H of a super-block: section H/2 (128 columns), quarters 2*(H%2) and 2*(H%2)+1 of that section
             auto half_step = [&](uint32_t step, auto h_tag) {
                 constexpr int H = decltype(h_tag)::value;
-                constexpr int buf = H & 1, wbuf = H / 2;
+                constexpr int wbuf = H / 2, ring = H;  // step % RING
                 const uint32_t b = step / 4;
-                fetch_a(step + 1 < ksteps ? step + 1 : step, Slot0{});
+                // Even steps request the slabs of the steps two and three ahead, as the first loads after their barrier; the
+                // only loads younger than those are the section (6) and, at H == 2, scale (4) loads of the same step, and
+                // for an odd step the two slabs and the loads of the even step before it. Loads complete in order.
+                constexpr int W[4] = {6, 0, 10, 0};
+                lds_barrier_after_loads<H % 2 == 0 ? W[(H + 2) % 4] : W[(H + 1) % 4] + 2 * MT + W[(H + 3) % 4]>();  // slab and this wave's section bytes are complete; every wave has left the other buffers
+                if (H % 2 == 0) { dma_a(step + 2, (ring + 2) % RING); dma_a(step + 3, (ring + 3) % RING); }
                 if (H % 2 == 0) fetch_w(step / 2 + 1);
                 if (H == 2) { scl_next[0] = load_scales(b + 1, 0); scl_next[1] = load_scales(b + 1, 1); }
-                lds_barrier();  // lds_a[buf] and this wave's section bytes are complete; every wave has left the other buffers
                 if (H % 2 == 0) {
     #pragma unroll
                     for (int j = 0; j < 2; ++j) {
@@ -301,16 +317,16 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
                     f16x8 f0[2], f1[2];
                     frags_q6k<Q>(raw[0], khalf, f0);
                     frags_q6k<Q>(raw[1], khalf, f1);
-                    mfma(buf, (Q % 2) * 32 + khalf * 16, f0[0], f1[0], H == 0 && Q == 0);
-                    mfma(buf, (Q % 2) * 32 + khalf * 16 + 8, f0[1], f1[1], false);
+                    mfma(ring, (Q % 2) * 2, f0[0], f1[0], H == 0 && Q == 0);
+                    mfma(ring, (Q % 2) * 2 + 1, f0[1], f1[1], false);
                 };
                 quarter(std::integral_constant<int, 2 * (H % 2)>{});
                 quarter(std::integral_constant<int, 2 * (H % 2) + 1>{});
                 if (H == 3) fold(scl[0].d, scl[1].d);
-                store_a(buf ^ 1, Slot0{});
                 if (H % 2 == 1) store_w(wbuf ^ 1);
                 if (H == 3) { scl[0] = scl_next[0]; scl[1] = scl_next[1]; }
             };
+            wait_all_loads();  // slabs 0 and 1 (the stores above already waited for younger loads)
             for (uint32_t b = 0; b < bpr; ++b) {
                 half_step(b * 4 + 0, std::integral_constant<int, 0>{});
                 half_step(b * 4 + 1, std::integral_constant<int, 1>{});
@@ -370,45 +386,48 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
             store_sx(0);
             auto pair_step = [&](uint32_t step, auto p_tag) {
                 constexpr int P = decltype(p_tag)::value;
-                constexpr int buf = P & 1, wbuf = P / 2;
+                constexpr int wbuf = P / 2, ring = P;  // step % RING
                 const uint32_t b = step / 4;
-                fetch_a(step + 1 < ksteps ? step + 1 : step, Slot0{});
+                // Even steps request the slabs of the steps two and three ahead, as the first loads after their barrier; the
+                // only loads younger than those are the other loads of the same step (W), and for an odd step the two slabs
+                // and the loads of the even step before it. Loads complete in order.
+                constexpr int W[4] = {5, 0, 8, 0};  // sums + half-block, -, half-block + headers, -
+                lds_barrier_after_loads<P % 2 == 0 ? W[(P + 2) % 4] : W[(P + 1) % 4] + 2 * MT + W[(P + 3) % 4]>();  // slab, this wave's weight bytes (and at P == 3 lds_sx[b & 1]) are complete; every wave has left the other buffers
+                if (P % 2 == 0) { dma_a(step + 2, (ring + 2) % RING); dma_a(step + 3, (ring + 3) % RING); }
                 if (P == 0) fetch_sx(b + 1 < bpr ? b + 1 : b);
                 if (P == 0 || P == 2) fetch_w_all(step / 2 + 1);
                 if (P == 2) {
     #pragma unroll
                     for (int j = 0; j < 2; ++j) hdr_next[j] = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, b + 1 < bpr ? b + 1 : b);
                 }
-                lds_barrier();  // lds_a[buf], this wave's weight bytes (and at P == 0 lds_sx[b & 1]) are complete; every wave has left the other buffers
                 const u32x4 raw0 = read_w(wbuf, 0, P & 1), raw1 = read_w(wbuf, 1, P & 1);
                 f16x8 f0[2], f1[2];
                 frags_q4k<P, 0>(raw0, hdr[0], f0);
                 frags_q4k<P, 0>(raw1, hdr[1], f1);
-                mfma(buf, khalf * 16, f0[0], f1[0], P == 0);
-                mfma(buf, khalf * 16 + 8, f0[1], f1[1], false);
+                mfma(ring, 0, f0[0], f1[0], P == 0);
+                mfma(ring, 1, f0[1], f1[1], false);
                 frags_q4k<P, 1>(raw0, hdr[0], f0);
                 frags_q4k<P, 1>(raw1, hdr[1], f1);
-                mfma(buf, 32 + khalf * 16, f0[0], f1[0], false);
-                mfma(buf, 32 + khalf * 16 + 8, f0[1], f1[1], false);
+                mfma(ring, 2, f0[0], f1[0], false);
+                mfma(ring, 3, f0[1], f1[1], false);
                 if (P == 3) {
                     fold(hdr[0].d, hdr[1].d);
                     // minima: acc -= dmin * sum_s Sx(hi + lo)[m, s] * mn[n, s]
                     const f16x8 m0 = minima_frag(hdr[0]), m1 = minima_frag(hdr[1]);
     #pragma unroll
                     for (int i = 0; i < MT; ++i) {
-                        const f16x8 sf = *reinterpret_cast<const f16x8*>(&lds_sx[b & 1][(i * 32 + col) * LDS_SX + khalf * 8]);
+                        const f16x8 sf = *reinterpret_cast<const f16x8*>(&lds_sx[(b & 1) * kTaskRows * LDS_SX + (i * 32 + col) * LDS_SX + khalf * 8]);
                         const f32x16 zero{};
                         blk[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m0, zero, 0, 0, 0);
                         blk[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m1, zero, 0, 0, 0);
                     }
                     fold(-hdr[0].dmin, -hdr[1].dmin);
                 }
-                // the slab of the next step (and everything requested before it) has to have arrived now
-                store_a(buf ^ 1, Slot0{});
-                if (P == 0) store_sx((b + 1) & 1);
+                if (P == 1) store_sx((b + 1) & 1);  // read at P == 3 of the next super-block; the buffer was last read at P == 3 of the one before
                 if (P == 1 || P == 3) store_w(wbuf ^ 1);  // read again two barriers from now; this buffer was last read a step ago
                 if (P == 3) { hdr[0] = hdr_next[0]; hdr[1] = hdr_next[1]; }
             };
+            wait_all_loads();  // slabs 0 and 1 (the stores above already waited for younger loads)
             for (uint32_t b = 0; b < bpr; ++b) {
                 pair_step(b * 4 + 0, std::integral_constant<int, 0>{});
                 pair_step(b * 4 + 1, std::integral_constant<int, 1>{});
@@ -419,6 +438,10 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
     };
     if (mt_live == 1) run(std::integral_constant<int, 1>{});
     else run(std::integral_constant<int, 2>{});
+    wait_all_loads();  // the last steps requested slabs that nobody reads: they must have landed before this LDS is reused or given away
+    __syncthreads();
+    if (tid < kTaskRows) row_dst[tid] = my_dst;
+    __syncthreads();
 
     // ---- epilogue. Accumulator v of tile (i, j): row = i*32 + 8*(v/4) + 4*khalf + v%4, column = col.
     uint32_t bad = 0;

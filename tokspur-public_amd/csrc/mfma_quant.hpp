@@ -15,6 +15,23 @@ enum BKind : int { B_Q4K_RAW = 0, B_Q4K_PLANAR = 1, B_Q6K_PLANAR = 2 };
 // Workgroup barrier that waits for this wave's LDS traffic only. __syncthreads() also drains every outstanding
 // global load, which would serialise the prefetch of the next K step behind the barrier.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// The same, after all but the YOUNGEST vector-memory operations of this wave have completed (they complete in issue
+// order): for data that a direct global -> LDS load is bringing in, which no register dependency waits for.
+template <int YOUNGEST>
+__device__ __forceinline__ void lds_barrier_after_loads() {
+    static_assert(YOUNGEST >= 0 && YOUNGEST < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(YOUNGEST) : "memory");
+}
+// 16 bytes per lane from global memory straight into LDS at lds_base + 16 * lane (lds_base uniform over the wave).
+// The compiler does not know this load: it counts in vmcnt like any other, so waits the compiler places for its own
+// loads are only ever longer than needed, and whoever reads the bytes waits for them with lds_barrier_after_loads.
+__device__ __forceinline__ void load_to_lds_16(const void* src, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(src) : "memory", "m0");
+}
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+    return uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)p));
+}
+__device__ __forceinline__ void wait_all_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 __device__ __forceinline__ f16x2 as_h2(uint32_t bits) { return __builtin_bit_cast(f16x2, bits); }
 __device__ __forceinline__ uint32_t as_u32(f16x2 v) { return __builtin_bit_cast(uint32_t, v); }
