@@ -374,6 +374,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
             auto read_w = [&](int wbuf, int j, int p2) {  // row j*32 + col, chunk 2*p2 + khalf
                 return *reinterpret_cast<const u32x4*>(my_w + wbuf * 4096 + ((j * 32 + col) * 4 + ((2 * p2 + khalf) ^ ((col >> 1) & 3))) * 16);
             };
+            const Q4Consts q4c = q4_consts();
             HdrQ4 hdr[2], hdr_next[2];
     #pragma unroll
             for (int j = 0; j < 2; ++j) {
@@ -402,12 +403,12 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
                 }
                 const u32x4 raw0 = read_w(wbuf, 0, P & 1), raw1 = read_w(wbuf, 1, P & 1);
                 f16x8 f0[2], f1[2];
-                frags_q4k<P, 0>(raw0, hdr[0], f0);
-                frags_q4k<P, 0>(raw1, hdr[1], f1);
+                frags_q4k_swapped<P, 0>(raw0, hdr[0], q4c, f0);
+                frags_q4k_swapped<P, 0>(raw1, hdr[1], q4c, f1);
                 mfma(ring, 0, f0[0], f1[0], P == 0);
                 mfma(ring, 1, f0[1], f1[1], false);
-                frags_q4k<P, 1>(raw0, hdr[0], f0);
-                frags_q4k<P, 1>(raw1, hdr[1], f1);
+                frags_q4k_swapped<P, 1>(raw0, hdr[0], q4c, f0);
+                frags_q4k_swapped<P, 1>(raw1, hdr[1], q4c, f1);
                 mfma(ring, 2, f0[0], f1[0], false);
                 mfma(ring, 3, f0[1], f1[1], false);
                 if (P == 3) {
@@ -517,6 +518,9 @@ __global__ __launch_bounds__(256) void to_f16_rows(const void* __restrict__ src,
         sum += __shfl_xor(sum, 1, kWave);
         sum += __shfl_xor(sum, 2, kWave);
         if (live) {
+            // Q4_K consumers (the ones that ask for sums) unpack a dword of nibbles into the column pairs (0, 2), (1, 3):
+            // their activations are stored in that order, columns 1 <-> 2 and 5 <-> 6 of every eight swapped
+            if (sx) out = f16x8{out[0], out[2], out[1], out[3], out[4], out[6], out[5], out[7]};
             *reinterpret_cast<f16x8*>(dst + r * columns + c8 * 8) = out;
             if (sx && (c8 & 3) == 0) {
                 const uint32_t sub = uint32_t(c8 / 4), b = sub / 8, s = sub % 8;

@@ -95,6 +95,33 @@ __device__ __forceinline__ void frags_q4k(const u32x4& raw, const HdrQ4& h, f16x
     frag[1] = scaled8_q4((raw[2] >> (4 * HI)) & M4, (raw[3] >> (4 * HI)) & M4, s2, bias);
 }
 
+// The same fragments with the columns of every eight in the order (0, 2, 1, 3, 4, 6, 5, 7), for activations stored in
+// that order: one mask-or per pair of weights instead of a mask and two byte permutes per four. Low nibbles become
+// 1024 + q, high nibbles stay in place as 1024 + 16 q and take the scale sc / 16 (exact: sc < 64).
+// (w & mask) | bits is one instruction (v_and_or_b32) only when the constants sit in registers: a VOP3 instruction of
+// this target takes no literal, and with two literals the compiler emits an and plus an or. The kernel therefore pins
+// the three constants to registers once and hands them to the unpacking.
+struct Q4Consts { uint32_t lo_mask, hi_mask, bits; };
+__device__ __forceinline__ Q4Consts q4_consts() {
+    Q4Consts c{0x000f000fu, 0x00f000f0u, 0x64006400u};
+    asm volatile("" : "+s"(c.lo_mask), "+s"(c.hi_mask), "+v"(c.bits));
+    return c;
+}
+template <int HI>
+__device__ __forceinline__ f16x8 scaled8_q4_swapped(uint32_t w0, uint32_t w1, f16x2 sc, f16x2 bias, const Q4Consts& c) {
+    const uint32_t m = HI ? c.hi_mask : c.lo_mask;
+    const f16x2 p0 = fma2(as_h2((w0 & m) | c.bits), sc, bias), p1 = fma2(as_h2(((w0 >> 8) & m) | c.bits), sc, bias);
+    const f16x2 p2 = fma2(as_h2((w1 & m) | c.bits), sc, bias), p3 = fma2(as_h2(((w1 >> 8) & m) | c.bits), sc, bias);
+    return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
+template <int P, int HI>
+__device__ __forceinline__ void frags_q4k_swapped(const u32x4& raw, const HdrQ4& h, const Q4Consts& c, f16x8 frag[2]) {
+    const uint32_t sc = (h.sc[P >> 1] >> ((P & 1) * 16 + HI * 8)) & 0xffu;
+    const f16x2 s2 = splat(float(sc) * (HI ? 0.0625f : 1.0f)), bias = splat(float(sc) * (HI ? -64.0f : -1024.0f));
+    frag[0] = scaled8_q4_swapped<HI>(raw[0], raw[1], s2, bias, c);
+    frag[1] = scaled8_q4_swapped<HI>(raw[2], raw[3], s2, bias, c);
+}
+
 // B operand of the minima term: the eight integer minima, the same in both k-halves (hi and lo sums).
 __device__ __forceinline__ f16x8 minima_frag(const HdrQ4& h) {
     constexpr uint32_t K = 0x64646464u;
