@@ -666,8 +666,7 @@ extern "C" int tsp_grouped_mm(uint32_t encoding, uint32_t layout, const void* ma
     auto* sx = reinterpret_cast<_Float16*>(ws + l.sx);
     auto* task_list = reinterpret_cast<uint32_t*>(ws + l.tasks);
     int rc = tsp_grouped_routes(ids, token_map, counts, experts, selected, tokens, error_word, stream);
-    if (rc == TSP_OK) rc = tsp_grouped_tasks(counts, tasks, experts, selected, tokens, 32, error_word, stream);
-    if (rc == TSP_OK) rc = tsp_grouped_tasks(counts, task_list, experts, selected, tokens, kTaskRows, error_word, stream);
+    if (rc == TSP_OK) rc = grouped_tasks_pair(counts, tasks, 32, task_list, kTaskRows, experts, selected, tokens, error_word, stream);
     if (rc == TSP_OK) rc = convert_rows(input, input_stride_bytes, 0, xh, sx, l.in_rows, columns, error_word, s);
     if (rc != TSP_OK) return rc;
     GemmArgs a{};
@@ -744,8 +743,7 @@ extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream
     auto* hbuf = reinterpret_cast<_Float16*>(ws + l.hbuf);
 
     rc = tsp_grouped_routes(m->ids, m->token_map, m->counts, m->experts, m->selected, m->tokens, m->error_word, stream);
-    if (rc == TSP_OK) rc = tsp_grouped_tasks(m->counts, m->tasks, m->experts, m->selected, m->tokens, 32, m->error_word, stream);
-    if (rc == TSP_OK) rc = tsp_grouped_tasks(m->counts, task_list, m->experts, m->selected, m->tokens, kTaskRows, m->error_word, stream);
+    if (rc == TSP_OK) rc = grouped_tasks_pair(m->counts, m->tasks, 32, task_list, kTaskRows, m->experts, m->selected, m->tokens, m->error_word, stream);
     if (rc == TSP_OK) rc = convert_rows(m->x, m->x_stride_bytes, 0, xh, sx, m->tokens, m->channels, m->error_word, s);
     if (rc != TSP_OK) return rc;
 

@@ -47,9 +47,12 @@ __global__ __launch_bounds__(256) void grouped_routes_kernel(const uint32_t* __r
 }
 
 // One block of 512 threads; experts <= 512.
-__global__ __launch_bounds__(512) void grouped_tasks_kernel(const uint32_t* __restrict__ counts, uint32_t* __restrict__ tasks,
-                                                            uint32_t experts, uint32_t selected, uint32_t tokens, uint32_t tile,
-                                                            uint32_t* error_word) {
+// Block b writes list b: the same counts tiled two ways in one launch (tasks1 may be null with a grid of one).
+__global__ __launch_bounds__(512) void grouped_tasks_kernel(const uint32_t* __restrict__ counts, uint32_t* __restrict__ tasks0, uint32_t tile0,
+                                                            uint32_t* __restrict__ tasks1, uint32_t tile1, uint32_t experts, uint32_t selected,
+                                                            uint32_t tokens, uint32_t* error_word) {
+    uint32_t* const tasks = blockIdx.x == 0 ? tasks0 : tasks1;
+    const uint32_t tile = blockIdx.x == 0 ? tile0 : tile1;
     __shared__ uint32_t tiles_scan[512];
     __shared__ uint32_t routes_scan[512];
     const uint32_t tid = threadIdx.x;
@@ -170,7 +173,17 @@ extern "C" int tsp_grouped_tasks(const uint32_t* counts, uint32_t* tasks, uint32
     TSP_REQUIRE(experts && experts <= 512 && selected && selected <= 16 && tokens && tokens <= 2048 && tile && tile <= 256,
                 "grouped tasks geometry");
     TSP_REQUIRE(counts && tasks && error_word, "null device pointer");
-    TSP_LAUNCH("grouped_tasks", static_cast<hipStream_t>(stream), grouped_tasks_kernel<<<1, 512, 0, static_cast<hipStream_t>(stream)>>>(counts, tasks, experts, selected, tokens, tile, error_word));
+    TSP_LAUNCH("grouped_tasks", static_cast<hipStream_t>(stream), grouped_tasks_kernel<<<1, 512, 0, static_cast<hipStream_t>(stream)>>>(counts, tasks, tile, nullptr, 0, experts, selected, tokens, error_word));
+    return launch_status("grouped_tasks");
+}
+
+// The caller's task list (tile0 rows per task) and a second one (tile1) from the same counts, in one launch.
+int tsp::grouped_tasks_pair(const uint32_t* counts, uint32_t* tasks0, uint32_t tile0, uint32_t* tasks1, uint32_t tile1, uint32_t experts,
+                            uint32_t selected, uint32_t tokens, uint32_t* error_word, void* stream) {
+    TSP_REQUIRE(experts && experts <= 512 && selected && selected <= 16 && tokens && tokens <= 2048 && tile0 && tile0 <= 256 && tile1 && tile1 <= 256,
+                "grouped tasks geometry");
+    TSP_REQUIRE(counts && tasks0 && tasks1 && error_word, "null device pointer");
+    TSP_LAUNCH("grouped_tasks", static_cast<hipStream_t>(stream), grouped_tasks_kernel<<<2, 512, 0, static_cast<hipStream_t>(stream)>>>(counts, tasks0, tile0, tasks1, tile1, experts, selected, tokens, error_word));
     return launch_status("grouped_tasks");
 }
 

@@ -154,6 +154,45 @@ __global__ __launch_bounds__(256) void mixture_rows(MixtureArgs a) {
     publish_error(bad, a.error_word);
 }
 
+// The same with four channels per thread (16-byte loads) and all expert rows of a token requested before the first
+// is used; SELECTED = 0 takes the count from the arguments.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+template <int SELECTED>
+__global__ __launch_bounds__(256) void mixture_rows_x4(MixtureArgs a) {
+    const uint32_t channel = (blockIdx.x * blockDim.x + threadIdx.x) * 4, row = blockIdx.y;
+    const uint32_t selected = SELECTED ? SELECTED : a.selected;
+    uint32_t bad = 0;
+    if (channel < a.channels && row < a.tokens) {
+        const float slogit = a.shared_logit[row];
+        if (nonfinite(slogit)) {
+            bad = TSP_ERRBIT_NONFINITE;
+        } else {
+            const float* ex = a.experts + uint64_t(row) * selected * a.channels + channel;
+            const float* w = a.weights + uint64_t(row) * selected;
+            const f32x4 sh = *reinterpret_cast<const f32x4*>(a.shared + uint64_t(row) * a.channels + channel);
+            const float gate = sigmoid_f(slogit);
+            f32x4 value = sh * gate;
+            auto add = [&](float wr, const f32x4& e) {
+                if (nonfinite(wr) || wr < 0.0f) bad = TSP_ERRBIT_NONFINITE;
+                value.x = __builtin_fmaf(wr, e.x, value.x); value.y = __builtin_fmaf(wr, e.y, value.y);
+                value.z = __builtin_fmaf(wr, e.z, value.z); value.w = __builtin_fmaf(wr, e.w, value.w);
+            };
+            if constexpr (SELECTED != 0) {
+                f32x4 e[SELECTED];
+#pragma unroll
+                for (int r = 0; r < SELECTED; ++r) e[r] = *reinterpret_cast<const f32x4*>(ex + uint64_t(r) * a.channels);
+#pragma unroll
+                for (int r = 0; r < SELECTED; ++r) add(w[r], e[r]);
+            } else {
+                for (uint32_t r = 0; r < selected; ++r) add(w[r], *reinterpret_cast<const f32x4*>(ex + uint64_t(r) * a.channels));
+            }
+            if (nonfinite(value.x) || nonfinite(value.y) || nonfinite(value.z) || nonfinite(value.w)) bad = TSP_ERRBIT_NONFINITE;
+            *reinterpret_cast<f32x4*>(reinterpret_cast<uint8_t*>(a.output) + row * a.output_stride_bytes + uint64_t(channel) * 4) = value;
+        }
+    }
+    publish_error(bad, a.error_word);
+}
+
 __global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ gate, const float* __restrict__ up,
                                                      float* __restrict__ out, uint64_t count, float scale, uint32_t* error_word) {
     uint32_t bad = 0;
@@ -218,7 +257,14 @@ extern "C" int tsp_mixture_batch(const float* experts, const float* weights, con
                     !ranges_overlap(output, out_span, shared_logit, uint64_t(tokens) * 4),
                 "mixture output overlaps an input");
     const MixtureArgs a{experts, weights, shared, shared_logit, output, output_stride_bytes, channels, selected, tokens, error_word};
-    TSP_LAUNCH("mixture_rows", static_cast<hipStream_t>(stream), mixture_rows<<<dim3((channels + 255) / 256, tokens), 256, 0, static_cast<hipStream_t>(stream)>>>(a));
+    const auto st = static_cast<hipStream_t>(stream);
+    const bool wide = channels % 4 == 0 && output_stride_bytes % 16 == 0 && (reinterpret_cast<uintptr_t>(experts) | reinterpret_cast<uintptr_t>(shared) |
+                                                                            reinterpret_cast<uintptr_t>(output)) % 16 == 0;
+    const dim3 grid4((channels / 4 + 255) / 256, tokens);
+    if (wide && selected == 10) TSP_LAUNCH("mixture_rows", st, mixture_rows_x4<10><<<grid4, 256, 0, st>>>(a));
+    else if (wide && selected == 8) TSP_LAUNCH("mixture_rows", st, mixture_rows_x4<8><<<grid4, 256, 0, st>>>(a));
+    else if (wide) TSP_LAUNCH("mixture_rows", st, mixture_rows_x4<0><<<grid4, 256, 0, st>>>(a));
+    else TSP_LAUNCH("mixture_rows", st, mixture_rows<<<dim3((channels + 255) / 256, tokens), 256, 0, st>>>(a));
     return launch_status("mixture");
 }
 
