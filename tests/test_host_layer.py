@@ -158,3 +158,66 @@ def test_host_class_library_exports_graph_operators():
         assert f"tokspur::HipGraph::{op}(" in names, op
     for fn in ("tokspur::encode_moe(", "tokspur::encode_moe_batch(", "tokspur::allocate_moe_scratch(", "tokspur::is_planar_moe("):
         assert fn in names, fn
+
+
+def test_gemm_staging_waits_match_the_compiled_load_order(tmp_path):
+    """The GEMM kernels bring activation slabs in with direct global -> LDS loads that no register dependency waits
+    for: each K step waits with `s_waitcnt vmcnt(N)` where N is the number of younger vector-memory operations, written
+    into the source as constants. This compiles gemm.hip to assembly and recounts, per kernel and loop: at an even step
+    N must equal the other loads of the even step before; at an odd step, those of the even step three back plus the
+    slab loads and the other loads of the step before."""
+    import importlib
+    import shutil
+    import subprocess
+    if shutil.which("hipcc") is None:
+        pytest.skip("hipcc not on PATH")
+    build = importlib.import_module("tokspur-public_amd.build")
+    asm = tmp_path / "gemm.s"
+    src = os.path.join(ROOT, "tokspur-public_amd", "csrc", "gemm.hip")
+    flags = [f for f in build.HIP_FLAGS if f != "-fPIC"]
+    subprocess.run(["hipcc", "-x", "hip", "-S", "--cuda-device-only", src, "-o", str(asm)] + flags, check=True,
+                   stdout=subprocess.PIPE, stderr=subprocess.PIPE)
+    kernels, name = {}, None
+    for text in asm.read_text().splitlines():
+        m = re.match(r"^(_Z\w*gemm_kernel\w*):", text)
+        if m:
+            name = m.group(1)
+            kernels[name] = []
+        elif name and text.strip().startswith("s_endpgm"):
+            name = None
+        elif name:
+            kernels[name].append(text)
+    assert len(kernels) >= 9
+    loops_checked = 0
+    for name, lines in kernels.items():
+        loops, current = [], None
+        for text in lines:
+            if "Loop Header" in text:
+                current = []
+                loops.append(current)
+            elif current is not None:
+                current.append(text.strip())
+                if text.strip().startswith("s_cbranch_scc"):
+                    current = None
+        for body in loops:
+            steps, waits = [], []  # per K step: [slab loads, other loads]; wait constant at the top of the step
+            for text in body:
+                m = re.match(r"s_waitcnt vmcnt\((\d+)\) lgkmcnt\(0\)", text)
+                if m:
+                    waits.append(int(m.group(1)))
+                    steps.append([0, 0])
+                elif text.startswith("global_load_lds") and steps:
+                    steps[-1][0] += 1
+                elif (text.startswith("global_load") or text.startswith("buffer_load")) and steps:
+                    steps[-1][1] += 1
+            if len(waits) != 4:
+                continue  # not a K loop
+            loops_checked += 1
+            for i in range(4):
+                if i % 2 == 0:
+                    want = steps[(i + 2) % 4][1]
+                    assert steps[i][0] > 0 and steps[(i + 1) % 4] == [0, 0], (name, steps)
+                else:
+                    want = steps[(i + 1) % 4][1] + steps[(i + 3) % 4][0] + steps[(i + 3) % 4][1]
+                assert waits[i] == want, (name, i, waits, steps)
+    assert loops_checked >= 18  # two loops (one or two row tiles) in each of the nine kernels

@@ -392,7 +392,8 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
                 // Even steps request the slabs of the steps two and three ahead, as the first loads after their barrier; the
                 // only loads younger than those are the other loads of the same step (W), and for an odd step the two slabs
                 // and the loads of the even step before it. Loads complete in order.
-                constexpr int W[4] = {5, 0, 8, 0};  // sums + half-block, -, half-block + headers, -
+                // sums + half-block, -, half-block + headers (planes: scales and d/dmin apart, two loads per tile; GGUF rows: one), -
+                constexpr int W[4] = {5, 0, BKIND == B_Q4K_PLANAR ? 8 : 6, 0};
                 lds_barrier_after_loads<P % 2 == 0 ? W[(P + 2) % 4] : W[(P + 1) % 4] + 2 * MT + W[(P + 3) % 4]>();  // slab, this wave's weight bytes (and at P == 3 lds_sx[b & 1]) are complete; every wave has left the other buffers
                 if (P % 2 == 0) { dma_a(step + 2, (ring + 2) % RING); dma_a(step + 3, (ring + 3) % RING); }
                 if (P == 0) fetch_sx(b + 1 < bpr ? b + 1 : b);
