@@ -2,11 +2,14 @@
 // (value descending, column ascending, -0 == +0), the number found, and the first non-finite and first
 // subnormal column. Rank 0 is the arg-max a greedy sampler needs.
 //
-// Two launches. Stage 1: one workgroup per (4096-column tile, row) sorts its tile and writes a partial row.
-// Stage 2: one workgroup per row sorts the partial rows' candidates and writes the final row. Both stages sort
-// 64-bit keys with a bitonic network in LDS: high word = the float mapped to an unsigned integer of the same
-// order (after -0 -> +0), low word = ~column, so that "largest key first" is exactly the ordering above.
-// Non-finite logits and padding get key 0, below every finite value's key.
+// Two launches. Stage 1: one workgroup per (4096-column tile, row); each of its four waves keeps the 64 largest keys
+// of its 1024 columns in registers, one key per lane, and the four lists are merged into a partial row. Stage 2: one
+// workgroup per row merges the partial rows' lists the same way and writes the final row. Keys are 64 bits: high word
+// = the float mapped to an unsigned integer of the same order (after -0 -> +0), low word = ~column, so that "largest
+// key first" is exactly the ordering above and no two keys are equal. Non-finite logits and padding get key 0, below
+// every finite value's key. A list is sorted with a bitonic network over the wave's lanes; two lists are merged by
+// sorting one of them ascending, taking the lane-wise maximum (the 64 largest of both, a bitonic sequence) and
+// running the last six steps of the network.
 #include "tsp_common.hpp"
 
 using namespace tsp;
@@ -21,7 +24,6 @@ struct TopKArgs {
     uint32_t rows, vocabulary, tiles;
     tsp_logit_topk_row* partial;  // [rows][tiles]
     tsp_logit_topk_row* out;      // [rows]
-    uint32_t sort_size;           // stage 2: power of two >= tiles * 64
 };
 
 __device__ __forceinline__ uint64_t make_key(float value, uint32_t column) {
@@ -32,34 +34,57 @@ __device__ __forceinline__ uint64_t make_key(float value, uint32_t column) {
     return (uint64_t(ordered) << 32) | uint32_t(~column);
 }
 
-// Descending bitonic sort of `n` (a power of two) keys in LDS by the whole workgroup.
-__device__ void sort_descending(uint64_t* keys, uint32_t n) {
-    for (uint32_t size = 2; size <= n; size <<= 1) {
-        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
-            __syncthreads();
-            for (uint32_t t = threadIdx.x; t < n / 2; t += blockDim.x) {
-                const uint32_t lo = 2 * t - (t & (stride - 1)), hi = lo + stride;
-                const bool descending = (lo & size) == 0;
-                const uint64_t a = keys[lo], b = keys[hi];
-                if ((a < b) == descending) { keys[lo] = b; keys[hi] = a; }
-            }
-        }
-    }
-    __syncthreads();
+__device__ __forceinline__ uint64_t exchange(uint64_t key, uint32_t stride, bool keep_larger) {
+    const uint64_t other = __shfl_xor(key, stride, kWave);
+    return (key > other) == keep_larger ? key : other;
 }
 
-__device__ void write_row(tsp_logit_topk_row* row, const uint64_t* keys, const float* logits_row, uint32_t vocabulary,
-                          uint32_t first_nonfinite, uint32_t first_subnormal) {
-    if (threadIdx.x < kCapacity) {
-        const uint64_t key = keys[threadIdx.x];
-        const uint32_t column = ~uint32_t(key);
-        const bool live = key != 0;
-        row->ids[threadIdx.x] = live ? column : 0u;
-        row->logits[threadIdx.x] = live ? logits_row[column] : -__builtin_inff();  // the raw value, -0 included
+// Bitonic sort of one key per lane: lane i ends with the i-th largest (DESCENDING) or i-th smallest key.
+template <bool DESCENDING>
+__device__ __forceinline__ uint64_t wave_sort(uint64_t key, uint32_t lane) {
+#pragma unroll
+    for (uint32_t size = 2; size <= kWave; size <<= 1) {
+#pragma unroll
+        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+            const bool block_descending = size == kWave ? DESCENDING : ((lane & size) == 0) == DESCENDING;
+            key = exchange(key, stride, ((lane & stride) == 0) == block_descending);
+        }
     }
-    if (threadIdx.x == 0) {
-        uint32_t count = 0;
-        while (count < kCapacity && keys[count] != 0) ++count;
+    return key;
+}
+
+// The 64 largest of a descending list and an ascending list, descending.
+__device__ __forceinline__ uint64_t wave_merge(uint64_t descending, uint64_t ascending, uint32_t lane) {
+    uint64_t key = descending > ascending ? descending : ascending;
+#pragma unroll
+    for (uint32_t stride = kWave >> 1; stride > 0; stride >>= 1) key = exchange(key, stride, (lane & stride) == 0);
+    return key;
+}
+
+__device__ __forceinline__ uint32_t wave_min(uint32_t v) {
+#pragma unroll
+    for (int m = 1; m < kWave; m <<= 1) {
+        const uint32_t o = __shfl_xor(v, m, kWave);
+        v = o < v ? o : v;
+    }
+    return v;
+}
+
+// Merges the four waves' descending lists through LDS (wave 0 ends with the workgroup's list) and writes the row.
+__device__ void merge_waves_and_write(uint64_t top, uint64_t (*lists)[kCapacity], tsp_logit_topk_row* row, const float* logits_row,
+                                      uint32_t vocabulary, uint32_t first_nonfinite, uint32_t first_subnormal) {
+    const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    lists[wave][lane] = top;
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (uint32_t w = 1; w < 4; ++w) top = wave_merge(top, lists[w][kWave - 1 - lane], lane);
+    const uint32_t column = ~uint32_t(top);
+    const bool live = top != 0;
+    row->ids[lane] = live ? column : 0u;
+    row->logits[lane] = live ? logits_row[column] : -__builtin_inff();  // the raw value, -0 included
+    const uint32_t count = __builtin_popcountll(__builtin_amdgcn_ballot_w64(live));
+    if (lane == 0) {
         row->vocabulary = vocabulary;
         row->count = count;
         row->first_nonfinite_col = first_nonfinite;
@@ -68,52 +93,75 @@ __device__ void write_row(tsp_logit_topk_row* row, const uint64_t* keys, const f
 }
 
 __global__ __launch_bounds__(256) void topk_stage1(TopKArgs a) {
-    __shared__ uint64_t keys[kTileSpan];
+    __shared__ uint64_t lists[4][kCapacity];
     __shared__ uint32_t first_nonfinite, first_subnormal;
-    const uint32_t tile = blockIdx.x, row = blockIdx.y;
+    const uint32_t tile = blockIdx.x, row = blockIdx.y, lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const float* logits_row = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(a.logits) + uint64_t(row) * a.stride_bytes);
     if (threadIdx.x == 0) { first_nonfinite = kNone; first_subnormal = kNone; }
     __syncthreads();
     uint32_t nonfinite = kNone, subnormal = kNone;
-    for (uint32_t i = threadIdx.x; i < kTileSpan; i += blockDim.x) {
-        const uint32_t column = tile * kTileSpan + i;
-        uint64_t key = 0;
-        if (column < a.vocabulary) {
-            const float v = logits_row[column];
-            const uint32_t bits = __float_as_uint(v);
-            if ((bits & 0x7f800000u) == 0x7f800000u) nonfinite = nonfinite < column ? nonfinite : column;
-            else if ((bits & 0x7f800000u) == 0 && (bits & 0x007fffffu) != 0) subnormal = subnormal < column ? subnormal : column;
-            key = make_key(v, column);
+    // 16 batches of 64 columns per wave, two independent running lists so that the exchanges of one hide the other's latency
+    uint64_t top[2] = {0, 0};
+#pragma unroll 1
+    for (uint32_t pair = 0; pair < 8; ++pair) {
+        uint64_t key[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t column = tile * kTileSpan + wave * 1024 + (pair * 2 + h) * kWave + lane;
+            key[h] = 0;
+            if (column < a.vocabulary) {
+                const float v = logits_row[column];
+                const uint32_t bits = __float_as_uint(v);
+                if ((bits & 0x7f800000u) == 0x7f800000u) nonfinite = nonfinite < column ? nonfinite : column;
+                else if ((bits & 0x7f800000u) == 0 && (bits & 0x007fffffu) != 0) subnormal = subnormal < column ? subnormal : column;
+                key[h] = make_key(v, column);
+            }
         }
-        keys[i] = key;
+        if (pair == 0) {
+            top[0] = wave_sort<true>(key[0], lane);
+            top[1] = wave_sort<true>(key[1], lane);
+        } else {
+            const uint64_t c0 = wave_sort<false>(key[0], lane), c1 = wave_sort<false>(key[1], lane);
+            top[0] = wave_merge(top[0], c0, lane);
+            top[1] = wave_merge(top[1], c1, lane);
+        }
     }
-    if (nonfinite != kNone) atomicMin(&first_nonfinite, nonfinite);
-    if (subnormal != kNone) atomicMin(&first_subnormal, subnormal);
-    sort_descending(keys, kTileSpan);
+    const uint64_t mine = wave_merge(top[0], __shfl(top[1], kWave - 1 - lane, kWave), lane);
+    nonfinite = wave_min(nonfinite);
+    subnormal = wave_min(subnormal);
+    if (lane == 0 && nonfinite != kNone) atomicMin(&first_nonfinite, nonfinite);
+    if (lane == 0 && subnormal != kNone) atomicMin(&first_subnormal, subnormal);
+    __syncthreads();
     const uint32_t begin = tile * kTileSpan, width = a.vocabulary - begin < kTileSpan ? a.vocabulary - begin : kTileSpan;
-    write_row(a.partial + uint64_t(row) * a.tiles + tile, keys, logits_row, width, first_nonfinite, first_subnormal);
+    merge_waves_and_write(mine, lists, a.partial + uint64_t(row) * a.tiles + tile, logits_row, width, first_nonfinite, first_subnormal);
 }
 
 __global__ __launch_bounds__(256) void topk_stage2(TopKArgs a) {
-    extern __shared__ uint64_t merged[];
+    __shared__ uint64_t lists[4][kCapacity];
     __shared__ uint32_t first_nonfinite, first_subnormal;
-    const uint32_t row = blockIdx.x;
+    const uint32_t row = blockIdx.x, lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const float* logits_row = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(a.logits) + uint64_t(row) * a.stride_bytes);
     const tsp_logit_topk_row* partial = a.partial + uint64_t(row) * a.tiles;
     if (threadIdx.x == 0) { first_nonfinite = kNone; first_subnormal = kNone; }
     __syncthreads();
-    for (uint32_t i = threadIdx.x; i < a.sort_size; i += blockDim.x) {
-        const uint32_t tile = i / kCapacity, slot = i % kCapacity;
-        uint64_t key = 0;
-        if (tile < a.tiles && slot < partial[tile].count) key = make_key(partial[tile].logits[slot], partial[tile].ids[slot]);
-        merged[i] = key;
+    // a partial row is a descending list (empty slots have key 0); read backwards it is ascending
+    auto list_key = [&](uint32_t tile, uint32_t slot) -> uint64_t {
+        return tile < a.tiles && slot < partial[tile].count ? make_key(partial[tile].logits[slot], partial[tile].ids[slot]) : 0;
+    };
+    uint64_t top[2] = {list_key(wave, lane), list_key(wave + 4, lane)};
+#pragma unroll 1
+    for (uint32_t tile = wave + 8; tile < a.tiles; tile += 8) {  // a pair per round; a tile past the end is an empty list
+        const uint64_t c0 = list_key(tile, kWave - 1 - lane), c1 = list_key(tile + 4, kWave - 1 - lane);
+        top[0] = wave_merge(top[0], c0, lane);
+        top[1] = wave_merge(top[1], c1, lane);
     }
+    const uint64_t mine = wave_merge(top[0], __shfl(top[1], kWave - 1 - lane, kWave), lane);
     for (uint32_t tile = threadIdx.x; tile < a.tiles; tile += blockDim.x) {
         if (partial[tile].first_nonfinite_col != kNone) atomicMin(&first_nonfinite, partial[tile].first_nonfinite_col);
         if (partial[tile].first_subnormal_col != kNone) atomicMin(&first_subnormal, partial[tile].first_subnormal_col);
     }
-    sort_descending(merged, a.sort_size);
-    write_row(a.out + row, merged, logits_row, a.vocabulary, first_nonfinite, first_subnormal);
+    __syncthreads();
+    merge_waves_and_write(mine, lists, a.out + row, logits_row, a.vocabulary, first_nonfinite, first_subnormal);
 }
 
 uint32_t tiles_for(uint32_t vocabulary) { return (vocabulary + kTileSpan - 1) / kTileSpan; }
@@ -155,18 +203,11 @@ extern "C" int tsp_logit_topk(const float* logits, uint64_t stride_bytes, uint32
                     !ranges_overlap(partial_scratch, need_scratch, out_rows, need_out),
                 "GPU logit top-k buffers overlap");
     TopKArgs a{logits, stride_bytes, rows, vocabulary, tiles, static_cast<tsp_logit_topk_row*>(partial_scratch),
-               static_cast<tsp_logit_topk_row*>(out_rows), 64};
-    while (a.sort_size < tiles * kCapacity) a.sort_size <<= 1;
+               static_cast<tsp_logit_topk_row*>(out_rows)};
     const auto s = static_cast<hipStream_t>(stream);
     TSP_LAUNCH("logit_topk_stage1", s, topk_stage1<<<dim3(tiles, rows), 256, 0, s>>>(a));
     int rc = launch_status("logit_topk_stage1");
     if (rc != TSP_OK) return rc;
-    const uint32_t lds_bytes = a.sort_size * 8;
-    static bool raised = false;
-    if (lds_bytes > 48 * 1024 && !raised) {
-        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&topk_stage2), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxTiles * kCapacity * 8));
-        raised = true;
-    }
-    TSP_LAUNCH("logit_topk_stage2", s, topk_stage2<<<rows, 256, lds_bytes, s>>>(a));
+    TSP_LAUNCH("logit_topk_stage2", s, topk_stage2<<<rows, 256, 0, s>>>(a));
     return launch_status("logit_topk_stage2");
 }
