@@ -680,7 +680,7 @@ extern "C" int tsp_grouped_mm(uint32_t encoding, uint32_t layout, const void* ma
 
 // ---------------------------------------------------------------- grouped MoE
 namespace {
-struct NaxLayout { uint64_t xh, sx, tasks, hbuf, total; uint32_t bound; };
+struct NaxLayout { uint64_t xh, sx, tasks, hbuf, meta, total; uint32_t bound; };
 NaxLayout nax_layout(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t channels, uint32_t hidden) {
     NaxLayout l{};
     l.bound = tokens * selected / kTaskRows + experts;
@@ -688,8 +688,38 @@ NaxLayout nax_layout(uint32_t tokens, uint32_t selected, uint32_t experts, uint3
     l.sx = align256(uint64_t(tokens) * channels * 2);
     l.tasks = l.sx + align256(uint64_t(tokens) * (channels / 256) * 32);
     l.hbuf = l.tasks + align256((2 + 2 * uint64_t(l.bound)) * 4);
-    l.total = l.hbuf + align256(uint64_t(l.bound) * kTaskRows * hidden * 2);
+    l.meta = l.hbuf + align256(uint64_t(l.bound) * kTaskRows * hidden * 2);  // union records of one chunk of eight tokens
+    l.total = l.meta + align256(2320 * 4);
     return l;
+}
+
+// The planar kinds the matrix-core kernels have no unpacking for (Q5_K / Q8_0 gate and up, Q5_1 / Q8_0 down) run
+// through the routed kernels for at most eight tokens, a chunk of eight tokens at a time: the same routes, tasks and
+// expert_down rows, computed in f32 on the vector units. h of a chunk (8 * selected rows of f32) borrows the buffer the
+// matrix-core path keeps its h rows in, which is never smaller.
+int grouped_moe_in_eights(const tsp_grouped_moe* m, const NaxLayout& l, void* stream) {
+    auto* ws = static_cast<uint8_t*>(m->workspace);
+    int rc = tsp_grouped_routes(m->ids, m->token_map, m->counts, m->experts, m->selected, m->tokens, m->error_word, stream);
+    if (rc == TSP_OK) rc = tsp_grouped_tasks(m->counts, m->tasks, m->experts, m->selected, m->tokens, 32, m->error_word, stream);
+    TSP_REQUIRE(uint64_t(8) * m->selected * m->hidden * 4 <= l.meta - l.hbuf, "planar v3 NAX scratch too small for requested batch");
+    for (uint32_t t0 = 0; rc == TSP_OK && t0 < m->tokens; t0 += 8) {
+        tsp_small_moe c{};
+        c.pair_lo = m->pair_lo; c.pair_hi = m->pair_hi; c.down = m->down;
+        c.gate_kind = m->gate_kind; c.up_kind = m->up_kind; c.down_kind = m->down_kind;
+        c.channels = m->channels; c.hidden = m->hidden; c.experts = m->experts; c.selected = m->selected;
+        c.tokens = m->tokens - t0 < 8 ? m->tokens - t0 : 8;
+        c.ids = m->ids + uint64_t(t0) * m->selected;
+        c.x = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(m->x) + uint64_t(t0) * m->x_stride_bytes);
+        c.x_stride_bytes = m->x_stride_bytes;
+        c.h = reinterpret_cast<float*>(ws + l.hbuf); c.h_stride_bytes = uint64_t(m->hidden) * 4;
+        c.y = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(m->y) + uint64_t(t0) * m->selected * m->y_stride_bytes);
+        c.y_stride_bytes = m->y_stride_bytes;
+        c.union_meta = reinterpret_cast<uint32_t*>(ws + l.meta);
+        c.error_word = m->error_word;
+        rc = tsp_planar_union_build(c.ids, c.union_meta, m->experts, m->selected, c.tokens, m->hidden, m->channels, m->error_word, stream);
+        if (rc == TSP_OK) rc = tsp_planar_moe_routed_m8(&c, stream);
+    }
+    return rc;
 }
 }  // namespace
 
@@ -699,8 +729,7 @@ extern "C" uint64_t tsp_planar_nax_workspace_bytes(uint32_t tokens, uint32_t sel
 
 extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream) {
     TSP_REQUIRE(m, "null grouped MoE description");
-    TSP_REQUIRE(m->gate_kind == TSP_KIND_Q4K_COLOC_GATE && m->up_kind == TSP_KIND_Q4K_COLOC_UP && m->down_kind == TSP_KIND_Q6K_PLANAR_X,
-                "planar v3 grouped MoE on the matrix cores takes Q4_K co-located gate/up and Q6_K planes for down");
+    const bool matrix_cores = m->gate_kind == TSP_KIND_Q4K_COLOC_GATE && m->up_kind == TSP_KIND_Q4K_COLOC_UP && m->down_kind == TSP_KIND_Q6K_PLANAR_X;
     TSP_REQUIRE(m->tokens >= 1 && m->tokens <= 2048 && m->selected >= 1 && m->selected <= 16 && m->selected <= m->experts &&
                     m->experts >= 2 && m->experts <= 512 && m->experts % 2 == 0 && m->channels % 256 == 0 && m->hidden % 256 == 0 &&
                     m->channels <= 65536 && m->hidden <= 65536,
@@ -711,6 +740,12 @@ extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream
     TSP_REQUIRE(m->pair_lo && m->pair_hi && m->down && m->ids && m->x && m->y && m->token_map && m->counts && m->tasks &&
                     m->workspace && m->error_word,
                 "null device pointer");
+    if (!matrix_cores) {
+        const NaxLayout lay = nax_layout(m->tokens, m->selected, m->experts, m->channels, m->hidden);
+        TSP_REQUIRE(m->workspace_bytes >= lay.total && reinterpret_cast<uintptr_t>(m->workspace) % 256 == 0,
+                    "planar v3 NAX scratch too small for requested batch");
+        return grouped_moe_in_eights(m, lay, stream);  // kinds, spans and overlaps are checked per chunk
+    }
     tsp_planar_spec gu, dn;
     int rc = tsp_make_expert_spec(12, m->channels, m->hidden, &gu);
     if (rc == TSP_OK) rc = tsp_make_expert_spec(14, m->hidden, m->channels, &dn);
