@@ -175,6 +175,13 @@ int tsp_gemv_rows(uint32_t encoding, uint32_t layout, const void* matrix, uint64
  * weight is decoded once for all rows. */
 int tsp_q8_matvec_many(uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* x, float* y,
                        uint32_t columns, uint32_t rows, uint32_t width, uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:860 `dense_mm_q8` (kernels/grouped_mm.metal:239-243; planner src/grouped_mm.cpp:48-54):
+ * out[t, :] = W in[t, :] for a dense Q8_0 matrix in GGUF rows (layout 0) or q8_lanes_v1 rows (layout 1), f32 rows in
+ * and out with byte strides. Decoded and accumulated in f32 (the engine stages halves); token rows that lie back to
+ * back share each weight read eight at a time. */
+int tsp_dense_mm_q8(uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* input, uint64_t input_stride_bytes,
+                    float* output, uint64_t output_stride_bytes, uint32_t tokens, uint32_t columns, uint32_t rows,
+                    uint32_t* error_word, void* stream);
 /* include/tokspur/graph.hpp:1093 `routed_gemv` (kernels/gemv.metal:198-227): per selected expert s,
  * y[s, :] = W[ids[s]] * x (x broadcast, or one x row per route). Raw GGUF expert stacks. */
 int tsp_routed_gemv(uint32_t encoding, const void* matrices, uint64_t matrices_bytes, const uint32_t* ids, const float* x,

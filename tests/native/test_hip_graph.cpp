@@ -204,6 +204,38 @@ std::vector<double> cpu_moe_token(const MoeFixture& f, const float* x, bool shar
     return out;
 }
 
+void test_dense_mm_q8_layouts() {
+    // graph.hpp:859-860: a dense Q8_0 matrix in GGUF rows and in q8_lanes_v1 rows, strided f32 rows in and out
+    const uint32_t K = 512, R = 160, M = 19;
+    HipGraph g(64u << 20);
+    const auto w = fixture(8, K, R, 1);
+    std::vector<uint8_t> lanes(w.size());
+    EXPECT(tsp_q8_lanes_pack_rows(K, w.data(), lanes.data(), w.size()) == TSP_OK);
+    const auto x = lcg_floats(21, size_t(M) * (K + 8));
+    const GpuView dw = g.upload(bytes_of(w), "w"), dl = g.upload(bytes_of(lanes), "lanes"), dx = g.upload(bytes_of(x), "x", false);
+    const std::vector<float> canary(size_t(M) * (R + 4), -7.0f);
+    const GpuView y0 = g.upload(bytes_of(canary), "y0", false), y1 = g.upload(bytes_of(canary), "y1", false);
+    EXPECT(throws_format([&] { g.configure_block_gemv(4); }));
+    g.configure_block_gemv(3);
+    g.configure_small_gemv(8);
+    g.prepare_dense_mm_q8(PrefillWeightLayout::q8_lanes_v1);
+    EXPECT(throws_format([&] { g.prepare_dense_mm_q8(PrefillWeightLayout::planar_v3); }));
+    const GpuRowsF32 in{dx, M, K, uint64_t(K + 8) * 4};
+    g.begin();
+    g.dense_mm_q8(PrefillWeightLayout::gguf, dw, in, {y0, M, R, uint64_t(R + 4) * 4});
+    g.dense_mm_q8(PrefillWeightLayout::q8_lanes_v1, dl, in, {y1, M, R, uint64_t(R + 4) * 4});
+    (void)g.submit();
+    const auto got0 = read_as<float>(g, y0), got1 = read_as<float>(g, y1);
+    for (uint32_t m = 0; m < M; ++m) {
+        std::vector<double> want(R);
+        orc_reference_gemv(8, w.data(), w.size(), K, R, x.data() + size_t(m) * (K + 8), K, want.data());
+        const std::vector<float> row0(got0.begin() + size_t(m) * (R + 4), got0.begin() + size_t(m) * (R + 4) + R);
+        const std::vector<float> row1(got1.begin() + size_t(m) * (R + 4), got1.begin() + size_t(m) * (R + 4) + R);
+        EXPECT(scaled_error(row0, want) <= 5e-5 && scaled_error(row1, want) <= 5e-5);
+        for (uint32_t pad = R; pad < R + 4; ++pad) EXPECT(got0[size_t(m) * (R + 4) + pad] == -7.0f && got1[size_t(m) * (R + 4) + pad] == -7.0f);
+    }
+}
+
 void test_encode_moe_single_token() {
     const MoeFixture f = make_moe(256, 256, 8, 3);
     HipGraph g(256u << 20);
@@ -319,6 +351,7 @@ void test_encode_moe_batch() {
 int main() {
     const std::pair<const char*, void (*)()> tests[] = {{"ledger and phases", test_ledger_and_phases},
                                                          {"gemv, route, mixture, top-k", test_gemv_route_mixture_topk},
+                                                         {"dense_mm_q8 in both row layouts", test_dense_mm_q8_layouts},
                                                          {"encode_moe single token", test_encode_moe_single_token},
                                                          {"encode_moe_batch", test_encode_moe_batch}};
     for (const auto& [name, fn] : tests) {

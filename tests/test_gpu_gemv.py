@@ -217,6 +217,25 @@ def test_gemv_refusals(gpu, tsp, synth):
 
 # ---------------------------------------------------------------------------------- Q8 many rows
 
+@pytest.mark.parametrize("tokens,cols,rows", [(1, 64, 5), (19, 512, 160), (40, 2048, 96)])
+def test_dense_mm_q8(gpu, tsp, orc, synth, tokens, cols, rows):
+    # graph.hpp:860 `dense_mm_q8`: a dense Q8_0 matrix times f32 rows, GGUF rows and q8_lanes_v1 rows; rows back to back
+    # (width groups 8, 4, 2, 1) and rows with padding (canaries stay)
+    w = synth.matrix(8, 1800 + cols, rows, cols)
+    lanes = tsp.q8_lanes_pack_rows(cols, w)
+    x = synth.activations_f32(1801 + tokens, (tokens, cols + 4))
+    want = np.stack([orc.reference_gemv(8, w, cols, rows, x[t, :cols]) for t in range(tokens)])
+    for matrix, layout in ((w, tsp.LAYOUT_GGUF), (lanes, tsp.LAYOUT_Q8_LANES_V1)):
+        packed = tsp.dense_mm_q8(gpu, layout, gpu.upload(matrix), gpu.upload(np.ascontiguousarray(x[:, :cols])), tokens, cols, rows).cpu().numpy()
+        assert scaled_error(packed, want) <= TOL and gpu.error() == 0
+        out = gpu.full((tokens, rows + 3), -5.0)
+        tsp.dense_mm_q8(gpu, layout, gpu.upload(matrix), gpu.upload(x), tokens, cols, rows, out=out, x_stride=(cols + 4) * 4, out_stride=(rows + 3) * 4)
+        got = out.cpu().numpy()
+        assert scaled_error(got[:, :rows], want) <= TOL and (got[:, rows:] == -5.0).all() and gpu.error() == 0
+    with pytest.raises(tsp.FormatError):
+        tsp.dense_mm_q8(gpu, tsp.LAYOUT_PLANAR_V3, gpu.upload(w), gpu.upload(x), tokens, cols, rows, x_stride=(cols + 4) * 4)
+
+
 @pytest.mark.parametrize("width", [1, 2, 4, 8])
 @pytest.mark.parametrize("cols,rows", [(2048, 37), (64, 5), (96, 7), (4096, 9)])
 def test_q8_matvec_many(gpu, tsp, orc, synth, width, cols, rows):

@@ -388,6 +388,16 @@ class GroupedMoe(C.Structure):
                 ("tasks", C.c_void_p), ("workspace", C.c_void_p), ("workspace_bytes", C.c_uint64), ("error_word", C.c_void_p)]
 
 
+def dense_mm_q8(dev, layout, matrix, x, tokens, columns, rows, out=None, x_stride=None, out_stride=None):
+    """Dense Q8_0 GEMM (`dense_mm_q8`): out[t] = W x[t], GGUF rows or q8_lanes_v1 rows, f32 rows with byte strides."""
+    out = dev.empty((tokens, rows)) if out is None else out
+    check(dll().tsp_dense_mm_q8(C.c_uint32(layout), dev.ptr(matrix), C.c_uint64(dev.nbytes(matrix)), dev.ptr(x),
+                                C.c_uint64(columns * 4 if x_stride is None else x_stride), dev.ptr(out),
+                                C.c_uint64(rows * 4 if out_stride is None else out_stride), C.c_uint32(tokens), C.c_uint32(columns),
+                                C.c_uint32(rows), dev.ptr(dev.err), dev.stream()))
+    return out
+
+
 def dense_mm_workspace_bytes(tokens, columns):
     f = dll().tsp_dense_mm_workspace_bytes
     f.restype = C.c_uint64

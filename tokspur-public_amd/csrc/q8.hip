@@ -189,3 +189,30 @@ extern "C" int tsp_q8_matvec_many(uint32_t layout, const void* matrix, uint64_t 
     default: return launch<8>(layout, a, s);
     }
 }
+
+extern "C" int tsp_dense_mm_q8(uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* input, uint64_t input_stride_bytes,
+                               float* output, uint64_t output_stride_bytes, uint32_t tokens, uint32_t columns, uint32_t rows,
+                               uint32_t* error_word, void* stream) {
+    TSP_REQUIRE(tokens && tokens <= 65536 && input_stride_bytes % 4 == 0 && output_stride_bytes % 4 == 0 &&
+                    input_stride_bytes >= uint64_t(columns) * 4 && output_stride_bytes >= uint64_t(rows) * 4,
+                "dense Q8_0 GEMM row geometry mismatch");
+    TSP_REQUIRE(input && output, "null device pointer");
+    const uint64_t in_span = uint64_t(tokens - 1) * input_stride_bytes + uint64_t(columns) * 4;
+    const uint64_t out_span = uint64_t(tokens - 1) * output_stride_bytes + uint64_t(rows) * 4;
+    TSP_REQUIRE(!ranges_overlap(output, out_span, matrix, matrix_bytes) && !ranges_overlap(output, out_span, input, in_span),
+                "dense Q8_0 GEMM output overlaps an input");
+    // Token rows that lie back to back go eight, four, two, one at a time (each weight decoded once for the group, the
+    // width sequence of src/q8_many.cpp:20-29); rows with padding between them go one by one.
+    const bool packed = input_stride_bytes == uint64_t(columns) * 4 && output_stride_bytes == uint64_t(rows) * 4;
+    for (uint32_t done = 0; done < tokens;) {
+        uint32_t width = 1;
+        if (packed) tsp_q8_many_width(tokens - done, &width);
+        const int rc = tsp_q8_matvec_many(layout, matrix, matrix_bytes,
+                                          reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(input) + uint64_t(done) * input_stride_bytes),
+                                          reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(output) + uint64_t(done) * output_stride_bytes),
+                                          columns, rows, width, error_word, stream);
+        if (rc != TSP_OK) return rc;
+        done += width;
+    }
+    return TSP_OK;
+}

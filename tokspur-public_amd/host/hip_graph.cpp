@@ -560,6 +560,34 @@ void HipGraph::dense_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView m
                        p.dense_workspace_bytes, p.error_word, p.stream));
 }
 
+void HipGraph::prepare_dense_mm_q8(PrefillWeightLayout layout) {
+    impl_->idle();
+    require(layout == PrefillWeightLayout::gguf || layout == PrefillWeightLayout::q8_lanes_v1, "dense Q8_0 GEMM layout");
+}
+
+void HipGraph::dense_mm_q8(PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output, bool) {
+    auto& p = *impl_; p.active();
+    require(layout == PrefillWeightLayout::gguf || layout == PrefillWeightLayout::q8_lanes_v1, "dense Q8_0 GEMM layout");
+    p.rows_fit(input, "dense Q8_0 GEMM geometry");
+    p.rows_fit(output, "dense Q8_0 GEMM geometry");
+    require(input.rows == output.rows && input.rows >= 1, "dense Q8_0 GEMM geometry");
+    validate_disjoint(std::array{matrix, input.view}, std::array{output.view});
+    check(tsp_dense_mm_q8(uint32_t(layout), p.device(matrix), matrix.bytes, reinterpret_cast<const float*>(p.device(input.view)), input.stride_bytes,
+                          reinterpret_cast<float*>(p.device(output.view, true)), output.stride_bytes, input.rows, input.columns, output.columns,
+                          p.error_word, p.stream));
+}
+
+void HipGraph::configure_small_gemv(uint32_t column_splits) {
+    impl_->idle();
+    require(column_splits == 0 || column_splits == 1 || column_splits == 4 || column_splits == 8 || column_splits == 16 || column_splits == 32,
+            "small GEMV column split count");
+}
+
+void HipGraph::configure_block_gemv(uint32_t formats) {
+    impl_->idle();
+    require(formats <= 3, "block GEMV format mask");
+}
+
 uint64_t HipGraph::logit_topk_scratch_bytes(uint32_t max_rows, uint32_t max_vocabulary) {
     const uint64_t bytes = tsp_logit_topk_scratch_bytes(max_rows, max_vocabulary);
     require(bytes > 0, "GPU logit top-k scratch bounds mismatch");

@@ -142,6 +142,14 @@ public:
                     GpuView token_map, GpuView counts, GpuView tasks, uint32_t experts, uint32_t selected, bool broadcast);
     // the same with experts = 1, selected = 1, broadcast: the dense dequant-GEMM (Q4_K rows or planes, Q6_K planes)
     void dense_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output);
+    // graph.hpp:859-860 `prepare_dense_mm_q8` / `dense_mm_q8`: out[m, :] = W x[m, :] for a dense Q8_0 matrix in GGUF rows or
+    // q8_lanes_v1 rows, f32 rows in and out (decoded and accumulated in f32, each weight read once per eight rows)
+    void prepare_dense_mm_q8(PrefillWeightLayout layout);
+    void dense_mm_q8(PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output, bool reuse_bf16 = false);
+    // graph.hpp:548-553 selectors of the engine's GEMV variants: same arithmetic here whatever they say, kept so that
+    // callers' set-up code runs unchanged (idle only, same accepted values)
+    void configure_small_gemv(uint32_t column_splits);
+    void configure_block_gemv(uint32_t formats);
     static uint64_t logit_topk_scratch_bytes(uint32_t max_rows, uint32_t max_vocabulary = 1u << 20);                 // graph.hpp:1030
     static uint64_t logit_topk_output_bytes(uint32_t max_rows);
     void prepare_logit_topk();
