@@ -346,6 +346,105 @@ void test_encode_moe_batch() {
     EXPECT(throws_format([&] { (void)g.submit(); }));
     release_moe_batch_scratch(g, scratch);
 }
+// CPU composition of the whole sublayer for one token with a dense Q8_0 shared expert (src/moe_mm_many.cpp:126-283 order)
+std::vector<double> cpu_moe_token_q8_shared(const MoeFixture& f, const std::vector<uint8_t>& sg, const std::vector<uint8_t>& su, const std::vector<uint8_t>& sd,
+                                            const float* x) {
+    const MoeShape s = f.shape;
+    std::vector<double> logits(s.experts), weights(s.selected), out(s.channels);
+    orc_reference_gemv(0, reinterpret_cast<const uint8_t*>(f.router.data()), f.router.size() * 4, s.channels, s.experts, x, s.channels, logits.data());
+    for (auto& v : logits) v = double(float(v));
+    std::vector<uint32_t> ids(s.selected);
+    orc_route_reference(logits.data(), s.experts, s.selected, 0, 1, ids.data(), weights.data());
+    std::vector<double> h(size_t(s.selected) * s.hidden), y(size_t(s.selected) * s.channels);
+    orc_moe_routed_reference(12, 14, f.gate.data(), f.up.data(), f.down.data(), s.channels, s.hidden, s.experts, ids.data(), 1, s.selected, x, s.channels, 1, 0,
+                             h.data(), y.data(), 1);
+    std::vector<double> g(s.hidden), u(s.hidden), sy(s.channels);
+    orc_reference_gemv(8, sg.data(), sg.size(), s.channels, s.hidden, x, s.channels, g.data());
+    orc_reference_gemv(8, su.data(), su.size(), s.channels, s.hidden, x, s.channels, u.data());
+    std::vector<float> act(s.hidden);
+    for (uint32_t i = 0; i < s.hidden; ++i) { const double v = g[i]; act[i] = float(v / (1.0 + std::exp(-v)) * u[i]); }
+    orc_reference_gemv(8, sd.data(), sd.size(), s.hidden, s.channels, act.data(), s.hidden, sy.data());
+    double shared_logit = 0;
+    orc_reference_gemv(0, reinterpret_cast<const uint8_t*>(f.shared_router.data()), f.shared_router.size() * 4, s.channels, 1, x, s.channels, &shared_logit);
+    orc_mixture_reference(y.data(), weights.data(), s.selected, sy.data(), s.channels, double(float(shared_logit)), out.data());
+    return out;
+}
+
+void test_encode_moe_mm_many() {
+    // planar Q4_K / Q6_K routed experts, dense Q8_0 shared expert (gate in q8_lanes_v1 rows, up and down in GGUF rows), F32 routers;
+    // 70 rows take the grouped GEMM, 5 rows the routed kernels for at most eight
+    const MoeFixture f = make_moe(256, 256, 8, 3);
+    const uint32_t capacity = 70;
+    HipGraph g(512u << 20);
+    MoeOnGraph m = upload_moe(g, f);
+    const auto sg = fixture(8, f.shape.channels, f.shape.hidden, 1), sd = fixture(8, f.shape.hidden, f.shape.channels, 1);
+    auto su = sg;
+    for (size_t at = 0; at < su.size(); at += 34) for (size_t i = 2; i < 34; ++i) su[at + i] = uint8_t(su[at + i] * 5 + 3);
+    std::vector<uint8_t> sg_lanes(sg.size());
+    EXPECT(tsp_q8_lanes_pack_rows(f.shape.channels, sg.data(), sg_lanes.data(), sg.size()) == TSP_OK);
+    m.w.shared_gate = {g.upload(bytes_of(sg_lanes), "shared gate"), 8};
+    m.w.shared_up = {g.upload(bytes_of(su), "shared up"), 8};
+    m.w.shared_down = {g.upload(bytes_of(sd), "shared down"), 8};
+    MoeMmLayouts layouts;
+    layouts.shared_gate = PrefillWeightLayout::q8_lanes_v1;
+    prepare_moe_mm_many(g, m.w, f.shape, capacity, layouts);
+    const MoeMmManyScratch scratch = allocate_moe_mm_many_scratch(g, f.shape, capacity);
+    EXPECT(scratch.capacity == capacity && moe_mm_many_bytes(f.shape, capacity).views[0] == uint64_t(capacity) * f.shape.experts * 4);
+    const uint32_t stride = f.shape.channels + 4;  // 16-byte multiple, as the composition demands
+    for (const uint32_t T : {70u, 5u}) {
+        std::vector<float> x = lcg_floats(400 + T, size_t(T) * stride);
+        for (auto& v : x) { uint32_t bad = 0; v = orc_bf16_to_f32(orc_round_bf16_bits(v, &bad)); }
+        const GpuView dx = g.upload(bytes_of(x), "x", false);
+        const std::vector<float> canary(size_t(T) * stride, -3.0f);
+        const GpuView dy = g.upload(bytes_of(canary), "y", false);
+        const uint64_t allocations = g.memory().allocations;
+        g.begin();
+        encode_moe_mm_many(g, m.w, scratch, {dx, T, f.shape.channels, uint64_t(stride) * 4}, {dy, T, f.shape.channels, uint64_t(stride) * 4}, f.shape,
+                           RouterMode::softmax, true, layouts);
+        (void)g.submit();
+        EXPECT(g.memory().allocations == allocations);
+        const auto y = read_as<float>(g, dy);
+        double worst = 0;
+        bool pads = true;
+        for (uint32_t t = 0; t < T; ++t) {
+            const auto want = cpu_moe_token_q8_shared(f, sg, su, sd, &x[size_t(t) * stride]);
+            double scale = 1;
+            for (double v : want) scale = std::max(scale, std::fabs(v));
+            for (uint32_t c = 0; c < f.shape.channels; ++c) worst = std::max(worst, std::fabs(double(y[size_t(t) * stride + c]) - want[c]) / scale);
+            for (uint32_t c = f.shape.channels; c < stride; ++c) pads = pads && y[size_t(t) * stride + c] == -3.0f;
+        }
+        std::printf("encode_moe_mm_many T=%u: max error / row max %.3e\n", T, worst);
+        EXPECT(worst <= 2e-3 && pads);
+        g.release(dx);
+        g.release(dy);
+    }
+    // rows beyond the scratch capacity are worked off in chunks; a scratch of another capacity is refused
+    {
+        const uint32_t T = 150;
+        std::vector<float> x = lcg_floats(777, size_t(T) * stride);
+        for (auto& v : x) { uint32_t bad = 0; v = orc_bf16_to_f32(orc_round_bf16_bits(v, &bad)); }
+        const GpuView dx = g.upload(bytes_of(x), "x", false), dy = g.zeros(uint64_t(T) * stride * 4, "y");
+        g.begin();
+        encode_moe_mm_many(g, m.w, scratch, {dx, T, f.shape.channels, uint64_t(stride) * 4}, {dy, T, f.shape.channels, uint64_t(stride) * 4}, f.shape,
+                           RouterMode::softmax, true, layouts);
+        (void)g.submit();
+        const auto y = read_as<float>(g, dy);
+        const auto want = cpu_moe_token_q8_shared(f, sg, su, sd, &x[size_t(149) * stride]);
+        double scale = 1, worst = 0;
+        for (double v : want) scale = std::max(scale, std::fabs(v));
+        for (uint32_t c = 0; c < f.shape.channels; ++c) worst = std::max(worst, std::fabs(double(y[size_t(149) * stride + c]) - want[c]) / scale);
+        EXPECT(worst <= 2e-3);
+        MoeMmManyScratch wrong = scratch;
+        wrong.capacity = capacity + 1;
+        g.begin();
+        EXPECT(throws_format([&] {
+            encode_moe_mm_many(g, m.w, wrong, {dx, 4, f.shape.channels, uint64_t(stride) * 4}, {dy, 4, f.shape.channels, uint64_t(stride) * 4}, f.shape,
+                               RouterMode::softmax, true, layouts);
+        }));
+        g.abort();
+    }
+    release_moe_mm_many_scratch(g, scratch);
+}
 }  // namespace
 
 int main() {
@@ -353,7 +452,8 @@ int main() {
                                                          {"gemv, route, mixture, top-k", test_gemv_route_mixture_topk},
                                                          {"dense_mm_q8 in both row layouts", test_dense_mm_q8_layouts},
                                                          {"encode_moe single token", test_encode_moe_single_token},
-                                                         {"encode_moe_batch", test_encode_moe_batch}};
+                                                         {"encode_moe_batch", test_encode_moe_batch},
+                                                         {"encode_moe_mm_many", test_encode_moe_mm_many}};
     for (const auto& [name, fn] : tests) {
         std::printf("== %s\n", name);
         std::fflush(stdout);

@@ -719,4 +719,98 @@ void encode_moe_batch(HipGraph& graph, const MoeWeights& w, const MoeBatchScratc
     graph.prefill_mixture_batch(s.expert_down, s.weights, s.shared_down, s.shared_logit, output, shape.selected);
 }
 
+// ------------------------------------------------------------------ encode_moe_mm_many
+MoeMmManyBytes moe_mm_many_bytes(MoeShape shape, uint32_t capacity, bool allow_nax_2k) {
+    shape_check(shape);
+    MoeMmManyBytes b;
+    check(tsp_moe_mm_many_bytes(shape.channels, shape.hidden, shape.experts, shape.selected, capacity, allow_nax_2k ? 1 : 0, b.views.data(), &b.total));
+    return b;
+}
+
+MoeMmManyScratch allocate_moe_mm_many_scratch(HipGraph& graph, MoeShape shape, uint32_t capacity, bool allow_nax_2k) {
+    const MoeMmManyBytes b = moe_mm_many_bytes(shape, capacity, allow_nax_2k);
+    std::array<GpuView, 13> v{};
+    size_t made = 0;
+    try {
+        for (; made < v.size(); ++made) v[made] = graph.zeros(b.views[made], "tiled mixture scratch");
+    } catch (...) {
+        for (size_t i = 0; i < made; ++i) graph.release(v[i]);
+        throw;
+    }
+    return {{v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], v[9]}, v[10], v[11], v[12], capacity};
+}
+
+void release_moe_mm_many_scratch(HipGraph& graph, const MoeMmManyScratch& scratch) {
+    for (const auto view : scratch.views()) graph.release(view);
+}
+
+void prepare_moe_mm_many(HipGraph& graph, const MoeWeights& w, MoeShape shape, uint32_t capacity, MoeMmLayouts l) {
+    shape_check(shape);
+    require(capacity >= 1, "tiled MoE capacity");
+    const uint32_t rows = capacity < 2048 ? capacity : 2048;
+    if (is_planar_moe(graph, w, shape)) {
+        graph.prepare_planar_moe_v3(w.gate.encoding, w.down.encoding, true, rows, shape.experts, shape.selected, shape.channels, shape.hidden);
+    } else {
+        graph.prepare_grouped_mm(w.gate.encoding, l.gate, rows, shape.selected, shape.experts, shape.channels > shape.hidden ? shape.channels : shape.hidden);
+    }
+    for (const auto layout : {l.shared_gate, l.shared_up, l.shared_down}) graph.prepare_dense_mm_q8(layout);
+}
+
+void encode_moe_mm_many(HipGraph& g, const MoeWeights& w, const MoeMmManyScratch& s, GpuRowsF32 input, GpuRowsF32 output, MoeShape shape,
+                        RouterMode mode, bool normalize_selected, MoeMmLayouts l) {
+    shape_check(shape);
+    const uint32_t chunk = s.capacity < 2048 ? s.capacity : 2048;
+    require(chunk > 0 && input.rows >= 1 && input.rows == output.rows && input.columns == shape.channels && output.columns == shape.channels,
+            "tiled MoE active rows/router mode");
+    if (input.rows > chunk) {  // src/moe_mm_many.cpp:134-143
+        for (uint32_t at = 0; at < input.rows; at += chunk) {
+            const uint32_t n = input.rows - at < chunk ? input.rows - at : chunk;
+            const GpuView in = g.slice(input.view, uint64_t(at) * input.stride_bytes, uint64_t(n - 1) * input.stride_bytes + uint64_t(input.columns) * 4);
+            const GpuView out = g.slice(output.view, uint64_t(at) * output.stride_bytes, uint64_t(n - 1) * output.stride_bytes + uint64_t(output.columns) * 4);
+            encode_moe_mm_many(g, w, s, {in, n, input.columns, input.stride_bytes}, {out, n, output.columns, output.stride_bytes}, shape, mode,
+                               normalize_selected, l);
+        }
+        return;
+    }
+    const MoeMmManyBytes b = moe_mm_many_bytes(shape, s.capacity, true);
+    const auto all = s.views();
+    for (size_t i = 0; i < all.size(); ++i) require(all[i].bytes == b.views[i], "tiled MoE scratch capacity extent");
+    const uint32_t n = input.rows;
+    for (const auto& r : {input, output})
+        require(r.stride_bytes >= uint64_t(shape.channels) * 4 && r.stride_bytes % 16 == 0 &&
+                    r.view.bytes >= uint64_t(n - 1) * r.stride_bytes + uint64_t(shape.channels) * 4,
+                "tiled MoE strided row extent");
+    const std::array<GpuView, 9> read{input.view, w.router.view, w.gate.view, w.up.view, w.down.view, w.shared_gate.view, w.shared_up.view,
+                                      w.shared_down.view, w.shared_router.view};
+    std::array<GpuView, 14> write{output.view};
+    std::copy(all.begin(), all.end(), write.begin() + 1);
+    g.validate_disjoint(read, write);
+    // the first `per_row * n` floats of a scratch view, flat or as n rows
+    const auto active = [&](GpuView v, uint64_t per_row) { return g.slice(v, 0, per_row * n * 4); };
+    const auto rows = [&](GpuView v, uint32_t count, uint32_t columns) { return GpuRowsF32{g.slice(v, 0, uint64_t(count) * columns * 4), count, columns, uint64_t(columns) * 4}; };
+    const GpuView logits = active(s.rows.logits, shape.experts), ids = active(s.rows.indices, shape.selected), weights = active(s.rows.weights, shape.selected);
+    g.gemv_rows(w.router.encoding, w.router.view, input, {logits, n, shape.experts, uint64_t(shape.experts) * 4});
+    g.prefill_route_batch(logits, ids, weights, shape.experts, shape.selected, n, mode, normalize_selected);
+    const GpuRowsF32 gate = rows(s.rows.gate, n * shape.selected, shape.hidden), down_rows = rows(s.rows.down, n * shape.selected, shape.channels);
+    if (is_planar_moe(g, w, shape)) {
+        if (n <= 8) g.planar_moe_routed_m8(w.gate.view, w.up.view, w.down.view, ids, input, gate, down_rows, shape.experts, shape.selected);
+        else g.planar_nax_grouped_moe(w.gate.view, w.up.view, w.down.view, ids, input, down_rows, s.token_map, s.counts, s.tasks, shape.experts, shape.selected);
+    } else {
+        const GpuRowsF32 up = rows(s.rows.up, n * shape.selected, shape.hidden);
+        g.grouped_mm(w.gate.encoding, l.gate, w.gate.view, ids, input, gate, s.token_map, s.counts, s.tasks, shape.experts, shape.selected, true);
+        g.grouped_mm(w.up.encoding, l.up, w.up.view, ids, input, up, s.token_map, s.counts, s.tasks, shape.experts, shape.selected, true);
+        g.swiglu(gate.view, up.view, gate.view);
+        g.grouped_mm(w.down.encoding, l.down, w.down.view, ids, gate, down_rows, s.token_map, s.counts, s.tasks, shape.experts, shape.selected, false);
+    }
+    const GpuRowsF32 sg = rows(s.rows.shared_gate, n, shape.hidden), su = rows(s.rows.shared_up, n, shape.hidden);
+    g.dense_mm_q8(l.shared_gate, w.shared_gate.view, input, sg);
+    g.dense_mm_q8(l.shared_up, w.shared_up.view, input, su);
+    g.swiglu(sg.view, su.view, sg.view);
+    g.dense_mm_q8(l.shared_down, w.shared_down.view, sg, rows(s.rows.shared_down, n, shape.channels));
+    const GpuView shared_logit = active(s.rows.shared_logit, 1);
+    g.gemv_rows(w.shared_router.encoding, w.shared_router.view, input, {shared_logit, n, 1, 4});
+    g.prefill_mixture_batch(active(s.rows.down, uint64_t(shape.selected) * shape.channels), weights, active(s.rows.shared_down, shape.channels),
+                            shared_logit, output, shape.selected);
+}
+
 }  // namespace tokspur

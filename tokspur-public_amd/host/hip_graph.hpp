@@ -188,4 +188,33 @@ void release_moe_batch_scratch(HipGraph& graph, const MoeBatchScratch& scratch);
 void encode_moe_batch(HipGraph& graph, const MoeWeights& weights, const MoeBatchScratch& scratch, GpuView logits, GpuRowsF32 input,
                       GpuRowsF32 output, MoeShape shape, RouterMode mode, bool normalize_selected);
 
+// ---- the whole prefill MoE sublayer for up to `capacity` token rows, include/tokspur/moe_mm_many.hpp:7-63 and
+// src/moe_mm_many.cpp:126-283 (default arm): router projection (F32 rows) -> batch top-k -> routed experts (planar: at most
+// eight rows through the routed kernels, more through the grouped GEMM; raw GGUF: grouped_mm x 2 + SwiGLU + grouped_mm) ->
+// shared expert as dense Q8_0 products -> shared router -> batch mixture. Rows beyond 2048 are worked off in chunks.
+struct MoeMmLayouts {
+    PrefillWeightLayout gate = PrefillWeightLayout::gguf, up = PrefillWeightLayout::gguf, down = PrefillWeightLayout::gguf;
+    PrefillWeightLayout shared_gate = PrefillWeightLayout::gguf, shared_up = PrefillWeightLayout::gguf, shared_down = PrefillWeightLayout::gguf;
+};
+struct MoeMmManyBytes {
+    std::array<uint64_t, 13> views{};
+    uint64_t total = 0;
+};
+struct MoeMmManyScratch {
+    MoeScratch rows;
+    GpuView token_map, counts, tasks;
+    uint32_t capacity = 0;
+    [[nodiscard]] std::array<GpuView, 13> views() const {
+        const auto r = rows.views();
+        return {r[0], r[1], r[2], r[3], r[4], r[5], r[6], r[7], r[8], r[9], token_map, counts, tasks};
+    }
+};
+MoeMmManyBytes moe_mm_many_bytes(MoeShape shape, uint32_t capacity, bool allow_nax_2k = true);
+MoeMmManyScratch allocate_moe_mm_many_scratch(HipGraph& graph, MoeShape shape, uint32_t capacity, bool allow_nax_2k = true);
+void release_moe_mm_many_scratch(HipGraph& graph, const MoeMmManyScratch& scratch);
+// idle only: sizes the workspaces the routed and shared products need for `capacity` rows
+void prepare_moe_mm_many(HipGraph& graph, const MoeWeights& weights, MoeShape shape, uint32_t capacity, MoeMmLayouts layouts = {});
+void encode_moe_mm_many(HipGraph& graph, const MoeWeights& weights, const MoeMmManyScratch& scratch, GpuRowsF32 input, GpuRowsF32 output,
+                        MoeShape shape, RouterMode mode, bool normalize_selected, MoeMmLayouts layouts = {});
+
 }  // namespace tokspur
