@@ -50,6 +50,8 @@ __device__ __forceinline__ f16x8 quants8(uint32_t w0, uint32_t w1) {
     return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
 }
 
+// DEPTH = (tile, group) items whose bytes are on their way while one is multiplied (1, 2 or 4; it divides the number of groups).
+template <int DEPTH>
 __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [hi plane][lo plane][8 weight tiles]
     __shared__ float wave_max[kWaves];
@@ -111,8 +113,9 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
         return *reinterpret_cast<const f16x8*>(plane + (arow * chunks + (chunk ^ arow)) * 8);
     };
     // chunk `id` of a group tile: row id / 17 of the wave's 32, bytes (id % 17) * 16 of that row's 272
-    uint2 stage[kStageLoads][2];
-    auto fetch_group = [&](uint32_t row0, uint32_t group) {
+    uint2 stage[DEPTH][kStageLoads][2];
+    auto fetch_group = [&](uint32_t row0, uint32_t group, auto set_tag) {
+        constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
         for (uint32_t t = 0; t < kStageLoads; ++t) {
             uint32_t id = t * kWave + lane;
@@ -120,18 +123,19 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
             uint32_t row = row0 + id / kGroupChunks;
             row = row < a.rows ? row : a.rows - 1;
             const uint4 v = *reinterpret_cast<const uint4*>(a.matrix + uint64_t(row) * row_bytes + group * kGroupBytes + (id % kGroupChunks) * 16);
-            stage[t][0] = uint2{v.x, v.y};
-            stage[t][1] = uint2{v.z, v.w};
+            stage[SET][t][0] = uint2{v.x, v.y};
+            stage[SET][t][1] = uint2{v.z, v.w};
         }
     };
-    auto store_group = [&]() {
+    auto store_group = [&](auto set_tag) {
+        constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
         for (uint32_t t = 0; t < kStageLoads; ++t) {
             uint32_t id = t * kWave + lane;
             id = id < 32 * kGroupChunks ? id : 32 * kGroupChunks - 1;
             uint8_t* at = tile + (id / kGroupChunks) * kTileStride + (id % kGroupChunks) * 16;  // 8-byte aligned
-            *reinterpret_cast<uint2*>(at) = stage[t][0];
-            *reinterpret_cast<uint2*>(at + 8) = stage[t][1];
+            *reinterpret_cast<uint2*>(at) = stage[SET][t][0];
+            *reinterpret_cast<uint2*>(at + 8) = stage[SET][t][1];
         }
     };
 
@@ -146,17 +150,27 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
         return uint32_t(__builtin_amdgcn_readfirstlane(int(t)));
     };
     uint32_t t = take_tile(), t_next = take_tile();
-    if (t < share_end) fetch_group(t * 32, 0);
+    if (t < share_end) {
+        fetch_group(t * 32, 0, std::integral_constant<int, 0>{});
+        if constexpr (DEPTH >= 2) fetch_group(t * 32, 1, std::integral_constant<int, 1 % DEPTH>{});
+        if constexpr (DEPTH >= 4) {
+            fetch_group(t * 32, 2, std::integral_constant<int, 2 % DEPTH>{});
+            fetch_group(t * 32, 3, std::integral_constant<int, 3 % DEPTH>{});
+        }
+    }
     for (; t < share_end; t = t_next, t_next = take_tile()) {
         const uint32_t row0 = t * 32;
         f32x16 acc;
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
-        for (uint32_t g = 0; g < groups; ++g) {
-            store_group();  // the previous item's reads were issued before this point; LDS serves a wave in order
-            const bool last = g + 1 == groups;
-            const uint32_t following = last ? (t_next < share_end ? t_next : t) : t;
-            fetch_group(following * 32, last ? 0 : g + 1);  // past the end: a harmless repeat of this tile's first group
+        // one item: its bytes go registers -> LDS tile, the item DEPTH ahead is requested into the freed registers, then the
+        // tile is multiplied. Items past the workgroup's share are a harmless repeat of this tile's first groups.
+        auto item = [&](uint32_t g, auto set_tag) {
+            store_group(set_tag);  // the previous item's reads were issued before this point; LDS serves a wave in order
+            const uint32_t ahead = g + DEPTH;
+            const bool wraps = ahead >= groups;
+            const uint32_t following = wraps ? (t_next < share_end ? t_next : t) : t;
+            fetch_group(following * 32, wraps ? ahead - groups : ahead, set_tag);
             const uint8_t* mine = tile + col * kTileStride + khalf * 16;
             auto block = [&](auto b_tag) {
                 constexpr int B = decltype(b_tag)::value;
@@ -193,6 +207,14 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
             block(std::integral_constant<int, 5>{});
             block(std::integral_constant<int, 6>{});
             block(std::integral_constant<int, 7>{});
+        };
+        for (uint32_t g = 0; g < groups; g += DEPTH) {  // the host picks a DEPTH that divides the number of groups
+            item(g, std::integral_constant<int, 0>{});
+            if constexpr (DEPTH >= 2) item(g + 1, std::integral_constant<int, 1 % DEPTH>{});
+            if constexpr (DEPTH >= 4) {
+                item(g + 2, std::integral_constant<int, 2 % DEPTH>{});
+                item(g + 3, std::integral_constant<int, 3 % DEPTH>{});
+            }
         }
         const uint32_t r = row0 + col;
 #pragma unroll
@@ -223,7 +245,9 @@ int q8_mfma(const void* matrix, const float* x, float* y, uint32_t columns, uint
     static bool raised = false;
     static int compute_units = 0;
     if (!raised) {
-        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    int(2 * kRows * 2048 * 2 + kWaves * kTileBytes)));
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     int(2 * kRows * 2048 * 2 + kWaves * kTileBytes)));
         int device = 0;
         TSP_HIP(hipGetDevice(&device));
@@ -233,7 +257,9 @@ int q8_mfma(const void* matrix, const float* x, float* y, uint32_t columns, uint
     const uint32_t tiles = (rows + 31) / 32;
     uint32_t grid = uint32_t(compute_units > 0 ? compute_units : 256);
     if (grid * kWaves > tiles) grid = (tiles + kWaves - 1) / kWaves;
-    TSP_LAUNCH("q8_mfma", s, q8_mfma_kernel<<<grid, kThreads, lds_bytes, s>>>(a));
+    // two items in flight measured best on MI355X (one: 72 us, two: 69 us, four: 75 us at 151 936 x 2048)
+    if ((columns / 256) % 2 == 0) TSP_LAUNCH("q8_mfma", s, q8_mfma_kernel<2><<<grid, kThreads, lds_bytes, s>>>(a));
+    else TSP_LAUNCH("q8_mfma", s, q8_mfma_kernel<1><<<grid, kThreads, lds_bytes, s>>>(a));
     return launch_status("q8_mfma");
 }
 
