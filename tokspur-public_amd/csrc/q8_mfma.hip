@@ -164,13 +164,16 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
         // one item: its bytes go registers -> LDS tile, the item DEPTH ahead is requested into the freed registers, then the
-        // tile is multiplied. Items past the workgroup's share are a harmless repeat of this tile's first groups.
+        // tile is multiplied.
         auto item = [&](uint32_t g, auto set_tag) {
             store_group(set_tag);  // the previous item's reads were issued before this point; LDS serves a wave in order
             const uint32_t ahead = g + DEPTH;
             const bool wraps = ahead >= groups;
-            const uint32_t following = wraps ? (t_next < share_end ? t_next : t) : t;
-            fetch_group(following * 32, wraps ? ahead - groups : ahead, set_tag);
+            // past the workgroup's share: ask again for the group at hand (its lines are in cache), nothing new comes from memory
+            const bool more = t_next < share_end;
+            const uint32_t following = wraps && more ? t_next : t;
+            const uint32_t group = !wraps ? ahead : more ? ahead - groups : g;
+            fetch_group(following * 32, group, set_tag);
             const uint8_t* mine = tile + col * kTileStride + khalf * 16;
             auto block = [&](auto b_tag) {
                 constexpr int B = decltype(b_tag)::value;
