@@ -293,7 +293,7 @@ def main():
                                        "launch": "HIP graph replay of eight steps" if graph2 is not None else "eager launches from Python"}
         state["i"] = 0
         configs["c2_moe_verify_t8"]["kernels_us"] = {k: round(v["avg_us"], 2) for k, v in profiled(capi, torch, step_c2, 8).items()}
-        # config 4: Q8_0 LM head, vocab 151936 x 2048, raw GGUF rows; M = 16 is two width-8 passes
+        # config 4: Q8_0 LM head, vocab 151936 x 2048, raw GGUF rows; M = 16 goes through the dense Q8_0 GEMM entry point (one pass, K halves summed)
         V = 151936
         w4 = gpu.upload(synth.matrix(8, synth.tensor_seed(4, 1), V, C))
         for m in (1, 4, 8, 16):
@@ -301,9 +301,10 @@ def main():
             y4 = gpu.empty((m, V))
 
             def lm_head():
-                for at in range(0, m, 8):
-                    width = min(8, m - at)
-                    gpu.q8_matvec_many(w4, x4[at:at + width], C, V, width, y=y4[at:at + width])
+                if m > 8:  # one pass over the matrix for up to sixteen rows
+                    capi.dense_mm_q8(gpu, capi.LAYOUT_GGUF, w4, x4, m, C, V, out=y4)
+                else:
+                    gpu.q8_matvec_many(w4, x4, C, V, m, y=y4)
 
             ms = timed(torch, lm_head, k2, 2)
             b4 = 330612736 + 615936 * m

@@ -178,7 +178,8 @@ int tsp_q8_matvec_many(uint32_t layout, const void* matrix, uint64_t matrix_byte
 /* include/tokspur/graph.hpp:860 `dense_mm_q8` (kernels/grouped_mm.metal:239-243; planner src/grouped_mm.cpp:48-54):
  * out[t, :] = W in[t, :] for a dense Q8_0 matrix in GGUF rows (layout 0) or q8_lanes_v1 rows (layout 1), f32 rows in
  * and out with byte strides. Decoded and accumulated in f32 (the engine stages halves); token rows that lie back to
- * back share each weight read eight at a time. */
+ * back share each weight read eight at a time, and up to sixteen at a time for GGUF rows of 1024 or 2048 columns
+ * (16-byte aligned buffers, at least 64 rows, a multiple of 4). */
 int tsp_dense_mm_q8(uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* input, uint64_t input_stride_bytes,
                     float* output, uint64_t output_stride_bytes, uint32_t tokens, uint32_t columns, uint32_t rows,
                     uint32_t* error_word, void* stream);

@@ -1,4 +1,4 @@
-// Q8_0 GEMV for up to eight token rows on the matrix cores (LM head, verify): y[m, r] = sum_k d[r, k/32] * q[r, k] * x[m, k].
+// Q8_0 GEMV for up to sixteen token rows on the matrix cores (LM head, verify): y[m, r] = sum_k d[r, k/32] * q[r, k] * x[m, k].
 //
 // A Q8_0 row is a run of 34-byte blocks (f16 scale + 32 int8). The int8 quants are exact halves, so a block is two
 // 32x32x16 MFMA steps of the integer quants against the activations; the block's scale multiplies the f32 result
@@ -15,6 +15,11 @@
 //
 // Workgroups are persistent (one per compute unit, 8 waves): the activations are staged once per workgroup, which owns
 // a contiguous share of the matrix's 32-row tiles; its waves take tiles from that share through a counter in LDS.
+//
+// Nine to sixteen token rows do not fit LDS for all of K beside the weight tiles, so that variant splits K in two:
+// even workgroups take the first half of the columns, odd ones the second, each over its share of the tiles, and both
+// add their f32 partial sums into an output the host cleared before the launch (two addends onto zero: the sum does
+// not depend on which arrives first). The matrix is still read once.
 #include "q8_mfma.hpp"
 
 #include <type_traits>
@@ -25,7 +30,6 @@ using namespace tsp;
 
 namespace {
 
-constexpr int kRows = 8;
 constexpr uint32_t kWaves = 8, kThreads = kWaves * kWave;
 constexpr uint32_t kGroupBlocks = 8, kGroupBytes = kGroupBlocks * 34, kGroupChunks = kGroupBytes / 16;  // 272 B = 17 chunks
 constexpr uint32_t kTileStride = 280;                     // bytes between rows of the LDS weight tile
@@ -50,17 +54,28 @@ __device__ __forceinline__ f16x8 quants8(uint32_t w0, uint32_t w1) {
     return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
 }
 
-// DEPTH = (tile, group) items whose bytes are on their way while one is multiplied (1, 2 or 4; it divides the number of groups).
-template <int DEPTH>
+__global__ void clear_rows(float4* out, uint64_t count4) {
+    const uint64_t i = uint64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < count4) out[i] = float4{0, 0, 0, 0};
+}
+
+// DEPTH = (tile, group) items whose bytes are on their way while one is multiplied (1, 2 or 4; it divides the number of groups
+// of a workgroup). ROWS = token rows staged (8: all of K per workgroup; 16: half of K per workgroup, sums added into y).
+template <int DEPTH, int ROWS>
 __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
+    constexpr int kRows = ROWS;
+    constexpr uint32_t KSPLIT = ROWS / 8;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [hi plane][lo plane][8 weight tiles]
     __shared__ float wave_max[kWaves];
     __shared__ uint32_t next_tile;
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const uint32_t col = lane % 32, khalf = lane / 32;
-    const uint32_t K = a.columns, chunks = K / 8, groups = K / 256, row_bytes = K / 32 * 34;
-    if (tid == 0) next_tile = uint32_t(uint64_t((a.rows + 31) / 32) * blockIdx.x / gridDim.x);
+    // K: the columns this workgroup multiplies, starting at column k0 (group g0 of the rows)
+    const uint32_t K = a.columns / KSPLIT, chunks = K / 8, groups = K / 256, row_bytes = a.columns / 32 * 34;
+    const uint32_t k0 = (blockIdx.x % KSPLIT) * K, g0 = k0 / 256;
+    const uint32_t sharer = blockIdx.x / KSPLIT, sharers = gridDim.x / KSPLIT;  // the host launches a multiple of KSPLIT
+    if (tid == 0) next_tile = uint32_t(uint64_t((a.rows + 31) / 32) * sharer / sharers);
     _Float16* const a_hi = reinterpret_cast<_Float16*>(lds);
     _Float16* const a_lo = a_hi + kRows * K;
     uint8_t* const tile = lds + 2 * kRows * K * 2 + wave * kTileBytes;
@@ -69,7 +84,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     uint32_t bad = 0;
     float biggest = 0;
     for (uint32_t i = tid; i < a.m * (K / 4); i += kThreads) {
-        const float4 v = reinterpret_cast<const float4*>(a.x)[i];
+        const float4 v = *reinterpret_cast<const float4*>(a.x + uint64_t(i / (K / 4)) * a.columns + k0 + (i % (K / 4)) * 4);
         if (nonfinite(v.x) || nonfinite(v.y) || nonfinite(v.z) || nonfinite(v.w)) bad = TSP_ERRBIT_NONFINITE;
         biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
     }
@@ -92,7 +107,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
         const uint32_t r = i / chunks, c = i % chunks;
         f16x8 hi{}, lo{};
         if (r < a.m) {
-            const float4* src = reinterpret_cast<const float4*>(a.x + uint64_t(r) * K + c * 8);
+            const float4* src = reinterpret_cast<const float4*>(a.x + uint64_t(r) * a.columns + k0 + c * 8);
             const float4 v0 = src[0], v1 = src[1];
             const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
@@ -108,7 +123,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     }
     __syncthreads();
 
-    const uint32_t arow = col & 7;
+    const uint32_t arow = col & (kRows - 1);
     auto a_frag = [&](const _Float16* plane, uint32_t chunk) {
         return *reinterpret_cast<const f16x8*>(plane + (arow * chunks + (chunk ^ arow)) * 8);
     };
@@ -122,7 +137,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
             id = id < 32 * kGroupChunks ? id : 32 * kGroupChunks - 1;  // the tail lanes repeat the last chunk
             uint32_t row = row0 + id / kGroupChunks;
             row = row < a.rows ? row : a.rows - 1;
-            const uint4 v = *reinterpret_cast<const uint4*>(a.matrix + uint64_t(row) * row_bytes + group * kGroupBytes + (id % kGroupChunks) * 16);
+            const uint4 v = *reinterpret_cast<const uint4*>(a.matrix + uint64_t(row) * row_bytes + (g0 + group) * kGroupBytes + (id % kGroupChunks) * 16);
             stage[SET][t][0] = uint2{v.x, v.y};
             stage[SET][t][1] = uint2{v.z, v.w};
         }
@@ -143,7 +158,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     // a counter in LDS (which wave computes a tile does not change the result). The bytes of the next (tile, group) item
     // are requested before the current one is multiplied, so a wave always holds its next tile index one step ahead.
     const uint32_t tiles = (a.rows + 31) / 32;
-    const uint32_t share_end = uint32_t(uint64_t(tiles) * (blockIdx.x + 1) / gridDim.x);
+    const uint32_t share_end = uint32_t(uint64_t(tiles) * (sharer + 1) / sharers);
     auto take_tile = [&]() {
         uint32_t t = 0;
         if (lane == 0) t = atomicAdd(&next_tile, 1u);
@@ -200,7 +215,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
                 part_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag(a_hi, chunk + 1), b1, part_hi, 0, 0, 0);
                 part_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag(a_lo, chunk + 1), b1, part_lo, 0, 0, 0);
 #pragma unroll
-                for (int v = 0; v < 4; ++v) acc[v] = __builtin_fmaf(scale_d, part_hi[v] + part_lo[v], acc[v]);  // rows 4 * khalf + v
+                for (int v = 0; v < kRows / 2; ++v) acc[v] = __builtin_fmaf(scale_d, part_hi[v] + part_lo[v], acc[v]);  // rows 8 * (v / 4) + 4 * khalf + v % 4
             };
             block(std::integral_constant<int, 0>{});
             block(std::integral_constant<int, 1>{});
@@ -221,12 +236,13 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
         }
         const uint32_t r = row0 + col;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const uint32_t m = 4 * khalf + v;
+        for (int v = 0; v < kRows / 2; ++v) {
+            const uint32_t m = 8 * (v / 4) + 4 * khalf + v % 4;
             if (m < a.m && r < a.rows) {
                 const float val = acc[v] * inv_scale;
                 if (nonfinite(val)) bad = TSP_ERRBIT_NONFINITE;
-                a.y[uint64_t(m) * a.rows + r] = val;
+                if constexpr (KSPLIT == 1) a.y[uint64_t(m) * a.rows + r] = val;
+                else unsafeAtomicAdd(a.y + uint64_t(m) * a.rows + r, val);
             }
         }
     }
@@ -242,16 +258,22 @@ bool q8_mfma_supported(const void* matrix, const float* x, uint32_t columns, uin
            reinterpret_cast<uintptr_t>(x) % 16 == 0;
 }
 
+bool q8_mfma_supported_16(const void* matrix, const float* x, const float* y, uint32_t columns, uint32_t rows) {
+    return q8_mfma_supported(matrix, x, columns, rows) && columns % 1024 == 0 && rows >= 64 && rows % 4 == 0 &&
+           reinterpret_cast<uintptr_t>(y) % 16 == 0;
+}
+
 int q8_mfma(const void* matrix, const float* x, float* y, uint32_t columns, uint32_t rows, uint32_t width, uint32_t* error_word, hipStream_t s) {
     const Q8MfmaArgs a{static_cast<const uint8_t*>(matrix), x, y, columns, rows, width, error_word};
-    const uint32_t lds_bytes = 2 * kRows * columns * 2 + kWaves * kTileBytes;
+    // 8 rows x all columns and 16 rows x half the columns stage the same number of bytes
+    const uint32_t lds_bytes = 2 * 8 * columns * 2 + kWaves * kTileBytes;
     static bool raised = false;
     static int compute_units = 0;
     if (!raised) {
-        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    int(2 * kRows * 2048 * 2 + kWaves * kTileBytes)));
-        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    int(2 * kRows * 2048 * 2 + kWaves * kTileBytes)));
+        const int most = int(2 * 8 * 2048 * 2 + kWaves * kTileBytes);
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<1, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<2, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<2, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
         int device = 0;
         TSP_HIP(hipGetDevice(&device));
         TSP_HIP(hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device));
@@ -259,10 +281,19 @@ int q8_mfma(const void* matrix, const float* x, float* y, uint32_t columns, uint
     }
     const uint32_t tiles = (rows + 31) / 32;
     uint32_t grid = uint32_t(compute_units > 0 ? compute_units : 256);
+    if (width > 8) {
+        // two workgroups (one per half of the columns) share each run of tiles; the output starts at zero
+        uint32_t pairs = grid / 2 ? grid / 2 : 1;
+        if (pairs * kWaves > tiles) pairs = (tiles + kWaves - 1) / kWaves;
+        const uint64_t count4 = uint64_t(width) * rows / 4;
+        TSP_LAUNCH("clear_rows", s, clear_rows<<<uint32_t((count4 + 255) / 256), 256, 0, s>>>(reinterpret_cast<float4*>(y), count4));
+        TSP_LAUNCH("q8_mfma", s, q8_mfma_kernel<2, 16><<<2 * pairs, kThreads, lds_bytes, s>>>(a));
+        return launch_status("q8_mfma");
+    }
     if (grid * kWaves > tiles) grid = (tiles + kWaves - 1) / kWaves;
     // two items in flight measured best on MI355X (one: 72 us, two: 69 us, four: 75 us at 151 936 x 2048)
-    if ((columns / 256) % 2 == 0) TSP_LAUNCH("q8_mfma", s, q8_mfma_kernel<2><<<grid, kThreads, lds_bytes, s>>>(a));
-    else TSP_LAUNCH("q8_mfma", s, q8_mfma_kernel<1><<<grid, kThreads, lds_bytes, s>>>(a));
+    if ((columns / 256) % 2 == 0) TSP_LAUNCH("q8_mfma", s, q8_mfma_kernel<2, 8><<<grid, kThreads, lds_bytes, s>>>(a));
+    else TSP_LAUNCH("q8_mfma", s, q8_mfma_kernel<1, 8><<<grid, kThreads, lds_bytes, s>>>(a));
     return launch_status("q8_mfma");
 }
 
