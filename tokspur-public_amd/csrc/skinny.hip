@@ -57,7 +57,8 @@ __device__ __forceinline__ bool load_task(const SkinnyArgs& a, uint32_t index, T
         for (int k = 0; k < kRows; ++k) t.src[k] = t.dst[k] = k;
         return index == 0;
     } else if (a.meta) {
-        if (index >= a.meta[6]) return false;
+        // every word is read before the record count is looked at (index < 128 always lies inside the block): one round trip, not two
+        const uint32_t live = a.meta[6];
         t.expert = a.meta[8 + index];
         t.count = a.meta[136 + index];
 #pragma unroll
@@ -66,7 +67,7 @@ __device__ __forceinline__ bool load_task(const SkinnyArgs& a, uint32_t index, T
             t.src[k] = SRC == SRC_RECORD_TOKENS ? token : route;
             t.dst[k] = route;
         }
-        return true;
+        return index < live;
     } else {
         if (index >= a.tokens * a.selected) return false;
         t.expert = a.ids[index];
@@ -358,6 +359,292 @@ __global__ __launch_bounds__(256 * KS, 2) void skinny_kernel(SkinnyArgs a) {
     publish_error(bad, a.error_word);
 }
 
+// ---------------------------------------------------------------- one super-block per wave
+// When a row has 1, 2, 4 or 8 super-blocks, a wave takes ONE super-block (256 columns) of 64 weight rows and nothing is
+// looped: its weight bytes are requested first, and while they travel the wave stages its own 256 columns of the
+// activation rows in a private corner of LDS (its own power-of-two scale: the partial sums are brought back to true
+// units before they meet), so no wave waits for another until the slices of a unit column add up at the end, in slice
+// order. A workgroup is the slices of one unit column (four or more waves: more unit columns when a row has fewer than
+// four super-blocks). Many short waves with every load in flight from the first instruction fill the chip better than
+// a few long pipelines here: these products move ~1 MB per expert and have about one expert per three compute units.
+constexpr uint32_t kSlice = 256;                                       // columns per wave
+constexpr uint32_t kWaveLds = 2 * kRows * kSlice * 2 + kRows * 32;      // hi plane, lo plane, sub-block sums: 8 448 B
+
+template <int BKIND, int OUT, int SRC>
+__global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs a) {  // four waves per SIMD: <= 128 registers per lane
+    constexpr bool Q6 = BKIND == B_Q6K_PLANAR;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [wave][hi plane][lo plane][sums]; partial sums over it at the end
+
+    const uint32_t tid = threadIdx.x, lane = tid % kWave, wv = tid / kWave;
+    const uint32_t col = lane % 32, khalf = lane / 32;
+    const uint32_t bpr = a.k / 256, ucols = blockDim.x / kWave / bpr;  // the host launches ucols * bpr waves
+    const uint32_t slice = wv % bpr, ucol = wv / bpr;
+    Task task;
+    if (!load_task<SRC>(a, blockIdx.y, task)) return;
+    if (task.expert >= a.experts || task.count == 0 || task.count > kRows) {
+        if (tid == 0 && blockIdx.x == 0 && (task.expert >= a.experts || task.count > kRows)) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+        return;
+    }
+
+    // ---- this wave's 256 columns of the activation rows (lane l: columns 4l .. 4l+3 of each row), requested first: loads
+    // come back in the order they were asked for, and these few cached bytes must not queue behind the weight bytes
+    uint32_t bad = 0;
+    float4 v[kRows];
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+        const uint32_t from = uint32_t(r) < task.count ? task.src[r] : task.src[0];  // uniform; a dead row re-reads row 0 and is zeroed
+        v[r] = *reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.x) + uint64_t(from) * a.x_stride + (slice * kSlice + lane * 4) * 4);
+    }
+
+    // ---- weight rows of this wave, and their bytes: requested before any arithmetic
+    const uint8_t* wbase[2];
+    uint32_t wrow[2], out_col[2];
+    bool col_live[2];
+    if constexpr (OUT == OUT_SWIGLU) {
+        const uint32_t unit = (blockIdx.x * ucols + ucol) * 32 + col;
+        const uint32_t half_e = a.experts / 2;
+        const uint8_t* pair = (task.expert < half_e ? a.w0 : a.w1) + uint64_t(task.expert < half_e ? task.expert : task.expert - half_e) * 2 * a.spec.planar_expert_bytes;
+        wbase[0] = pair; wbase[1] = pair + a.spec.planar_expert_bytes;
+        col_live[0] = col_live[1] = unit < a.n;
+        wrow[0] = wrow[1] = col_live[0] ? unit : a.n - 1;
+        out_col[0] = out_col[1] = unit;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t n = (blockIdx.x * ucols + ucol) * 64 + j * 32 + col;
+            col_live[j] = n < a.n;
+            wrow[j] = col_live[j] ? n : a.n - 1;
+            out_col[j] = n;
+            wbase[j] = a.w0 + uint64_t(task.expert) * a.spec.planar_expert_bytes;
+        }
+    }
+    struct BlockQ6 { u32x4 la[2], lb[2], qh[2]; uint32_t sc[4]; float d; };
+    struct BlockQ4 { u32x4 pair[4]; HdrQ4 hdr; };
+    using Block = std::conditional_t<Q6, BlockQ6, BlockQ4>;
+    Block cur[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint64_t at = uint64_t(wrow[j]) * bpr + slice;
+        if constexpr (Q6) {
+            const uint8_t* ql = wbase[j] + a.spec.qs_offset + at * 128 + khalf * 16;
+            const uint8_t* qh = wbase[j] + a.spec.qh_offset + at * 64 + khalf * 16;
+#pragma unroll
+            for (int sec = 0; sec < 2; ++sec) {
+                cur[j].la[sec] = *reinterpret_cast<const u32x4*>(ql + sec * 64);
+                cur[j].lb[sec] = *reinterpret_cast<const u32x4*>(ql + sec * 64 + 32);
+                cur[j].qh[sec] = *reinterpret_cast<const u32x4*>(qh + sec * 32);
+            }
+            const uint4 sc16 = *reinterpret_cast<const uint4*>(wbase[j] + a.spec.sm_offset + at * 16);
+            cur[j].sc[0] = sc16.x; cur[j].sc[1] = sc16.y; cur[j].sc[2] = sc16.z; cur[j].sc[3] = sc16.w;
+            cur[j].d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(wbase[j] + a.spec.dm_offset + at * 2));
+        } else {
+            constexpr uint32_t BLK = BKIND == B_Q4K_PLANAR ? 128 : 144, QS_AT = BKIND == B_Q4K_PLANAR ? 0 : 16;
+            const uint8_t* qs = wbase[j] + (BKIND == B_Q4K_PLANAR ? a.spec.qs_offset : 0) + at * BLK + QS_AT + khalf * 16;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) cur[j].pair[p] = *reinterpret_cast<const u32x4*>(qs + p * 32);
+            cur[j].hdr = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, slice);
+        }
+    }
+
+    __builtin_amdgcn_sched_barrier(0);  // every request above is out before the first wait below
+
+    // ---- stage the activation rows while the weight bytes travel
+    uint8_t* const mine = lds + wv * kWaveLds;
+    _Float16* const a_hi = reinterpret_cast<_Float16*>(mine);
+    _Float16* const a_lo = a_hi + kRows * kSlice;
+    _Float16* const sums = a_lo + kRows * kSlice;  // [row][8 hi, 8 lo] of (sub-block sum / 32), Q4_K only
+    float biggest = 0;
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+        if (uint32_t(r) >= task.count) v[r] = float4{0, 0, 0, 0};
+        if (nonfinite(v[r].x) || nonfinite(v[r].y) || nonfinite(v[r].z) || nonfinite(v[r].w)) bad = TSP_ERRBIT_NONFINITE;
+        biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v[r].x), fabsf(v[r].y)), fmaxf(fabsf(v[r].z), fabsf(v[r].w))));
+    }
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1) biggest = fmaxf(biggest, __shfl_xor(biggest, step, kWave));
+    // scale = 2^(13 - exponent(biggest)): the largest |x * scale| is below 2^15, the sub-block sums / 32 below 2^15 too
+    float scale = 1.0f, inv_scale = 1.0f;
+    if (biggest > 0 && !nonfinite(biggest)) {
+        const int e = int((__float_as_uint(biggest) >> 23) & 0xffu) - 127;
+        int shift = 13 - e;
+        shift = shift > 100 ? 100 : shift < -100 ? -100 : shift;
+        scale = __uint_as_float(uint32_t(127 + shift) << 23);
+        inv_scale = __uint_as_float(uint32_t(127 - shift) << 23);
+    }
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+        const float s4[4] = {v[r].x * scale, v[r].y * scale, v[r].z * scale, v[r].w * scale};
+        f16x4 hi, lo;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            hi[e] = _Float16(s4[e]);
+            lo[e] = _Float16(s4[e] - float(hi[e]));
+        }
+        // 16-byte chunk c = l / 2 of row r sits at position c ^ r; this lane owns half of it
+        const uint32_t at = (r * 32 + ((lane / 2) ^ r)) * 8 + (lane % 2) * 4;
+        *reinterpret_cast<f16x4*>(a_hi + at) = hi;
+        *reinterpret_cast<f16x4*>(a_lo + at) = lo;
+        if constexpr (!Q6) {
+            float sum = (s4[0] + s4[1]) + (s4[2] + s4[3]);  // eight neighbouring lanes hold one 32-column sub-block
+            sum += __shfl_xor(sum, 1, kWave);
+            sum += __shfl_xor(sum, 2, kWave);
+            sum += __shfl_xor(sum, 4, kWave);
+            if (lane % 8 == 0) {
+                const float s32 = sum * 0.03125f;
+                const _Float16 h = _Float16(s32);
+                sums[r * 16 + lane / 8] = h;
+                sums[r * 16 + 8 + lane / 8] = _Float16(s32 - float(h));
+            }
+        }
+    }
+    // the planes are read back by other lanes of this same wave only: LDS serves a wave's requests in order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    f32x16 blk[2];
+    float acc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};  // rows 4 * khalf + v of tile j
+    const uint32_t arow = col & 7;
+    auto a_frag = [&](const _Float16* plane, uint32_t chunk) {
+        return *reinterpret_cast<const f16x8*>(plane + (arow * 32 + (chunk ^ arow)) * 8);
+    };
+    auto mfma = [&](uint32_t chunk, const f16x8& b0, const f16x8& b1, bool first) {
+        const f16x8 ah = a_frag(a_hi, chunk), al = a_frag(a_lo, chunk);
+        if (first) {
+            const f32x16 zero{};
+            blk[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b0, zero, 0, 0, 0);
+            blk[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b1, zero, 0, 0, 0);
+        } else {
+            blk[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b0, blk[0], 0, 0, 0);
+            blk[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b1, blk[1], 0, 0, 0);
+        }
+        blk[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b0, blk[0], 0, 0, 0);
+        blk[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b1, blk[1], 0, 0, 0);
+    };
+    auto fold = [&](float d0, float d1) {
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) {
+            acc[0][v4] = __builtin_fmaf(d0, blk[0][v4], acc[0][v4]);
+            acc[1][v4] = __builtin_fmaf(d1, blk[1][v4], acc[1][v4]);
+        }
+    };
+    if constexpr (Q6) {
+        auto section = [&](auto sec_tag) {
+            constexpr int SEC = decltype(sec_tag)::value;
+            RawQ6 raw[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                raw[j].la = cur[j].la[SEC]; raw[j].lb = cur[j].lb[SEC]; raw[j].qh = cur[j].qh[SEC];
+                raw[j].sc[0] = cur[j].sc[SEC * 2]; raw[j].sc[1] = cur[j].sc[SEC * 2 + 1];
+            }
+            auto quarter = [&](auto q_tag) {
+                constexpr int Q = decltype(q_tag)::value;
+                f16x8 f0[2], f1[2];
+                frags_q6k<Q>(raw[0], khalf, f0);
+                frags_q6k<Q>(raw[1], khalf, f1);
+                const uint32_t chunk = SEC * 16 + Q * 4 + khalf * 2;  // columns SEC*128 + Q*32 + 16h of the slice
+                mfma(chunk, f0[0], f1[0], SEC == 0 && Q == 0);
+                mfma(chunk + 1, f0[1], f1[1], false);
+            };
+            quarter(std::integral_constant<int, 0>{});
+            quarter(std::integral_constant<int, 1>{});
+            quarter(std::integral_constant<int, 2>{});
+            quarter(std::integral_constant<int, 3>{});
+        };
+        section(std::integral_constant<int, 0>{});
+        section(std::integral_constant<int, 1>{});
+        fold(cur[0].d, cur[1].d);
+    } else {
+        auto pair_step = [&](auto p_tag) {
+            constexpr int P = decltype(p_tag)::value;
+            f16x8 f0[2], f1[2];
+            const uint32_t chunk = P * 8 + khalf * 2;  // columns P*64 + 16h of the slice
+            frags_q4k<P, 0>(cur[0].pair[P], cur[0].hdr, f0);
+            frags_q4k<P, 0>(cur[1].pair[P], cur[1].hdr, f1);
+            mfma(chunk, f0[0], f1[0], P == 0);
+            mfma(chunk + 1, f0[1], f1[1], false);
+            frags_q4k<P, 1>(cur[0].pair[P], cur[0].hdr, f0);
+            frags_q4k<P, 1>(cur[1].pair[P], cur[1].hdr, f1);
+            mfma(chunk + 4, f0[0], f1[0], false);
+            mfma(chunk + 5, f0[1], f1[1], false);
+        };
+        pair_step(std::integral_constant<int, 0>{});
+        pair_step(std::integral_constant<int, 1>{});
+        pair_step(std::integral_constant<int, 2>{});
+        pair_step(std::integral_constant<int, 3>{});
+        fold(cur[0].hdr.d, cur[1].hdr.d);
+        // minima: acc -= 32 * dmin * sum_s (Sx / 32)(hi + lo)[m, s] * mn[n, s]
+        const f16x8 m0 = minima_frag(cur[0].hdr), m1 = minima_frag(cur[1].hdr);
+        const f16x8 sf = *reinterpret_cast<const f16x8*>(sums + arow * 16 + khalf * 8);
+        const f32x16 zero{};
+        blk[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m0, zero, 0, 0, 0);
+        blk[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m1, zero, 0, 0, 0);
+        fold(-32.0f * cur[0].hdr.dmin, -32.0f * cur[1].hdr.dmin);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) acc[j][v4] *= inv_scale;  // exact: a power of two
+
+    // ---- the slices of a unit column meet in LDS, added in slice order; the planes are free once every wave is here
+    if (bpr > 1) {
+        float* const partial = reinterpret_cast<float*>(lds);  // [slice - 1][unit column][tile][v][lane]
+        __syncthreads();
+        if (slice > 0) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4) partial[((((slice - 1) * ucols + ucol) * 2 + j) * 4 + v4) * kWave + lane] = acc[j][v4];
+        }
+        __syncthreads();
+        if (slice > 0) { publish_error(bad, a.error_word); return; }
+        for (uint32_t s = 1; s < bpr; ++s)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4) acc[j][v4] += partial[((((s - 1) * ucols + ucol) * 2 + j) * 4 + v4) * kWave + lane];
+    }
+    // ---- epilogue: accumulator v of tile j is row 4 * khalf + v, weight row `col`
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+        const uint32_t r = 4 * khalf + v4;
+        if (r >= task.count) continue;
+        const uint32_t dst = khalf ? task.dst[4 + v4] : task.dst[v4];
+        uint8_t* orow = reinterpret_cast<uint8_t*>(a.out) + uint64_t(dst) * a.out_stride;
+        if constexpr (OUT == OUT_SWIGLU) {
+            if (!col_live[0]) continue;
+            const float g = acc[0][v4], u = acc[1][v4];
+            const float sg = g >= 0 ? 1.0f / (1.0f + expf(-g)) : expf(g) / (1.0f + expf(g));
+            const float h = (g * sg) * u;
+            if (nonfinite(g) || nonfinite(u) || nonfinite(h)) bad = TSP_ERRBIT_NONFINITE;
+            reinterpret_cast<float*>(orow)[out_col[0]] = h;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (!col_live[j]) continue;
+                const float val = acc[j][v4];
+                if (nonfinite(val)) bad = TSP_ERRBIT_NONFINITE;
+                reinterpret_cast<float*>(orow)[out_col[j]] = val;
+            }
+        }
+    }
+    publish_error(bad, a.error_word);
+}
+
+template <int BKIND, int OUT, int SRC>
+int launch_flat(const char* name, const SkinnyArgs& a, uint32_t tasks, hipStream_t s) {
+    const uint32_t bpr = a.k / 256, waves = bpr < 4 ? 4 : bpr, ucols = waves / bpr;
+    const uint32_t per_group = ucols * (OUT == OUT_SWIGLU ? 32 : 64), col_tiles = (a.n + per_group - 1) / per_group;
+    static bool raised = false;
+    if (!raised) {
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&flat_kernel<BKIND, OUT, SRC>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    int(8 * kWaveLds)));
+        raised = true;
+    }
+    TSP_LAUNCH(name, s, flat_kernel<BKIND, OUT, SRC><<<dim3(col_tiles, tasks), waves * kWave, waves * kWaveLds, s>>>(a));
+    return launch_status(name);
+}
+
 uint32_t lds_bytes(uint32_t columns, bool sums) { return 2 * kRows * columns * 2 + (sums ? kRows * (columns / 256) * 32 : 0); }
 
 template <int BKIND, int OUT, int SRC, int KS>
@@ -376,6 +663,8 @@ int launch_sliced(const char* name, const SkinnyArgs& a, uint32_t col_tiles, uin
 // Two K slices whenever the super-blocks split evenly: the task tiles of these products number about one per compute unit.
 template <int BKIND, int OUT, int SRC>
 int launch(const char* name, const SkinnyArgs& a, uint32_t col_tiles, uint32_t tasks, hipStream_t s) {
+    const uint32_t bpr = a.k / 256;
+    if (bpr == 1 || bpr == 2 || bpr == 4 || bpr == 8) return launch_flat<BKIND, OUT, SRC>(name, a, tasks, s);
     if ((a.k / 256) % 2 == 0) return launch_sliced<BKIND, OUT, SRC, 2>(name, a, col_tiles, tasks, s);
     return launch_sliced<BKIND, OUT, SRC, 1>(name, a, col_tiles, tasks, s);
 }
