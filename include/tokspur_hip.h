@@ -183,6 +183,16 @@ int tsp_q8_matvec_many(uint32_t layout, const void* matrix, uint64_t matrix_byte
 int tsp_dense_mm_q8(uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* input, uint64_t input_stride_bytes,
                     float* output, uint64_t output_stride_bytes, uint32_t tokens, uint32_t columns, uint32_t rows,
                     uint32_t* error_word, void* stream);
+/* The same product for many token rows at once (a prefill chunk's shared expert), where one pass over the matrix per
+ * sixteen rows no longer pays: the matrix is decoded once into halves (d * q rounded to nearest, as the engine's kernel
+ * stages them, kernels/grouped_mm.metal:239-243), the rows are rounded to halves, and a matrix-core GEMM with f32
+ * accumulation multiplies them. Columns in multiples of 64; `workspace` (16-byte aligned, at least
+ * tsp_dense_mm_q8_workspace_bytes) is scratch for the call and must not overlap the other buffers. Results agree with
+ * tsp_dense_mm_q8 to the GEMM tolerance (2e-3 of the row scale), not bit for bit. */
+uint64_t tsp_dense_mm_q8_workspace_bytes(uint32_t tokens, uint32_t columns, uint32_t rows);
+int tsp_dense_mm_q8_staged(uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* input, uint64_t input_stride_bytes,
+                           float* output, uint64_t output_stride_bytes, uint32_t tokens, uint32_t columns, uint32_t rows,
+                           void* workspace, uint64_t workspace_bytes, uint32_t* error_word, void* stream);
 /* include/tokspur/graph.hpp:1093 `routed_gemv` (kernels/gemv.metal:198-227): per selected expert s,
  * y[s, :] = W[ids[s]] * x (x broadcast, or one x row per route). Raw GGUF expert stacks. */
 int tsp_routed_gemv(uint32_t encoding, const void* matrices, uint64_t matrices_bytes, const uint32_t* ids, const float* x,

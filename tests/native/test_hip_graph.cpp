@@ -234,6 +234,39 @@ void test_dense_mm_q8_layouts() {
         EXPECT(scaled_error(row0, want) <= 5e-5 && scaled_error(row1, want) <= 5e-5);
         for (uint32_t pad = R; pad < R + 4; ++pad) EXPECT(got0[size_t(m) * (R + 4) + pad] == -7.0f && got1[size_t(m) * (R + 4) + pad] == -7.0f);
     }
+    // prepared with bounds, 32 rows or more go through the staged form (halves on the matrix cores): same values to the GEMM
+    // tolerance, same canaries, and the scratch is charged to the graph's budget (it grows when prepared again with wider bounds)
+    const uint32_t M2 = 45;
+    const auto x2 = lcg_floats(22, size_t(M2) * (K + 8));
+    const GpuView dx2 = g.upload(bytes_of(x2), "x2", false);
+    const std::vector<float> canary2(size_t(M2) * (R + 4), -7.0f);
+    const GpuView y2 = g.upload(bytes_of(canary2), "y2", false), y3 = g.upload(bytes_of(canary2), "y3", false);
+    const uint64_t before = g.memory().live_bytes;
+    g.prepare_dense_mm_q8(PrefillWeightLayout::gguf, 32, K, R);
+    const uint64_t small = g.memory().live_bytes - before;
+    EXPECT(small == tsp_dense_mm_q8_workspace_bytes(32, K, R));
+    g.prepare_dense_mm_q8(PrefillWeightLayout::gguf, M2, K, R);
+    EXPECT(g.memory().live_bytes - before == tsp_dense_mm_q8_workspace_bytes(M2, K, R));
+    EXPECT(throws_format([&] { g.prepare_dense_mm_q8(PrefillWeightLayout::gguf, 0, K, R); }));
+    const GpuRowsF32 in2{dx2, M2, K, uint64_t(K + 8) * 4};
+    g.begin();
+    g.dense_mm_q8(PrefillWeightLayout::gguf, dw, in2, {y2, M2, R, uint64_t(R + 4) * 4});
+    g.dense_mm_q8(PrefillWeightLayout::q8_lanes_v1, dl, in2, {y3, M2, R, uint64_t(R + 4) * 4});
+    (void)g.submit();
+    const auto got2 = read_as<float>(g, y2), got3 = read_as<float>(g, y3);
+    for (uint32_t m = 0; m < M2; ++m) {
+        std::vector<double> want(R);
+        orc_reference_gemv(8, w.data(), w.size(), K, R, x2.data() + size_t(m) * (K + 8), K, want.data());
+        double scale = 1, worst = 0;  // the GEMM tolerance: 2e-3 of the row's largest magnitude
+        for (double v : want) scale = std::max(scale, std::fabs(v));
+        for (uint32_t r = 0; r < R; ++r) {
+            worst = std::max(worst, std::fabs(double(got2[size_t(m) * (R + 4) + r]) - want[r]) / scale);
+            worst = std::max(worst, std::fabs(double(got3[size_t(m) * (R + 4) + r]) - want[r]) / scale);
+        }
+        if (m == 0) std::printf("dense_mm_q8 staged: row 0 max error / row max %.3e\n", worst);
+        EXPECT(worst <= 2e-3);
+        for (uint32_t pad = R; pad < R + 4; ++pad) EXPECT(got2[size_t(m) * (R + 4) + pad] == -7.0f && got3[size_t(m) * (R + 4) + pad] == -7.0f);
+    }
 }
 
 void test_encode_moe_single_token() {

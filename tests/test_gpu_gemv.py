@@ -238,6 +238,41 @@ def test_dense_mm_q8(gpu, tsp, orc, synth, tokens, cols, rows):
         tsp.dense_mm_q8(gpu, tsp.LAYOUT_PLANAR_V3, gpu.upload(w), gpu.upload(x), tokens, cols, rows, x_stride=(cols + 4) * 4)
 
 
+@pytest.mark.parametrize("tokens,cols,rows", [(1, 64, 5), (70, 128, 33), (200, 2048, 512), (129, 512, 2048), (64, 4096, 64)])
+def test_dense_mm_q8_staged(gpu, tsp, orc, synth, tokens, cols, rows):
+    # the many-row form of graph.hpp:860 `dense_mm_q8`: matrix and rows as halves, one matrix-core GEMM. Both layouts, rows with
+    # padding on both sides (canaries stay), tiles that overhang the matrix on either edge, and agreement with the streaming
+    # entry point.
+    w = synth.matrix(8, 1900 + cols, rows, cols)
+    lanes = tsp.q8_lanes_pack_rows(cols, w)
+    x = synth.activations_f32(1901 + tokens, (tokens, cols + 4))
+    sample = np.unique(np.linspace(0, tokens - 1, min(tokens, 24)).astype(int))
+    want = np.stack([orc.reference_gemv(8, w, cols, rows, x[t, :cols]) for t in sample])
+    scale = np.maximum(1.0, np.sqrt((want ** 2).mean(axis=1, keepdims=True)))
+    streamed = tsp.dense_mm_q8(gpu, tsp.LAYOUT_GGUF, gpu.upload(w), gpu.upload(np.ascontiguousarray(x[:, :cols])), tokens, cols, rows).cpu().numpy()
+    for matrix, layout in ((w, tsp.LAYOUT_GGUF), (lanes, tsp.LAYOUT_Q8_LANES_V1)):
+        out = gpu.full((tokens, rows + 3), -5.0)
+        tsp.dense_mm_q8_staged(gpu, layout, gpu.upload(matrix), gpu.upload(x), tokens, cols, rows, out=out, x_stride=(cols + 4) * 4,
+                               out_stride=(rows + 3) * 4)
+        got = out.cpu().numpy()
+        assert gpu.error() == 0 and (got[:, rows:] == -5.0).all()
+        assert float(np.max(np.abs(got[sample, :rows] - want) / np.maximum(scale, np.abs(want)))) <= 2e-3  # the GEMM tolerance
+        row_scale = np.maximum(1.0, np.sqrt((streamed ** 2).mean(axis=1, keepdims=True)))
+        assert float(np.max(np.abs(got[:, :rows] - streamed) / np.maximum(row_scale, np.abs(streamed)))) <= 2e-3
+        nmse = float(((got[:, :rows] - streamed) ** 2).sum() / max((streamed ** 2).sum(), 1e-30))
+        assert nmse <= 1e-6, nmse
+    with pytest.raises(tsp.FormatError):  # columns not a multiple of 64
+        tsp.dense_mm_q8_staged(gpu, tsp.LAYOUT_GGUF, gpu.upload(synth.matrix(8, 3, 4, 96)), gpu.zeros((2, 96)), 2, 96, 4)
+    with pytest.raises(tsp.FormatError):  # workspace too small
+        tsp.dense_mm_q8_staged(gpu, tsp.LAYOUT_GGUF, gpu.upload(w), gpu.upload(x), tokens, cols, rows, x_stride=(cols + 4) * 4,
+                               workspace=gpu.empty(256, "uint8"))
+    x_bad = np.ascontiguousarray(x[:, :cols]).copy()
+    x_bad[tokens // 2, cols // 2] = np.inf
+    tsp.dense_mm_q8_staged(gpu, tsp.LAYOUT_GGUF, gpu.upload(w), gpu.upload(x_bad), tokens, cols, rows)
+    assert gpu.error() & tsp.ERRBIT_NONFINITE
+    gpu.clear_error()
+
+
 @pytest.mark.parametrize("width", [1, 2, 4, 8])
 @pytest.mark.parametrize("cols,rows", [(2048, 37), (64, 5), (96, 7), (4096, 9)])
 def test_q8_matvec_many(gpu, tsp, orc, synth, width, cols, rows):

@@ -398,6 +398,19 @@ def dense_mm_q8(dev, layout, matrix, x, tokens, columns, rows, out=None, x_strid
     return out
 
 
+def dense_mm_q8_staged(dev, layout, matrix, x, tokens, columns, rows, out=None, x_stride=None, out_stride=None, workspace=None):
+    """Dense Q8_0 GEMM for many rows: matrix and rows staged as halves in `workspace`, one matrix-core GEMM."""
+    f = dll().tsp_dense_mm_q8_workspace_bytes
+    f.restype = C.c_uint64
+    out = dev.empty((tokens, rows)) if out is None else out
+    workspace = dev.empty(f(C.c_uint32(tokens), C.c_uint32(columns), C.c_uint32(rows)), "uint8") if workspace is None else workspace
+    check(dll().tsp_dense_mm_q8_staged(C.c_uint32(layout), dev.ptr(matrix), C.c_uint64(dev.nbytes(matrix)), dev.ptr(x),
+                                       C.c_uint64(columns * 4 if x_stride is None else x_stride), dev.ptr(out),
+                                       C.c_uint64(rows * 4 if out_stride is None else out_stride), C.c_uint32(tokens), C.c_uint32(columns),
+                                       C.c_uint32(rows), dev.ptr(workspace), C.c_uint64(dev.nbytes(workspace)), dev.ptr(dev.err), dev.stream()))
+    return out
+
+
 def dense_mm_workspace_bytes(tokens, columns):
     f = dll().tsp_dense_mm_workspace_bytes
     f.restype = C.c_uint64

@@ -68,6 +68,8 @@ struct HipGraph::Impl {
     uint64_t dense_workspace_bytes = 0;
     void* grouped_workspace = nullptr;
     uint64_t grouped_workspace_bytes = 0;
+    void* q8_workspace = nullptr;
+    uint64_t q8_workspace_bytes = 0;
     uint32_t prepared_gate_up = 0, prepared_down = 0;
 
     void same_thread() const { require(std::this_thread::get_id() == thread, "GPU graph used from another thread"); }
@@ -142,7 +144,7 @@ HipGraph::~HipGraph() {
     (void)hipStreamSynchronize(impl_->stream);
     for (auto& a : impl_->slots)
         if (a.live) (void)hipFree(a.device);
-    for (void* p : {impl_->union_meta, impl_->nax_workspace, impl_->dense_workspace, impl_->grouped_workspace, static_cast<void*>(impl_->error_word)})
+    for (void* p : {impl_->union_meta, impl_->nax_workspace, impl_->dense_workspace, impl_->grouped_workspace, impl_->q8_workspace, static_cast<void*>(impl_->error_word)})
         if (p) (void)hipFree(p);
     (void)hipEventDestroy(impl_->started);
     (void)hipEventDestroy(impl_->finished);
@@ -560,9 +562,22 @@ void HipGraph::dense_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView m
                        p.dense_workspace_bytes, p.error_word, p.stream));
 }
 
-void HipGraph::prepare_dense_mm_q8(PrefillWeightLayout layout) {
+void HipGraph::prepare_dense_mm_q8(PrefillWeightLayout layout, uint32_t max_tokens, uint32_t max_columns, uint32_t max_rows) {
     impl_->idle();
     require(layout == PrefillWeightLayout::gguf || layout == PrefillWeightLayout::q8_lanes_v1, "dense Q8_0 GEMM layout");
+    if (max_tokens == 0 && max_columns == 0 && max_rows == 0) return;
+    require(max_tokens >= 1 && max_tokens <= 65536 && max_columns >= 32 && max_columns <= 65536 && max_rows >= 1 && max_rows <= 1000000,
+            "dense Q8_0 GEMM preparation bounds mismatch");
+    const uint64_t bytes = tsp_dense_mm_q8_workspace_bytes(max_tokens, max_columns, max_rows);
+    if (bytes <= impl_->q8_workspace_bytes) return;
+    if (impl_->q8_workspace) {  // idle: nothing in flight reads the old scratch
+        hip(hipFree(impl_->q8_workspace), "hipFree");
+        impl_->live_bytes -= impl_->q8_workspace_bytes;
+        impl_->q8_workspace = nullptr;
+        impl_->q8_workspace_bytes = 0;
+    }
+    impl_->q8_workspace = impl_->raw(bytes);
+    impl_->q8_workspace_bytes = bytes;
 }
 
 void HipGraph::dense_mm_q8(PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output, bool) {
@@ -572,6 +587,13 @@ void HipGraph::dense_mm_q8(PrefillWeightLayout layout, GpuView matrix, GpuRowsF3
     p.rows_fit(output, "dense Q8_0 GEMM geometry");
     require(input.rows == output.rows && input.rows >= 1, "dense Q8_0 GEMM geometry");
     validate_disjoint(std::array{matrix, input.view}, std::array{output.view});
+    if (input.rows >= 32 && input.columns % 64 == 0 && p.q8_workspace &&
+        tsp_dense_mm_q8_workspace_bytes(input.rows, input.columns, output.columns) <= p.q8_workspace_bytes) {
+        check(tsp_dense_mm_q8_staged(uint32_t(layout), p.device(matrix), matrix.bytes, reinterpret_cast<const float*>(p.device(input.view)),
+                                     input.stride_bytes, reinterpret_cast<float*>(p.device(output.view, true)), output.stride_bytes, input.rows,
+                                     input.columns, output.columns, p.q8_workspace, p.q8_workspace_bytes, p.error_word, p.stream));
+        return;
+    }
     check(tsp_dense_mm_q8(uint32_t(layout), p.device(matrix), matrix.bytes, reinterpret_cast<const float*>(p.device(input.view)), input.stride_bytes,
                           reinterpret_cast<float*>(p.device(output.view, true)), output.stride_bytes, input.rows, input.columns, output.columns,
                           p.error_word, p.stream));
@@ -753,7 +775,8 @@ void prepare_moe_mm_many(HipGraph& graph, const MoeWeights& w, MoeShape shape, u
     } else {
         graph.prepare_grouped_mm(w.gate.encoding, l.gate, rows, shape.selected, shape.experts, shape.channels > shape.hidden ? shape.channels : shape.hidden);
     }
-    for (const auto layout : {l.shared_gate, l.shared_up, l.shared_down}) graph.prepare_dense_mm_q8(layout);
+    const uint32_t widest = shape.channels > shape.hidden ? shape.channels : shape.hidden;
+    for (const auto layout : {l.shared_gate, l.shared_up, l.shared_down}) graph.prepare_dense_mm_q8(layout, rows, widest, widest);
 }
 
 void encode_moe_mm_many(HipGraph& g, const MoeWeights& w, const MoeMmManyScratch& s, GpuRowsF32 input, GpuRowsF32 output, MoeShape shape,

@@ -143,8 +143,11 @@ public:
     // the same with experts = 1, selected = 1, broadcast: the dense dequant-GEMM (Q4_K rows or planes, Q6_K planes)
     void dense_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output);
     // graph.hpp:859-860 `prepare_dense_mm_q8` / `dense_mm_q8`: out[m, :] = W x[m, :] for a dense Q8_0 matrix in GGUF rows or
-    // q8_lanes_v1 rows, f32 rows in and out (decoded and accumulated in f32, each weight read once per eight rows)
-    void prepare_dense_mm_q8(PrefillWeightLayout layout);
+    // q8_lanes_v1 rows, f32 rows in and out (decoded and accumulated in f32, each weight read once per eight rows).
+    // Preparing with bounds (not in the engine's signature) sizes a scratch for the many-row form: from 32 rows on, with
+    // columns in multiples of 64 and within the bounds, matrix and rows are staged as halves and one matrix-core GEMM
+    // multiplies them (the engine's kernel stages halves too); the bounds may grow by preparing again.
+    void prepare_dense_mm_q8(PrefillWeightLayout layout, uint32_t max_tokens = 0, uint32_t max_columns = 0, uint32_t max_rows = 0);
     void dense_mm_q8(PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output, bool reuse_bf16 = false);
     // graph.hpp:548-553 selectors of the engine's GEMV variants: same arithmetic here whatever they say, kept so that
     // callers' set-up code runs unchanged (idle only, same accepted values)
