@@ -67,7 +67,8 @@ def test_routed_m8_all_singletons(gpu, tsp, orc, gu, dn):
     assert gpu.error() == 0
 
 
-@pytest.mark.parametrize("channels,hidden", [(2048, 512), (1024, 256), (512, 1024)])
+# rows of 1, 2, 4, 8 super-blocks take the one-block-per-wave kernel, (768, 1280) the looped one on both sides
+@pytest.mark.parametrize("channels,hidden", [(2048, 512), (1024, 256), (512, 1024), (256, 2048), (768, 1280)])
 @pytest.mark.parametrize("tokens", [1, 2, 3, 5, 8])
 def test_routed_m8_fast_arms(gpu, tsp, orc, synth, channels, hidden, tokens):
     """Q4_K co-located gate/up with Q6_K planes for down: the shapes the register-resident kernels take,

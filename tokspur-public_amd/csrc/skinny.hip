@@ -11,7 +11,9 @@
 // near 2^14 and split as hi + lo halves (22 significant bits); both halves multiply the same integer weight
 // fragment and accumulate into the same f32 accumulator. Nothing else is rounded before the f32 scaling.
 //
-// One workgroup = one task (a weight matrix and up to 8 rows) x 256 weight rows (128 hidden units for gate/up).
+// Two kernels. Rows of 1, 2, 4 or 8 super-blocks (every shape the engine's models have) take flat_kernel further down: one
+// super-block per wave, no loop. The looped skinny_kernel serves the other row lengths:
+// one workgroup = one task (a weight matrix and up to 8 rows) x 256 weight rows (128 hidden units for gate/up).
 // The rows are staged once, for all of K, in LDS (hi and lo planes, 16-byte chunks XOR-swizzled by row so the
 // eight rows of a fragment read fall in different banks); after that the four waves run independently, with no
 // barrier in the K loop, each streaming its own 64 weight rows with one super-block of loads in flight.
