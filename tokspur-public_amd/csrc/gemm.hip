@@ -24,6 +24,7 @@
 //     two and three steps ahead, into a ring of four slabs; one LDS-only barrier per K step.
 //   * For gate/up the two column tiles of a wave are the gate rows and the up rows of the same 32 hidden
 //     units, so SwiGLU is an element-wise epilogue on accumulator registers.
+#include "grouping_device.hpp"
 #include "mfma_quant.hpp"
 
 #include <type_traits>
@@ -489,13 +490,15 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
 // f32 rows -> bf16 (RNE) -> f16, or bf16 rows -> f16, plus the per-sub-block (32 column) sums of the converted
 // values as hi + lo f16 pairs: sx[row][block][0..7] = hi, [8..15] = lo. A thread converts 8 columns; four
 // neighbouring lanes share one sub-block. Values outside the f16 range are flagged.
+// `block` of `blocks` workgroups share the rows (any workgroup size that is a multiple of the wave).
 template <bool FROM_BF16>
-__global__ __launch_bounds__(256) void to_f16_rows(const void* __restrict__ src, uint64_t src_stride_bytes, _Float16* __restrict__ dst,
-                                                   _Float16* __restrict__ sx, uint32_t rows, uint32_t columns, uint32_t* error_word) {
+__device__ __forceinline__ void to_f16_rows_block(const void* __restrict__ src, uint64_t src_stride_bytes, _Float16* __restrict__ dst,
+                                                  _Float16* __restrict__ sx, uint32_t rows, uint32_t columns, uint32_t* error_word,
+                                                  uint32_t block, uint32_t blocks) {
     uint32_t bad = 0;
     const uint64_t chunks = uint64_t(rows) * (columns / 8);
     const uint64_t span = (chunks + 3) / 4 * 4;  // whole groups of four lanes stay in the loop together
-    for (uint64_t i = blockIdx.x * uint64_t(blockDim.x) + threadIdx.x; i < span; i += uint64_t(gridDim.x) * blockDim.x) {
+    for (uint64_t i = block * uint64_t(blockDim.x) + threadIdx.x; i < span; i += uint64_t(blocks) * blockDim.x) {
         const bool live = i < chunks;
         const uint64_t r = live ? i / (columns / 8) : 0, c8 = live ? i % (columns / 8) : 0;
         const uint8_t* row = static_cast<const uint8_t*>(src) + r * src_stride_bytes;
@@ -536,6 +539,28 @@ __global__ __launch_bounds__(256) void to_f16_rows(const void* __restrict__ src,
     publish_error(bad, error_word);
 }
 
+template <bool FROM_BF16>
+__global__ __launch_bounds__(256) void to_f16_rows(const void* __restrict__ src, uint64_t src_stride_bytes, _Float16* __restrict__ dst,
+                                                   _Float16* __restrict__ sx, uint32_t rows, uint32_t columns, uint32_t* error_word) {
+    to_f16_rows_block<FROM_BF16>(src, src_stride_bytes, dst, sx, rows, columns, error_word, blockIdx.x, gridDim.x);
+}
+
+// The two task lists of a grouped product (workgroups 0 and 1) and the row conversion (all other workgroups) in one launch:
+// neither needs the other, both need only what the route permutation before them wrote or nothing at all, and a launch of
+// its own costs each of these small kernels more than its work.
+struct TaskLists { const uint32_t* counts; uint32_t* tasks0; uint32_t tile0; uint32_t* tasks1; uint32_t tile1; uint32_t experts, selected, tokens; };
+__global__ __launch_bounds__(512) void tasks_and_rows(TaskLists t, const void* __restrict__ src, uint64_t src_stride_bytes, _Float16* __restrict__ dst,
+                                                      _Float16* __restrict__ sx, uint32_t rows, uint32_t columns, uint32_t* error_word) {
+    __shared__ uint32_t tiles_scan[512];
+    __shared__ uint32_t routes_scan[512];
+    if (blockIdx.x < 2) {
+        grouped_tasks_block(t.counts, blockIdx.x == 0 ? t.tasks0 : t.tasks1, blockIdx.x == 0 ? t.tile0 : t.tile1, t.experts, t.selected, t.tokens,
+                            error_word, tiles_scan, routes_scan);
+    } else {
+        to_f16_rows_block<false>(src, src_stride_bytes, dst, sx, rows, columns, error_word, blockIdx.x - 2, gridDim.x - 2);
+    }
+}
+
 template <int BKIND, int EPI, int ROWS>
 int launch(const GemmArgs& a, uint32_t col_tiles, uint32_t tasks, hipStream_t s) {
     constexpr const char* name = EPI == EPI_SWIGLU ? "gemm_gate_up_swiglu" : ROWS == ROWS_TASK_SLOTS ? "gemm_down" : ROWS == ROWS_ROUTES ? "gemm_grouped" : "gemm_dense";
@@ -554,6 +579,15 @@ int convert_rows(const void* src, uint64_t stride, int from_bf16, _Float16* dst,
     if (from_bf16) TSP_LAUNCH("to_f16_rows", s, to_f16_rows<true><<<grid, 256, 0, s>>>(src, stride, dst, sx, rows, columns, err));
     else TSP_LAUNCH("to_f16_rows", s, to_f16_rows<false><<<grid, 256, 0, s>>>(src, stride, dst, sx, rows, columns, err));
     return launch_status("to_f16_rows");
+}
+
+// f32 rows only; the caller has checked the task geometry (experts <= 512, tiles <= 256)
+int lists_and_rows(const TaskLists& t, const void* src, uint64_t stride, _Float16* dst, _Float16* sx, uint32_t rows, uint32_t columns,
+                   uint32_t* err, hipStream_t s) {
+    const uint64_t chunks = uint64_t(rows) * (columns / 8);
+    const uint32_t grid = 2 + uint32_t((chunks + 511) / 512 > 8192 ? 8192 : (chunks + 511) / 512);
+    TSP_LAUNCH("tasks_and_rows", s, tasks_and_rows<<<grid, 512, 0, s>>>(t, src, stride, dst, sx, rows, columns, err));
+    return launch_status("tasks_and_rows");
 }
 
 uint64_t align256(uint64_t v) { return (v + 255) / 256 * 256; }
@@ -667,8 +701,8 @@ extern "C" int tsp_grouped_mm(uint32_t encoding, uint32_t layout, const void* ma
     auto* sx = reinterpret_cast<_Float16*>(ws + l.sx);
     auto* task_list = reinterpret_cast<uint32_t*>(ws + l.tasks);
     int rc = tsp_grouped_routes(ids, token_map, counts, experts, selected, tokens, error_word, stream);
-    if (rc == TSP_OK) rc = grouped_tasks_pair(counts, tasks, 32, task_list, kTaskRows, experts, selected, tokens, error_word, stream);
-    if (rc == TSP_OK) rc = convert_rows(input, input_stride_bytes, 0, xh, sx, l.in_rows, columns, error_word, s);
+    if (rc == TSP_OK) rc = lists_and_rows(TaskLists{counts, tasks, 32, task_list, kTaskRows, experts, selected, tokens}, input, input_stride_bytes, xh, sx,
+                                          l.in_rows, columns, error_word, s);
     if (rc != TSP_OK) return rc;
     GemmArgs a{};
     a.a = xh; a.a_stride = columns; a.sx = sx; a.w0 = static_cast<const uint8_t*>(matrices); a.raw_expert_bytes = expert_bytes;
@@ -779,8 +813,8 @@ extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream
     auto* hbuf = reinterpret_cast<_Float16*>(ws + l.hbuf);
 
     rc = tsp_grouped_routes(m->ids, m->token_map, m->counts, m->experts, m->selected, m->tokens, m->error_word, stream);
-    if (rc == TSP_OK) rc = grouped_tasks_pair(m->counts, m->tasks, 32, task_list, kTaskRows, m->experts, m->selected, m->tokens, m->error_word, stream);
-    if (rc == TSP_OK) rc = convert_rows(m->x, m->x_stride_bytes, 0, xh, sx, m->tokens, m->channels, m->error_word, s);
+    if (rc == TSP_OK) rc = lists_and_rows(TaskLists{m->counts, m->tasks, 32, task_list, kTaskRows, m->experts, m->selected, m->tokens}, m->x,
+                                          m->x_stride_bytes, xh, sx, m->tokens, m->channels, m->error_word, s);
     if (rc != TSP_OK) return rc;
 
     GemmArgs g{};

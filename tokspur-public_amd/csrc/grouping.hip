@@ -8,7 +8,7 @@
 //  grouped_tasks   tiles(e) = ceil(min(counts[e], T) / tile); exclusive scan over experts; task i of
 //                  expert e is (e, i*tile); unused slots up to the bound are 0xFFFFFFFF.
 //  union_build     for T*S <= 128 routes: records (expert, <= cap routes) in first-use order.
-#include "tsp_common.hpp"
+#include "grouping_device.hpp"
 
 using namespace tsp;
 
@@ -46,44 +46,14 @@ __global__ __launch_bounds__(256) void grouped_routes_kernel(const uint32_t* __r
     publish_error(bad, error_word);
 }
 
-// One block of 512 threads; experts <= 512.
 // Block b writes list b: the same counts tiled two ways in one launch (tasks1 may be null with a grid of one).
 __global__ __launch_bounds__(512) void grouped_tasks_kernel(const uint32_t* __restrict__ counts, uint32_t* __restrict__ tasks0, uint32_t tile0,
                                                             uint32_t* __restrict__ tasks1, uint32_t tile1, uint32_t experts, uint32_t selected,
                                                             uint32_t tokens, uint32_t* error_word) {
-    uint32_t* const tasks = blockIdx.x == 0 ? tasks0 : tasks1;
-    const uint32_t tile = blockIdx.x == 0 ? tile0 : tile1;
     __shared__ uint32_t tiles_scan[512];
     __shared__ uint32_t routes_scan[512];
-    const uint32_t tid = threadIdx.x;
-    const uint32_t bound = tokens * selected / tile + experts;
-    uint32_t bad = 0;
-    const uint32_t count = tid < experts ? counts[tid] : 0;
-    if (count > tokens) bad = TSP_ERRBIT_INDEX;
-    const uint32_t n = ((count < tokens ? count : tokens) + tile - 1) / tile;
-    tiles_scan[tid] = n;
-    routes_scan[tid] = count;
-    __syncthreads();
-    for (uint32_t step = 1; step < 512; step <<= 1) {  // inclusive Hillis-Steele scan
-        const uint32_t a = tid >= step ? tiles_scan[tid - step] : 0, b = tid >= step ? routes_scan[tid - step] : 0;
-        __syncthreads();
-        tiles_scan[tid] += a;
-        routes_scan[tid] += b;
-        __syncthreads();
-    }
-    const uint32_t total = tiles_scan[511], routes = routes_scan[511];
-    const uint32_t offset = tiles_scan[tid] - n;
-    for (uint32_t i = tid; i < bound; i += 512) { tasks[2 + 2 * i] = 0xffffffffu; tasks[3 + 2 * i] = 0xffffffffu; }
-    __syncthreads();
-    if (tid < experts)
-        for (uint32_t i = 0; i < n; ++i)
-            if (offset + i < bound) { tasks[2 + 2 * (offset + i)] = tid; tasks[3 + 2 * (offset + i)] = i * tile; }
-    if (tid == 0) {
-        tasks[0] = total < bound ? total : bound;
-        tasks[1] = routes;
-        if (total > bound || routes != tokens * selected) bad = TSP_ERRBIT_INDEX;
-    }
-    publish_error(bad, error_word);
+    grouped_tasks_block(counts, blockIdx.x == 0 ? tasks0 : tasks1, blockIdx.x == 0 ? tile0 : tile1, experts, selected, tokens, error_word,
+                        tiles_scan, routes_scan);
 }
 
 // 128 threads, one per flat route (T*S <= 128). meta layout in 32-bit words: [0..7] header,
@@ -174,16 +144,6 @@ extern "C" int tsp_grouped_tasks(const uint32_t* counts, uint32_t* tasks, uint32
                 "grouped tasks geometry");
     TSP_REQUIRE(counts && tasks && error_word, "null device pointer");
     TSP_LAUNCH("grouped_tasks", static_cast<hipStream_t>(stream), grouped_tasks_kernel<<<1, 512, 0, static_cast<hipStream_t>(stream)>>>(counts, tasks, tile, nullptr, 0, experts, selected, tokens, error_word));
-    return launch_status("grouped_tasks");
-}
-
-// The caller's task list (tile0 rows per task) and a second one (tile1) from the same counts, in one launch.
-int tsp::grouped_tasks_pair(const uint32_t* counts, uint32_t* tasks0, uint32_t tile0, uint32_t* tasks1, uint32_t tile1, uint32_t experts,
-                            uint32_t selected, uint32_t tokens, uint32_t* error_word, void* stream) {
-    TSP_REQUIRE(experts && experts <= 512 && selected && selected <= 16 && tokens && tokens <= 2048 && tile0 && tile0 <= 256 && tile1 && tile1 <= 256,
-                "grouped tasks geometry");
-    TSP_REQUIRE(counts && tasks0 && tasks1 && error_word, "null device pointer");
-    TSP_LAUNCH("grouped_tasks", static_cast<hipStream_t>(stream), grouped_tasks_kernel<<<2, 512, 0, static_cast<hipStream_t>(stream)>>>(counts, tasks0, tile0, tasks1, tile1, experts, selected, tokens, error_word));
     return launch_status("grouped_tasks");
 }
 

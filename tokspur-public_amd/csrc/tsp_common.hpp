@@ -111,8 +111,4 @@ __device__ __forceinline__ void publish_error(uint32_t bad, uint32_t* error_word
 
 #endif  // __HIPCC__
 
-// grouping.hip: the caller's task list and a second tiling of the same counts in one launch
-int grouped_tasks_pair(const uint32_t* counts, uint32_t* tasks0, uint32_t tile0, uint32_t* tasks1, uint32_t tile1, uint32_t experts,
-                       uint32_t selected, uint32_t tokens, uint32_t* error_word, void* stream);
-
 }  // namespace tsp
