@@ -119,9 +119,10 @@ def main():
     su = synth.matrix(12, synth.tensor_seed(3, 21), H, C)
     sd = synth.matrix(14, synth.tensor_seed(3, 22), C, H)
     ws = capi.PlanarMoeWeights(gpu, 12, 14, C, H, 2, np.concatenate([sg, sg]), np.concatenate([su, su]), np.concatenate([sd, sd]))
+    shared = capi.PlanarSharedExpert(gpu, C, H, sg, su, sd)
     d_logits, d_x = gpu.upload(logits), gpu.upload(x)
     ids, wts = gpu.zeros((T, S), "int32"), gpu.zeros((T, S))
-    scratch, scratch_s = capi.GroupedScratch(gpu, T, S, E, C, H), capi.GroupedScratch(gpu, T, 1, 2, C, H)
+    scratch, scratch_s = capi.GroupedScratch(gpu, T, S, E, C, H, with_shared=True), capi.GroupedScratch(gpu, T, 1, 2, C, H)
     y, ys, out = gpu.empty((T * S, C)), gpu.empty((T, C)), gpu.empty((T, C))
     ids_shared, shared_logit = gpu.zeros(T, "int32"), gpu.full(T, 20.0)
 
@@ -130,7 +131,7 @@ def main():
 
     side = torch.cuda.Stream()  # default priority: the shared expert only needs x, so it runs beside the routed experts
 
-    def step_c3():
+    def step_two_streams():  # the shared expert as a grouped product of its own beside the routed experts
         main = torch.cuda.current_stream()
         side.wait_stream(main)
         with torch.cuda.stream(side):
@@ -140,7 +141,17 @@ def main():
         main.wait_stream(side)
         gpu.mixture(y, wts, ys, shared_logit, C, S, tokens=T, out=out)
 
+    def step_c3():  # the shared expert's rows ride in the routed experts' two GEMM launches
+        gpu.route(d_logits, S, 0, True, tokens=T, out=(ids, wts))
+        capi.planar_nax_grouped_moe(gpu, w, ids, d_x, T, S, scratch, y=y, shared=shared, shared_y=ys)
+        gpu.mixture(y, wts, ys, shared_logit, C, S, tokens=T, out=out)
+
+    two_streams_ms_step = timed(torch, step_two_streams, args.steps, args.warmup)
+    torch.cuda.synchronize()
+    reference_out = out.clone()
     eager_ms_step = timed(torch, step_c3, args.steps, args.warmup)
+    torch.cuda.synchronize()
+    assert torch.equal(out, reference_out), "the two ways of running the shared expert disagree"
     graph = None if args.no_graph else graph_of(torch, step_c3, out)
     graph_ms_step = timed(torch, graph.replay, args.steps, args.warmup) if graph is not None else None
     if graph_ms_step is None or graph_ms_step >= eager_ms_step:
@@ -177,8 +188,10 @@ def main():
         "hbm_gbps": bytes_step / (ms_step * 1e-3) / 1e9, "hbm_frac": bytes_step / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "expert_loads": {"nonempty": nonempty, "min": int(counts.min()), "median": int(np.median(counts)), "max": int(counts.max())},
         "kernels_us": {k: round(v["avg_us"], 2) for k, v in prof.items()},
-        "launch": "HIP graph replay of the step's kernels on two streams" if graph is not None else "eager launches from Python",
-        "eager_ms_per_step": eager_ms_step, "graph_ms_per_step": graph_ms_step}}
+        "launch": "HIP graph replay of the step's kernels" if graph is not None else "eager launches from Python",
+        "eager_ms_per_step": eager_ms_step, "graph_ms_per_step": graph_ms_step,
+        "shared_expert": "rides in the routed experts' gate/up and down launches (same bits as run beside them on a second stream: "
+                         f"{two_streams_ms_step:.3f} ms per step that way, eager)"}}
 
     # ------------------------------------------------------------------ CPU baseline (rank 0, bounded sample)
     cpu = None

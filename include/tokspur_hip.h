@@ -327,6 +327,21 @@ uint64_t tsp_planar_nax_workspace_bytes(uint32_t tokens, uint32_t selected, uint
  * permutation -> prefix-sum tasks -> gather -> ragged grouped gate/up GEMM with fused SwiGLU (h carried as
  * the half nearest h / 256) -> grouped down GEMM -> scatter of f32 rows to y[rid]. */
 int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* moe, void* stream);
+/* The same call with the layer's always-on expert riding in the two GEMM launches instead of running as dense GEMMs of
+ * its own beside them (src/moe_mm_many.cpp:152-187 runs it as three `dense_mm_q8`; this is for a shared expert kept in
+ * the routed experts' formats): `gate` and `up` are one Pack v3 Q4_K expert each (the halves of a co-located pair,
+ * src/planar_pack_v3.cpp:1061-1123, need not be adjacent), `down` one Q6_K planes expert; every token is a row of it,
+ * and y [tokens, channels] receives down(silu(gate x) * up x), to be handed to `tsp_prefill_mixture_batch` as `shared`.
+ * Only with the Q4_K co-located / Q6_K planes kinds; the workspace is tsp_planar_nax_shared_workspace_bytes. */
+typedef struct tsp_shared_expert {
+    const void* gate;
+    const void* up;
+    const void* down;
+    float* y;
+    uint64_t y_stride_bytes;
+} tsp_shared_expert;
+uint64_t tsp_planar_nax_shared_workspace_bytes(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t channels, uint32_t hidden);
+int tsp_planar_nax_grouped_moe_shared(const tsp_grouped_moe* moe, const tsp_shared_expert* shared, void* stream);
 
 /* ------------------------------------------------------------------ row top-k of the logits */
 

@@ -229,6 +229,50 @@ def test_grouped_moe_reference_cases(gpu, tsp, orc, synth, n):
     assert max_rel_error(y, declared) <= 2e-3 and nmse(y, declared) <= 1e-7
 
 
+@pytest.mark.parametrize("n", [1, 33, 70, 200])
+def test_grouped_moe_with_always_on_expert(gpu, tsp, orc, synth, n):
+    """The layer's always-on expert riding in the grouped launches (every token is a row of it): the routed rows are the
+    same bits as without it, its own rows are the same bits as a separate call that routes every token to it, both agree
+    with the CPU composition, the caller's task list is unchanged, padding of a strided output stays."""
+    channels, hidden, experts, selected = 512, 256, 8, 3
+    gate = synth.matrix(12, 3101, hidden * experts, channels)
+    up = synth.matrix(12, 3102, hidden * experts, channels)
+    down = synth.matrix(14, 3103, channels * experts, hidden)
+    sg, su, sd = synth.matrix(12, 3104, hidden, channels), synth.matrix(12, 3105, hidden, channels), synth.matrix(14, 3106, channels, hidden)
+    w = tsp.PlanarMoeWeights(gpu, 12, 14, channels, hidden, experts, gate, up, down)
+    shared = tsp.PlanarSharedExpert(gpu, channels, hidden, sg, su, sd)
+    rng = np.random.default_rng(n)
+    ids = np.stack([rng.permutation(experts)[:selected] for _ in range(n)]).astype(np.uint32).reshape(-1)
+    x = synth.round_bf16(synth.activations_f32(3107 + n, (n, channels)))
+    d_ids, d_x = gpu.upload(ids), gpu.upload(x)
+    plain = tsp.planar_nax_grouped_moe(gpu, w, d_ids, d_x, n, selected, tsp.GroupedScratch(gpu, n, selected, experts, channels, hidden)).cpu().numpy()
+    scratch = tsp.GroupedScratch(gpu, n, selected, experts, channels, hidden, with_shared=True)
+    padded = gpu.full((n, channels + 8), -4.0)
+    y, _ = tsp.planar_nax_grouped_moe(gpu, w, d_ids, d_x, n, selected, scratch, shared=shared, shared_y=padded, shared_y_stride=(channels + 8) * 4)
+    assert gpu.error() == 0
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), plain.view(np.uint32))
+    got = padded.cpu().numpy()
+    assert (got[:, channels:] == -4.0).all()
+    want_counts = orc.grouped_routes(ids, experts, selected, n)[1]
+    assert np.array_equal(scratch.tasks.cpu().numpy().view(np.uint32), orc.grouped_tasks(want_counts, experts, selected, n, 32)[0])
+    # the same expert as the only choice of every token, through the plain call (two copies: co-located halves come in pairs)
+    alone = tsp.PlanarMoeWeights(gpu, 12, 14, channels, hidden, 2, np.concatenate([sg, sg]), np.concatenate([su, su]), np.concatenate([sd, sd]))
+    zeros = gpu.upload(np.zeros(n, dtype=np.uint32))
+    separate = tsp.planar_nax_grouped_moe(gpu, alone, zeros, d_x, n, 1, tsp.GroupedScratch(gpu, n, 1, 2, channels, hidden)).cpu().numpy()
+    assert np.array_equal(got[:, :channels].view(np.uint32), separate.view(np.uint32))
+    _, declared = orc.moe_routed_reference(12, 14, sg, su, sd, channels, hidden, 1, np.zeros(n, dtype=np.uint32), n, 1, x, stage=12, threads=8)
+    _, unrounded = orc.moe_routed_reference(12, 14, sg, su, sd, channels, hidden, 1, np.zeros(n, dtype=np.uint32), n, 1, x, stage=0, threads=8)
+    assert max_rel_error(got[:, :channels], declared) <= 2e-3 and nmse(got[:, :channels], declared) <= 1e-7
+    assert nmse(got[:, :channels], unrounded) <= 2e-3
+    with pytest.raises(tsp.FormatError):  # the smaller scratch of the plain call is refused
+        tsp.planar_nax_grouped_moe(gpu, w, d_ids, d_x, n, selected, tsp.GroupedScratch(gpu, n, selected, experts, channels, hidden), shared=shared)
+    if n == 33:
+        other = tsp.PlanarMoeWeights(gpu, 13, 7, channels, hidden, experts, synth.matrix(13, 1, hidden * experts, channels),
+                                     synth.matrix(13, 2, hidden * experts, channels), synth.matrix(7, 3, channels * experts, hidden))
+        with pytest.raises(tsp.FormatError):  # only beside the Q4_K / Q6_K kinds
+            tsp.planar_nax_grouped_moe(gpu, other, d_ids, d_x, n, selected, scratch, shared=shared)
+
+
 def test_grouped_moe_exact_when_products_fit_half(gpu, tsp, orc, synth):
     """With Q6_K sub-scales in [-64, 63] every integer product sc * (q - 32) is exact in f16, and the grouped MoE
     then differs from the f32-dequantised CPU reference (bf16 x, h as half(h / 256)) only by f32 accumulation and

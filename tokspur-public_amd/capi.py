@@ -461,16 +461,38 @@ def dense_mm(dev, encoding, layout, matrix, x, tokens, columns, rows, out=None, 
 
 
 class GroupedScratch:
-    """Caller-owned outputs and scratch of planar_nax_grouped_moe for a given capacity."""
+    """Caller-owned outputs and scratch of planar_nax_grouped_moe for a given capacity (with_shared: room for the
+    always-on expert's rows as well)."""
 
-    def __init__(self, dev, tokens, selected, experts, channels, hidden):
+    def __init__(self, dev, tokens, selected, experts, channels, hidden, with_shared=False):
         self.token_map = dev.zeros(experts * tokens, "int32")
         self.counts = dev.zeros(experts, "int32")
         self.tasks = dev.zeros(2 + 2 * (tokens * selected // 32 + experts), "int32")
-        self.workspace = dev.empty(planar_nax_workspace_bytes(tokens, selected, experts, channels, hidden), "uint8")
+        f = dll().tsp_planar_nax_shared_workspace_bytes
+        f.restype = C.c_uint64
+        size = (f(C.c_uint32(tokens), C.c_uint32(selected), C.c_uint32(experts), C.c_uint32(channels), C.c_uint32(hidden)) if with_shared
+                else planar_nax_workspace_bytes(tokens, selected, experts, channels, hidden))
+        self.workspace = dev.empty(size, "uint8")
 
 
-def planar_nax_grouped_moe(dev, w, ids, x, tokens, selected, scratch, y=None, x_stride=None, y_stride=None):
+class SharedExpert(C.Structure):
+    _fields_ = [("gate", C.c_void_p), ("up", C.c_void_p), ("down", C.c_void_p), ("y", C.c_void_p), ("y_stride_bytes", C.c_uint64)]
+
+
+class PlanarSharedExpert:
+    """One always-on expert in the routed experts' formats: Q4_K gate and up as one Pack v3 expert each, Q6_K planes down."""
+
+    def __init__(self, dev, channels, hidden, gate_raw, up_raw, down_raw):
+        self.channels, self.hidden = channels, hidden
+        gu, dn = make_expert_spec(12, channels, hidden), make_expert_spec(14, hidden, channels)
+        self.gate, self.up = dev.upload(pack_experts(gu, gate_raw, 1)), dev.upload(pack_experts(gu, up_raw, 1))
+        self.down = dev.upload(pack_experts(dn, down_raw, 1))
+
+
+def planar_nax_grouped_moe(dev, w, ids, x, tokens, selected, scratch, y=None, x_stride=None, y_stride=None, shared=None, shared_y=None,
+                           shared_y_stride=None):
+    """`planar_nax_grouped_moe`; with `shared` (a PlanarSharedExpert) the always-on expert rides in the same launches and its
+    rows come back as the second result."""
     y = dev.empty((tokens * selected, w.channels)) if y is None else y
     gate_kind, up_kind = COLOC_KINDS[w.gu_type]
     m = GroupedMoe(w.pair_lo.data_ptr(), w.pair_hi.data_ptr(), w.down.data_ptr(), gate_kind, up_kind, DOWN_KINDS[w.dn_type],
@@ -478,8 +500,14 @@ def planar_nax_grouped_moe(dev, w, ids, x, tokens, selected, scratch, y=None, x_
                    w.channels * 4 if x_stride is None else x_stride, y.data_ptr(), w.channels * 4 if y_stride is None else y_stride,
                    scratch.token_map.data_ptr(), scratch.counts.data_ptr(), scratch.tasks.data_ptr(), scratch.workspace.data_ptr(),
                    dev.nbytes(scratch.workspace), dev.err.data_ptr())
-    check(dll().tsp_planar_nax_grouped_moe(C.byref(m), dev.stream()))
-    return y
+    if shared is None:
+        check(dll().tsp_planar_nax_grouped_moe(C.byref(m), dev.stream()))
+        return y
+    shared_y = dev.empty((tokens, w.channels)) if shared_y is None else shared_y
+    e = SharedExpert(shared.gate.data_ptr(), shared.up.data_ptr(), shared.down.data_ptr(), shared_y.data_ptr(),
+                     w.channels * 4 if shared_y_stride is None else shared_y_stride)
+    check(dll().tsp_planar_nax_grouped_moe_shared(C.byref(m), C.byref(e), dev.stream()))
+    return y, shared_y
 
 
 class KernelTime(C.Structure):

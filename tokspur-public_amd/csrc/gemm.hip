@@ -60,6 +60,12 @@ struct GemmArgs {
     uint64_t raw_expert_bytes;       // raw GGUF expert stacks: bytes between experts (0 for one dense matrix)
     uint32_t broadcast;              // ROWS_ROUTES: one input row per token instead of one per route
     uint32_t col_tiles, task_slots;  // logical grid: column tiles x tasks, launched as one linear grid
+    // an always-on expert riding in the same launch: tasks whose expert id is `experts` take every token as their rows,
+    // these weights (gate / up halves, or the down matrix) and, for the down product, these output rows
+    const uint8_t* shared_w0;
+    const uint8_t* shared_w1;
+    void* shared_out;
+    uint64_t shared_out_stride;
 };
 
 // ---------------------------------------------------------------- the kernel
@@ -108,6 +114,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
 
     // ---- task resolution
     uint32_t expert = 0, nrows = 0;
+    bool shared = false;
     uint32_t my_dst = 0xffffffffu;  // output row of activation row `tid` (threads 0..63), parked in a register during the loop
     if (tid == 0) task_bad = 0;
     __syncthreads();
@@ -117,7 +124,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
         nrows = a.m - row0 < kTaskRows ? a.m - row0 : kTaskRows;
         if (tid < kTaskRows) { row_src[tid] = row0 + (tid < nrows ? tid : 0); my_dst = row0 + tid; }
     } else {
-        const uint32_t bound = a.tokens * a.selected / kTaskRows + a.experts;
+        const uint32_t bound = a.tokens * a.selected / kTaskRows + a.experts + (a.shared_w0 ? (a.tokens + kTaskRows - 1) / kTaskRows : 0);
         const uint32_t live = a.tasks[0];
         if (live > bound || a.tasks[1] != a.tokens * a.selected) {
             if (tid == 0 && bx == 0 && task == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
@@ -126,23 +133,29 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
         if (task >= live) return;
         expert = a.tasks[2 + 2 * task];
         const uint32_t start = a.tasks[3 + 2 * task];
-        const uint32_t count = expert < a.experts ? a.counts[expert] : 0;
-        if (expert >= a.experts || count > a.tokens || start >= count) {
+        shared = a.shared_w0 != nullptr && expert == a.experts;
+        const uint32_t count = shared ? a.tokens : expert < a.experts ? a.counts[expert] : 0;
+        if ((expert >= a.experts && !shared) || count > a.tokens || start >= count) {
             if (tid == 0 && bx == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
             return;
         }
         nrows = count - start < kTaskRows ? count - start : kTaskRows;
         if (tid < kTaskRows) {
             // rows past the task's end re-read its first row: their accumulators are never stored
-            uint32_t rid = a.token_map[uint64_t(expert) * a.tokens + start + (tid < nrows ? tid : 0)];
-            if (rid >= a.tokens * a.selected || a.ids[rid] != expert) { rid = 0xffffffffu; task_bad = 1; }
+            uint32_t rid;
+            if (shared) {
+                rid = (start + (tid < nrows ? tid : 0)) * a.selected;  // "route 0" of the token: row_src below divides it back
+            } else {
+                rid = a.token_map[uint64_t(expert) * a.tokens + start + (tid < nrows ? tid : 0)];
+                if (rid >= a.tokens * a.selected || a.ids[rid] != expert) { rid = 0xffffffffu; task_bad = 1; }
+            }
             // activation row: the route's token (gate/up, broadcast grouped GEMM), the route itself (grouped GEMM with one input
             // row per route) or the task's slot in the intermediate buffer (down); output row: task slot or route
             const uint32_t safe = rid == 0xffffffffu ? 0 : rid;
             row_src[tid] = ROWS == ROWS_GATHER_TOKENS ? safe / a.selected
                          : ROWS == ROWS_ROUTES       ? (a.broadcast ? safe / a.selected : safe)
                                                      : task * kTaskRows + (tid < nrows ? tid : 0);
-            my_dst = ROWS == ROWS_GATHER_TOKENS ? task * kTaskRows + tid : rid;
+            my_dst = ROWS == ROWS_GATHER_TOKENS ? task * kTaskRows + tid : shared ? rid / a.selected : rid;
         }
     }
     __syncthreads();
@@ -158,7 +171,8 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
         const uint32_t unit = bx * 128 + wave * 32 + col;
         const uint32_t half_e = a.experts / 2;
         const uint8_t* pair = (expert < half_e ? a.w0 : a.w1) + uint64_t(expert < half_e ? expert : expert - half_e) * 2 * a.spec.planar_expert_bytes;
-        wbase[0] = pair; wbase[1] = pair + a.spec.planar_expert_bytes;
+        wbase[0] = shared ? a.shared_w0 : pair;
+        wbase[1] = shared ? a.shared_w1 : pair + a.spec.planar_expert_bytes;
         col_live[0] = col_live[1] = unit < a.n;
         wrow[0] = wrow[1] = col_live[0] ? unit : a.n - 1;
         out_col[0] = out_col[1] = unit;
@@ -169,7 +183,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
             col_live[j] = n < a.n;
             wrow[j] = col_live[j] ? n : a.n - 1;
             out_col[j] = n;
-            wbase[j] = a.w0 + uint64_t(expert) * (BKIND == B_Q4K_RAW ? a.raw_expert_bytes : a.spec.planar_expert_bytes);
+            wbase[j] = shared ? a.shared_w0 : a.w0 + uint64_t(expert) * (BKIND == B_Q4K_RAW ? a.raw_expert_bytes : a.spec.planar_expert_bytes);
         }
     }
     const uint32_t bpr = a.k / 256;
@@ -473,7 +487,8 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
                     if (!col_live[j]) continue;
                     const float val = acc[i][j][v] * a.out_scale;
                     if (nonfinite(val)) bad = TSP_ERRBIT_NONFINITE;
-                    uint8_t* orow = static_cast<uint8_t*>(a.out) + uint64_t(dst) * a.out_stride;
+                    uint8_t* orow = shared && ROWS == ROWS_TASK_SLOTS ? static_cast<uint8_t*>(a.shared_out) + uint64_t(dst) * a.shared_out_stride
+                                                                      : static_cast<uint8_t*>(a.out) + uint64_t(dst) * a.out_stride;
                     if constexpr (EPI == EPI_F32) {
                         reinterpret_cast<float*>(orow)[out_col[j]] = val;
                     } else {
@@ -548,14 +563,17 @@ __global__ __launch_bounds__(256) void to_f16_rows(const void* __restrict__ src,
 // The two task lists of a grouped product (workgroups 0 and 1) and the row conversion (all other workgroups) in one launch:
 // neither needs the other, both need only what the route permutation before them wrote or nothing at all, and a launch of
 // its own costs each of these small kernels more than its work.
-struct TaskLists { const uint32_t* counts; uint32_t* tasks0; uint32_t tile0; uint32_t* tasks1; uint32_t tile1; uint32_t experts, selected, tokens; };
+struct TaskLists {
+    const uint32_t* counts; uint32_t* tasks0; uint32_t tile0; uint32_t* tasks1; uint32_t tile1; uint32_t experts, selected, tokens;
+    bool every_token1;  // list 1 also holds the always-on expert's tasks
+};
 __global__ __launch_bounds__(512) void tasks_and_rows(TaskLists t, const void* __restrict__ src, uint64_t src_stride_bytes, _Float16* __restrict__ dst,
                                                       _Float16* __restrict__ sx, uint32_t rows, uint32_t columns, uint32_t* error_word) {
     __shared__ uint32_t tiles_scan[512];
     __shared__ uint32_t routes_scan[512];
     if (blockIdx.x < 2) {
         grouped_tasks_block(t.counts, blockIdx.x == 0 ? t.tasks0 : t.tasks1, blockIdx.x == 0 ? t.tile0 : t.tile1, t.experts, t.selected, t.tokens,
-                            error_word, tiles_scan, routes_scan);
+                            error_word, tiles_scan, routes_scan, blockIdx.x == 1 && t.every_token1);
     } else {
         to_f16_rows_block<false>(src, src_stride_bytes, dst, sx, rows, columns, error_word, blockIdx.x - 2, gridDim.x - 2);
     }
@@ -701,7 +719,7 @@ extern "C" int tsp_grouped_mm(uint32_t encoding, uint32_t layout, const void* ma
     auto* sx = reinterpret_cast<_Float16*>(ws + l.sx);
     auto* task_list = reinterpret_cast<uint32_t*>(ws + l.tasks);
     int rc = tsp_grouped_routes(ids, token_map, counts, experts, selected, tokens, error_word, stream);
-    if (rc == TSP_OK) rc = lists_and_rows(TaskLists{counts, tasks, 32, task_list, kTaskRows, experts, selected, tokens}, input, input_stride_bytes, xh, sx,
+    if (rc == TSP_OK) rc = lists_and_rows(TaskLists{counts, tasks, 32, task_list, kTaskRows, experts, selected, tokens, false}, input, input_stride_bytes, xh, sx,
                                           l.in_rows, columns, error_word, s);
     if (rc != TSP_OK) return rc;
     GemmArgs a{};
@@ -715,9 +733,9 @@ extern "C" int tsp_grouped_mm(uint32_t encoding, uint32_t layout, const void* ma
 // ---------------------------------------------------------------- grouped MoE
 namespace {
 struct NaxLayout { uint64_t xh, sx, tasks, hbuf, meta, total; uint32_t bound; };
-NaxLayout nax_layout(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t channels, uint32_t hidden) {
+NaxLayout nax_layout(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t channels, uint32_t hidden, bool shared = false) {
     NaxLayout l{};
-    l.bound = tokens * selected / kTaskRows + experts;
+    l.bound = tokens * selected / kTaskRows + experts + (shared ? (tokens + kTaskRows - 1) / kTaskRows : 0);
     l.xh = 0;
     l.sx = align256(uint64_t(tokens) * channels * 2);
     l.tasks = l.sx + align256(uint64_t(tokens) * (channels / 256) * 32);
@@ -761,7 +779,23 @@ extern "C" uint64_t tsp_planar_nax_workspace_bytes(uint32_t tokens, uint32_t sel
     return nax_layout(tokens, selected, experts, channels, hidden).total;
 }
 
-extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream) {
+namespace {
+int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void* stream);
+}
+
+extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream) { return grouped_moe(m, nullptr, stream); }
+
+extern "C" uint64_t tsp_planar_nax_shared_workspace_bytes(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t channels, uint32_t hidden) {
+    return nax_layout(tokens, selected, experts, channels, hidden, true).total;
+}
+
+extern "C" int tsp_planar_nax_grouped_moe_shared(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void* stream) {
+    TSP_REQUIRE(shared, "null shared expert description");
+    return grouped_moe(m, shared, stream);
+}
+
+namespace {
+int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void* stream) {
     TSP_REQUIRE(m, "null grouped MoE description");
     const bool matrix_cores = m->gate_kind == TSP_KIND_Q4K_COLOC_GATE && m->up_kind == TSP_KIND_Q4K_COLOC_UP && m->down_kind == TSP_KIND_Q6K_PLANAR_X;
     TSP_REQUIRE(m->tokens >= 1 && m->tokens <= 2048 && m->selected >= 1 && m->selected <= 16 && m->selected <= m->experts &&
@@ -774,6 +808,7 @@ extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream
     TSP_REQUIRE(m->pair_lo && m->pair_hi && m->down && m->ids && m->x && m->y && m->token_map && m->counts && m->tasks &&
                     m->workspace && m->error_word,
                 "null device pointer");
+    TSP_REQUIRE(!shared || matrix_cores, "the always-on expert rides only with Q4_K co-located gate/up and Q6_K planes down");
     if (!matrix_cores) {
         const NaxLayout lay = nax_layout(m->tokens, m->selected, m->experts, m->channels, m->hidden);
         TSP_REQUIRE(m->workspace_bytes >= lay.total && reinterpret_cast<uintptr_t>(m->workspace) % 256 == 0,
@@ -786,8 +821,25 @@ extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream
     if (rc != TSP_OK) return rc;
     TSP_REQUIRE(gu.planar_expert_bytes < (1ull << 32) && dn.planar_expert_bytes < (1ull << 32),
                 "planar v3 grouped MoE addresses weight rows with 32-bit offsets: one expert must be under 4 GiB");
-    const NaxLayout l = nax_layout(m->tokens, m->selected, m->experts, m->channels, m->hidden);
+    const NaxLayout l = nax_layout(m->tokens, m->selected, m->experts, m->channels, m->hidden, shared != nullptr);
     TSP_REQUIRE(m->workspace_bytes >= l.total, "planar v3 NAX scratch too small for requested batch");
+    if (shared) {
+        TSP_REQUIRE(shared->gate && shared->up && shared->down && shared->y, "null device pointer");
+        TSP_REQUIRE(reinterpret_cast<uintptr_t>(shared->gate) % 16 == 0 && reinterpret_cast<uintptr_t>(shared->up) % 16 == 0 &&
+                        reinterpret_cast<uintptr_t>(shared->down) % 16 == 0,
+                    "planar v3 matrices require 16-byte alignment (workspace 256)");
+        TSP_REQUIRE(shared->y_stride_bytes >= uint64_t(m->channels) * 4 && shared->y_stride_bytes % 4 == 0, "planar v3 NAX grouped MoE shape or stride mismatch");
+        const uint64_t sy_span = uint64_t(m->tokens - 1) * shared->y_stride_bytes + uint64_t(m->channels) * 4;
+        const void* others[] = {m->pair_lo, m->pair_hi, m->down, m->x, m->ids, shared->gate, shared->up, shared->down, m->y, m->token_map, m->counts, m->tasks, m->workspace};
+        const uint64_t spans[] = {uint64_t(m->experts) * gu.planar_expert_bytes, uint64_t(m->experts) * gu.planar_expert_bytes, uint64_t(m->experts) * dn.planar_expert_bytes,
+                                  uint64_t(m->tokens - 1) * m->x_stride_bytes + uint64_t(m->channels) * 4, uint64_t(m->tokens) * m->selected * 4,
+                                  gu.planar_expert_bytes, gu.planar_expert_bytes, dn.planar_expert_bytes,
+                                  uint64_t(m->tokens * m->selected - 1) * m->y_stride_bytes + uint64_t(m->channels) * 4, uint64_t(m->experts) * m->tokens * 4,
+                                  uint64_t(m->experts) * 4, (2 + 2 * (uint64_t(m->tokens) * m->selected / 32 + m->experts)) * 4, l.total};
+        for (int i = 0; i < 13; ++i) TSP_REQUIRE(!ranges_overlap(shared->y, sy_span, others[i], spans[i]), "planar v3 NAX grouped MoE outputs overlap inputs");
+        for (int i = 8; i < 13; ++i)
+            for (int w = 5; w < 8; ++w) TSP_REQUIRE(!ranges_overlap(others[i], spans[i], others[w], spans[w]), "planar v3 NAX grouped MoE outputs overlap inputs");
+    }
     TSP_REQUIRE(reinterpret_cast<uintptr_t>(m->workspace) % 256 == 0 && reinterpret_cast<uintptr_t>(m->pair_lo) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(m->pair_hi) % 16 == 0 && reinterpret_cast<uintptr_t>(m->down) % 16 == 0,
                 "planar v3 matrices require 16-byte alignment (workspace 256)");
@@ -813,7 +865,7 @@ extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream
     auto* hbuf = reinterpret_cast<_Float16*>(ws + l.hbuf);
 
     rc = tsp_grouped_routes(m->ids, m->token_map, m->counts, m->experts, m->selected, m->tokens, m->error_word, stream);
-    if (rc == TSP_OK) rc = lists_and_rows(TaskLists{m->counts, m->tasks, 32, task_list, kTaskRows, m->experts, m->selected, m->tokens}, m->x,
+    if (rc == TSP_OK) rc = lists_and_rows(TaskLists{m->counts, m->tasks, 32, task_list, kTaskRows, m->experts, m->selected, m->tokens, shared != nullptr}, m->x,
                                           m->x_stride_bytes, xh, sx, m->tokens, m->channels, m->error_word, s);
     if (rc != TSP_OK) return rc;
 
@@ -822,6 +874,7 @@ extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream
     g.spec = gu; g.experts = m->experts; g.tasks = task_list; g.counts = m->counts; g.token_map = m->token_map; g.ids = m->ids;
     g.tokens = m->tokens; g.selected = m->selected; g.n = m->hidden; g.k = m->channels; g.out = hbuf; g.out_scale = 1.0f;
     g.error_word = m->error_word;
+    if (shared) { g.shared_w0 = static_cast<const uint8_t*>(shared->gate); g.shared_w1 = static_cast<const uint8_t*>(shared->up); }
     rc = launch<B_Q4K_PLANAR, EPI_SWIGLU, ROWS_GATHER_TOKENS>(g, (m->hidden + 127) / 128, l.bound, s);
     if (rc != TSP_OK) return rc;
 
@@ -830,5 +883,7 @@ extern "C" int tsp_planar_nax_grouped_moe(const tsp_grouped_moe* m, void* stream
     d.tasks = task_list; d.counts = m->counts; d.token_map = m->token_map; d.ids = m->ids; d.tokens = m->tokens; d.selected = m->selected;
     d.n = m->channels; d.k = m->hidden; d.out = m->y; d.out_stride = m->y_stride_bytes; d.out_scale = 256.0f;  // undo the 2^-8 carried by h
     d.error_word = m->error_word;
+    if (shared) { d.shared_w0 = static_cast<const uint8_t*>(shared->down); d.shared_out = shared->y; d.shared_out_stride = shared->y_stride_bytes; }
     return launch<B_Q6K_PLANAR, EPI_F32, ROWS_TASK_SLOTS>(d, (m->channels + 255) / 256, l.bound, s);
 }
+}  // namespace
