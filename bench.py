@@ -286,7 +286,7 @@ def main():
             gpu.route(lg, S, 0, True, tokens=T2, out=(ids2, wts2))
             used.append(len(set(ids2.cpu().numpy().reshape(-1).tolist())))
 
-        def step_c2():
+        def step_c2_two_streams():  # the shared expert as a routed call of its own beside the routed experts
             lg, xx = sets[state["i"] % len(sets)]
             state["i"] += 1
             main = torch.cuda.current_stream()
@@ -298,6 +298,22 @@ def main():
             main.wait_stream(side)
             gpu.mixture(y2, wts2, ys2, sl2, C, S, tokens=T2, out=out2)
 
+        def step_c2():  # the shared expert as one more record of the routed experts' two launches
+            lg, xx = sets[state["i"] % len(sets)]
+            state["i"] += 1
+            gpu.route(lg, S, 0, True, tokens=T2, out=(ids2, wts2))
+            capi.planar_moe_routed_m8(gpu, w, ids2, xx, T2, S, h=h2, y=y2, shared=shared, shared_h=hs2, shared_y=ys2)
+            gpu.mixture(y2, wts2, ys2, sl2, C, S, tokens=T2, out=out2)
+
+        two_streams_ms = timed(torch, step_c2_two_streams, 48, 16)
+        state["i"] = 0
+        step_c2_two_streams()
+        torch.cuda.synchronize()
+        reference_out2 = out2.clone()
+        state["i"] = 0
+        step_c2()
+        torch.cuda.synchronize()
+        assert torch.equal(out2, reference_out2), "the two ways of running the shared expert disagree (config 2)"
         eager_ms = timed(torch, step_c2, 48, 16)
         state["i"] = len(sets) - 1  # the check inside graph_of runs the last set once more, then the capture starts at set 0
         graph2 = None if args.no_graph else graph_of(torch, step_c2, out2, times=len(sets))
@@ -310,7 +326,8 @@ def main():
         configs["c2_moe_verify_t8"] = {"us": ms * 1e3, "eager_us": eager_ms * 1e3, "graph_us": None if graph_ms is None else graph_ms * 1e3,
                                        "distinct_experts_mean": float(np.mean(used)),
                                        "hbm_gbps": b2 / (ms * 1e-3) / 1e9, "hbm_frac": b2 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                                       "launch": "HIP graph replay of eight steps" if graph2 is not None else "eager launches from Python"}
+                                       "launch": "HIP graph replay of eight steps" if graph2 is not None else "eager launches from Python",
+                                       "two_streams_us": two_streams_ms * 1e3}
         state["i"] = 0
         configs["c2_moe_verify_t8"]["kernels_us"] = {k: round(v["avg_us"], 2) for k, v in profiled(capi, torch, step_c2, 8).items()}
         # config 4: Q8_0 LM head, vocab 151936 x 2048, raw GGUF rows; M = 16 goes through the dense Q8_0 GEMM entry point (one pass, K halves summed)

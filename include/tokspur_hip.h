@@ -272,6 +272,21 @@ int tsp_planar_moe_gate_up_swiglu_m8(const tsp_small_moe* moe, void* stream);
 /* include/tokspur/graph.hpp:475 `planar_moe_routed_m8` (kernels/planar_moe_v3.metal:1572-1803):
  * the above followed by y[rid, :] = Wd[e] h[rid, :]. */
 int tsp_planar_moe_routed_m8(const tsp_small_moe* moe, void* stream);
+/* The same call with the layer's always-on expert riding in the two launches as one more record whose rows are the
+ * tokens (no counterpart: the engine runs the shared expert as GEMVs of its own, src/moe.cpp:71-78). gate, up: one
+ * Pack v3 Q4_K expert each; down: one Q6_K planes expert; h [tokens, hidden] and y [tokens, channels] are its rows
+ * (h 16-byte aligned). Only with Q4_K co-located gate/up and Q6_K planes down. Rows are bit-identical to a separate
+ * call that routes every token to that expert. */
+typedef struct tsp_shared_rows {
+    const void* gate;
+    const void* up;
+    const void* down;
+    float* h;
+    uint64_t h_stride_bytes;
+    float* y;
+    uint64_t y_stride_bytes;
+} tsp_shared_rows;
+int tsp_planar_moe_routed_m8_shared(const tsp_small_moe* moe, const tsp_shared_rows* shared, void* stream);
 
 /* ------------------------------------------------------------------ device: prefill dequant-GEMM (matrix cores) */
 

@@ -94,6 +94,43 @@ def test_routed_m8_fast_arms(gpu, tsp, orc, synth, channels, hidden, tokens):
     assert (h[:, hidden:] == -5.0).all() and (y[:, channels:] == -6.0).all() and gpu.error() == 0
 
 
+@pytest.mark.parametrize("channels,hidden", [(2048, 512), (512, 256), (768, 1280)])
+@pytest.mark.parametrize("tokens", [1, 3, 8])
+def test_routed_m8_with_always_on_expert(gpu, tsp, orc, synth, channels, hidden, tokens):
+    """The layer's always-on expert as one more record of the two launches (its rows are the tokens): the routed rows are
+    the same bits as without it, its rows the same bits as a separate call that routes every token to it, and they agree
+    with the CPU composition; padding of a strided output stays."""
+    experts, selected = 8, 3
+    gate = synth.matrix(12, 41, hidden * experts, channels)
+    up = synth.matrix(12, 42, hidden * experts, channels)
+    down = synth.matrix(14, 43, channels * experts, hidden)
+    sg, su, sd = synth.matrix(12, 44, hidden, channels), synth.matrix(12, 45, hidden, channels), synth.matrix(14, 46, channels, hidden)
+    w = tsp.PlanarMoeWeights(gpu, 12, 14, channels, hidden, experts, gate, up, down)
+    shared = tsp.PlanarSharedExpert(gpu, channels, hidden, sg, su, sd)
+    rng = np.random.default_rng(tokens + channels)
+    ids = np.stack([rng.permutation(experts)[:selected] for _ in range(tokens)]).astype(np.uint32).reshape(-1)
+    x = (synth.activations_f32(47 + tokens, (tokens, channels)) * 0.25).astype(np.float32)
+    d_ids, d_x = gpu.upload(ids), gpu.upload(x)
+    h0, y0 = tsp.planar_moe_routed_m8(gpu, w, d_ids, d_x, tokens, selected)
+    padded = gpu.full((tokens, channels + 4), -2.0)
+    h1, y1, _ = tsp.planar_moe_routed_m8(gpu, w, d_ids, d_x, tokens, selected, shared=shared, shared_y=padded, shared_y_stride=(channels + 4) * 4)
+    assert gpu.error() == 0
+    assert np.array_equal(h1.cpu().numpy().view(np.uint32), h0.cpu().numpy().view(np.uint32))
+    assert np.array_equal(y1.cpu().numpy().view(np.uint32), y0.cpu().numpy().view(np.uint32))
+    got = padded.cpu().numpy()
+    assert (got[:, channels:] == -2.0).all()
+    alone = tsp.PlanarMoeWeights(gpu, 12, 14, channels, hidden, 2, np.concatenate([sg, sg]), np.concatenate([su, su]), np.concatenate([sd, sd]))
+    zeros = np.zeros(tokens, dtype=np.uint32)
+    _, separate = tsp.planar_moe_routed_m8(gpu, alone, gpu.upload(zeros), d_x, tokens, 1)
+    assert np.array_equal(got[:, :channels].view(np.uint32), separate.cpu().numpy().view(np.uint32))
+    _, ref_y = orc.moe_routed_reference(12, 14, sg, su, sd, channels, hidden, 1, zeros, tokens, 1, x, threads=4)
+    assert nmse(got[:, :channels], ref_y) <= 1e-6
+    other = tsp.PlanarMoeWeights(gpu, 13, 7, 256, 256, 2, synth.matrix(13, 1, 512, 256), synth.matrix(13, 2, 512, 256), synth.matrix(7, 3, 512, 256))
+    small = tsp.PlanarSharedExpert(gpu, 256, 256, synth.matrix(12, 4, 256, 256), synth.matrix(12, 5, 256, 256), synth.matrix(14, 6, 256, 256))
+    with pytest.raises(tsp.FormatError):  # only beside the Q4_K / Q6_K kinds
+        tsp.planar_moe_routed_m8(gpu, other, gpu.upload(np.zeros(2, dtype=np.uint32)), gpu.zeros((2, 256)), 2, 1, shared=small)
+
+
 def test_routed_m8_sticky_errors_and_refusals(gpu, tsp, orc, synth):
     channels, hidden, experts, selected = 512, 256, 4, 2
     gate = synth.matrix(12, 31, hidden * experts, channels)

@@ -371,12 +371,27 @@ def planar_moe_gate_up_swiglu_m8(dev, w, ids, x, tokens, selected, h=None, **str
     return h
 
 
-def planar_moe_routed_m8(dev, w, ids, x, tokens, selected, h=None, y=None, **strides):
+class SharedRows(C.Structure):
+    _fields_ = [("gate", C.c_void_p), ("up", C.c_void_p), ("down", C.c_void_p), ("h", C.c_void_p), ("h_stride_bytes", C.c_uint64),
+                ("y", C.c_void_p), ("y_stride_bytes", C.c_uint64)]
+
+
+def planar_moe_routed_m8(dev, w, ids, x, tokens, selected, h=None, y=None, shared=None, shared_h=None, shared_y=None, shared_y_stride=None,
+                         **strides):
+    """`planar_moe_routed_m8`; with `shared` (a PlanarSharedExpert) the always-on expert rides in the same launches and
+    its rows [tokens, channels] come back as the third result."""
     h = dev.empty((tokens * selected, w.hidden)) if h is None else h
     y = dev.empty((tokens * selected, w.channels)) if y is None else y
     m = _small_moe(dev, w, ids, x, tokens, selected, h, y, **strides)
-    check(dll().tsp_planar_moe_routed_m8(C.byref(m), dev.stream()))
-    return h, y
+    if shared is None:
+        check(dll().tsp_planar_moe_routed_m8(C.byref(m), dev.stream()))
+        return h, y
+    shared_h = dev.empty((tokens, w.hidden)) if shared_h is None else shared_h
+    shared_y = dev.empty((tokens, w.channels)) if shared_y is None else shared_y
+    e = SharedRows(shared.gate.data_ptr(), shared.up.data_ptr(), shared.down.data_ptr(), shared_h.data_ptr(), w.hidden * 4,
+                   shared_y.data_ptr(), w.channels * 4 if shared_y_stride is None else shared_y_stride)
+    check(dll().tsp_planar_moe_routed_m8_shared(C.byref(m), C.byref(e), dev.stream()))
+    return h, y, shared_y
 
 
 class GroupedMoe(C.Structure):

@@ -408,15 +408,22 @@ uint32_t record_slots(const SmallMoeArgs& a) {
     return routes < 128 ? routes : 128;
 }
 
-SkinnyMoe skinny_view(const SmallMoeArgs& a) {
-    return SkinnyMoe{a.pair_lo, a.pair_hi, a.down, a.ids, a.meta, a.x, a.h, a.y, a.x_stride, a.h_stride, a.y_stride,
-                     a.channels, a.hidden, a.experts, a.selected, a.tokens, record_slots(a), a.gu, a.dn, a.error_word};
+SkinnyMoe skinny_view(const SmallMoeArgs& a, const tsp_shared_rows* shared = nullptr) {
+    SkinnyMoe v{a.pair_lo, a.pair_hi, a.down, a.ids, a.meta, a.x, a.h, a.y, a.x_stride, a.h_stride, a.y_stride,
+                a.channels, a.hidden, a.experts, a.selected, a.tokens, record_slots(a), a.gu, a.dn, a.error_word};
+    if (shared) {
+        v.shared_gate = static_cast<const uint8_t*>(shared->gate); v.shared_up = static_cast<const uint8_t*>(shared->up);
+        v.shared_down = static_cast<const uint8_t*>(shared->down);
+        v.shared_h = shared->h; v.shared_h_stride = shared->h_stride_bytes; v.shared_y = shared->y; v.shared_y_stride = shared->y_stride_bytes;
+    }
+    return v;
 }
 
-int launch_gate_up(const SmallMoeArgs& a, hipStream_t s) {
+int launch_gate_up(const SmallMoeArgs& a, hipStream_t s, const tsp_shared_rows* shared = nullptr) {
     const uint32_t records = record_slots(a);
     if (skinny_moe_supported(a.gu.source_type, a.dn.source_type, a.channels, a.hidden, a.x, a.x_stride, a.h, a.h_stride, false))
-        return skinny_moe_gate_up(skinny_view(a), s);
+        return skinny_moe_gate_up(skinny_view(a, shared), s);
+    TSP_REQUIRE(!shared, "the always-on expert rides only on the matrix-core small-row kernels");
     const bool x_aligned = reinterpret_cast<uintptr_t>(a.x) % 16 == 0 && a.x_stride % 16 == 0;
     if (a.gu.source_type == 12 && x_aligned && (a.channels == 512 || a.channels == 1024 || a.channels == 2048)) {
         const uint32_t bpr = a.channels / 256;
@@ -442,10 +449,11 @@ int launch_gate_up(const SmallMoeArgs& a, hipStream_t s) {
     return launch_status("gate_up_generic");
 }
 
-int launch_down(const SmallMoeArgs& a, hipStream_t s) {
+int launch_down(const SmallMoeArgs& a, hipStream_t s, const tsp_shared_rows* shared = nullptr) {
     const uint32_t records = record_slots(a);
     if (a.dn.source_type == 14 && a.hidden % 256 == 0 && a.hidden <= 2048 && reinterpret_cast<uintptr_t>(a.h) % 16 == 0 && a.h_stride % 16 == 0)
-        return skinny_moe_down(skinny_view(a), s);
+        return skinny_moe_down(skinny_view(a, shared), s);
+    TSP_REQUIRE(!shared, "the always-on expert rides only on the matrix-core small-row kernels");
     const bool h_aligned = reinterpret_cast<uintptr_t>(a.h) % 16 == 0 && a.h_stride % 16 == 0;
     if (a.dn.source_type == 14 && h_aligned && (a.hidden == 256 || a.hidden == 512 || a.hidden == 1024)) {
         const uint32_t bpr = a.hidden / 256;
@@ -496,4 +504,39 @@ extern "C" int tsp_planar_moe_routed_m8(const tsp_small_moe* m, void* stream) {
     rc = launch_gate_up(a, s);
     if (rc != TSP_OK) return rc;
     return launch_down(a, s);
+}
+
+extern "C" int tsp_planar_moe_routed_m8_shared(const tsp_small_moe* m, const tsp_shared_rows* shared, void* stream) {
+    TSP_REQUIRE(shared, "null shared expert description");
+    SmallMoeArgs a{};
+    int rc = fill_common(m, &a, true);
+    if (rc != TSP_OK) return rc;
+    TSP_REQUIRE(shared->gate && shared->up && shared->down && shared->h && shared->y, "null device pointer");
+    TSP_REQUIRE(skinny_moe_supported(a.gu.source_type, a.dn.source_type, a.channels, a.hidden, a.x, a.x_stride, a.h, a.h_stride, true) &&
+                    a.gu.source_type == 12 && a.dn.source_type == 14,
+                "the always-on expert rides only with Q4_K co-located gate/up and Q6_K planes down, 16-byte aligned rows");
+    TSP_REQUIRE(reinterpret_cast<uintptr_t>(shared->gate) % 16 == 0 && reinterpret_cast<uintptr_t>(shared->up) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(shared->down) % 16 == 0 && reinterpret_cast<uintptr_t>(shared->h) % 16 == 0 &&
+                    shared->h_stride_bytes % 16 == 0 && shared->h_stride_bytes >= uint64_t(m->hidden) * 4 && shared->y_stride_bytes % 4 == 0 &&
+                    shared->y_stride_bytes >= uint64_t(m->channels) * 4,
+                "planar v3 small MoE shape or stride mismatch");
+    const uint64_t h_span = uint64_t(m->tokens - 1) * shared->h_stride_bytes + uint64_t(m->hidden) * 4;
+    const uint64_t y_span = uint64_t(m->tokens - 1) * shared->y_stride_bytes + uint64_t(m->channels) * 4;
+    const uint32_t routes = m->tokens * m->selected;
+    const void* others[] = {m->x, m->ids, m->h, m->y, shared->gate, shared->up, shared->down, m->union_meta};
+    const uint64_t spans[] = {uint64_t(m->tokens - 1) * m->x_stride_bytes + uint64_t(m->channels) * 4, uint64_t(routes) * 4,
+                              uint64_t(routes - 1) * m->h_stride_bytes + uint64_t(m->hidden) * 4, uint64_t(routes - 1) * m->y_stride_bytes + uint64_t(m->channels) * 4,
+                              a.gu.planar_expert_bytes, a.gu.planar_expert_bytes, a.dn.planar_expert_bytes, m->union_meta ? 9280u : 0u};
+    for (int i = 0; i < 8; ++i)
+        TSP_REQUIRE(!ranges_overlap(shared->h, h_span, others[i], spans[i]) && !ranges_overlap(shared->y, y_span, others[i], spans[i]),
+                    "planar v3 small MoE outputs overlap inputs");
+    TSP_REQUIRE(!ranges_overlap(shared->h, h_span, shared->y, y_span), "planar v3 small MoE outputs overlap inputs");
+    const auto s = static_cast<hipStream_t>(stream);
+    if (m->tokens > 1) {
+        rc = tsp_planar_union_build(m->ids, m->union_meta, m->experts, m->selected, m->tokens, m->hidden, m->channels, m->error_word, stream);
+        if (rc != TSP_OK) return rc;
+    }
+    rc = launch_gate_up(a, s, shared);
+    if (rc != TSP_OK) return rc;
+    return launch_down(a, s, shared);
 }

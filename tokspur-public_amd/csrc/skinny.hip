@@ -46,14 +46,31 @@ struct SkinnyArgs {
     float* out;            // rows out_stride bytes apart
     uint64_t out_stride;
     uint32_t* error_word;
+    // an always-on expert riding in the same launch: the workgroups of task index `shared_index` take every token as a
+    // row, these weights (gate / up, or down in shared_w0), these input rows and these output rows
+    const uint8_t* shared_w0;
+    const uint8_t* shared_w1;
+    const float* shared_x;
+    uint64_t shared_x_stride;
+    float* shared_out;
+    uint64_t shared_out_stride;
+    uint32_t shared_index;
 };
+
+// The always-on expert's task: row k is token k.
+__device__ __forceinline__ bool is_shared_task(const SkinnyArgs& a, uint32_t index) { return a.shared_w0 != nullptr && index == a.shared_index; }
 
 struct Task { uint32_t expert, count, src[kRows], dst[kRows]; };
 
 // Task `index`: the dense rows, a union record, or a single route when there is no union block.
 template <int SRC>
 __device__ __forceinline__ bool load_task(const SkinnyArgs& a, uint32_t index, Task& t) {
-    if constexpr (SRC == SRC_DENSE) {
+    if (is_shared_task(a, index)) {
+        t.expert = 0; t.count = a.tokens;
+#pragma unroll
+        for (int k = 0; k < kRows; ++k) t.src[k] = t.dst[k] = uint32_t(k) < a.tokens ? k : 0;
+        return a.tokens <= kRows;
+    } else if constexpr (SRC == SRC_DENSE) {
         t.expert = 0; t.count = a.m;
 #pragma unroll
         for (int k = 0; k < kRows; ++k) t.src[k] = t.dst[k] = k;
@@ -84,7 +101,10 @@ __device__ __forceinline__ bool load_task(const SkinnyArgs& a, uint32_t index, T
 // slices' partial sums meet in LDS at the end (fixed order, so results do not depend on timing). With about one task
 // tile per compute unit, slicing K is what puts more than one wave on each SIMD.
 template <int BKIND, int OUT, int SRC, int KS>
-__global__ __launch_bounds__(256 * KS, 2) void skinny_kernel(SkinnyArgs a) {
+__global__ __launch_bounds__(256 * KS, 2) void skinny_kernel(SkinnyArgs args) {
+    SkinnyArgs a = args;
+    const bool shared = is_shared_task(a, blockIdx.y);
+    if (shared) { a.x = a.shared_x; a.x_stride = a.shared_x_stride; a.out = a.shared_out; a.out_stride = a.shared_out_stride; }
     constexpr bool Q6 = BKIND == B_Q6K_PLANAR;
     constexpr uint32_t THREADS = 256 * KS;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [hi plane][lo plane][activation sums]
@@ -173,7 +193,8 @@ __global__ __launch_bounds__(256 * KS, 2) void skinny_kernel(SkinnyArgs a) {
         const uint32_t unit = blockIdx.x * 128 + wave * 32 + col;
         const uint32_t half_e = a.experts / 2;
         const uint8_t* pair = (task.expert < half_e ? a.w0 : a.w1) + uint64_t(task.expert < half_e ? task.expert : task.expert - half_e) * 2 * a.spec.planar_expert_bytes;
-        wbase[0] = pair; wbase[1] = pair + a.spec.planar_expert_bytes;
+        wbase[0] = shared ? a.shared_w0 : pair;
+        wbase[1] = shared ? a.shared_w1 : pair + a.spec.planar_expert_bytes;
         col_live[0] = col_live[1] = unit < a.n;
         wrow[0] = wrow[1] = col_live[0] ? unit : a.n - 1;
         out_col[0] = out_col[1] = unit;
@@ -184,7 +205,7 @@ __global__ __launch_bounds__(256 * KS, 2) void skinny_kernel(SkinnyArgs a) {
             col_live[j] = n < a.n;
             wrow[j] = col_live[j] ? n : a.n - 1;
             out_col[j] = n;
-            wbase[j] = BKIND == B_Q4K_RAW ? a.w0 : a.w0 + uint64_t(task.expert) * a.spec.planar_expert_bytes;
+            wbase[j] = shared ? a.shared_w0 : BKIND == B_Q4K_RAW ? a.w0 : a.w0 + uint64_t(task.expert) * a.spec.planar_expert_bytes;
         }
     }
 
@@ -373,7 +394,10 @@ constexpr uint32_t kSlice = 256;                                       // column
 constexpr uint32_t kWaveLds = 2 * kRows * kSlice * 2 + kRows * 32;      // hi plane, lo plane, sub-block sums: 8 448 B
 
 template <int BKIND, int OUT, int SRC>
-__global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs a) {  // four waves per SIMD: <= 128 registers per lane
+__global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // four waves per SIMD: <= 128 registers per lane
+    SkinnyArgs a = args;
+    const bool shared = is_shared_task(a, blockIdx.y);
+    if (shared) { a.x = a.shared_x; a.x_stride = a.shared_x_stride; a.out = a.shared_out; a.out_stride = a.shared_out_stride; }
     constexpr bool Q6 = BKIND == B_Q6K_PLANAR;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [wave][hi plane][lo plane][sums]; partial sums over it at the end
 
@@ -406,7 +430,8 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs a) {  // four w
         const uint32_t unit = (blockIdx.x * ucols + ucol) * 32 + col;
         const uint32_t half_e = a.experts / 2;
         const uint8_t* pair = (task.expert < half_e ? a.w0 : a.w1) + uint64_t(task.expert < half_e ? task.expert : task.expert - half_e) * 2 * a.spec.planar_expert_bytes;
-        wbase[0] = pair; wbase[1] = pair + a.spec.planar_expert_bytes;
+        wbase[0] = shared ? a.shared_w0 : pair;
+        wbase[1] = shared ? a.shared_w1 : pair + a.spec.planar_expert_bytes;
         col_live[0] = col_live[1] = unit < a.n;
         wrow[0] = wrow[1] = col_live[0] ? unit : a.n - 1;
         out_col[0] = out_col[1] = unit;
@@ -417,7 +442,7 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs a) {  // four w
             col_live[j] = n < a.n;
             wrow[j] = col_live[j] ? n : a.n - 1;
             out_col[j] = n;
-            wbase[j] = a.w0 + uint64_t(task.expert) * a.spec.planar_expert_bytes;
+            wbase[j] = shared ? a.shared_w0 : a.w0 + uint64_t(task.expert) * a.spec.planar_expert_bytes;
         }
     }
     struct BlockQ6 { u32x4 la[2], lb[2], qh[2]; uint32_t sc[4]; float d; };
@@ -689,7 +714,11 @@ int skinny_moe_gate_up(const SkinnyMoe& m, hipStream_t s) {
     a.x = m.x; a.x_stride = m.x_stride; a.w0 = m.pair_lo; a.w1 = m.pair_hi; a.spec = m.gu; a.experts = m.experts; a.selected = m.selected;
     a.tokens = m.tokens; a.ids = m.ids; a.meta = m.meta; a.n = m.hidden; a.k = m.channels; a.out = m.h; a.out_stride = m.h_stride;
     a.error_word = m.error_word;
-    return launch<B_Q4K_PLANAR, OUT_SWIGLU, SRC_RECORD_TOKENS>("skinny_gate_up_swiglu", a, (m.hidden + 127) / 128, m.records, s);
+    if (m.shared_gate) {
+        a.shared_w0 = m.shared_gate; a.shared_w1 = m.shared_up; a.shared_x = m.x; a.shared_x_stride = m.x_stride;
+        a.shared_out = m.shared_h; a.shared_out_stride = m.shared_h_stride; a.shared_index = m.records;
+    }
+    return launch<B_Q4K_PLANAR, OUT_SWIGLU, SRC_RECORD_TOKENS>("skinny_gate_up_swiglu", a, (m.hidden + 127) / 128, m.records + (m.shared_gate ? 1 : 0), s);
 }
 
 int skinny_moe_down(const SkinnyMoe& m, hipStream_t s) {
@@ -697,7 +726,11 @@ int skinny_moe_down(const SkinnyMoe& m, hipStream_t s) {
     a.x = m.h; a.x_stride = m.h_stride; a.w0 = m.down; a.spec = m.dn; a.experts = m.experts; a.selected = m.selected;
     a.tokens = m.tokens; a.ids = m.ids; a.meta = m.meta; a.n = m.channels; a.k = m.hidden; a.out = m.y; a.out_stride = m.y_stride;
     a.error_word = m.error_word;
-    return launch<B_Q6K_PLANAR, OUT_ROWS, SRC_RECORD_ROUTES>("skinny_down", a, (m.channels + 255) / 256, m.records, s);
+    if (m.shared_down) {
+        a.shared_w0 = m.shared_down; a.shared_x = m.shared_h; a.shared_x_stride = m.shared_h_stride;
+        a.shared_out = m.shared_y; a.shared_out_stride = m.shared_y_stride; a.shared_index = m.records;
+    }
+    return launch<B_Q6K_PLANAR, OUT_ROWS, SRC_RECORD_ROUTES>("skinny_down", a, (m.channels + 255) / 256, m.records + (m.shared_down ? 1 : 0), s);
 }
 
 }  // namespace tsp

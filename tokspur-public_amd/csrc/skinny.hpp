@@ -17,6 +17,13 @@ struct SkinnyMoe {
     uint32_t channels, hidden, experts, selected, tokens, records;
     tsp_planar_spec gu, dn;
     uint32_t* error_word;
+    // optional always-on expert riding in the same launches (one Pack v3 expert each; rows = the tokens)
+    const uint8_t* shared_gate = nullptr;
+    const uint8_t* shared_up = nullptr;
+    const uint8_t* shared_down = nullptr;
+    float* shared_h = nullptr;  // [tokens, hidden]
+    float* shared_y = nullptr;  // [tokens, channels]
+    uint64_t shared_h_stride = 0, shared_y_stride = 0;
 };
 
 // Q4_K co-located gate/up (and Q6_K planar down when with_down), columns a multiple of 256 up to 2048, 16-byte aligned rows.
