@@ -352,7 +352,7 @@ void test_encode_moe_batch() {
     encode_moe_batch(g, m.w, scratch, dl, {dx, T, f.shape.channels, uint64_t(stride) * 4}, {dy, T, f.shape.channels, uint64_t(stride) * 4}, f.shape,
                      RouterMode::softmax, true);
     const BatchResult r = g.submit();
-    EXPECT(r.dispatches == 5 && g.memory().allocations == allocations);
+    EXPECT(r.dispatches == 4 && g.memory().allocations == allocations);  // route, grouped MoE with the shared expert riding, shared router, mixture
     const auto y = read_as<float>(g, dy);
     double worst = 0;
     bool pads = true;

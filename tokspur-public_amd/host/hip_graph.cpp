@@ -265,7 +265,7 @@ void HipGraph::prepare_planar_moe_v3(uint32_t gate_up_encoding, uint32_t down_en
     if (!impl_->union_meta) impl_->union_meta = impl_->raw(9280);
     if (prepare_nax) {
         const uint32_t channels = (max_channels + 255) / 256 * 256, hidden = (max_hidden + 255) / 256 * 256;
-        const uint64_t bytes = tsp_planar_nax_workspace_bytes(max_nax_tokens, max_selected, max_experts, channels, hidden);
+        const uint64_t bytes = tsp_planar_nax_shared_workspace_bytes(max_nax_tokens, max_selected, max_experts, channels, hidden);  // room for an always-on expert's rows too
         if (bytes > impl_->nax_workspace_bytes) {
             require(impl_->nax_workspace == nullptr, "planar v3 NAX scratch is sized once");
             impl_->nax_workspace = impl_->raw(bytes);
@@ -484,7 +484,7 @@ void HipGraph::planar_moe_routed_m8(GpuView pair_lo, GpuView pair_hi, GpuView do
 
 void HipGraph::planar_nax_grouped_moe(GpuView pair_lo, GpuView pair_hi, GpuView down_weights, GpuView indices, GpuRowsF32 input,
                                       GpuRowsF32 expert_down, GpuView token_map, GpuView counts, GpuView tasks, uint32_t experts,
-                                      uint32_t selected) {
+                                      uint32_t selected, const SharedPlanarExpert* shared) {
     auto& p = *impl_; p.active();
     const PlanarEntry* lo = p.planar_of(pair_lo);
     const PlanarEntry* hi = p.planar_of(pair_hi);
@@ -500,7 +500,8 @@ void HipGraph::planar_nax_grouped_moe(GpuView pair_lo, GpuView pair_hi, GpuView 
     require(token_map.bytes >= checked_mul(checked_mul(experts, tokens), 4) && counts.bytes >= uint64_t(experts) * 4 &&
                 tasks.bytes >= (2 + 2 * (uint64_t(tokens) * selected / 32 + experts)) * 4,
             "planar v3 NAX grouped MoE routing scratch too small");
-    const uint64_t need = tsp_planar_nax_workspace_bytes(tokens, selected, experts, input.columns, lo->shape.rows);
+    const uint64_t need = shared ? tsp_planar_nax_shared_workspace_bytes(tokens, selected, experts, input.columns, lo->shape.rows)
+                                 : tsp_planar_nax_workspace_bytes(tokens, selected, experts, input.columns, lo->shape.rows);
     require(need <= p.nax_workspace_bytes, "planar v3 NAX scratch too small for requested batch");
     validate_disjoint(std::array{pair_lo, pair_hi, down_weights, indices, input.view}, std::array{expert_down.view, token_map, counts, tasks});
     tsp_grouped_moe m{};
@@ -514,7 +515,28 @@ void HipGraph::planar_nax_grouped_moe(GpuView pair_lo, GpuView pair_hi, GpuView 
     m.counts = reinterpret_cast<uint32_t*>(p.device(counts, true));
     m.tasks = reinterpret_cast<uint32_t*>(p.device(tasks, true));
     m.workspace = p.nax_workspace; m.workspace_bytes = p.nax_workspace_bytes; m.error_word = p.error_word;
-    check(tsp_planar_nax_grouped_moe(&m, p.stream));
+    if (!shared) {
+        check(tsp_planar_nax_grouped_moe(&m, p.stream));
+        return;
+    }
+    const PlanarEntry* sp = p.planar_of(shared->pair);
+    const PlanarEntry* sd = p.planar_of(shared->down);
+    require(sp && sd, "planar v3 NAX grouped MoE requires registered matrices and prepared scratch");
+    p.rows_fit(shared->rows, "planar v3 NAX grouped MoE shape or stride mismatch");
+    require(sp->shape.kind == lo->shape.kind && sd->shape.kind == dn->shape.kind && sp->shape.columns == lo->shape.columns &&
+                sp->shape.rows == lo->shape.rows && sd->shape.columns == dn->shape.columns && sd->shape.rows == dn->shape.rows &&
+                shared->rows.rows == tokens && shared->rows.columns == input.columns,
+            "planar v3 NAX grouped MoE shape or stride mismatch");
+    validate_disjoint(std::array{pair_lo, pair_hi, down_weights, indices, input.view, shared->pair, shared->down},
+                      std::array{expert_down.view, token_map, counts, tasks, shared->rows.view});
+    tsp_planar_spec gu{};
+    check(tsp_make_expert_spec(12, input.columns, lo->shape.rows, &gu));
+    tsp_shared_expert e{};
+    e.gate = p.device(shared->pair);                                             // a co-located pair tensor holds [gate_0, up_0, gate_1, ...]
+    e.up = static_cast<const uint8_t*>(e.gate) + gu.planar_expert_bytes;
+    e.down = p.device(shared->down);
+    e.y = reinterpret_cast<float*>(p.device(shared->rows.view, true)); e.y_stride_bytes = shared->rows.stride_bytes;
+    check(tsp_planar_nax_grouped_moe_shared(&m, &e, p.stream));
 }
 
 void HipGraph::prepare_grouped_mm(uint32_t encoding, PrefillWeightLayout layout, uint32_t max_tokens, uint32_t max_selected, uint32_t max_experts,
@@ -730,13 +752,25 @@ void encode_moe_batch(HipGraph& graph, const MoeWeights& w, const MoeBatchScratc
     shape_check(shape);
     const uint32_t tokens = input.rows;
     graph.prefill_route_batch(logits, s.indices, s.weights, shape.experts, shape.selected, tokens, mode, normalize_selected);
-    graph.planar_nax_grouped_moe(w.gate.view, w.up.view, w.down.view, s.indices, input,
-                                 {s.expert_down, tokens * shape.selected, shape.channels, uint64_t(shape.channels) * 4}, s.token_map, s.counts, s.tasks,
-                                 shape.experts, shape.selected);
-    // the shared expert is a two-expert planar stack of which every token selects expert 0 (shared_indices stay zero)
-    graph.planar_nax_grouped_moe(w.shared_gate.view, w.shared_up.view, w.shared_down.view, s.shared_indices, input,
-                                 {s.shared_down, tokens, shape.channels, uint64_t(shape.channels) * 4}, s.shared_token_map, s.shared_counts,
-                                 s.shared_tasks, 2, 1);
+    // The shared expert is expert 0 of a two-expert planar stack. Beside Q4_K / Q6_K routed experts of the same kinds it rides in
+    // their two GEMM launches; otherwise it is a grouped product of its own in which every token selects expert 0
+    // (shared_indices stay zero).
+    const auto routed = graph.planar_matrix_shape(w.gate.view), routed_down = graph.planar_matrix_shape(w.down.view);
+    const auto own = graph.planar_matrix_shape(w.shared_gate.view), own_down = graph.planar_matrix_shape(w.shared_down.view);
+    const bool rides = routed && routed_down && own && own_down && routed->kind == TSP_KIND_Q4K_COLOC_GATE && own->kind == routed->kind &&
+                       routed_down->kind == TSP_KIND_Q6K_PLANAR_X && own_down->kind == routed_down->kind;
+    const GpuRowsF32 expert_down{s.expert_down, tokens * shape.selected, shape.channels, uint64_t(shape.channels) * 4};
+    const GpuRowsF32 shared_rows{s.shared_down, tokens, shape.channels, uint64_t(shape.channels) * 4};
+    if (rides) {
+        const HipGraph::SharedPlanarExpert shared{w.shared_gate.view, w.shared_down.view, shared_rows};
+        graph.planar_nax_grouped_moe(w.gate.view, w.up.view, w.down.view, s.indices, input, expert_down, s.token_map, s.counts, s.tasks,
+                                     shape.experts, shape.selected, &shared);
+    } else {
+        graph.planar_nax_grouped_moe(w.gate.view, w.up.view, w.down.view, s.indices, input, expert_down, s.token_map, s.counts, s.tasks,
+                                     shape.experts, shape.selected);
+        graph.planar_nax_grouped_moe(w.shared_gate.view, w.shared_up.view, w.shared_down.view, s.shared_indices, input, shared_rows,
+                                     s.shared_token_map, s.shared_counts, s.shared_tasks, 2, 1);
+    }
     graph.gemv_rows(w.shared_router.encoding, w.shared_router.view, input, {s.shared_logit, tokens, 1, 4});
     graph.prefill_mixture_batch(s.expert_down, s.weights, s.shared_down, s.shared_logit, output, shape.selected);
 }

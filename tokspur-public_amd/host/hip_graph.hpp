@@ -132,9 +132,13 @@ public:
                                       GpuRowsF32 expert_hidden, uint32_t experts, uint32_t selected);               // graph.hpp:472
     void planar_moe_routed_m8(GpuView pair_lo, GpuView pair_hi, GpuView down_weights, GpuView indices, GpuRowsF32 input,
                               GpuRowsF32 expert_hidden, GpuRowsF32 expert_down, uint32_t experts, uint32_t selected);  // 475
+    // `shared` (not in the engine's signature): an always-on expert kept in the routed experts' formats rides in the two GEMM
+    // launches, every token one of its rows. Its gate and up are expert 0 of a registered co-located pair tensor, its down
+    // expert 0 of a registered Q6_K planes tensor; `rows` [tokens, channels] receives down(silu(gate x) * up x).
+    struct SharedPlanarExpert { GpuView pair; GpuView down; GpuRowsF32 rows; };
     void planar_nax_grouped_moe(GpuView pair_lo, GpuView pair_hi, GpuView down_weights, GpuView indices, GpuRowsF32 input,
                                 GpuRowsF32 expert_down, GpuView token_map, GpuView counts, GpuView tasks, uint32_t experts,
-                                uint32_t selected);                                                                  // graph.hpp:478
+                                uint32_t selected, const SharedPlanarExpert* shared = nullptr);                      // graph.hpp:478
     // graph.hpp:750-753 `prepare_grouped_mm` / `grouped_mm`: raw GGUF Q4_K expert stacks, one output row per route
     void prepare_grouped_mm(uint32_t encoding, PrefillWeightLayout layout, uint32_t max_tokens = 2048, uint32_t max_selected = 10,
                             uint32_t max_experts = 512, uint32_t max_columns = 2560);
