@@ -449,8 +449,8 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
     struct BlockQ4 { u32x4 pair[4]; HdrQ4 hdr; };
     using Block = std::conditional_t<Q6, BlockQ6, BlockQ4>;
     Block cur[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    auto load_tile = [&](auto j_tag) {
+        constexpr int j = decltype(j_tag)::value;
         const uint64_t at = uint64_t(wrow[j]) * bpr + slice;
         if constexpr (Q6) {
             const uint8_t* ql = wbase[j] + a.spec.qs_offset + at * 128 + khalf * 16;
@@ -471,8 +471,11 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
             for (int p = 0; p < 4; ++p) cur[j].pair[p] = *reinterpret_cast<const u32x4*>(qs + p * 32);
             cur[j].hdr = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, slice);
         }
-    }
-
+    };
+    // Q6_K blocks are 29 registers per tile: with the 32 of the activation rows both tiles at once do not fit the 128 of
+    // four waves per SIMD, so the second tile is requested once the rows are staged (it queues behind the first anyway)
+    load_tile(std::integral_constant<int, 0>{});
+    if constexpr (!Q6) load_tile(std::integral_constant<int, 1>{});
     __builtin_amdgcn_sched_barrier(0);  // every request above is out before the first wait below
 
     // ---- stage the activation rows while the weight bytes travel
@@ -528,6 +531,10 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if constexpr (Q6) {
+        load_tile(std::integral_constant<int, 1>{});
+        __builtin_amdgcn_sched_barrier(0);
+    }
 
     f32x16 blk[2];
     float acc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};  // rows 4 * khalf + v of tile j
