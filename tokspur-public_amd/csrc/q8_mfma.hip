@@ -1,17 +1,18 @@
 // Q8_0 GEMV for up to sixteen token rows on the matrix cores (LM head, verify): y[m, r] = sum_k d[r, k/32] * q[r, k] * x[m, k].
 //
-// A Q8_0 row is a run of 34-byte blocks (f16 scale + 32 int8). The int8 quants are exact halves, so a block is two
-// 32x32x16 MFMA steps of the integer quants against the activations; the block's scale multiplies the f32 result
-// once (4 fused multiply-adds per lane for the eight live rows). The activations are scaled by a power of two and
-// split into hi + lo halves, staged once in LDS for all of K, so the result carries 22 significant bits of x: this
-// is the f32 GEMV of the engine to within f32 accumulation error, at ~1.3 VALU operations per weight byte whatever the
-// number of token rows.
+// A Q8_0 row is a run of 34-byte blocks (f16 scale + 32 int8). The int8 quants are exact halves, so a block is one
+// 16x16x32 MFMA step per 16 weight rows: the block's 32 columns are the instruction's whole K, a lane (n, kq) supplies the
+// eight quants 8 kq .. 8 kq + 7 of weight row n, and the sixteen operand rows on the other side are the token rows (eight
+// of them repeated when there are only eight). The block's scale multiplies the f32 result once (4 fused multiply-adds per
+// lane and 16 weight rows). The activations are scaled by a power of two and split into hi + lo halves, staged once in
+// LDS for all of K, so the result carries 22 significant bits of x: this is the f32 GEMV of the engine to within f32
+// accumulation error, at ~1.3 VALU operations per weight byte whatever the number of token rows.
 //
 // Raw rows are only 2-byte aligned inside, so the bytes travel global -> registers -> LDS -> registers: a wave reads
 // its 32 weight rows x 8 blocks (272 contiguous bytes per row, 16-byte aligned because 8 blocks = 17 x 16 bytes) with
 // whole-chunk loads by consecutive lanes, parks them in a wave-private LDS tile whose row stride (280 bytes) spreads
-// the rows over all banks, and each lane then picks its 16 quants of a block with aligned dword reads and a byte
-// funnel shift. The next group of 8 blocks is in flight while the current one is multiplied.
+// the rows over all banks, and each lane then picks its 8 quants of a block (for each half of the tile's 32 rows) with
+// aligned dword reads and a byte funnel shift. The next group of 8 blocks is in flight while the current one is multiplied.
 //
 // Workgroups are persistent (one per compute unit, 8 waves): the activations are staged once per workgroup, which owns
 // a contiguous share of the matrix's 32-row tiles; its waves take tiles from that share through a counter in LDS.
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     __shared__ uint32_t next_tile;
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-    const uint32_t col = lane % 32, khalf = lane / 32;
+    const uint32_t n16 = lane % 16, kq = lane / 16;  // 16x16x32 MFMA: operand row / column lane % 16, columns 8 kq .. 8 kq + 7 of the block
     // K: the columns this workgroup multiplies, starting at column k0 (group g0 of the rows)
     const uint32_t K = a.columns / KSPLIT, chunks = K / 8, groups = K / 256, row_bytes = a.columns / 32 * 34;
     const uint32_t k0 = (blockIdx.x % KSPLIT) * K, g0 = k0 / 256;
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     }
     __syncthreads();
 
-    const uint32_t arow = col & (kRows - 1);
+    const uint32_t arow = n16 & (kRows - 1);
     auto a_frag = [&](const _Float16* plane, uint32_t chunk) {
         return *reinterpret_cast<const f16x8*>(plane + (arow * chunks + (chunk ^ arow)) * 8);
     };
@@ -175,9 +176,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     }
     for (; t < share_end; t = t_next, t_next = take_tile()) {
         const uint32_t row0 = t * 32;
-        f32x16 acc;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+        float acc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};  // [16-row half of the tile][token row 4 kq + v]
         // one item: its bytes go registers -> LDS tile, the item DEPTH ahead is requested into the freed registers, then the
         // tile is multiplied.
         auto item = [&](uint32_t g, auto set_tag) {
@@ -189,33 +188,42 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
             const uint32_t following = wraps && more ? t_next : t;
             const uint32_t group = !wraps ? ahead : more ? ahead - groups : g;
             fetch_group(following * 32, group, set_tag);
-            const uint8_t* mine = tile + col * kTileStride + khalf * 16;
+            const uint8_t* mine = tile + n16 * kTileStride + kq * 8;
             auto block = [&](auto b_tag) {
                 constexpr int B = decltype(b_tag)::value;
-                // quants at byte 34 B + 2 + 16 h of the row: dword aligned for odd B, 2 bytes past a dword for even B
+                // the lane's eight quants of the block, for rows n16 and n16 + 16 of the tile: bytes 34 B + 2 + 8 kq .. + 8 of the
+                // row, dword aligned for odd B, 2 bytes past a dword for even B
                 constexpr uint32_t Q_AT = 34 * B + 2, ALIGNED = Q_AT & ~3u;
-                uint32_t w[4];
-                if constexpr (Q_AT % 4 == 0) {
+                f16x8 b_frag[2];
+                float scale_d[2];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) w[i] = *reinterpret_cast<const uint32_t*>(mine + ALIGNED + 4 * i);
-                } else {
-                    uint32_t d[5];
+                for (int nt = 0; nt < 2; ++nt) {
+                    const uint8_t* row = mine + nt * 16 * kTileStride;
+                    uint32_t w[2];
+                    if constexpr (Q_AT % 4 == 0) {
+                        w[0] = *reinterpret_cast<const uint32_t*>(row + ALIGNED);
+                        w[1] = *reinterpret_cast<const uint32_t*>(row + ALIGNED + 4);
+                    } else {
+                        uint32_t d[3];
 #pragma unroll
-                    for (int i = 0; i < 5; ++i) d[i] = *reinterpret_cast<const uint32_t*>(mine + ALIGNED + 4 * i);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) w[i] = __builtin_amdgcn_alignbyte(d[i + 1], d[i], 2);
+                        for (int i = 0; i < 3; ++i) d[i] = *reinterpret_cast<const uint32_t*>(row + ALIGNED + 4 * i);
+                        w[0] = __builtin_amdgcn_alignbyte(d[1], d[0], 2);
+                        w[1] = __builtin_amdgcn_alignbyte(d[2], d[1], 2);
+                    }
+                    b_frag[nt] = quants8(w[0], w[1]);
+                    scale_d[nt] = half_bits_to_float(*reinterpret_cast<const uint16_t*>(tile + (nt * 16 + n16) * kTileStride + 34 * B));
                 }
-                const float scale_d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(tile + col * kTileStride + 34 * B));
-                const f16x8 b0 = quants8(w[0], w[1]), b1 = quants8(w[2], w[3]);
-                const uint32_t chunk = g * 32 + B * 4 + khalf * 2;  // columns g*256 + B*32 + 16h
-                const f32x16 zero{};
-                // two independent accumulation chains (hi and lo halves of the rows) per block
-                f32x16 part_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag(a_hi, chunk), b0, zero, 0, 0, 0);
-                f32x16 part_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag(a_lo, chunk), b0, zero, 0, 0, 0);
-                part_hi = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag(a_hi, chunk + 1), b1, part_hi, 0, 0, 0);
-                part_lo = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag(a_lo, chunk + 1), b1, part_lo, 0, 0, 0);
+                const uint32_t chunk = g * 32 + B * 4 + kq;  // columns g*256 + B*32 + 8 kq
+                const f16x8 ah = a_frag(a_hi, chunk), al = a_frag(a_lo, chunk);
+                const f32x4 zero{};
 #pragma unroll
-                for (int v = 0; v < kRows / 2; ++v) acc[v] = __builtin_fmaf(scale_d, part_hi[v] + part_lo[v], acc[v]);  // rows 8 * (v / 4) + 4 * khalf + v % 4
+                for (int nt = 0; nt < 2; ++nt) {
+                    // independent products of the hi and lo halves of the rows with the block's integer quants
+                    const f32x4 part_hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, b_frag[nt], zero, 0, 0, 0);
+                    const f32x4 part_lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, b_frag[nt], zero, 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[nt][v] = __builtin_fmaf(scale_d[nt], part_hi[v] + part_lo[v], acc[nt][v]);  // rows 4 kq + v
+                }
             };
             block(std::integral_constant<int, 0>{});
             block(std::integral_constant<int, 1>{});
@@ -234,15 +242,18 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
                 item(g + 3, std::integral_constant<int, 3 % DEPTH>{});
             }
         }
-        const uint32_t r = row0 + col;
 #pragma unroll
-        for (int v = 0; v < kRows / 2; ++v) {
-            const uint32_t m = 8 * (v / 4) + 4 * khalf + v % 4;
-            if (m < a.m && r < a.rows) {
-                const float val = acc[v] * inv_scale;
-                if (nonfinite(val)) bad = TSP_ERRBIT_NONFINITE;
-                if constexpr (KSPLIT == 1) a.y[uint64_t(m) * a.rows + r] = val;
-                else unsafeAtomicAdd(a.y + uint64_t(m) * a.rows + r, val);
+        for (int nt = 0; nt < 2; ++nt) {
+            const uint32_t r = row0 + nt * 16 + n16;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const uint32_t m = 4 * kq + v;  // lanes with 4 kq >= kRows hold repeats of rows 0 .. kRows - 1
+                if (m < kRows && m < a.m && r < a.rows) {
+                    const float val = acc[nt][v] * inv_scale;
+                    if (nonfinite(val)) bad = TSP_ERRBIT_NONFINITE;
+                    if constexpr (KSPLIT == 1) a.y[uint64_t(m) * a.rows + r] = val;
+                    else unsafeAtomicAdd(a.y + uint64_t(m) * a.rows + r, val);
+                }
             }
         }
     }
