@@ -398,7 +398,7 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
     SkinnyArgs a = args;
     const bool shared = is_shared_task(a, blockIdx.y);
     if (shared) { a.x = a.shared_x; a.x_stride = a.shared_x_stride; a.out = a.shared_out; a.out_stride = a.shared_out_stride; }
-    constexpr bool Q6 = BKIND == B_Q6K_PLANAR;
+    static_assert(BKIND != B_Q6K_PLANAR, "Q6_K planes take flat16_kernel");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [wave][hi plane][lo plane][sums]; partial sums over it at the end
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wv = tid / kWave;
@@ -445,44 +445,26 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
             wbase[j] = shared ? a.shared_w0 : a.w0 + uint64_t(task.expert) * a.spec.planar_expert_bytes;
         }
     }
-    struct BlockQ6 { u32x4 la[2], lb[2], qh[2]; uint32_t sc[4]; float d; };
-    struct BlockQ4 { u32x4 pair[4]; HdrQ4 hdr; };
-    using Block = std::conditional_t<Q6, BlockQ6, BlockQ4>;
+    struct Block { u32x4 pair[4]; HdrQ4 hdr; };
     Block cur[2];
     auto load_tile = [&](auto j_tag) {
         constexpr int j = decltype(j_tag)::value;
         const uint64_t at = uint64_t(wrow[j]) * bpr + slice;
-        if constexpr (Q6) {
-            const uint8_t* ql = wbase[j] + a.spec.qs_offset + at * 128 + khalf * 16;
-            const uint8_t* qh = wbase[j] + a.spec.qh_offset + at * 64 + khalf * 16;
+        constexpr uint32_t BLK = BKIND == B_Q4K_PLANAR ? 128 : 144, QS_AT = BKIND == B_Q4K_PLANAR ? 0 : 16;
+        const uint8_t* qs = wbase[j] + (BKIND == B_Q4K_PLANAR ? a.spec.qs_offset : 0) + at * BLK + QS_AT + khalf * 16;
 #pragma unroll
-            for (int sec = 0; sec < 2; ++sec) {
-                cur[j].la[sec] = *reinterpret_cast<const u32x4*>(ql + sec * 64);
-                cur[j].lb[sec] = *reinterpret_cast<const u32x4*>(ql + sec * 64 + 32);
-                cur[j].qh[sec] = *reinterpret_cast<const u32x4*>(qh + sec * 32);
-            }
-            const uint4 sc16 = *reinterpret_cast<const uint4*>(wbase[j] + a.spec.sm_offset + at * 16);
-            cur[j].sc[0] = sc16.x; cur[j].sc[1] = sc16.y; cur[j].sc[2] = sc16.z; cur[j].sc[3] = sc16.w;
-            cur[j].d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(wbase[j] + a.spec.dm_offset + at * 2));
-        } else {
-            constexpr uint32_t BLK = BKIND == B_Q4K_PLANAR ? 128 : 144, QS_AT = BKIND == B_Q4K_PLANAR ? 0 : 16;
-            const uint8_t* qs = wbase[j] + (BKIND == B_Q4K_PLANAR ? a.spec.qs_offset : 0) + at * BLK + QS_AT + khalf * 16;
-#pragma unroll
-            for (int p = 0; p < 4; ++p) cur[j].pair[p] = *reinterpret_cast<const u32x4*>(qs + p * 32);
-            cur[j].hdr = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, slice);
-        }
+        for (int p = 0; p < 4; ++p) cur[j].pair[p] = *reinterpret_cast<const u32x4*>(qs + p * 32);
+        cur[j].hdr = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, slice);
     };
-    // Q6_K blocks are 29 registers per tile: with the 32 of the activation rows both tiles at once do not fit the 128 of
-    // four waves per SIMD, so the second tile is requested once the rows are staged (it queues behind the first anyway)
     load_tile(std::integral_constant<int, 0>{});
-    if constexpr (!Q6) load_tile(std::integral_constant<int, 1>{});
+    load_tile(std::integral_constant<int, 1>{});
     __builtin_amdgcn_sched_barrier(0);  // every request above is out before the first wait below
 
     // ---- stage the activation rows while the weight bytes travel
     uint8_t* const mine = lds + wv * kWaveLds;
     _Float16* const a_hi = reinterpret_cast<_Float16*>(mine);
     _Float16* const a_lo = a_hi + kRows * kSlice;
-    _Float16* const sums = a_lo + kRows * kSlice;  // [row][8 hi, 8 lo] of (sub-block sum / 32), Q4_K only
+    _Float16* const sums = a_lo + kRows * kSlice;  // [row][8 hi, 8 lo] of (sub-block sum / 32)
     float biggest = 0;
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
@@ -514,27 +496,21 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
         const uint32_t at = (r * 32 + ((lane / 2) ^ r)) * 8 + (lane % 2) * 4;
         *reinterpret_cast<f16x4*>(a_hi + at) = hi;
         *reinterpret_cast<f16x4*>(a_lo + at) = lo;
-        if constexpr (!Q6) {
-            float sum = (s4[0] + s4[1]) + (s4[2] + s4[3]);  // eight neighbouring lanes hold one 32-column sub-block
-            sum += __shfl_xor(sum, 1, kWave);
-            sum += __shfl_xor(sum, 2, kWave);
-            sum += __shfl_xor(sum, 4, kWave);
-            if (lane % 8 == 0) {
-                const float s32 = sum * 0.03125f;
-                const _Float16 h = _Float16(s32);
-                sums[r * 16 + lane / 8] = h;
-                sums[r * 16 + 8 + lane / 8] = _Float16(s32 - float(h));
-            }
+        float sum = (s4[0] + s4[1]) + (s4[2] + s4[3]);  // eight neighbouring lanes hold one 32-column sub-block
+        sum += __shfl_xor(sum, 1, kWave);
+        sum += __shfl_xor(sum, 2, kWave);
+        sum += __shfl_xor(sum, 4, kWave);
+        if (lane % 8 == 0) {
+            const float s32 = sum * 0.03125f;
+            const _Float16 h = _Float16(s32);
+            sums[r * 16 + lane / 8] = h;
+            sums[r * 16 + 8 + lane / 8] = _Float16(s32 - float(h));
         }
     }
     // the planes are read back by other lanes of this same wave only: LDS serves a wave's requests in order
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    if constexpr (Q6) {
-        load_tile(std::integral_constant<int, 1>{});
-        __builtin_amdgcn_sched_barrier(0);
-    }
 
     f32x16 blk[2];
     float acc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};  // rows 4 * khalf + v of tile j
@@ -562,59 +538,31 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
             acc[1][v4] = __builtin_fmaf(d1, blk[1][v4], acc[1][v4]);
         }
     };
-    if constexpr (Q6) {
-        auto section = [&](auto sec_tag) {
-            constexpr int SEC = decltype(sec_tag)::value;
-            RawQ6 raw[2];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                raw[j].la = cur[j].la[SEC]; raw[j].lb = cur[j].lb[SEC]; raw[j].qh = cur[j].qh[SEC];
-                raw[j].sc[0] = cur[j].sc[SEC * 2]; raw[j].sc[1] = cur[j].sc[SEC * 2 + 1];
-            }
-            auto quarter = [&](auto q_tag) {
-                constexpr int Q = decltype(q_tag)::value;
-                f16x8 f0[2], f1[2];
-                frags_q6k<Q>(raw[0], khalf, f0);
-                frags_q6k<Q>(raw[1], khalf, f1);
-                const uint32_t chunk = SEC * 16 + Q * 4 + khalf * 2;  // columns SEC*128 + Q*32 + 16h of the slice
-                mfma(chunk, f0[0], f1[0], SEC == 0 && Q == 0);
-                mfma(chunk + 1, f0[1], f1[1], false);
-            };
-            quarter(std::integral_constant<int, 0>{});
-            quarter(std::integral_constant<int, 1>{});
-            quarter(std::integral_constant<int, 2>{});
-            quarter(std::integral_constant<int, 3>{});
-        };
-        section(std::integral_constant<int, 0>{});
-        section(std::integral_constant<int, 1>{});
-        fold(cur[0].d, cur[1].d);
-    } else {
-        auto pair_step = [&](auto p_tag) {
-            constexpr int P = decltype(p_tag)::value;
-            f16x8 f0[2], f1[2];
-            const uint32_t chunk = P * 8 + khalf * 2;  // columns P*64 + 16h of the slice
-            frags_q4k<P, 0>(cur[0].pair[P], cur[0].hdr, f0);
-            frags_q4k<P, 0>(cur[1].pair[P], cur[1].hdr, f1);
-            mfma(chunk, f0[0], f1[0], P == 0);
-            mfma(chunk + 1, f0[1], f1[1], false);
-            frags_q4k<P, 1>(cur[0].pair[P], cur[0].hdr, f0);
-            frags_q4k<P, 1>(cur[1].pair[P], cur[1].hdr, f1);
-            mfma(chunk + 4, f0[0], f1[0], false);
-            mfma(chunk + 5, f0[1], f1[1], false);
-        };
-        pair_step(std::integral_constant<int, 0>{});
-        pair_step(std::integral_constant<int, 1>{});
-        pair_step(std::integral_constant<int, 2>{});
-        pair_step(std::integral_constant<int, 3>{});
-        fold(cur[0].hdr.d, cur[1].hdr.d);
-        // minima: acc -= 32 * dmin * sum_s (Sx / 32)(hi + lo)[m, s] * mn[n, s]
-        const f16x8 m0 = minima_frag(cur[0].hdr), m1 = minima_frag(cur[1].hdr);
-        const f16x8 sf = *reinterpret_cast<const f16x8*>(sums + arow * 16 + khalf * 8);
-        const f32x16 zero{};
-        blk[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m0, zero, 0, 0, 0);
-        blk[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m1, zero, 0, 0, 0);
-        fold(-32.0f * cur[0].hdr.dmin, -32.0f * cur[1].hdr.dmin);
-    }
+    auto pair_step = [&](auto p_tag) {
+        constexpr int P = decltype(p_tag)::value;
+        f16x8 f0[2], f1[2];
+        const uint32_t chunk = P * 8 + khalf * 2;  // columns P*64 + 16h of the slice
+        frags_q4k<P, 0>(cur[0].pair[P], cur[0].hdr, f0);
+        frags_q4k<P, 0>(cur[1].pair[P], cur[1].hdr, f1);
+        mfma(chunk, f0[0], f1[0], P == 0);
+        mfma(chunk + 1, f0[1], f1[1], false);
+        frags_q4k<P, 1>(cur[0].pair[P], cur[0].hdr, f0);
+        frags_q4k<P, 1>(cur[1].pair[P], cur[1].hdr, f1);
+        mfma(chunk + 4, f0[0], f1[0], false);
+        mfma(chunk + 5, f0[1], f1[1], false);
+    };
+    pair_step(std::integral_constant<int, 0>{});
+    pair_step(std::integral_constant<int, 1>{});
+    pair_step(std::integral_constant<int, 2>{});
+    pair_step(std::integral_constant<int, 3>{});
+    fold(cur[0].hdr.d, cur[1].hdr.d);
+    // minima: acc -= 32 * dmin * sum_s (Sx / 32)(hi + lo)[m, s] * mn[n, s]
+    const f16x8 m0 = minima_frag(cur[0].hdr), m1 = minima_frag(cur[1].hdr);
+    const f16x8 sf = *reinterpret_cast<const f16x8*>(sums + arow * 16 + khalf * 8);
+    const f32x16 zero{};
+    blk[0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m0, zero, 0, 0, 0);
+    blk[1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(sf, m1, zero, 0, 0, 0);
+    fold(-32.0f * cur[0].hdr.dmin, -32.0f * cur[1].hdr.dmin);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -665,17 +613,230 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
     publish_error(bad, a.error_word);
 }
 
+// The same kernel for Q6_K planes on 16x16x32 MFMA tiles: sixteen operand rows hold the (at most eight) token rows with
+// half the idle rows of the 32x32x16 tile, an instruction covers 32 columns, and a wave's 64 weight rows are four tiles
+// of 16. Lane (n, kq) of a tile owns weight row n and a quarter of the super-block: section s = kq / 2 (128 columns) and
+// the 16-byte half h = kq % 2 of each of its 32-byte groups, i.e. the same 16-byte pieces the 32x32x16 layout gives a
+// lane, for one section instead of two. Eight instructions (times hi and lo) per tile and super-block, half the
+// matrix-pipe time of the wider tile, and the result registers shrink from 16 to 4 per tile: the whole block fits the
+// 128 registers of four waves per SIMD without spilling (the Q4_K form of this layout did not: its four headers and
+// per-position scales cost more than the tile saves, 56 us against 37 for config 2's gate/up).
+template <int BKIND, int OUT, int SRC>
+__global__ __launch_bounds__(512, 4) void flat16_kernel(SkinnyArgs args) {  // four waves per SIMD: <= 128 registers per lane
+    SkinnyArgs a = args;
+    const bool shared = is_shared_task(a, blockIdx.y);
+    if (shared) { a.x = a.shared_x; a.x_stride = a.shared_x_stride; a.out = a.shared_out; a.out_stride = a.shared_out_stride; }
+    static_assert(BKIND == B_Q6K_PLANAR, "Q6_K planes only");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [wave][hi plane][lo plane][sums]; partial sums over it at the end
+
+    const uint32_t tid = threadIdx.x, lane = tid % kWave, wv = tid / kWave;
+    const uint32_t n16 = lane % 16, kq = lane / 16, sec = kq / 2, half = kq % 2;
+    const uint32_t bpr = a.k / 256, ucols = blockDim.x / kWave / bpr;  // the host launches ucols * bpr waves
+    const uint32_t slice = wv % bpr, ucol = wv / bpr;
+    Task task;
+    if (!load_task<SRC>(a, blockIdx.y, task)) return;
+    if (task.expert >= a.experts || task.count == 0 || task.count > kRows) {
+        if (tid == 0 && blockIdx.x == 0 && (task.expert >= a.experts || task.count > kRows)) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+        return;
+    }
+
+    // ---- this wave's 256 columns of the activation rows (lane l: columns 4l .. 4l+3 of each row), requested first: loads
+    // come back in the order they were asked for, and these few cached bytes must not queue behind the weight bytes
+    uint32_t bad = 0;
+    float4 v[kRows];
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+        const uint32_t from = uint32_t(r) < task.count ? task.src[r] : task.src[0];  // uniform; a dead row re-reads row 0 and is zeroed
+        v[r] = *reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.x) + uint64_t(from) * a.x_stride + (slice * kSlice + lane * 4) * 4);
+    }
+
+    // ---- weight rows of this wave (tiles 0, 1: gate units, tiles 2, 3: the same units of up; or 64 rows of down)
+    const uint8_t* wbase[4];
+    uint32_t wrow[4], out_col[4];
+    bool col_live[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+        if constexpr (OUT == OUT_SWIGLU) {
+            const uint32_t unit = (blockIdx.x * ucols + ucol) * 32 + (nt % 2) * 16 + n16;
+            const uint32_t half_e = a.experts / 2;
+            const uint8_t* pair = (task.expert < half_e ? a.w0 : a.w1) + uint64_t(task.expert < half_e ? task.expert : task.expert - half_e) * 2 * a.spec.planar_expert_bytes;
+            wbase[nt] = nt < 2 ? (shared ? a.shared_w0 : pair) : (shared ? a.shared_w1 : pair + a.spec.planar_expert_bytes);
+            col_live[nt] = unit < a.n;
+            wrow[nt] = col_live[nt] ? unit : a.n - 1;
+            out_col[nt] = unit;
+        } else {
+            const uint32_t n = (blockIdx.x * ucols + ucol) * 64 + nt * 16 + n16;
+            col_live[nt] = n < a.n;
+            wrow[nt] = col_live[nt] ? n : a.n - 1;
+            out_col[nt] = n;
+            wbase[nt] = shared ? a.shared_w0 : a.w0 + uint64_t(task.expert) * a.spec.planar_expert_bytes;
+        }
+    }
+    struct Tile { RawQ6 raw; float d; };  // the lane's pieces of section sec
+    Tile cur[4];
+    auto load_tile = [&](auto nt_tag) {
+        constexpr int nt = decltype(nt_tag)::value;
+        const uint64_t at = uint64_t(wrow[nt]) * bpr + slice;
+        const uint8_t* ql = wbase[nt] + a.spec.qs_offset + at * 128 + sec * 64 + half * 16;
+        cur[nt].raw.la = *reinterpret_cast<const u32x4*>(ql);
+        cur[nt].raw.lb = *reinterpret_cast<const u32x4*>(ql + 32);
+        cur[nt].raw.qh = *reinterpret_cast<const u32x4*>(wbase[nt] + a.spec.qh_offset + at * 64 + sec * 32 + half * 16);
+        const uint2 sc8 = *reinterpret_cast<const uint2*>(wbase[nt] + a.spec.sm_offset + at * 16 + sec * 8);
+        cur[nt].raw.sc[0] = sc8.x; cur[nt].raw.sc[1] = sc8.y;
+        cur[nt].d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(wbase[nt] + a.spec.dm_offset + at * 2));
+    };
+    load_tile(std::integral_constant<int, 0>{});
+    load_tile(std::integral_constant<int, 1>{});
+    load_tile(std::integral_constant<int, 2>{});
+    load_tile(std::integral_constant<int, 3>{});
+    __builtin_amdgcn_sched_barrier(0);  // every request above is out before the first wait below
+
+    // ---- stage the activation rows while the weight bytes travel
+    uint8_t* const mine = lds + wv * kWaveLds;
+    _Float16* const a_hi = reinterpret_cast<_Float16*>(mine);
+    _Float16* const a_lo = a_hi + kRows * kSlice;
+    float biggest = 0;
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+        if (uint32_t(r) >= task.count) v[r] = float4{0, 0, 0, 0};
+        if (nonfinite(v[r].x) || nonfinite(v[r].y) || nonfinite(v[r].z) || nonfinite(v[r].w)) bad = TSP_ERRBIT_NONFINITE;
+        biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v[r].x), fabsf(v[r].y)), fmaxf(fabsf(v[r].z), fabsf(v[r].w))));
+    }
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1) biggest = fmaxf(biggest, __shfl_xor(biggest, step, kWave));
+    // scale = 2^(13 - exponent(biggest)): the largest |x * scale| is below 2^15, the sub-block sums / 32 below 2^15 too
+    float scale = 1.0f, inv_scale = 1.0f;
+    if (biggest > 0 && !nonfinite(biggest)) {
+        const int e = int((__float_as_uint(biggest) >> 23) & 0xffu) - 127;
+        int shift = 13 - e;
+        shift = shift > 100 ? 100 : shift < -100 ? -100 : shift;
+        scale = __uint_as_float(uint32_t(127 + shift) << 23);
+        inv_scale = __uint_as_float(uint32_t(127 - shift) << 23);
+    }
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+        const float s4[4] = {v[r].x * scale, v[r].y * scale, v[r].z * scale, v[r].w * scale};
+        f16x4 hi, lo;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            hi[e] = _Float16(s4[e]);
+            lo[e] = _Float16(s4[e] - float(hi[e]));
+        }
+        // 16-byte chunk c = l / 2 of row r sits at position c ^ r; this lane owns half of it
+        const uint32_t at = (r * 32 + ((lane / 2) ^ r)) * 8 + (lane % 2) * 4;
+        *reinterpret_cast<f16x4*>(a_hi + at) = hi;
+        *reinterpret_cast<f16x4*>(a_lo + at) = lo;
+    }
+    // the planes are read back by other lanes of this same wave only: LDS serves a wave's requests in order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // ---- one super-block: operand row lane % 16 is token row (lane % 16) % 8; result register v of a lane is token row 4 kq + v
+    const uint32_t arow = n16 & 7;
+    auto a_frag = [&](const _Float16* plane, uint32_t chunk) {
+        return *reinterpret_cast<const f16x8*>(plane + (arow * 32 + (chunk ^ arow)) * 8);
+    };
+    f32x4 blk[4];
+    // quarter Q of section sec: two 8-column fragments per tile (f = 0, 1) at chunk base + f
+    auto quarter = [&](auto q_tag, bool first) {
+        constexpr int Q = decltype(q_tag)::value;
+        const uint32_t chunk = sec * 16 + Q * 4 + half * 2;  // columns sec*128 + Q*32 + 16 half (+ 8 f)
+        const f16x8 ah0 = a_frag(a_hi, chunk), al0 = a_frag(a_lo, chunk), ah1 = a_frag(a_hi, chunk + 1), al1 = a_frag(a_lo, chunk + 1);
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            f16x8 f[2];
+            frags_q6k<Q>(cur[nt].raw, half, f);
+            if (first) {
+                const f32x4 zero{};
+                blk[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah0, f[0], zero, 0, 0, 0);
+            } else {
+                blk[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah0, f[0], blk[nt], 0, 0, 0);
+            }
+            blk[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al0, f[0], blk[nt], 0, 0, 0);
+            blk[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah1, f[1], blk[nt], 0, 0, 0);
+            blk[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al1, f[1], blk[nt], 0, 0, 0);
+        }
+    };
+    quarter(std::integral_constant<int, 0>{}, true);
+    quarter(std::integral_constant<int, 1>{}, false);
+    quarter(std::integral_constant<int, 2>{}, false);
+    quarter(std::integral_constant<int, 3>{}, false);
+    float acc[4][4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) acc[nt][v4] = cur[nt].d * blk[nt][v4];
+    }
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) acc[nt][v4] *= inv_scale;  // exact: a power of two
+
+    // ---- the slices of a unit column meet in LDS, added in slice order; the planes are free once every wave is here
+    if (bpr > 1) {
+        float* const partial = reinterpret_cast<float*>(lds);  // [slice - 1][unit column][tile][v][lane]
+        __syncthreads();
+        if (slice > 0) {
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4) partial[((((slice - 1) * ucols + ucol) * 4 + nt) * 4 + v4) * kWave + lane] = acc[nt][v4];
+        }
+        __syncthreads();
+        if (slice > 0) { publish_error(bad, a.error_word); return; }
+        for (uint32_t s = 1; s < bpr; ++s)
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4) acc[nt][v4] += partial[((((s - 1) * ucols + ucol) * 4 + nt) * 4 + v4) * kWave + lane];
+    }
+    // ---- epilogue: register v of tile nt is token row 4 kq + v (lanes kq >= 2 hold repeats), weight row n16 of the tile
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+        const uint32_t r = 4 * kq + v4;
+        if (kq >= 2 || r >= task.count) continue;
+        const uint32_t dst = kq ? task.dst[4 + v4] : task.dst[v4];
+        uint8_t* orow = reinterpret_cast<uint8_t*>(a.out) + uint64_t(dst) * a.out_stride;
+        if constexpr (OUT == OUT_SWIGLU) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                if (!col_live[u]) continue;
+                const float g = acc[u][v4], up = acc[2 + u][v4];
+                const float sg = g >= 0 ? 1.0f / (1.0f + expf(-g)) : expf(g) / (1.0f + expf(g));
+                const float h = (g * sg) * up;
+                if (nonfinite(g) || nonfinite(up) || nonfinite(h)) bad = TSP_ERRBIT_NONFINITE;
+                reinterpret_cast<float*>(orow)[out_col[u]] = h;
+            }
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) {
+                if (!col_live[nt]) continue;
+                const float val = acc[nt][v4];
+                if (nonfinite(val)) bad = TSP_ERRBIT_NONFINITE;
+                reinterpret_cast<float*>(orow)[out_col[nt]] = val;
+            }
+        }
+    }
+    publish_error(bad, a.error_word);
+}
+
 template <int BKIND, int OUT, int SRC>
 int launch_flat(const char* name, const SkinnyArgs& a, uint32_t tasks, hipStream_t s) {
     const uint32_t bpr = a.k / 256, waves = bpr < 4 ? 4 : bpr, ucols = waves / bpr;
     const uint32_t per_group = ucols * (OUT == OUT_SWIGLU ? 32 : 64), col_tiles = (a.n + per_group - 1) / per_group;
     static bool raised = false;
     if (!raised) {
-        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&flat_kernel<BKIND, OUT, SRC>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    int(8 * kWaveLds)));
+        if constexpr (BKIND == B_Q6K_PLANAR)
+            TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&flat16_kernel<BKIND, OUT, SRC>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        int(8 * kWaveLds)));
+        else
+            TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&flat_kernel<BKIND, OUT, SRC>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        int(8 * kWaveLds)));
         raised = true;
     }
-    TSP_LAUNCH(name, s, flat_kernel<BKIND, OUT, SRC><<<dim3(col_tiles, tasks), waves * kWave, waves * kWaveLds, s>>>(a));
+    if constexpr (BKIND == B_Q6K_PLANAR) TSP_LAUNCH(name, s, flat16_kernel<BKIND, OUT, SRC><<<dim3(col_tiles, tasks), waves * kWave, waves * kWaveLds, s>>>(a));
+    else TSP_LAUNCH(name, s, flat_kernel<BKIND, OUT, SRC><<<dim3(col_tiles, tasks), waves * kWave, waves * kWaveLds, s>>>(a));
     return launch_status(name);
 }
 
