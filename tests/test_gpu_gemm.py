@@ -409,3 +409,23 @@ def test_config3_moe_grouped_prefill(gpu, tsp, orc, synth):
         want = orc.mixture_reference(yh[t].astype(np.float64), wh[t].astype(np.float64), np.zeros(C), 0.0)
         assert max_rel_error(out[t], want) <= 1e-5
     assert gpu.error() == 0
+    # the step as the bench runs it: the shared expert's rows riding in the same two launches. Routed rows unchanged to the
+    # bit; shared rows against the CPU composition on sampled tokens; the combine with the engine's gate sigmoid(shared_logit)
+    sg, su = synth.matrix(12, synth.tensor_seed(3, 20), H, C), synth.matrix(12, synth.tensor_seed(3, 21), H, C)
+    sd = synth.matrix(14, synth.tensor_seed(3, 22), C, H)
+    shared = tsp.PlanarSharedExpert(gpu, C, H, sg, su, sd)
+    riding = tsp.GroupedScratch(gpu, T, S, E, C, H, with_shared=True)
+    y2, ys = tsp.planar_nax_grouped_moe(gpu, w, ids_d, gpu.upload(x), T, S, riding, shared=shared)
+    assert gpu.error() == 0 and bool((y2.view(dtype=gpu.torch.int32) == y.view(dtype=gpu.torch.int32)).all())
+    tokens = np.arange(0, T, 173)
+    zeros = np.zeros(len(tokens), dtype=np.uint32)
+    _, want_s = orc.moe_routed_reference(12, 14, sg, su, sd, C, H, 1, zeros, len(tokens), 1, x[tokens], stage=12, threads=8)
+    got_s = ys.cpu().numpy()[tokens]
+    assert max_rel_error(got_s, want_s) <= 2e-3 and nmse(got_s, want_s) <= 1e-7
+    logit = gpu.upload(np.linspace(-3, 3, T).astype(np.float32))
+    out2 = gpu.mixture(y2, wts_d, ys, logit, C, S, tokens=T).cpu().numpy()
+    ysh, lh = ys.cpu().numpy(), np.linspace(-3, 3, T).astype(np.float32)
+    for t in range(0, T, 211):
+        want = orc.mixture_reference(yh[t].astype(np.float64), wh[t].astype(np.float64), ysh[t].astype(np.float64), float(lh[t]))
+        assert max_rel_error(out2[t], want) <= 1e-5
+    assert gpu.error() == 0
