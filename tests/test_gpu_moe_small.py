@@ -193,6 +193,12 @@ def test_config2_moe_verify(gpu, tsp, orc, synth):
     _, ys = tsp.planar_moe_routed_m8(gpu, ws, gpu.zeros(T, "int32"), gpu.upload(x), T, 1)
     out = gpu.mixture(y, wts_d, ys, gpu.full(T, 20.0), C, S, tokens=T).cpu().numpy()
     assert gpu.error() == 0
+    # the same step as the bench runs it: the shared expert as one more record of the routed experts' two launches
+    riding = tsp.PlanarSharedExpert(gpu, C, H, sg, su, sd)
+    h2, y2, ys2 = tsp.planar_moe_routed_m8(gpu, w, ids_d, gpu.upload(x), T, S, shared=riding)
+    assert gpu.error() == 0
+    assert np.array_equal(y2.cpu().numpy().view(np.uint32), y.cpu().numpy().view(np.uint32))
+    assert np.array_equal(ys2.cpu().numpy().view(np.uint32), ys.cpu().numpy().view(np.uint32))
 
     # oracle: per-route experts through compact stacks (expert index = position in `used`)
     pos = {e: i for i, e in enumerate(used)}
