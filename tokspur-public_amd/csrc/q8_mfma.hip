@@ -278,18 +278,17 @@ int q8_mfma(const void* matrix, const float* x, float* y, uint32_t columns, uint
     const Q8MfmaArgs a{static_cast<const uint8_t*>(matrix), x, y, columns, rows, width, error_word};
     // 8 rows x all columns and 16 rows x half the columns stage the same number of bytes
     const uint32_t lds_bytes = 2 * 8 * columns * 2 + kWaves * kTileBytes;
-    static bool raised = false;
-    static int compute_units = 0;
-    if (!raised) {
+    static std::atomic<uint64_t> raised{0};
+    static int units_of[64] = {};
+    int device = 0;
+    if (first_use_on_device(raised, &device)) {
         const int most = int(2 * 8 * 2048 * 2 + kWaves * kTileBytes);
         TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<1, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
         TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<2, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
         TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<2, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
-        int device = 0;
-        TSP_HIP(hipGetDevice(&device));
-        TSP_HIP(hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device));
-        raised = true;
+        TSP_HIP(hipDeviceGetAttribute(&units_of[device], hipDeviceAttributeMultiprocessorCount, device));
     }
+    const int compute_units = units_of[device];
     const uint32_t tiles = (rows + 31) / 32;
     uint32_t grid = uint32_t(compute_units > 0 ? compute_units : 256);
     if (width > 8) {
