@@ -2,9 +2,10 @@
 // (value descending, column ascending, -0 == +0), the number found, and the first non-finite and first
 // subnormal column. Rank 0 is the arg-max a greedy sampler needs.
 //
-// Two launches. Stage 1: one workgroup per (4096-column tile, row); each of its four waves keeps the 64 largest keys
-// of its 1024 columns in registers, one key per lane, and the four lists are merged into a partial row. Stage 2: one
-// workgroup per row merges the partial rows' lists the same way and writes the final row. Keys are 64 bits: high word
+// Two launches. Stage 1: one workgroup per (4096-column tile, row); each of its sixteen waves keeps the 64 largest keys
+// of its 256 columns in registers, one key per lane, and the sixteen lists are merged pairwise (a tree through LDS) into
+// a partial row. Stage 2: one workgroup per row merges the partial rows' lists the same way and writes the final row. A
+// sort or merge is a chain of dependent cross-lane exchanges, so what shortens it is more waves with shorter chains. Keys are 64 bits: high word
 // = the float mapped to an unsigned integer of the same order (after -0 -> +0), low word = ~column, so that "largest
 // key first" is exactly the ordering above and no two keys are equal. Non-finite logits and padding get key 0, below
 // every finite value's key. A list is sorted with a bitonic network over the wave's lanes; two lists are merged by
@@ -17,6 +18,7 @@ using namespace tsp;
 namespace {
 
 constexpr uint32_t kCapacity = 64, kTileSpan = 4096, kMaxTiles = 256, kNone = 0xffffffffu;
+constexpr uint32_t kWaves = 16, kThreads = kWaves * kWave, kWaveSpan = kTileSpan / kWaves;  // 256 columns per wave of stage 1
 
 struct TopKArgs {
     const float* logits;
@@ -70,15 +72,23 @@ __device__ __forceinline__ uint32_t wave_min(uint32_t v) {
     return v;
 }
 
-// Merges the four waves' descending lists through LDS (wave 0 ends with the workgroup's list) and writes the row.
+// Merges the waves' descending lists pairwise through LDS (wave 0 ends with the workgroup's list) and writes the row.
+// Every thread of the workgroup calls it (barriers inside).
 __device__ void merge_waves_and_write(uint64_t top, uint64_t (*lists)[kCapacity], tsp_logit_topk_row* row, const float* logits_row,
                                       uint32_t vocabulary, uint32_t first_nonfinite, uint32_t first_subnormal) {
     const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     lists[wave][lane] = top;
     __syncthreads();
-    if (wave != 0) return;
 #pragma unroll
-    for (uint32_t w = 1; w < 4; ++w) top = wave_merge(top, lists[w][kWave - 1 - lane], lane);
+    for (uint32_t step = 1; step < kWaves; step <<= 1) {
+        const bool merges = wave % (2 * step) == 0;
+        if (merges) top = wave_merge(top, lists[wave + step][kWave - 1 - lane], lane);
+        if (2 * step < kWaves) {
+            if (merges) lists[wave][lane] = top;  // its own slot: nobody else reads it at this level
+            __syncthreads();
+        }
+    }
+    if (wave != 0) return;
     const uint32_t column = ~uint32_t(top);
     const bool live = top != 0;
     row->ids[lane] = live ? column : 0u;
@@ -92,22 +102,22 @@ __device__ void merge_waves_and_write(uint64_t top, uint64_t (*lists)[kCapacity]
     }
 }
 
-__global__ __launch_bounds__(256) void topk_stage1(TopKArgs a) {
-    __shared__ uint64_t lists[4][kCapacity];
+__global__ __launch_bounds__(kThreads) void topk_stage1(TopKArgs a) {
+    __shared__ uint64_t lists[kWaves][kCapacity];
     __shared__ uint32_t first_nonfinite, first_subnormal;
     const uint32_t tile = blockIdx.x, row = blockIdx.y, lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const float* logits_row = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(a.logits) + uint64_t(row) * a.stride_bytes);
     if (threadIdx.x == 0) { first_nonfinite = kNone; first_subnormal = kNone; }
     __syncthreads();
     uint32_t nonfinite = kNone, subnormal = kNone;
-    // 16 batches of 64 columns per wave, two independent running lists so that the exchanges of one hide the other's latency
+    // 4 batches of 64 columns per wave, two independent running lists so that the exchanges of one hide the other's latency
     uint64_t top[2] = {0, 0};
 #pragma unroll 1
-    for (uint32_t pair = 0; pair < 8; ++pair) {
+    for (uint32_t pair = 0; pair < kWaveSpan / (2 * kWave); ++pair) {
         uint64_t key[2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const uint32_t column = tile * kTileSpan + wave * 1024 + (pair * 2 + h) * kWave + lane;
+            const uint32_t column = tile * kTileSpan + wave * kWaveSpan + (pair * 2 + h) * kWave + lane;
             key[h] = 0;
             if (column < a.vocabulary) {
                 const float v = logits_row[column];
@@ -136,8 +146,8 @@ __global__ __launch_bounds__(256) void topk_stage1(TopKArgs a) {
     merge_waves_and_write(mine, lists, a.partial + uint64_t(row) * a.tiles + tile, logits_row, width, first_nonfinite, first_subnormal);
 }
 
-__global__ __launch_bounds__(256) void topk_stage2(TopKArgs a) {
-    __shared__ uint64_t lists[4][kCapacity];
+__global__ __launch_bounds__(kThreads) void topk_stage2(TopKArgs a) {
+    __shared__ uint64_t lists[kWaves][kCapacity];
     __shared__ uint32_t first_nonfinite, first_subnormal;
     const uint32_t row = blockIdx.x, lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const float* logits_row = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(a.logits) + uint64_t(row) * a.stride_bytes);
@@ -148,10 +158,10 @@ __global__ __launch_bounds__(256) void topk_stage2(TopKArgs a) {
     auto list_key = [&](uint32_t tile, uint32_t slot) -> uint64_t {
         return tile < a.tiles && slot < partial[tile].count ? make_key(partial[tile].logits[slot], partial[tile].ids[slot]) : 0;
     };
-    uint64_t top[2] = {list_key(wave, lane), list_key(wave + 4, lane)};
+    uint64_t top[2] = {list_key(wave, lane), list_key(wave + kWaves, lane)};
 #pragma unroll 1
-    for (uint32_t tile = wave + 8; tile < a.tiles; tile += 8) {  // a pair per round; a tile past the end is an empty list
-        const uint64_t c0 = list_key(tile, kWave - 1 - lane), c1 = list_key(tile + 4, kWave - 1 - lane);
+    for (uint32_t tile = wave + 2 * kWaves; tile < a.tiles; tile += 2 * kWaves) {  // a pair per round; a tile past the end is an empty list
+        const uint64_t c0 = list_key(tile, kWave - 1 - lane), c1 = list_key(tile + kWaves, kWave - 1 - lane);
         top[0] = wave_merge(top[0], c0, lane);
         top[1] = wave_merge(top[1], c1, lane);
     }
@@ -205,9 +215,9 @@ extern "C" int tsp_logit_topk(const float* logits, uint64_t stride_bytes, uint32
     TopKArgs a{logits, stride_bytes, rows, vocabulary, tiles, static_cast<tsp_logit_topk_row*>(partial_scratch),
                static_cast<tsp_logit_topk_row*>(out_rows)};
     const auto s = static_cast<hipStream_t>(stream);
-    TSP_LAUNCH("logit_topk_stage1", s, topk_stage1<<<dim3(tiles, rows), 256, 0, s>>>(a));
+    TSP_LAUNCH("logit_topk_stage1", s, topk_stage1<<<dim3(tiles, rows), kThreads, 0, s>>>(a));
     int rc = launch_status("logit_topk_stage1");
     if (rc != TSP_OK) return rc;
-    TSP_LAUNCH("logit_topk_stage2", s, topk_stage2<<<rows, 256, 0, s>>>(a));
+    TSP_LAUNCH("logit_topk_stage2", s, topk_stage2<<<rows, kThreads, 0, s>>>(a));
     return launch_status("logit_topk_stage2");
 }
