@@ -36,31 +36,59 @@ __device__ __forceinline__ uint64_t make_key(float value, uint32_t column) {
     return (uint64_t(ordered) << 32) | uint32_t(~column);
 }
 
-__device__ __forceinline__ uint64_t exchange(uint64_t key, uint32_t stride, bool keep_larger) {
-    const uint64_t other = __shfl_xor(key, stride, kWave);
+template <int CTRL>
+__device__ __forceinline__ uint64_t dpp_u64(uint64_t v) {
+    const uint32_t lo = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v)), CTRL, 0xf, 0xf, true));
+    const uint32_t hi = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v >> 32)), CTRL, 0xf, 0xf, true));
+    return (uint64_t(hi) << 32) | lo;
+}
+
+// The key of lane (lane ^ STRIDE). Strides 1, 2, 4 and 8 stay inside a row of 16 lanes and use the data-parallel
+// primitives (quad permutes, row rotations), whose latency is a fraction of a trip through the LDS crossbar; a sort is
+// a chain of 21 dependent exchanges, 18 of them with these strides.
+template <uint32_t STRIDE>
+__device__ __forceinline__ uint64_t partner(uint64_t key, uint32_t lane) {
+    if constexpr (STRIDE == 1) return dpp_u64<0xB1>(key);        // quad_perm [1, 0, 3, 2]
+    else if constexpr (STRIDE == 2) return dpp_u64<0x4E>(key);   // quad_perm [2, 3, 0, 1]
+    else if constexpr (STRIDE == 8) return dpp_u64<0x128>(key);  // row_ror:8
+    else if constexpr (STRIDE == 4) {
+        const uint64_t below = dpp_u64<0x124>(key), above = dpp_u64<0x12C>(key);  // row_ror:4 = lane - 4, row_ror:12 = lane + 4 (mod 16)
+        return (lane & 4) ? below : above;
+    } else return __shfl_xor(key, STRIDE, kWave);
+}
+
+template <uint32_t STRIDE>
+__device__ __forceinline__ uint64_t exchange(uint64_t key, uint32_t lane, bool keep_larger) {
+    const uint64_t other = partner<STRIDE>(key, lane);
     return (key > other) == keep_larger ? key : other;
+}
+
+// The strides SIZE / 2, SIZE / 4, ..., 1 of one bitonic merge step over blocks of SIZE lanes.
+template <uint32_t SIZE, uint32_t STRIDE, bool DESCENDING>
+__device__ __forceinline__ uint64_t merge_strides(uint64_t key, uint32_t lane) {
+    if constexpr (STRIDE == 0) return key;
+    else {
+        const bool block_descending = SIZE == kWave ? DESCENDING : ((lane & SIZE) == 0) == DESCENDING;
+        key = exchange<STRIDE>(key, lane, ((lane & STRIDE) == 0) == block_descending);
+        return merge_strides<SIZE, STRIDE / 2, DESCENDING>(key, lane);
+    }
 }
 
 // Bitonic sort of one key per lane: lane i ends with the i-th largest (DESCENDING) or i-th smallest key.
 template <bool DESCENDING>
 __device__ __forceinline__ uint64_t wave_sort(uint64_t key, uint32_t lane) {
-#pragma unroll
-    for (uint32_t size = 2; size <= kWave; size <<= 1) {
-#pragma unroll
-        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
-            const bool block_descending = size == kWave ? DESCENDING : ((lane & size) == 0) == DESCENDING;
-            key = exchange(key, stride, ((lane & stride) == 0) == block_descending);
-        }
-    }
-    return key;
+    key = merge_strides<2, 1, DESCENDING>(key, lane);
+    key = merge_strides<4, 2, DESCENDING>(key, lane);
+    key = merge_strides<8, 4, DESCENDING>(key, lane);
+    key = merge_strides<16, 8, DESCENDING>(key, lane);
+    key = merge_strides<32, 16, DESCENDING>(key, lane);
+    return merge_strides<64, 32, DESCENDING>(key, lane);
 }
 
 // The 64 largest of a descending list and an ascending list, descending.
 __device__ __forceinline__ uint64_t wave_merge(uint64_t descending, uint64_t ascending, uint32_t lane) {
-    uint64_t key = descending > ascending ? descending : ascending;
-#pragma unroll
-    for (uint32_t stride = kWave >> 1; stride > 0; stride >>= 1) key = exchange(key, stride, (lane & stride) == 0);
-    return key;
+    const uint64_t key = descending > ascending ? descending : ascending;
+    return merge_strides<64, 32, true>(key, lane);
 }
 
 __device__ __forceinline__ uint32_t wave_min(uint32_t v) {
