@@ -24,10 +24,20 @@ __global__ __launch_bounds__(256) void grouped_routes_kernel(const uint32_t* __r
         const uint32_t token = base + tid;
         uint32_t slot = 0xffffffffu, matches = 0;
         if (token < tokens) {
-            for (uint32_t i = 0; i < selected; ++i) {
-                const uint32_t id = ids[uint64_t(token) * selected + i];
-                if (id >= experts) bad = TSP_ERRBIT_INDEX;
-                if (id == expert) { slot = i; ++matches; }
+            const uint32_t* row = ids + uint64_t(token) * selected;
+            if (selected % 2 == 0) {  // rows of an even number of ids are 8-byte aligned: half as many loads
+                for (uint32_t i = 0; i < selected; i += 2) {
+                    const uint2 pair = *reinterpret_cast<const uint2*>(row + i);
+                    if (pair.x >= experts || pair.y >= experts) bad = TSP_ERRBIT_INDEX;
+                    if (pair.x == expert) { slot = i; ++matches; }
+                    if (pair.y == expert) { slot = i + 1; ++matches; }
+                }
+            } else {
+                for (uint32_t i = 0; i < selected; ++i) {
+                    const uint32_t id = row[i];
+                    if (id >= experts) bad = TSP_ERRBIT_INDEX;
+                    if (id == expert) { slot = i; ++matches; }
+                }
             }
         }
         if (matches > 1) bad = TSP_ERRBIT_INDEX;
