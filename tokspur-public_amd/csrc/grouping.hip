@@ -14,13 +14,15 @@ using namespace tsp;
 
 namespace {
 
-__global__ __launch_bounds__(256) void grouped_routes_kernel(const uint32_t* __restrict__ ids, uint32_t* __restrict__ token_map,
+constexpr uint32_t kRouteThreads = 1024;  // tokens looked at per pass of one expert's workgroup
+
+__global__ __launch_bounds__(kRouteThreads) void grouped_routes_kernel(const uint32_t* __restrict__ ids, uint32_t* __restrict__ token_map,
                                                              uint32_t* __restrict__ counts, uint32_t experts, uint32_t selected,
                                                              uint32_t tokens, uint32_t* error_word) {
-    __shared__ uint32_t wave_totals[4];
+    __shared__ uint32_t wave_totals[kRouteThreads / kWave];
     const uint32_t expert = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     uint32_t accumulated = 0, bad = 0;
-    for (uint32_t base = 0; base < tokens; base += 256) {
+    for (uint32_t base = 0; base < tokens; base += kRouteThreads) {
         const uint32_t token = base + tid;
         uint32_t slot = 0xffffffffu, matches = 0;
         if (token < tokens) {
@@ -47,7 +49,7 @@ __global__ __launch_bounds__(256) void grouped_routes_kernel(const uint32_t* __r
         if (lane == 0) wave_totals[wave] = __builtin_popcountll(mask);
         __syncthreads();
         uint32_t before = 0, chunk = 0;
-        for (uint32_t w = 0; w < 4; ++w) { if (w < wave) before += wave_totals[w]; chunk += wave_totals[w]; }
+        for (uint32_t w = 0; w < kRouteThreads / kWave; ++w) { if (w < wave) before += wave_totals[w]; chunk += wave_totals[w]; }
         if (found) token_map[uint64_t(expert) * tokens + accumulated + before + prefix] = token * selected + slot;
         accumulated += chunk;
         __syncthreads();
@@ -144,7 +146,7 @@ extern "C" int tsp_grouped_routes(const uint32_t* ids, uint32_t* token_map, uint
     TSP_REQUIRE(experts && experts <= 512 && selected && selected <= 16 && selected <= experts && tokens && tokens <= 2048,
                 "grouped routes geometry");
     TSP_REQUIRE(ids && token_map && counts && error_word, "null device pointer");
-    TSP_LAUNCH("grouped_routes", static_cast<hipStream_t>(stream), grouped_routes_kernel<<<experts, 256, 0, static_cast<hipStream_t>(stream)>>>(ids, token_map, counts, experts, selected, tokens, error_word));
+    TSP_LAUNCH("grouped_routes", static_cast<hipStream_t>(stream), grouped_routes_kernel<<<experts, kRouteThreads, 0, static_cast<hipStream_t>(stream)>>>(ids, token_map, counts, experts, selected, tokens, error_word));
     return launch_status("grouped_routes");
 }
 
