@@ -73,8 +73,9 @@ __global__ __launch_bounds__(512) void grouped_tasks_kernel(const uint32_t* __re
 __global__ __launch_bounds__(128) void union_build_kernel(const uint32_t* __restrict__ ids, uint32_t* __restrict__ meta,
                                                           uint32_t experts, uint32_t selected, uint32_t tokens, uint32_t hidden,
                                                           uint32_t channels, uint32_t* error_word) {
-    __shared__ uint32_t sid[128];
-    __shared__ uint32_t record_of[128];
+    __shared__ __align__(16) uint32_t sid[128];
+    __shared__ __align__(16) uint32_t rank_of[128];
+    __shared__ __align__(16) uint32_t record_of[128];
     __shared__ uint32_t wave_leaders[2];
     __shared__ uint32_t any_bad;
     const uint32_t f = threadIdx.x, total = tokens * selected;
@@ -93,11 +94,17 @@ __global__ __launch_bounds__(128) void union_build_kernel(const uint32_t* __rest
         return;
     }
     const uint32_t cap = tokens <= 4 ? 4u : 8u;
+    // All 128 slots are compared, four per LDS read and with no dependence between the reads, so the scan costs one LDS
+    // latency and not one per route; the slots past the last route hold 0xffffffff and match no live route.
     uint32_t rank = 0, same = 0;
-    if (live) {
-        for (uint32_t g = 0; g < total; ++g) {
-            const bool eq = sid[g] == mine;
-            rank += (eq && g < f) ? 1u : 0u;
+#pragma unroll
+    for (uint32_t g = 0; g < 128; g += 4) {
+        const uint4 four = *reinterpret_cast<const uint4*>(&sid[g]);
+        const uint32_t id4[4] = {four.x, four.y, four.z, four.w};
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            const bool eq = id4[i] == mine;
+            rank += (eq && g + i < f) ? 1u : 0u;
             same += eq ? 1u : 0u;
         }
     }
@@ -109,17 +116,22 @@ __global__ __launch_bounds__(128) void union_build_kernel(const uint32_t* __rest
     const uint32_t record = (wave ? wave_leaders[0] : 0u) + __builtin_popcountll(mask & ((1ull << lane) - 1ull));
     const uint32_t records = wave_leaders[0] + wave_leaders[1];
     record_of[f] = leader ? record : 0xffffffffu;
+    rank_of[f] = rank;
     __syncthreads();
     if (live) {
         // my record is the one opened by the route of my expert whose rank is rank - rank % cap
         const uint32_t want = rank - rank % cap;
-        uint32_t seen = 0, rec = record;
+        uint32_t rec = record;
         if (!leader) {
-            for (uint32_t g = 0; g < f; ++g) {
-                if (sid[g] == mine) {
-                    if (seen == want) { rec = record_of[g]; break; }
-                    ++seen;
-                }
+#pragma unroll
+            for (uint32_t g = 0; g < 128; g += 4) {
+                const uint4 id4 = *reinterpret_cast<const uint4*>(&sid[g]);
+                const uint4 rank4 = *reinterpret_cast<const uint4*>(&rank_of[g]);
+                const uint4 rec4 = *reinterpret_cast<const uint4*>(&record_of[g]);
+                if (id4.x == mine && rank4.x == want) rec = rec4.x;
+                if (id4.y == mine && rank4.y == want) rec = rec4.y;
+                if (id4.z == mine && rank4.z == want) rec = rec4.z;
+                if (id4.w == mine && rank4.w == want) rec = rec4.w;
             }
         }
         const uint32_t slot = rank % cap;

@@ -1,7 +1,7 @@
 // Router top-k with softmax / sigmoid weights, the weighted mixture (combine) and SwiGLU.
 //
-// Top-k is integer-exact: k rounds of arg-max over f32 logits compared as given, exact ties to the
-// lower expert id. One 64-lane wave owns one token row and keeps the row's logits in registers
+// Top-k is integer-exact: k rounds of arg-max over f32 logits compared as given (as 32-bit integers of
+// the same order), exact ties to the lower expert id. One 64-lane wave owns one token row and keeps the row's logits in registers
 // (lane i holds experts i, i+64, ...), so a round is a per-lane scan plus two wave reductions and
 // no barrier. Weights use accurate expf/logf; their association differs from a sequential sum but
 // they are compared to the double reference under tolerance, never bit for bit.
@@ -25,38 +25,32 @@ __device__ __forceinline__ float route_activation(float logit, float maximum, ui
     return sigmoid_f(logit);
 }
 
-// A candidate as one 64-bit key: high word = the logit mapped to an unsigned integer of the same order (-0 as +0), low
-// word = ~expert, so the largest key is the largest logit and, among equal logits, the lowest expert id. 0 = no candidate.
-__device__ __forceinline__ uint64_t route_key(float logit, uint32_t expert) {
+// A logit as an unsigned integer of the same order (-0 as +0). Every finite or infinite logit maps above 0, so 0 = no candidate.
+__device__ __forceinline__ uint32_t ordered_logit(float logit) {
     uint32_t bits = __float_as_uint(logit);
     if ((bits & 0x7fffffffu) == 0) bits = 0;
-    const uint32_t ordered = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
-    return (uint64_t(ordered) << 32) | uint32_t(~expert);
+    return (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
 }
-__device__ __forceinline__ float route_key_logit(uint64_t key) {
-    const uint32_t ordered = uint32_t(key >> 32);
+__device__ __forceinline__ float logit_of_ordered(uint32_t ordered) {
     return __uint_as_float((ordered & 0x80000000u) ? (ordered & 0x7fffffffu) : ~ordered);
 }
-template <int Ctrl>
-__device__ __forceinline__ uint64_t dpp_max_u64(uint64_t v) {
-    const uint32_t lo = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v)), Ctrl, 0xf, 0xf, true));
-    const uint32_t hi = uint32_t(__builtin_amdgcn_update_dpp(0, int(uint32_t(v >> 32)), Ctrl, 0xf, 0xf, true));
-    const uint64_t other = (uint64_t(hi) << 32) | lo;
-    return other > v ? other : v;
+// Four cross-lane steps inside each row of 16 lanes leave the row's result in all its lanes; the four rows meet in scalar registers.
+template <int Ctrl, bool MAX>
+__device__ __forceinline__ uint32_t dpp_step_u32(uint32_t v) {
+    const uint32_t other = uint32_t(__builtin_amdgcn_update_dpp(int(v), int(v), Ctrl, 0xf, 0xf, false));
+    return MAX ? (other > v ? other : v) : (other < v ? other : v);
 }
-// Largest key of the wave, uniform: four cross-lane steps inside each row of 16 lanes, then the four rows by scalar reads.
-__device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-    v = dpp_max_u64<0xB1>(v);   // quad_perm [1,0,3,2]
-    v = dpp_max_u64<0x4E>(v);   // quad_perm [2,3,0,1]
-    v = dpp_max_u64<0x141>(v);  // row_half_mirror
-    v = dpp_max_u64<0x140>(v);  // row_mirror
-    uint64_t best = 0;
+template <bool MAX>
+__device__ __forceinline__ uint32_t wave_extreme_u32(uint32_t v) {
+    v = dpp_step_u32<0xB1, MAX>(v);   // quad_perm [1,0,3,2]
+    v = dpp_step_u32<0x4E, MAX>(v);   // quad_perm [2,3,0,1]
+    v = dpp_step_u32<0x141, MAX>(v);  // row_half_mirror
+    v = dpp_step_u32<0x140, MAX>(v);  // row_mirror
+    uint32_t best = uint32_t(__builtin_amdgcn_readlane(int(v), 0));
 #pragma unroll
-    for (int row = 0; row < 4; ++row) {
-        const uint32_t lo = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(v)), row * 16));
-        const uint32_t hi = uint32_t(__builtin_amdgcn_readlane(int(uint32_t(v >> 32)), row * 16));
-        const uint64_t k = (uint64_t(hi) << 32) | lo;
-        best = k > best ? k : best;
+    for (int row = 1; row < 4; ++row) {
+        const uint32_t r = uint32_t(__builtin_amdgcn_readlane(int(v), row * 16));
+        best = MAX ? (r > best ? r : best) : (r < best ? r : best);
     }
     return best;
 }
@@ -73,34 +67,49 @@ __global__ __launch_bounds__(64) void route_rows(const float* __restrict__ logit
     const uint32_t row = blockIdx.x, lane = threadIdx.x;
     if (row >= tokens) return;
     const float* row_logits = logits + uint64_t(row) * experts;
-    uint64_t cand[CAND];
+    uint32_t cand[CAND];
     uint32_t bad = 0;
 #pragma unroll
     for (int k = 0; k < CAND; ++k) {
         const uint32_t i = lane + k * kWave;
-        uint64_t key = 0;
+        uint32_t key = 0;
         if (i < experts) {
             float v = row_logits[i];
             if (nonfinite(v)) { bad |= TSP_ERRBIT_NONFINITE; v = -INFINITY; }
-            key = route_key(v, i);
+            key = ordered_logit(v);
         }
         cand[k] = key;
     }
     // chosen logit j is kept by lane j (selected <= 64)
     float chosen_mine = 0, chosen_first = 0;
     for (uint32_t s = 0; s < selected; ++s) {
-        uint64_t best = 0;
+        uint32_t local = 0;
 #pragma unroll
-        for (int k = 0; k < CAND; ++k) best = cand[k] > best ? cand[k] : best;
-        best = wave_max_u64(best);
-        uint32_t chosen = ~uint32_t(best);
-        if (best == 0 || chosen >= experts) { bad |= TSP_ERRBIT_INDEX; chosen = 0; }
+        for (int k = 0; k < CAND; ++k) local = cand[k] > local ? cand[k] : local;
+        const uint32_t best = wave_extreme_u32<true>(local);
+        // the lowest expert id that holds the largest logit: lane + 64 * (first slot of the lane that holds it)
+        uint32_t first_slot = CAND;
+#pragma unroll
+        for (int k = CAND - 1; k >= 0; --k) first_slot = cand[k] == best ? uint32_t(k) : first_slot;
+        const bool holds = best != 0 && first_slot < uint32_t(CAND);
+        const uint64_t holders = __builtin_amdgcn_ballot_w64(holds);
+        uint32_t chosen = 0;
+        if (holders == 0) {
+            bad |= TSP_ERRBIT_INDEX;
+        } else if ((holders & (holders - 1)) == 0) {  // one lane holds it: no tie between lanes to settle
+            const int winner = __builtin_ctzll(holders);
+            chosen = uint32_t(winner) + kWave * uint32_t(__builtin_amdgcn_readlane(int(first_slot), winner));
+        } else {
+            chosen = wave_extreme_u32<false>(holds ? lane + kWave * first_slot : 0xffffffffu);
+        }
+        if (chosen >= experts) { bad |= TSP_ERRBIT_INDEX; chosen = 0; }
         if (lane == 0) indices[uint64_t(row) * selected + s] = chosen;
-        const float value = best == 0 ? row_logits[chosen] : route_key_logit(best);
+        const float value = holders == 0 ? row_logits[chosen] : logit_of_ordered(best);
         if (s == 0) chosen_first = value;
         if (s == lane) chosen_mine = value;
+        const uint32_t taken = (holders != 0 && chosen % kWave == lane) ? chosen / kWave : uint32_t(CAND);
 #pragma unroll
-        for (int k = 0; k < CAND; ++k) if (cand[k] == best) cand[k] = 0;
+        for (int k = 0; k < CAND; ++k) cand[k] = uint32_t(k) == taken ? 0u : cand[k];
     }
     const float act = lane < selected ? route_activation(chosen_mine, chosen_first, mode, normalize) : 0.0f;
     float sum = mode ? 1.0f : 0.0f;
