@@ -134,8 +134,7 @@ __global__ __launch_bounds__(256 * KS, 2) void skinny_kernel(SkinnyArgs args) {
             biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
         }
     }
-#pragma unroll
-    for (int step = 32; step >= 1; step >>= 1) biggest = fmaxf(biggest, __shfl_xor(biggest, step, kWave));
+    biggest = wave_largest(biggest);
     if (lane == 0) wave_max[tid / kWave] = biggest;
     __syncthreads();
     biggest = wave_max[0];
@@ -171,8 +170,8 @@ __global__ __launch_bounds__(256 * KS, 2) void skinny_kernel(SkinnyArgs args) {
         *reinterpret_cast<f16x8*>(a_lo + at) = lo;
         if constexpr (!Q6) {
             // four neighbouring lanes hold the four chunks of one 32-column sub-block (chunks is a multiple of 32)
-            sum += __shfl_xor(sum, 1, kWave);
-            sum += __shfl_xor(sum, 2, kWave);
+            sum = dpp_add<0xB1>(sum);
+            sum = dpp_add<0x4E>(sum);
             if ((c & 3) == 0) {
                 const float s32 = sum * 0.03125f;
                 const _Float16 h = _Float16(s32);
@@ -472,8 +471,7 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
         if (nonfinite(v[r].x) || nonfinite(v[r].y) || nonfinite(v[r].z) || nonfinite(v[r].w)) bad = TSP_ERRBIT_NONFINITE;
         biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v[r].x), fabsf(v[r].y)), fmaxf(fabsf(v[r].z), fabsf(v[r].w))));
     }
-#pragma unroll
-    for (int step = 32; step >= 1; step >>= 1) biggest = fmaxf(biggest, __shfl_xor(biggest, step, kWave));
+    biggest = wave_largest(biggest);
     // scale = 2^(13 - exponent(biggest)): the largest |x * scale| is below 2^15, the sub-block sums / 32 below 2^15 too
     float scale = 1.0f, inv_scale = 1.0f;
     if (biggest > 0 && !nonfinite(biggest)) {
@@ -497,9 +495,7 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
         *reinterpret_cast<f16x4*>(a_hi + at) = hi;
         *reinterpret_cast<f16x4*>(a_lo + at) = lo;
         float sum = (s4[0] + s4[1]) + (s4[2] + s4[3]);  // eight neighbouring lanes hold one 32-column sub-block
-        sum += __shfl_xor(sum, 1, kWave);
-        sum += __shfl_xor(sum, 2, kWave);
-        sum += __shfl_xor(sum, 4, kWave);
+        sum = octet_sum(sum);
         if (lane % 8 == 0) {
             const float s32 = sum * 0.03125f;
             const _Float16 h = _Float16(s32);
@@ -702,8 +698,7 @@ __global__ __launch_bounds__(512, 4) void flat16_kernel(SkinnyArgs args) {  // f
         if (nonfinite(v[r].x) || nonfinite(v[r].y) || nonfinite(v[r].z) || nonfinite(v[r].w)) bad = TSP_ERRBIT_NONFINITE;
         biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v[r].x), fabsf(v[r].y)), fmaxf(fabsf(v[r].z), fabsf(v[r].w))));
     }
-#pragma unroll
-    for (int step = 32; step >= 1; step >>= 1) biggest = fmaxf(biggest, __shfl_xor(biggest, step, kWave));
+    biggest = wave_largest(biggest);
     // scale = 2^(13 - exponent(biggest)): the largest |x * scale| is below 2^15, the sub-block sums / 32 below 2^15 too
     float scale = 1.0f, inv_scale = 1.0f;
     if (biggest > 0 && !nonfinite(biggest)) {

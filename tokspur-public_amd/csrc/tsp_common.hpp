@@ -99,6 +99,23 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (a + b) + (c + d);
 }
 
+// Largest of the wave's 64 values (NaNs are passed over, as fmaxf does); the result is uniform.
+template <int Ctrl>
+__device__ __forceinline__ float dpp_max(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), Ctrl, 0xf, 0xf, true);
+    return fmaxf(v, __int_as_float(moved));
+}
+__device__ __forceinline__ float wave_largest(float v) {
+    v = dpp_max<0xB1>(v);
+    v = dpp_max<0x4E>(v);
+    v = dpp_max<0x141>(v);
+    v = dpp_max<0x140>(v);
+    const int bits = __float_as_int(v);
+    const float a = __int_as_float(__builtin_amdgcn_readlane(bits, 0)), b = __int_as_float(__builtin_amdgcn_readlane(bits, 16));
+    const float c = __int_as_float(__builtin_amdgcn_readlane(bits, 32)), d = __int_as_float(__builtin_amdgcn_readlane(bits, 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
 // Sum over aligned groups of 8 lanes; every lane of a group receives the group's sum.
 __device__ __forceinline__ float octet_sum(float v) {
     v = dpp_add<0xB1>(v);
