@@ -474,7 +474,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
             if constexpr (EPI == EPI_SWIGLU) {
                 if (!col_live[0]) continue;
                 const float g = acc[i][0][v], u = acc[i][1][v];
-                const float sg = g >= 0 ? 1.0f / (1.0f + expf(-g)) : expf(g) / (1.0f + expf(g));
+                const float sg = sigmoid_stable(g);
                 const float h = (g * sg) * u;
                 // h is carried between the two GEMMs as the half nearest to h * 2^-8: 11 significant bits for
                 // 0.016 <= |h| < 1.6e7, an absolute step of 2^-16 below that

@@ -52,7 +52,7 @@ __device__ __forceinline__ bool load_record(const SmallMoeArgs& a, uint32_t inde
 }
 
 __device__ __forceinline__ float silu_mul(float g, float u) {
-    const float s = g >= 0 ? 1.0f / (1.0f + expf(-g)) : expf(g) / (1.0f + expf(g));
+    const float s = sigmoid_stable(g);
     return (g * s) * u;
 }
 

@@ -364,7 +364,7 @@ __global__ __launch_bounds__(256 * KS, 2) void skinny_kernel(SkinnyArgs args) {
         if constexpr (OUT == OUT_SWIGLU) {
             if (!col_live[0]) continue;
             const float g = acc[0][v] * inv_scale, u = acc[1][v] * inv_scale;
-            const float sg = g >= 0 ? 1.0f / (1.0f + expf(-g)) : expf(g) / (1.0f + expf(g));
+            const float sg = sigmoid_stable(g);
             const float h = (g * sg) * u;
             if (nonfinite(g) || nonfinite(u) || nonfinite(h)) bad = TSP_ERRBIT_NONFINITE;
             reinterpret_cast<float*>(orow)[out_col[0]] = h;
@@ -417,8 +417,11 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
     float4 v[kRows];
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
-        const uint32_t from = uint32_t(r) < task.count ? task.src[r] : task.src[0];  // uniform; a dead row re-reads row 0 and is zeroed
-        v[r] = *reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.x) + uint64_t(from) * a.x_stride + (slice * kSlice + lane * 4) * 4);
+        // a record rarely fills its eight rows: the rows past its count are neither read nor staged. Their places in LDS keep
+        // whatever was there; a token row of the product depends on its own operand row only, and those rows are never stored.
+        v[r] = float4{0, 0, 0, 0};
+        if (uint32_t(r) < task.count)  // uniform
+            v[r] = *reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.x) + uint64_t(task.src[r]) * a.x_stride + (slice * kSlice + lane * 4) * 4);
     }
 
     // ---- weight rows of this wave, and their bytes: requested before any arithmetic
@@ -467,7 +470,6 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
     float biggest = 0;
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
-        if (uint32_t(r) >= task.count) v[r] = float4{0, 0, 0, 0};
         if (nonfinite(v[r].x) || nonfinite(v[r].y) || nonfinite(v[r].z) || nonfinite(v[r].w)) bad = TSP_ERRBIT_NONFINITE;
         biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v[r].x), fabsf(v[r].y)), fmaxf(fabsf(v[r].z), fabsf(v[r].w))));
     }
@@ -483,6 +485,7 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
     }
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
+        if (uint32_t(r) >= task.count) continue;
         const float s4[4] = {v[r].x * scale, v[r].y * scale, v[r].z * scale, v[r].w * scale};
         f16x4 hi, lo;
 #pragma unroll
@@ -592,7 +595,7 @@ __global__ __launch_bounds__(512, 4) void flat_kernel(SkinnyArgs args) {  // fou
         if constexpr (OUT == OUT_SWIGLU) {
             if (!col_live[0]) continue;
             const float g = acc[0][v4], u = acc[1][v4];
-            const float sg = g >= 0 ? 1.0f / (1.0f + expf(-g)) : expf(g) / (1.0f + expf(g));
+            const float sg = sigmoid_stable(g);
             const float h = (g * sg) * u;
             if (nonfinite(g) || nonfinite(u) || nonfinite(h)) bad = TSP_ERRBIT_NONFINITE;
             reinterpret_cast<float*>(orow)[out_col[0]] = h;
@@ -642,8 +645,11 @@ __global__ __launch_bounds__(512, 4) void flat16_kernel(SkinnyArgs args) {  // f
     float4 v[kRows];
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
-        const uint32_t from = uint32_t(r) < task.count ? task.src[r] : task.src[0];  // uniform; a dead row re-reads row 0 and is zeroed
-        v[r] = *reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.x) + uint64_t(from) * a.x_stride + (slice * kSlice + lane * 4) * 4);
+        // a record rarely fills its eight rows: the rows past its count are neither read nor staged. Their places in LDS keep
+        // whatever was there; a token row of the product depends on its own operand row only, and those rows are never stored.
+        v[r] = float4{0, 0, 0, 0};
+        if (uint32_t(r) < task.count)  // uniform
+            v[r] = *reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.x) + uint64_t(task.src[r]) * a.x_stride + (slice * kSlice + lane * 4) * 4);
     }
 
     // ---- weight rows of this wave (tiles 0, 1: gate units, tiles 2, 3: the same units of up; or 64 rows of down)
@@ -694,7 +700,6 @@ __global__ __launch_bounds__(512, 4) void flat16_kernel(SkinnyArgs args) {  // f
     float biggest = 0;
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
-        if (uint32_t(r) >= task.count) v[r] = float4{0, 0, 0, 0};
         if (nonfinite(v[r].x) || nonfinite(v[r].y) || nonfinite(v[r].z) || nonfinite(v[r].w)) bad = TSP_ERRBIT_NONFINITE;
         biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v[r].x), fabsf(v[r].y)), fmaxf(fabsf(v[r].z), fabsf(v[r].w))));
     }
@@ -710,6 +715,7 @@ __global__ __launch_bounds__(512, 4) void flat16_kernel(SkinnyArgs args) {  // f
     }
 #pragma unroll
     for (int r = 0; r < kRows; ++r) {
+        if (uint32_t(r) >= task.count) continue;
         const float s4[4] = {v[r].x * scale, v[r].y * scale, v[r].z * scale, v[r].w * scale};
         f16x4 hi, lo;
 #pragma unroll
@@ -798,7 +804,7 @@ __global__ __launch_bounds__(512, 4) void flat16_kernel(SkinnyArgs args) {  // f
             for (int u = 0; u < 2; ++u) {
                 if (!col_live[u]) continue;
                 const float g = acc[u][v4], up = acc[2 + u][v4];
-                const float sg = g >= 0 ? 1.0f / (1.0f + expf(-g)) : expf(g) / (1.0f + expf(g));
+                const float sg = sigmoid_stable(g);
                 const float h = (g * sg) * up;
                 if (nonfinite(g) || nonfinite(up) || nonfinite(h)) bad = TSP_ERRBIT_NONFINITE;
                 reinterpret_cast<float*>(orow)[out_col[u]] = h;

@@ -99,6 +99,12 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (a + b) + (c + d);
 }
 
+// 1 / (1 + e^-g) with a single exponential that never overflows: e = e^-|g| is the small one of e^g and e^-g.
+__device__ __forceinline__ float sigmoid_stable(float g) {
+    const float e = expf(-fabsf(g));
+    return (g >= 0 ? 1.0f : e) / (1.0f + e);
+}
+
 // Largest of the wave's 64 values (NaNs are passed over, as fmaxf does); the result is uniform.
 template <int Ctrl>
 __device__ __forceinline__ float dpp_max(float v) {
