@@ -10,7 +10,7 @@
 //
 // Raw rows are only 2-byte aligned inside, so the bytes travel global -> registers -> LDS -> registers: a wave reads
 // its 32 weight rows x 8 blocks (272 contiguous bytes per row, 16-byte aligned because 8 blocks = 17 x 16 bytes) with
-// whole-chunk loads by consecutive lanes, parks them in a wave-private LDS tile whose row stride (280 bytes) spreads
+// whole-chunk loads by consecutive lanes, parks them in a wave-private LDS tile whose row stride (272 bytes: unpadded) spreads
 // the rows over all banks, and each lane then picks its 8 quants of a block (for each half of the tile's 32 rows) with
 // aligned dword reads and a byte funnel shift. The next group of 8 blocks is in flight while the current one is multiplied.
 //
@@ -33,8 +33,10 @@ namespace {
 
 constexpr uint32_t kWaves = 8, kThreads = kWaves * kWave;
 constexpr uint32_t kGroupBlocks = 8, kGroupBytes = kGroupBlocks * 34, kGroupChunks = kGroupBytes / 16;  // 272 B = 17 chunks
-constexpr uint32_t kTileStride = 280;                     // bytes between rows of the LDS weight tile
-constexpr uint32_t kTileBytes = 32 * kTileStride;         // 8 960 B per wave
+// Bytes between rows of the LDS weight tile: 68 dwords = 4 mod 64 banks, so the sixteen rows times two column quarters that a
+// half-wave reads one dword of land in 32 different banks, and the tile is written as the contiguous run of chunks it is.
+constexpr uint32_t kTileStride = kGroupBytes;
+constexpr uint32_t kTileBytes = 32 * kTileStride;         // 8 704 B per wave
 constexpr uint32_t kStageLoads = (32 * kGroupChunks + kWave - 1) / kWave;  // 9 chunk loads per lane and group (the last half used)
 
 struct Q8MfmaArgs {
@@ -149,9 +151,8 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
         for (uint32_t t = 0; t < kStageLoads; ++t) {
             uint32_t id = t * kWave + lane;
             id = id < 32 * kGroupChunks ? id : 32 * kGroupChunks - 1;
-            uint8_t* at = tile + (id / kGroupChunks) * kTileStride + (id % kGroupChunks) * 16;  // 8-byte aligned
-            *reinterpret_cast<uint2*>(at) = stage[SET][t][0];
-            *reinterpret_cast<uint2*>(at + 8) = stage[SET][t][1];
+            uint8_t* at = tile + (id / kGroupChunks) * kTileStride + (id % kGroupChunks) * 16;
+            *reinterpret_cast<uint4*>(at) = uint4{stage[SET][t][0].x, stage[SET][t][0].y, stage[SET][t][1].x, stage[SET][t][1].y};
         }
     };
 
@@ -218,11 +219,11 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
                 const f32x4 zero{};
 #pragma unroll
                 for (int nt = 0; nt < 2; ++nt) {
-                    // independent products of the hi and lo halves of the rows with the block's integer quants
-                    const f32x4 part_hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, b_frag[nt], zero, 0, 0, 0);
+                    // the lo halves of the rows first, the hi halves on top of them: one f32 result per block to scale
                     const f32x4 part_lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, b_frag[nt], zero, 0, 0, 0);
+                    const f32x4 part = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, b_frag[nt], part_lo, 0, 0, 0);
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) acc[nt][v] = __builtin_fmaf(scale_d[nt], part_hi[v] + part_lo[v], acc[nt][v]);  // rows 4 kq + v
+                    for (int v = 0; v < 4; ++v) acc[nt][v] = __builtin_fmaf(scale_d[nt], part[v], acc[nt][v]);  // rows 4 kq + v
                 }
             };
             block(std::integral_constant<int, 0>{});
