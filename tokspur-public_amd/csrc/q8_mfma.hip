@@ -126,21 +126,38 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     }
     __syncthreads();
 
+    // The activation chunk of block B of group g, columns 8 kq .. 8 kq + 7, is chunk g * 32 + B * 4 + kq of row `arow`, kept at
+    // position chunk ^ arow. arow < kRows only flips the low bits, which B % kVariants and kq decide: the lane keeps one
+    // address per variant and the rest of the chunk index is an offset known when the code is compiled (B) or uniform (g).
     const uint32_t arow = n16 & (kRows - 1);
-    auto a_frag = [&](const _Float16* plane, uint32_t chunk) {
-        return *reinterpret_cast<const f16x8*>(plane + (arow * chunks + (chunk ^ arow)) * 8);
-    };
-    // chunk `id` of a group tile: row id / 17 of the wave's 32, bytes (id % 17) * 16 of that row's 272
+    constexpr uint32_t kVariants = kRows / 4;
+    uint32_t a_at[kVariants];  // in halves, from the start of a plane
+#pragma unroll
+    for (uint32_t v = 0; v < kVariants; ++v) a_at[v] = (arow * chunks + ((v * 4 + kq) ^ arow)) * 8;
+    // chunk `id` of a group tile: row id / 17 of the wave's 32, bytes (id % 17) * 16 of that row's 272. The byte offsets from
+    // the tile's first row and the group's first byte never change, so a request is a uniform address plus a lane offset.
+    uint32_t chunk_at[kStageLoads];
+#pragma unroll
+    for (uint32_t t = 0; t < kStageLoads; ++t) {
+        uint32_t id = t * kWave + lane;
+        id = id < 32 * kGroupChunks ? id : 32 * kGroupChunks - 1;  // the tail lanes repeat the last chunk
+        chunk_at[t] = (id / kGroupChunks) * row_bytes + (id % kGroupChunks) * 16;
+    }
     uint2 stage[DEPTH][kStageLoads][2];
     auto fetch_group = [&](uint32_t row0, uint32_t group, auto set_tag) {
         constexpr int SET = decltype(set_tag)::value;
+        const uint8_t* from = a.matrix + uint64_t(row0) * row_bytes + uint64_t(g0 + group) * kGroupBytes;  // uniform
+        const bool whole = row0 + 32 <= a.rows;                                                           // uniform
 #pragma unroll
         for (uint32_t t = 0; t < kStageLoads; ++t) {
-            uint32_t id = t * kWave + lane;
-            id = id < 32 * kGroupChunks ? id : 32 * kGroupChunks - 1;  // the tail lanes repeat the last chunk
-            uint32_t row = row0 + id / kGroupChunks;
-            row = row < a.rows ? row : a.rows - 1;
-            const uint4 v = *reinterpret_cast<const uint4*>(a.matrix + uint64_t(row) * row_bytes + (g0 + group) * kGroupBytes + (id % kGroupChunks) * 16);
+            uint32_t at = chunk_at[t];
+            if (!whole) {  // the matrix's last tile: rows past the end repeat the last row
+                uint32_t id = t * kWave + lane;
+                id = id < 32 * kGroupChunks ? id : 32 * kGroupChunks - 1;
+                const uint32_t row = row0 + id / kGroupChunks < a.rows ? id / kGroupChunks : a.rows - 1 - row0;
+                at = row * row_bytes + (id % kGroupChunks) * 16;
+            }
+            const uint4 v = *reinterpret_cast<const uint4*>(from + at);
             stage[SET][t][0] = uint2{v.x, v.y};
             stage[SET][t][1] = uint2{v.z, v.w};
         }
@@ -214,8 +231,9 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
                     b_frag[nt] = quants8(w[0], w[1]);
                     scale_d[nt] = half_bits_to_float(*reinterpret_cast<const uint16_t*>(tile + (nt * 16 + n16) * kTileStride + 34 * B));
                 }
-                const uint32_t chunk = g * 32 + B * 4 + kq;  // columns g*256 + B*32 + 8 kq
-                const f16x8 ah = a_frag(a_hi, chunk), al = a_frag(a_lo, chunk);
+                // columns g * 256 + B * 32 + 8 kq of the lane's token row
+                const uint32_t at = a_at[B % kVariants] + (g * 32 + (B / kVariants) * kVariants * 4) * 8;
+                const f16x8 ah = *reinterpret_cast<const f16x8*>(a_hi + at), al = *reinterpret_cast<const f16x8*>(a_lo + at);
                 const f32x4 zero{};
 #pragma unroll
                 for (int nt = 0; nt < 2; ++nt) {
