@@ -15,7 +15,9 @@
 // aligned dword reads and a byte funnel shift. The next group of 8 blocks is in flight while the current one is multiplied.
 //
 // Workgroups are persistent (one per compute unit, 8 waves): the activations are staged once per workgroup, which owns
-// a contiguous share of the matrix's 32-row tiles; its waves take tiles from that share through a counter in LDS.
+// a contiguous share of the matrix's 32-row tiles; its waves take tiles from that share through a counter in LDS. A
+// lane asks for its share of the token rows first and for its wave's first weight bytes second, and stages the rows
+// while the weights travel. Every address inside the loop is a uniform base plus a lane offset fixed before the loop.
 //
 // Nine to sixteen token rows do not fit LDS for all of K beside the weight tiles, so that variant splits K in two:
 // even workgroups take the first half of the columns, odd ones the second, each over its share of the tiles, and both
@@ -79,61 +81,27 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     const uint32_t k0 = (blockIdx.x % KSPLIT) * K, g0 = k0 / 256;
     const uint32_t sharer = blockIdx.x / KSPLIT, sharers = gridDim.x / KSPLIT;  // the host launches a multiple of KSPLIT
     if (tid == 0) next_tile = uint32_t(uint64_t((a.rows + 31) / 32) * sharer / sharers);
+    __syncthreads();  // the tile counter is set before any wave takes from it
     _Float16* const a_hi = reinterpret_cast<_Float16*>(lds);
     _Float16* const a_lo = a_hi + kRows * K;
     uint8_t* const tile = lds + 2 * kRows * K * 2 + wave * kTileBytes;
 
-    // ---- stage the token rows: largest magnitude -> power-of-two scale -> hi/lo halves, 16-byte chunks swizzled by row
+    // ---- the token rows: this lane's 16-byte chunks are requested first (they come from cache and return first), then the
+    // wave's first weight bytes, and only then the arithmetic: largest magnitude -> power-of-two scale -> hi/lo halves,
+    // 16-byte chunks swizzled by row. The weights travel while the rows are staged.
+    constexpr uint32_t kMine = 4;  // chunks per lane: kRows * K / 8 <= 2048 = 4 * kThreads for K <= 2048 (8 rows) or 1024 (16 rows)
     uint32_t bad = 0;
-    float biggest = 0;
-    for (uint32_t i = tid; i < a.m * (K / 4); i += kThreads) {
-        const float4 v = *reinterpret_cast<const float4*>(a.x + uint64_t(i / (K / 4)) * a.columns + k0 + (i % (K / 4)) * 4);
-        if (nonfinite(v.x) || nonfinite(v.y) || nonfinite(v.z) || nonfinite(v.w)) bad = TSP_ERRBIT_NONFINITE;
-        biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
-    }
+    float4 xv[kMine][2];
 #pragma unroll
-    for (int step = 32; step >= 1; step >>= 1) biggest = fmaxf(biggest, __shfl_xor(biggest, step, kWave));
-    if (lane == 0) wave_max[wave] = biggest;
-    __syncthreads();
-    biggest = wave_max[0];
-#pragma unroll
-    for (uint32_t w = 1; w < kWaves; ++w) biggest = fmaxf(biggest, wave_max[w]);
-    float scale = 1.0f, inv_scale = 1.0f;
-    if (biggest > 0 && !nonfinite(biggest)) {
-        const int e = int((__float_as_uint(biggest) >> 23) & 0xffu) - 127;
-        int shift = 13 - e;
-        shift = shift > 100 ? 100 : shift < -100 ? -100 : shift;
-        scale = __uint_as_float(uint32_t(127 + shift) << 23);
-        inv_scale = __uint_as_float(uint32_t(127 - shift) << 23);
-    }
-    for (uint32_t i = tid; i < kRows * chunks; i += kThreads) {
-        const uint32_t r = i / chunks, c = i % chunks;
-        f16x8 hi{}, lo{};
-        if (r < a.m) {
+    for (uint32_t j = 0; j < kMine; ++j) {
+        const uint32_t i = tid + j * kThreads, r = i / chunks, c = i % chunks;
+        xv[j][0] = xv[j][1] = float4{0, 0, 0, 0};
+        if (i < kRows * chunks && r < a.m) {
             const float4* src = reinterpret_cast<const float4*>(a.x + uint64_t(r) * a.columns + k0 + c * 8);
-            const float4 v0 = src[0], v1 = src[1];
-            const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float s = v[e] * scale;
-                hi[e] = _Float16(s);
-                lo[e] = _Float16(s - float(hi[e]));
-            }
+            xv[j][0] = src[0];
+            xv[j][1] = src[1];
         }
-        const uint32_t at = (r * chunks + (c ^ r)) * 8;
-        *reinterpret_cast<f16x8*>(a_hi + at) = hi;
-        *reinterpret_cast<f16x8*>(a_lo + at) = lo;
     }
-    __syncthreads();
-
-    // The activation chunk of block B of group g, columns 8 kq .. 8 kq + 7, is chunk g * 32 + B * 4 + kq of row `arow`, kept at
-    // position chunk ^ arow. arow < kRows only flips the low bits, which B % kVariants and kq decide: the lane keeps one
-    // address per variant and the rest of the chunk index is an offset known when the code is compiled (B) or uniform (g).
-    const uint32_t arow = n16 & (kRows - 1);
-    constexpr uint32_t kVariants = kRows / 4;
-    uint32_t a_at[kVariants];  // in halves, from the start of a plane
-#pragma unroll
-    for (uint32_t v = 0; v < kVariants; ++v) a_at[v] = (arow * chunks + ((v * 4 + kq) ^ arow)) * 8;
     // chunk `id` of a group tile: row id / 17 of the wave's 32, bytes (id % 17) * 16 of that row's 272. The byte offsets from
     // the tile's first row and the group's first byte never change, so a request is a uniform address plus a lane offset.
     uint32_t chunk_at[kStageLoads];
@@ -162,17 +130,6 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
             stage[SET][t][1] = uint2{v.z, v.w};
         }
     };
-    auto store_group = [&](auto set_tag) {
-        constexpr int SET = decltype(set_tag)::value;
-#pragma unroll
-        for (uint32_t t = 0; t < kStageLoads; ++t) {
-            uint32_t id = t * kWave + lane;
-            id = id < 32 * kGroupChunks ? id : 32 * kGroupChunks - 1;
-            uint8_t* at = tile + (id / kGroupChunks) * kTileStride + (id % kGroupChunks) * 16;
-            *reinterpret_cast<uint4*>(at) = uint4{stage[SET][t][0].x, stage[SET][t][0].y, stage[SET][t][1].x, stage[SET][t][1].y};
-        }
-    };
-
     // Each workgroup owns a contiguous share of the 32-row tiles and its waves take the next free tile of that share from
     // a counter in LDS (which wave computes a tile does not change the result). The bytes of the next (tile, group) item
     // are requested before the current one is multiplied, so a wave always holds its next tile index one step ahead.
@@ -192,6 +149,68 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
             fetch_group(t * 32, 3, std::integral_constant<int, 3 % DEPTH>{});
         }
     }
+    __builtin_amdgcn_sched_barrier(0);  // every request above is out before the first wait below
+    float biggest = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < kMine; ++j) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float4 v = xv[j][h];
+            if (nonfinite(v.x) || nonfinite(v.y) || nonfinite(v.z) || nonfinite(v.w)) bad = TSP_ERRBIT_NONFINITE;
+            biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        }
+    }
+    biggest = wave_largest(biggest);
+    if (lane == 0) wave_max[wave] = biggest;
+    __syncthreads();
+    biggest = wave_max[0];
+#pragma unroll
+    for (uint32_t w = 1; w < kWaves; ++w) biggest = fmaxf(biggest, wave_max[w]);
+    float scale = 1.0f, inv_scale = 1.0f;
+    if (biggest > 0 && !nonfinite(biggest)) {
+        const int e = int((__float_as_uint(biggest) >> 23) & 0xffu) - 127;
+        int shift = 13 - e;
+        shift = shift > 100 ? 100 : shift < -100 ? -100 : shift;
+        scale = __uint_as_float(uint32_t(127 + shift) << 23);
+        inv_scale = __uint_as_float(uint32_t(127 - shift) << 23);
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < kMine; ++j) {
+        const uint32_t i = tid + j * kThreads, r = i / chunks, c = i % chunks;
+        if (i >= kRows * chunks) break;
+        const float v[8] = {xv[j][0].x, xv[j][0].y, xv[j][0].z, xv[j][0].w, xv[j][1].x, xv[j][1].y, xv[j][1].z, xv[j][1].w};
+        f16x8 hi, lo;  // zeros for the rows past a.m
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float sv = v[e] * scale;
+            hi[e] = _Float16(sv);
+            lo[e] = _Float16(sv - float(hi[e]));
+        }
+        const uint32_t at = (r * chunks + (c ^ r)) * 8;
+        *reinterpret_cast<f16x8*>(a_hi + at) = hi;
+        *reinterpret_cast<f16x8*>(a_lo + at) = lo;
+    }
+    __syncthreads();
+
+    // The activation chunk of block B of group g, columns 8 kq .. 8 kq + 7, is chunk g * 32 + B * 4 + kq of row `arow`, kept at
+    // position chunk ^ arow. arow < kRows only flips the low bits, which B % kVariants and kq decide: the lane keeps one
+    // address per variant and the rest of the chunk index is an offset known when the code is compiled (B) or uniform (g).
+    const uint32_t arow = n16 & (kRows - 1);
+    constexpr uint32_t kVariants = kRows / 4;
+    uint32_t a_at[kVariants];  // in halves, from the start of a plane
+#pragma unroll
+    for (uint32_t v = 0; v < kVariants; ++v) a_at[v] = (arow * chunks + ((v * 4 + kq) ^ arow)) * 8;
+    auto store_group = [&](auto set_tag) {
+        constexpr int SET = decltype(set_tag)::value;
+#pragma unroll
+        for (uint32_t t = 0; t < kStageLoads; ++t) {
+            uint32_t id = t * kWave + lane;
+            id = id < 32 * kGroupChunks ? id : 32 * kGroupChunks - 1;
+            uint8_t* at = tile + (id / kGroupChunks) * kTileStride + (id % kGroupChunks) * 16;
+            *reinterpret_cast<uint4*>(at) = uint4{stage[SET][t][0].x, stage[SET][t][0].y, stage[SET][t][1].x, stage[SET][t][1].y};
+        }
+    };
+
     for (; t < share_end; t = t_next, t_next = take_tile()) {
         const uint32_t row0 = t * 32;
         float acc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}};  // [16-row half of the tile][token row 4 kq + v]
