@@ -99,7 +99,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path is built and measured on a single MI355X (--gpus 1); "
-              "how it would shard is described in DESIGN.md", file=sys.stderr)
+              "across GPUs the experts would be sharded and the routed rows exchanged all-to-all, which is not built here",
+              file=sys.stderr)
         sys.exit(2)
 
     import torch
