@@ -379,6 +379,19 @@ uint64_t tsp_logit_topk_output_bytes(uint32_t max_rows);
 int tsp_logit_topk(const float* logits, uint64_t stride_bytes, uint32_t rows, uint32_t vocabulary, void* partial_scratch,
                    uint64_t scratch_bytes, void* out_rows, uint64_t out_bytes, void* stream);
 
+/* `tsp_logit_topk` for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid it) and so have no scratch buffer to hand over. No counterpart in the reference. The partial rows
+ * live in a device array inside the library (540 672 bytes per device, held until the process ends); the call allocates
+ * and frees nothing. At most TSP_LOGIT_TOPK_STATIC_MAX_ROWS rows of at most TSP_LOGIT_TOPK_STATIC_MAX_VOCABULARY
+ * columns; larger shapes are refused with TSP_ERR_FORMAT. Results are bit-identical to tsp_logit_topk. Every call on one
+ * device shares that device's array: calls that overlap in time on one device (two streams, two threads) race. The
+ * first call on a device looks the array's address up, which may not be done under stream capture: make one call
+ * before capturing. */
+#define TSP_LOGIT_TOPK_STATIC_MAX_ROWS 16u
+#define TSP_LOGIT_TOPK_STATIC_MAX_VOCABULARY 262144u
+int tsp_logit_topk_static(const float* logits, uint64_t stride_bytes, uint32_t rows, uint32_t vocabulary, void* out_rows,
+                          uint64_t out_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

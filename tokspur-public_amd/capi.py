@@ -573,6 +573,16 @@ def logit_topk(dev, logits, rows, vocabulary, stride_bytes=None, scratch=None, o
     return out
 
 
+def logit_topk_static(dev, logits, rows, vocabulary, stride_bytes=None, out=None):
+    """`tsp_logit_topk_static`: the same rows with the partial rows kept in the library's own device array (no scratch
+    argument, nothing allocated by the call when `out` is given)."""
+    stride_bytes = vocabulary * 4 if stride_bytes is None else stride_bytes
+    out = dev.empty(logit_topk_output_bytes(rows), "uint8") if out is None else out
+    check(dll().tsp_logit_topk_static(dev.ptr(logits), C.c_uint64(stride_bytes), C.c_uint32(rows), C.c_uint32(vocabulary), dev.ptr(out),
+                                      C.c_uint64(dev.nbytes(out)), dev.stream()))
+    return out
+
+
 def calibration_copy(dev, dst, src):
     """Plain copy kernel of a known size (scales a profiler's HBM byte counters)."""
     check(dll().tsp_calibration_copy(dev.ptr(dst), dev.ptr(src), C.c_uint64(dev.nbytes(src)), dev.stream()))

@@ -204,6 +204,14 @@ __global__ __launch_bounds__(kThreads) void topk_stage2(TopKArgs a) {
 
 uint32_t tiles_for(uint32_t vocabulary) { return (vocabulary + kTileSpan - 1) / kTileSpan; }
 
+int launch_topk(const TopKArgs& a, hipStream_t s) {
+    TSP_LAUNCH("logit_topk_stage1", s, topk_stage1<<<dim3(a.tiles, a.rows), kThreads, 0, s>>>(a));
+    const int rc = launch_status("logit_topk_stage1");
+    if (rc != TSP_OK) return rc;
+    TSP_LAUNCH("logit_topk_stage2", s, topk_stage2<<<a.rows, kThreads, 0, s>>>(a));
+    return launch_status("logit_topk_stage2");
+}
+
 }  // namespace
 
 extern "C" uint64_t tsp_logit_topk_scratch_bytes(uint32_t max_rows, uint32_t max_vocabulary) {
@@ -242,10 +250,50 @@ extern "C" int tsp_logit_topk(const float* logits, uint64_t stride_bytes, uint32
                 "GPU logit top-k buffers overlap");
     TopKArgs a{logits, stride_bytes, rows, vocabulary, tiles, static_cast<tsp_logit_topk_row*>(partial_scratch),
                static_cast<tsp_logit_topk_row*>(out_rows)};
-    const auto s = static_cast<hipStream_t>(stream);
-    TSP_LAUNCH("logit_topk_stage1", s, topk_stage1<<<dim3(tiles, rows), kThreads, 0, s>>>(a));
-    int rc = launch_status("logit_topk_stage1");
+    return launch_topk(a, static_cast<hipStream_t>(stream));
+}
+
+// ---------------------------------------------------------------- the same operator for callers that cannot allocate
+// The partial rows live in a file-scope device array instead of a caller's buffer. In host code the array's name is only
+// a handle: its device address is asked for once per device (each device holds its own copy at its own address) and kept.
+namespace {
+constexpr uint32_t kStaticRows = 16, kStaticTiles = 64;  // 16 rows x 262 144 columns: 540 672 bytes per device
+}
+static __device__ __align__(256) uint8_t scratch[uint64_t(kStaticRows) * kStaticTiles * sizeof(tsp_logit_topk_row)];
+namespace {
+std::atomic<void*> g_scratch_at[64];
+int static_scratch(void** at) {
+    int device = 0;
+    TSP_HIP(hipGetDevice(&device));
+    TSP_REQUIRE(device >= 0 && device < 64, "GPU logit top-k: device ordinal out of range");
+    void* p = g_scratch_at[device].load(std::memory_order_acquire);
+    if (!p) {
+        TSP_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        TSP_REQUIRE(p != nullptr, "GPU logit top-k: the static scratch array has no device address");
+        g_scratch_at[device].store(p, std::memory_order_release);
+    }
+    *at = p;
+    return TSP_OK;
+}
+}  // namespace
+
+static_assert(kStaticRows == TSP_LOGIT_TOPK_STATIC_MAX_ROWS && kStaticTiles * kTileSpan == TSP_LOGIT_TOPK_STATIC_MAX_VOCABULARY, "limits in the header");
+
+extern "C" int tsp_logit_topk_static(const float* logits, uint64_t stride_bytes, uint32_t rows, uint32_t vocabulary, void* out_rows,
+                                     uint64_t out_bytes, void* stream) {
+    TSP_REQUIRE(rows >= 1 && rows <= kStaticRows && vocabulary >= 1 && vocabulary <= kStaticTiles * kTileSpan,
+                "GPU logit top-k without a scratch argument takes at most %u rows of at most %u columns", kStaticRows, kStaticTiles * kTileSpan);
+    TSP_REQUIRE(stride_bytes >= uint64_t(vocabulary) * 4 && stride_bytes % 4 == 0, "GPU logit top-k geometry mismatch");
+    TSP_REQUIRE(logits && out_rows, "null device pointer");
+    const uint32_t tiles = tiles_for(vocabulary);
+    const uint64_t in_bytes = uint64_t(rows - 1) * stride_bytes + uint64_t(vocabulary) * 4, need_out = uint64_t(rows) * sizeof(tsp_logit_topk_row);
+    TSP_REQUIRE(out_bytes >= need_out && reinterpret_cast<uintptr_t>(logits) % 4 == 0 && reinterpret_cast<uintptr_t>(out_rows) % 4 == 0,
+                "GPU logit top-k buffer span or alignment mismatch");
+    TSP_REQUIRE(!ranges_overlap(logits, in_bytes, out_rows, need_out), "GPU logit top-k buffers overlap");
+    void* partial = nullptr;
+    const int rc = static_scratch(&partial);
     if (rc != TSP_OK) return rc;
-    TSP_LAUNCH("logit_topk_stage2", s, topk_stage2<<<rows, kThreads, 0, s>>>(a));
-    return launch_status("logit_topk_stage2");
+    // every partial row stage 2 reads is written by stage 1 of the same call: nothing has to start at zero
+    TopKArgs a{logits, stride_bytes, rows, vocabulary, tiles, static_cast<tsp_logit_topk_row*>(partial), static_cast<tsp_logit_topk_row*>(out_rows)};
+    return launch_topk(a, static_cast<hipStream_t>(stream));
 }
