@@ -1,0 +1,306 @@
+// Grouped gate/up GEMM with fused SwiGLU for 2048-column Q4_K experts, activations resident in registers.
+//
+// The ragged grouped product is bound by the expert weights streaming in from HBM, so the kernel is built around that
+// stream and keeps everything else off the memory pipeline:
+//
+//   * One persistent workgroup of eight waves per CU. The launch's work, the (task, 32 hidden units) items in task order,
+//     is cut into equal contiguous shares, one per workgroup; consecutive shares go to workgroups of the same XCD so that
+//     the tasks of one expert meet in one L2.
+//   * The K dimension is split over the waves: wave w owns super-block w (columns 256 w .. 256 w + 255) of every weight
+//     row. Its A operands, the task's <= 64 activation rows of those 256 columns, are loaded ONCE per task into registers
+//     (64 or 128 VGPRs as MFMA fragments) and stay there while all of the expert's rows stream past. No activation byte is
+//     read twice per task and none passes through LDS.
+//   * Weights go global -> LDS directly (no registers in between), a tile of 32 rows x one 128-byte line of nibbles +
+//     the rows' scale bytes and d/dmin per request, into a wave-private ring of two stages. Eight neighbouring lanes fetch
+//     one whole cache line. Nothing but these requests and the epilogue's stores uses the vector memory counter inside
+//     the loop, so each wave waits with an exact count, and since the ring is private no barrier guards it.
+//   * A wave's product over its super-block, d * sum(x * sc*q) - dmin * sum(Sx * mn), is a partial result of a 32 x 32
+//     tile; the eight partials add up through LDS in wave order (a fixed order: results are reproducible bit for bit) with
+//     one barrier per tile, and the threads that hold gate and up of the same hidden units apply SwiGLU and store h / 256
+//     as halves, the format the down GEMM reads.
+//   * What bounds the kernel is the vector unit: a SIMD issues one vector instruction per four cycles whichever of its
+//     two waves it comes from, and unpacking costs about one and a half of them per weight (mask-or, packed multiply-add,
+//     a share of the shifts and of the scale set-up). Everything else a wave executes per tile is kept short for that
+//     reason: scales are set up two sub-blocks at a time, the sigmoid uses the hardware exponential and reciprocal, and
+//     the tasks of at most 32 rows (most of them) run in a loop of their own that keeps every address in registers.
+#include "gate_up_resident.hpp"
+#include "mfma_quant.hpp"
+
+#include <type_traits>
+
+using namespace tsp;
+
+namespace {
+
+constexpr int kWaves = 8, kThreads = kWaves * kWave;
+constexpr int kTaskRows = 64;              // rows of a task (the grouped GEMMs' own task list)
+constexpr int kStageBytes = 5120;          // 32 rows x 128 B of nibbles, 32 x 16 B of scales / minima, 32 x 16 B holding d / dmin
+constexpr int kStages = 2;
+constexpr int kPartialBytes = 4096;        // one wave's 32 x 32 f32 partial tile
+constexpr int kPhaseBytes = kWaves * kPartialBytes;
+constexpr int kTileLoads = 5;              // direct-to-LDS requests per tile and wave
+
+struct TaskInfo { uint32_t expert, start, nrows; bool shared, ok; };
+
+__device__ __forceinline__ TaskInfo resolve_task(const ResidentGateUpArgs& a, uint32_t task) {
+    TaskInfo t;
+    t.expert = a.tasks[2 + 2 * task];
+    t.start = a.tasks[3 + 2 * task];
+    t.shared = a.shared_gate != nullptr && t.expert == a.experts;
+    const uint32_t count = t.shared ? a.tokens : t.expert < a.experts ? a.counts[t.expert] : 0;
+    t.ok = (t.expert < a.experts || t.shared) && count <= a.tokens && t.start < count;
+    t.nrows = t.ok ? (count - t.start < kTaskRows ? count - t.start : kTaskRows) : 0;
+    if (!t.ok) { t.expert = 0; t.start = 0; t.shared = false; }  // addresses stay inside the tensors; nothing of it is stored
+    return t;
+}
+
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gate_up_resident_kernel(ResidentGateUpArgs a) {
+    // LDS: [2 phases][8 waves][4 KB partial tile] | [8 waves][2 stages][5 KB weight tile] | row tables of two tasks
+    constexpr int kStagesAt = 2 * kPhaseBytes;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kStagesAt + kWaves * kStages * kStageBytes + 2 * kTaskRows * 4];
+    uint32_t* const row_ok = reinterpret_cast<uint32_t*>(lds_raw + kStagesAt + kWaves * kStages * kStageBytes);  // [2][64]
+
+    const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const uint32_t n = lane % 32, khalf = lane / 32;
+    constexpr uint32_t bpr = 8;  // 2048 columns
+    const uint32_t units = a.hidden / 32;
+
+    // ---- the launch's task list must be whole before anything is addressed through it
+    const uint32_t bound = a.task_slots;
+    const uint32_t listed = a.tasks[0];
+    if (listed > bound || a.tasks[1] != a.tokens * a.selected || a.classes[0] + a.classes[1] != listed) {
+        if (tid == 0 && blockIdx.x == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+        return;
+    }
+    const uint32_t groups = gridDim.x, share = (blockIdx.x % 8) * (groups / 8) + blockIdx.x / 8;
+
+    uint8_t* const my_stage = lds_raw + kStagesAt + wave * (kStages * kStageBytes);
+
+    const uint32_t my_stage_lds = __builtin_amdgcn_readfirstlane(lds_address(my_stage));
+
+    // ---- per-lane parts of the request addresses (the per-tile parts are uniform and stay in scalar registers)
+    // nibbles: request q covers rows 8q .. 8q+7 of the tile, eight lanes per row; lane l sits at 16-byte slot l % 8 of
+    // its row in LDS and fetches chunk (l % 8) ^ (row % 8), so that the fragment reads below spread over all banks
+    const uint32_t qs_lane = uint32_t(a.spec.qs_offset) + (lane / 8) * (bpr * 128) + wave * 128 + (((lane % 8) ^ ((lane / 8) & 7)) * 16);
+    // lanes 0..31: scales and minima of row l (16 B); lanes 32..63: the 16 bytes holding d / dmin of row l - 32
+    const uint32_t hdr_lane = lane < 32 ? uint32_t(a.spec.sm_offset) + lane * (bpr * 16) + wave * 16
+                                        : uint32_t(a.spec.dm_offset) + (lane - 32) * (bpr * 4) + (wave / 4) * 16;
+    const uint32_t hdr_unit_step = lane < 32 ? 32 * bpr * 16 : 32 * bpr * 4;
+
+    auto weight_bases = [&](const TaskInfo& t, const uint8_t*& gate, const uint8_t*& up) {
+        if (t.shared) { gate = a.shared_gate; up = a.shared_up; return; }
+        const uint32_t half_e = a.experts / 2;
+        const uint8_t* pair = (t.expert < half_e ? a.pair_lo : a.pair_hi) + uint64_t(t.expert < half_e ? t.expert : t.expert - half_e) * 2 * a.spec.planar_expert_bytes;
+        gate = pair;
+        up = pair + a.spec.planar_expert_bytes;
+    };
+    auto request_tile = [&](const uint8_t* base, uint32_t unit, uint32_t stage_offset) {  // base: one expert (under 4 GiB), uniform
+        const uint8_t* qs = base + uint64_t(unit) * (32 * bpr * 128);
+        const uint32_t dst = my_stage_lds + stage_offset;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) load_to_lds_16(qs + q * (8 * bpr * 128), qs_lane, dst + q * 1024);
+        load_to_lds_16(base, hdr_lane + unit * hdr_unit_step, dst + 4096);
+    };
+
+    uint32_t bad = 0, phase = 0;
+    const Q4Consts q4c = q4_consts();
+    const Q4ScaleConsts q4s = q4_scale_consts();
+
+    // The tasks come in two kinds, those of at most 32 rows (one row tile: 64 registers of activations) and those of 33..64
+    // (two row tiles, 128 registers), each with its own loop so that neither carries the other's registers. A workgroup takes
+    // the same share of either kind's (task, unit) items: equal work for every workgroup whatever the mix of kinds.
+    auto pass = [&](auto mt_tag) {
+        constexpr int MT = decltype(mt_tag)::value;
+        const uint32_t of_kind = a.classes[MT - 1];
+        const uint32_t* list = a.classes + 2 + (MT - 1) * bound;
+        const uint32_t items = of_kind * units;
+        const uint32_t it0 = uint32_t(uint64_t(items) * share / groups), it1 = uint32_t(uint64_t(items) * (share + 1) / groups);
+        if (it0 >= it1) return;
+        const uint32_t k0 = it0 / units, k1 = (it1 - 1) / units;  // first and last position in the kind's list
+        auto first_unit = [&](uint32_t k) { return k == k0 ? it0 % units : 0; };
+        auto end_unit = [&](uint32_t k) { return k == k1 ? (it1 - 1) % units + 1 : units; };
+        auto task_at = [&](uint32_t k) { const uint32_t t = list[k]; return t < listed ? t : 0; };
+
+        f16x8 A[MT][16];   // activation fragments: [row tile][k16 step of the super-block]
+        f16x8 sxA[MT];     // activation sums (k-half 0: the eight sub-block sums' high halves, k-half 1: the residuals)
+        // ---- the request cursor runs two tiles ahead of the arithmetic: (list position, unit, gate or up)
+        uint32_t rk = k0, runit = first_unit(k0), rj = 0, rstage = 0;
+        bool rdone = false;
+        const uint8_t *rgate, *rup;
+        weight_bases(resolve_task(a, task_at(k0)), rgate, rup);
+        auto request_next = [&]() {  // past the end of the share the last tile is requested again (unused)
+            request_tile(rj == 0 ? rgate : rup, runit, rstage);
+            rstage = rstage + kStageBytes == kStages * kStageBytes ? 0 : rstage + kStageBytes;
+            if (rdone) return;
+            if (rj == 0) { rj = 1; return; }
+            if (runit + 1 < end_unit(rk)) { rj = 0; ++runit; return; }
+            if (rk == k1) { rdone = true; return; }
+            ++rk;
+            rj = 0;
+            runit = 0;
+            weight_bases(resolve_task(a, task_at(rk)), rgate, rup);
+        };
+        request_next();
+        request_next();
+        uint32_t stage = 0;  // byte offset of the stage the next tile sits in
+
+        uint32_t task = 0;
+        TaskInfo cur{};
+        auto load_rows = [&](uint32_t k) {  // the task at list position k: its activation rows, this wave's 256 columns of them, into registers
+            task = task_at(k);
+            cur = resolve_task(a, task);
+            if (!cur.ok && tid == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const uint32_t r = i * 32 + n, rr = r < cur.nrows ? r : 0;
+                uint32_t token;
+                bool ok = true;
+                if (cur.shared) {
+                    token = cur.start + rr;
+                } else {
+                    const uint32_t rid = a.token_map[uint64_t(cur.expert) * a.tokens + cur.start + rr];
+                    ok = rid < a.tokens * a.selected && a.ids[rid < a.tokens * a.selected ? rid : 0] == cur.expert;
+                    token = ok ? rid / a.selected : 0;
+                }
+                if (!cur.ok) { token = 0; ok = false; }
+                if (!ok && cur.ok) bad |= TSP_ERRBIT_INDEX;
+                if (wave == 0 && khalf == 0) row_ok[(k & 1) * kTaskRows + r] = ok && r < cur.nrows;
+                const _Float16* row = a.xh + uint64_t(token) * (bpr * 256) + wave * 256 + khalf * 16;
+#pragma unroll
+                for (int t = 0; t < 16; ++t) A[i][t] = *reinterpret_cast<const f16x8*>(row + (t / 4) * 64 + ((t / 2) % 2) * 32 + (t % 2) * 8);
+                sxA[i] = *reinterpret_cast<const f16x8*>(a.sx + (uint64_t(token) * bpr + wave) * 16 + khalf * 8);
+            }
+        };
+
+        // ---- one tile: unpack, multiply, add the eight waves' partial results up, and for an up tile apply SwiGLU and store
+        float gate_sum[MT][2];
+        auto tile = [&](uint32_t k, uint32_t unit, auto j_tag) {
+            constexpr int J = decltype(j_tag)::value;
+            // wait for the tile's five requests (the five of the other stage may still be in flight)
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 1) * kTileLoads) : "memory");
+            // With two row tiles everything a lane derives from its id is derived again per tile from this one register:
+            // hoisted out of the loops these addresses would occupy a dozen registers next to the 128 of the activations.
+            uint32_t lane_now = lane;
+            if constexpr (MT == 2) asm volatile("" : "+v"(lane_now));
+            const uint32_t n = lane_now % 32, khalf = lane_now / 32;
+            const uint8_t* st = my_stage + stage;
+            u32x4 raw[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) raw[p] = *reinterpret_cast<const u32x4*>(st + n * 128 + (((2 * p + khalf) ^ (n & 7)) * 16));
+            const uint4 sm = *reinterpret_cast<const uint4*>(st + 4096 + n * 16);
+            const uint32_t dm = *reinterpret_cast<const uint32_t*>(st + 4096 + 512 + n * 16 + (wave % 4) * 4);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            // the stage is free again: the tile two ahead goes there
+            request_next();
+            stage = stage + kStageBytes == kStages * kStageBytes ? 0 : stage + kStageBytes;
+            const float d = half_bits_to_float(dm & 0xffffu), dmin = half_bits_to_float(dm >> 16);
+
+            f32x16 blk[MT];
+            auto steps = [&](auto p_tag) {
+                constexpr int P = decltype(p_tag)::value;
+                // the scales of sub-blocks 2P (low nibbles) and 2P + 1 (high nibbles, in place as 16 q: scale / 16) as one pair
+                const Q4PairScale sc = q4_pair_scale<P>(sm.x, sm.y, q4s);
+#pragma unroll
+                for (int hi = 0; hi < 2; ++hi) {
+                    f16x8 f[2];
+                    frags_q4k_pair(raw[P], sc, hi, q4c, f);
+#pragma unroll
+                    for (int ff = 0; ff < 2; ++ff)
+#pragma unroll
+                        for (int i = 0; i < MT; ++i) {
+                            if (P == 0 && hi == 0 && ff == 0) {
+                                const f32x16 zero{};
+                                blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][0], f[0], zero, 0, 0, 0);
+                            } else {
+                                blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][P * 4 + hi * 2 + ff], f[ff], blk[i], 0, 0, 0);
+                            }
+                        }
+                }
+            };
+            steps(std::integral_constant<int, 0>{});
+            steps(std::integral_constant<int, 1>{});
+            steps(std::integral_constant<int, 2>{});
+            steps(std::integral_constant<int, 3>{});
+            HdrQ4 hdr;
+            hdr.mn[0] = sm.z; hdr.mn[1] = sm.w;
+            const f16x8 mn = minima_frag(hdr);
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                // partial = d * blk - dmin * sum_s Sx(hi + lo)[m, s] * mn[n, s]
+                const f32x16 zero{};
+                const f32x16 mblk = __builtin_amdgcn_mfma_f32_32x32x16_f16(sxA[i], mn, zero, 0, 0, 0);
+                uint8_t* out = lds_raw + (phase & 1) * kPhaseBytes + wave * kPartialBytes + lane_now * 16;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    f32x4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf(-dmin, mblk[4 * c + e], d * blk[i][4 * c + e]);
+                    *reinterpret_cast<f32x4*>(out + c * 1024) = v;
+                }
+                lds_barrier();
+                // thread tid adds up elements 2 tid, 2 tid + 1 of the eight partial tiles, in wave order
+                const uint8_t* in = lds_raw + (phase & 1) * kPhaseBytes + (wave * kWave + lane_now) * 8;
+                float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll
+                for (int w = 0; w < kWaves; ++w) {
+                    const float2 p2 = *reinterpret_cast<const float2*>(in + w * kPartialBytes);
+                    s0 += p2.x; s1 += p2.y;
+                }
+                ++phase;
+                if constexpr (J == 0) {
+                    gate_sum[i][0] = s0; gate_sum[i][1] = s1;
+                } else {
+                    // element 2 tid + e of the tile is accumulator 4 (wave / 2) + 2 (lane % 2) + e of fragment lane
+                    // 32 (wave % 2) + lane / 2: task row 32 i + 4 wave + 2 (lane % 2) + e, hidden unit lane / 2 of the tile
+                    const float up_sum[2] = {s0, s1};
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const uint32_t r = i * 32 + 4 * wave + 2 * (lane_now % 2) + e;
+                        const float g = gate_sum[i][e], u = up_sum[e];
+                        const float h = (g * sigmoid_fast(g)) * u;
+                        // h travels to the down GEMM as the half nearest to h * 2^-8
+                        const _Float16 carried = _Float16(h * 0.00390625f);
+                        if (row_ok[(k & 1) * kTaskRows + r]) {
+                            if (nonfinite(g) || nonfinite(u) || nonfinite(h) || (__builtin_bit_cast(uint16_t, carried) & 0x7c00u) == 0x7c00u) bad |= TSP_ERRBIT_NONFINITE;
+                            a.hbuf[(uint64_t(task) * kTaskRows + r) * a.hidden + unit * 32 + lane_now / 2] = carried;
+                        }
+                    }
+                }
+            }
+        };
+
+        for (uint32_t k = k0; k <= k1; ++k) {
+            load_rows(k);
+            const uint32_t u1 = end_unit(k);
+            for (uint32_t unit = first_unit(k); unit < u1; ++unit) {
+                tile(k, unit, std::integral_constant<int, 0>{});
+                tile(k, unit, std::integral_constant<int, 1>{});
+            }
+        }
+        wait_all_loads();  // the last requests fetched tiles nobody reads: they must have landed before the stages are reused or given away
+    };
+    pass(std::integral_constant<int, 2>{});
+    pass(std::integral_constant<int, 1>{});
+    publish_error(bad, a.error_word);
+}
+
+}  // namespace
+
+namespace tsp {
+
+bool resident_gate_up_takes(uint32_t channels, uint32_t hidden) { return channels == 2048 && hidden % 32 == 0 && hidden >= 32; }
+
+int launch_resident_gate_up(const ResidentGateUpArgs& a, hipStream_t s) {
+    static std::atomic<uint64_t> seen{0};
+    static int cus[64];
+    int device = 0;
+    if (first_use_on_device(seen, &device) || cus[device] == 0) {
+        int n = 0;
+        TSP_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device));
+        cus[device] = n >= 8 ? n / 8 * 8 : 8;
+    }
+    TSP_LAUNCH("gemm_gate_up_swiglu", s, gate_up_resident_kernel<<<cus[device], kThreads, 0, s>>>(a));
+    return launch_status("gate_up_resident");
+}
+
+}  // namespace tsp

@@ -24,6 +24,7 @@
 //     two and three steps ahead, into a ring of four slabs; one LDS-only barrier per K step.
 //   * For gate/up the two column tiles of a wave are the gate rows and the up rows of the same 32 hidden
 //     units, so SwiGLU is an element-wise epilogue on accumulator registers.
+#include "gate_up_resident.hpp"
 #include "grouping_device.hpp"
 #include "mfma_quant.hpp"
 
@@ -566,14 +567,17 @@ __global__ __launch_bounds__(256) void to_f16_rows(const void* __restrict__ src,
 struct TaskLists {
     const uint32_t* counts; uint32_t* tasks0; uint32_t tile0; uint32_t* tasks1; uint32_t tile1; uint32_t experts, selected, tokens;
     bool every_token1;  // list 1 also holds the always-on expert's tasks
+    uint32_t* classes1;  // list 1 is a 64-row list: its tasks by number of rows (task_class_lists_block), or null
 };
 __global__ __launch_bounds__(512) void tasks_and_rows(TaskLists t, const void* __restrict__ src, uint64_t src_stride_bytes, _Float16* __restrict__ dst,
                                                       _Float16* __restrict__ sx, uint32_t rows, uint32_t columns, uint32_t* error_word) {
     __shared__ uint32_t tiles_scan[512];
     __shared__ uint32_t routes_scan[512];
+    __shared__ uint32_t third_scan[512];
     if (blockIdx.x < 2) {
         grouped_tasks_block(t.counts, blockIdx.x == 0 ? t.tasks0 : t.tasks1, blockIdx.x == 0 ? t.tile0 : t.tile1, t.experts, t.selected, t.tokens,
                             error_word, tiles_scan, routes_scan, blockIdx.x == 1 && t.every_token1);
+        if (blockIdx.x == 1 && t.classes1) task_class_lists_block(t.counts, t.classes1, t.experts, t.selected, t.tokens, t.every_token1, tiles_scan, routes_scan, third_scan);
     } else {
         to_f16_rows_block<false>(src, src_stride_bytes, dst, sx, rows, columns, error_word, blockIdx.x - 2, gridDim.x - 2);
     }
@@ -719,7 +723,7 @@ extern "C" int tsp_grouped_mm(uint32_t encoding, uint32_t layout, const void* ma
     auto* sx = reinterpret_cast<_Float16*>(ws + l.sx);
     auto* task_list = reinterpret_cast<uint32_t*>(ws + l.tasks);
     int rc = tsp_grouped_routes(ids, token_map, counts, experts, selected, tokens, error_word, stream);
-    if (rc == TSP_OK) rc = lists_and_rows(TaskLists{counts, tasks, 32, task_list, kTaskRows, experts, selected, tokens, false}, input, input_stride_bytes, xh, sx,
+    if (rc == TSP_OK) rc = lists_and_rows(TaskLists{counts, tasks, 32, task_list, kTaskRows, experts, selected, tokens, false, nullptr}, input, input_stride_bytes, xh, sx,
                                           l.in_rows, columns, error_word, s);
     if (rc != TSP_OK) return rc;
     GemmArgs a{};
@@ -732,14 +736,15 @@ extern "C" int tsp_grouped_mm(uint32_t encoding, uint32_t layout, const void* ma
 
 // ---------------------------------------------------------------- grouped MoE
 namespace {
-struct NaxLayout { uint64_t xh, sx, tasks, hbuf, meta, total; uint32_t bound; };
+struct NaxLayout { uint64_t xh, sx, tasks, classes, hbuf, meta, total; uint32_t bound; };
 NaxLayout nax_layout(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t channels, uint32_t hidden, bool shared = false) {
     NaxLayout l{};
     l.bound = tokens * selected / kTaskRows + experts + (shared ? (tokens + kTaskRows - 1) / kTaskRows : 0);
     l.xh = 0;
     l.sx = align256(uint64_t(tokens) * channels * 2);
     l.tasks = l.sx + align256(uint64_t(tokens) * (channels / 256) * 32);
-    l.hbuf = l.tasks + align256((2 + 2 * uint64_t(l.bound)) * 4);
+    l.classes = l.tasks + align256((2 + 2 * uint64_t(l.bound)) * 4);  // the 64-row tasks by number of rows: two counts, two index lists
+    l.hbuf = l.classes + align256((2 + 2 * uint64_t(l.bound)) * 4);
     l.meta = l.hbuf + align256(uint64_t(l.bound) * kTaskRows * hidden * 2);  // union records of one chunk of eight tokens
     l.total = l.meta + align256(2320 * 4);
     return l;
@@ -865,7 +870,7 @@ int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void*
     auto* hbuf = reinterpret_cast<_Float16*>(ws + l.hbuf);
 
     rc = tsp_grouped_routes(m->ids, m->token_map, m->counts, m->experts, m->selected, m->tokens, m->error_word, stream);
-    if (rc == TSP_OK) rc = lists_and_rows(TaskLists{m->counts, m->tasks, 32, task_list, kTaskRows, m->experts, m->selected, m->tokens, shared != nullptr}, m->x,
+    if (rc == TSP_OK) rc = lists_and_rows(TaskLists{m->counts, m->tasks, 32, task_list, kTaskRows, m->experts, m->selected, m->tokens, shared != nullptr, reinterpret_cast<uint32_t*>(ws + l.classes)}, m->x,
                                           m->x_stride_bytes, xh, sx, m->tokens, m->channels, m->error_word, s);
     if (rc != TSP_OK) return rc;
 
@@ -875,7 +880,16 @@ int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void*
     g.tokens = m->tokens; g.selected = m->selected; g.n = m->hidden; g.k = m->channels; g.out = hbuf; g.out_scale = 1.0f;
     g.error_word = m->error_word;
     if (shared) { g.shared_w0 = static_cast<const uint8_t*>(shared->gate); g.shared_w1 = static_cast<const uint8_t*>(shared->up); }
-    rc = launch<B_Q4K_PLANAR, EPI_SWIGLU, ROWS_GATHER_TOKENS>(g, (m->hidden + 127) / 128, l.bound, s);
+    if (resident_gate_up_takes(m->channels, m->hidden)) {
+        ResidentGateUpArgs r{};
+        r.xh = xh; r.sx = sx; r.pair_lo = g.w0; r.pair_hi = g.w1; r.shared_gate = g.shared_w0; r.shared_up = g.shared_w1; r.spec = gu;
+        r.experts = m->experts; r.tokens = m->tokens; r.selected = m->selected; r.hidden = m->hidden;
+        r.tasks = task_list; r.classes = reinterpret_cast<const uint32_t*>(ws + l.classes); r.counts = m->counts; r.token_map = m->token_map; r.ids = m->ids; r.task_slots = l.bound;
+        r.hbuf = hbuf; r.error_word = m->error_word;
+        rc = launch_resident_gate_up(r, s);
+    } else {
+        rc = launch<B_Q4K_PLANAR, EPI_SWIGLU, ROWS_GATHER_TOKENS>(g, (m->hidden + 127) / 128, l.bound, s);
+    }
     if (rc != TSP_OK) return rc;
 
     GemmArgs d{};

@@ -30,6 +30,10 @@ __device__ __forceinline__ void lds_barrier_after_loads() {
 __device__ __forceinline__ void load_to_lds_16(const void* src, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(src) : "memory", "m0");
 }
+// The same with the global address as a uniform base (scalar registers) plus a 32-bit byte offset per lane.
+__device__ __forceinline__ void load_to_lds_16(const void* uniform_base, uint32_t lane_offset, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(lane_offset), "s"(uniform_base) : "memory", "m0");
+}
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
     return uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)p));
 }
@@ -122,6 +126,37 @@ __device__ __forceinline__ void frags_q4k_swapped(const u32x4& raw, const HdrQ4&
     const f16x2 s2 = splat(float(sc) * (HI ? 0.0625f : 1.0f)), bias = splat(float(sc) * (HI ? -64.0f : -1024.0f));
     frag[0] = scaled8_q4_swapped<HI>(raw[0], raw[1], s2, bias, c);
     frag[1] = scaled8_q4_swapped<HI>(raw[2], raw[3], s2, bias, c);
+}
+
+// The same unpacking with the scale set-up shared by a pair of sub-blocks: the six-bit scales of sub-blocks 2P and 2P + 1 sit
+// in neighbouring bytes of the header; one byte permute puts them under 0x64 (1024 + sc as halves, side by side), one packed
+// add takes the 1024 off, and two packed multiplies make (sc, sc / 16) and (-1024 sc, -64 sc): the factors and the
+// offsets of the low-nibble and the high-nibble products. Four instructions per pair instead of ten per sub-block.
+struct Q4ScaleConsts { uint32_t sel[2]; uint32_t k64; f16x2 off, mul, bias; };
+__device__ __forceinline__ Q4ScaleConsts q4_scale_consts() {
+    // selector bytes: 0..3 pick a byte of the header word, 4..7 a byte of the constant 0x64646464
+    Q4ScaleConsts c{{0x04010400u, 0x04030402u}, 0x64646464u, f16x2{_Float16(-1024.0f), _Float16(-1024.0f)},
+                    f16x2{_Float16(1.0f), _Float16(0.0625f)}, f16x2{_Float16(-1024.0f), _Float16(-64.0f)}};
+    asm volatile("" : "+s"(c.sel[0]), "+s"(c.sel[1]), "+v"(c.k64));
+    return c;
+}
+struct Q4PairScale { f16x2 mul, bias; };  // [0]: low nibbles (sub-block 2P), [1]: high nibbles (sub-block 2P + 1)
+template <int P>
+__device__ __forceinline__ Q4PairScale q4_pair_scale(uint32_t sc_lo4, uint32_t sc_hi4, const Q4ScaleConsts& c) {
+    const uint32_t word = P < 2 ? sc_lo4 : sc_hi4;  // scales 0..3 | 4..7, one per byte
+    const f16x2 sc = as_h2(__builtin_amdgcn_perm(c.k64, word, c.sel[P & 1])) + c.off;  // (sc[2P], sc[2P + 1])
+    return Q4PairScale{sc * c.mul, sc * c.bias};
+}
+__device__ __forceinline__ void frags_q4k_pair(const u32x4& raw, const Q4PairScale& s, int hi, const Q4Consts& c, f16x8 frag[2]) {
+    const f16x2 s2 = hi ? f16x2{s.mul[1], s.mul[1]} : f16x2{s.mul[0], s.mul[0]};
+    const f16x2 bias = hi ? f16x2{s.bias[1], s.bias[1]} : f16x2{s.bias[0], s.bias[0]};
+    if (hi) {
+        frag[0] = scaled8_q4_swapped<1>(raw[0], raw[1], s2, bias, c);
+        frag[1] = scaled8_q4_swapped<1>(raw[2], raw[3], s2, bias, c);
+    } else {
+        frag[0] = scaled8_q4_swapped<0>(raw[0], raw[1], s2, bias, c);
+        frag[1] = scaled8_q4_swapped<0>(raw[2], raw[3], s2, bias, c);
+    }
 }
 
 // B operand of the minima term: the eight integer minima, the same in both k-halves (hi and lo sums).
