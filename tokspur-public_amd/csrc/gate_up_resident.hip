@@ -18,11 +18,13 @@
 //     tile; the eight partials add up through LDS in wave order (a fixed order: results are reproducible bit for bit) with
 //     one barrier per tile, and the threads that hold gate and up of the same hidden units apply SwiGLU and store h / 256
 //     as halves, the format the down GEMM reads.
-//   * What bounds the kernel is the vector unit: a SIMD issues one vector instruction per four cycles whichever of its
-//     two waves it comes from, and unpacking costs about one and a half of them per weight (mask-or, packed multiply-add,
-//     a share of the shifts and of the scale set-up). Everything else a wave executes per tile is kept short for that
-//     reason: scales are set up two sub-blocks at a time, the sigmoid uses the hardware exponential and reciprocal, and
-//     the tasks of at most 32 rows (most of them) run in a loop of their own that keeps every address in registers.
+//   * A wave issues at most one instruction every four cycles and two waves share a SIMD, so what a wave executes per
+//     tile is kept short: unpacking is one mask-or and one packed multiply-add per pair of weights, scales are set up two
+//     sub-blocks at a time, the sigmoid uses the hardware exponential and reciprocal, every lane stores (rows a task
+//     does not have land in slots nobody reads), and the tasks of at most 32 rows run in a loop of their own that keeps
+//     every address in registers. Measured with the arithmetic, the requests or the barrier taken out in turn, no single
+//     one of them bounds the kernel: what is left is the chain of latencies of one tile (arrival, LDS, matrix results,
+//     barrier, sum) at two waves per SIMD.
 #include "gate_up_resident.hpp"
 #include "mfma_quant.hpp"
 
@@ -55,10 +57,9 @@ __device__ __forceinline__ TaskInfo resolve_task(const ResidentGateUpArgs& a, ui
 }
 
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gate_up_resident_kernel(ResidentGateUpArgs a) {
-    // LDS: [2 phases][8 waves][4 KB partial tile] | [8 waves][2 stages][5 KB weight tile] | row tables of two tasks
+    // LDS: [2 phases][8 waves][4 KB partial tile] | [8 waves][2 stages][5 KB weight tile]
     constexpr int kStagesAt = 2 * kPhaseBytes;
-    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kStagesAt + kWaves * kStages * kStageBytes + 2 * kTaskRows * 4];
-    uint32_t* const row_ok = reinterpret_cast<uint32_t*>(lds_raw + kStagesAt + kWaves * kStages * kStageBytes);  // [2][64]
+    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kStagesAt + kWaves * kStages * kStageBytes];
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const uint32_t n = lane % 32, khalf = lane / 32;
@@ -150,25 +151,33 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             task = task_at(k);
             cur = resolve_task(a, task);
             if (!cur.ok && tid == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+            // first every row's token (two dependent look-ups), then all the row loads at once
+            uint32_t token[MT];
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
                 const uint32_t r = i * 32 + n, rr = r < cur.nrows ? r : 0;
-                uint32_t token;
+                token[i] = cur.shared ? cur.start + rr : a.token_map[uint64_t(cur.expert) * a.tokens + cur.start + rr];
+            }
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
                 bool ok = true;
-                if (cur.shared) {
-                    token = cur.start + rr;
-                } else {
-                    const uint32_t rid = a.token_map[uint64_t(cur.expert) * a.tokens + cur.start + rr];
+                if (!cur.shared) {
+                    const uint32_t rid = token[i];
                     ok = rid < a.tokens * a.selected && a.ids[rid < a.tokens * a.selected ? rid : 0] == cur.expert;
-                    token = ok ? rid / a.selected : 0;
+                    token[i] = ok ? rid / a.selected : 0;
                 }
-                if (!cur.ok) { token = 0; ok = false; }
+                // A row past the task's end repeats its first row and a row whose route does not check out stands in for token
+                // 0: their h lands in slots of the task's 64 that nobody reads, or the batch is refused. So every lane stores,
+                // every wave issues the same number of stores per unit, and the waits below can count them.
+                if (!cur.ok) { token[i] = 0; ok = false; }
                 if (!ok && cur.ok) bad |= TSP_ERRBIT_INDEX;
-                if (wave == 0 && khalf == 0) row_ok[(k & 1) * kTaskRows + r] = ok && r < cur.nrows;
-                const _Float16* row = a.xh + uint64_t(token) * (bpr * 256) + wave * 256 + khalf * 16;
+            }
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const _Float16* row = a.xh + uint64_t(token[i]) * (bpr * 256) + wave * 256 + khalf * 16;
 #pragma unroll
                 for (int t = 0; t < 16; ++t) A[i][t] = *reinterpret_cast<const f16x8*>(row + (t / 4) * 64 + ((t / 2) % 2) * 32 + (t % 2) * 8);
-                sxA[i] = *reinterpret_cast<const f16x8*>(a.sx + (uint64_t(token) * bpr + wave) * 16 + khalf * 8);
+                sxA[i] = *reinterpret_cast<const f16x8*>(a.sx + (uint64_t(token[i]) * bpr + wave) * 16 + khalf * 8);
             }
         };
 
@@ -176,8 +185,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         float gate_sum[MT][2];
         auto tile = [&](uint32_t k, uint32_t unit, auto j_tag) {
             constexpr int J = decltype(j_tag)::value;
-            // wait for the tile's five requests (the five of the other stage may still be in flight)
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 1) * kTileLoads) : "memory");
+            // wait for the tile's five requests: younger than those are the five of the other stage and, for a gate tile, the
+            // stores of the unit before (loads complete in order; a store that completes early only ends the wait sooner)
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 1) * kTileLoads + (J == 0 ? 2 * MT : 0)) : "memory");
             // With two row tiles everything a lane derives from its id is derived again per tile from this one register:
             // hoisted out of the loops these addresses would occupy a dozen registers next to the 128 of the activations.
             uint32_t lane_now = lane;
@@ -260,10 +270,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                         const float h = (g * sigmoid_fast(g)) * u;
                         // h travels to the down GEMM as the half nearest to h * 2^-8
                         const _Float16 carried = _Float16(h * 0.00390625f);
-                        if (row_ok[(k & 1) * kTaskRows + r]) {
-                            if (nonfinite(g) || nonfinite(u) || nonfinite(h) || (__builtin_bit_cast(uint16_t, carried) & 0x7c00u) == 0x7c00u) bad |= TSP_ERRBIT_NONFINITE;
-                            a.hbuf[(uint64_t(task) * kTaskRows + r) * a.hidden + unit * 32 + lane_now / 2] = carried;
-                        }
+                        if (nonfinite(g) || nonfinite(u) || nonfinite(h) || (__builtin_bit_cast(uint16_t, carried) & 0x7c00u) == 0x7c00u) bad |= TSP_ERRBIT_NONFINITE;
+                        a.hbuf[(uint64_t(task) * kTaskRows + r) * a.hidden + unit * 32 + lane_now / 2] = carried;
                     }
                 }
             }
