@@ -18,7 +18,7 @@ that one, so against it the engine's own rel-L2 limit of 5e-3 applies."""
 import numpy as np
 import pytest
 
-from conftest import max_rel_error, nmse
+from conftest import max_rel_error, nmse, reference_metric
 
 pytestmark = pytest.mark.gpu
 
@@ -118,6 +118,11 @@ def test_config1_dense_q4k_gemm(gpu, tsp, orc, synth, tokens):
     print(f"config1 M={tokens}: max rel error vs half-staged reference {err:.2e}, vs f32-dequantised {err_un:.2e}, "
           f"NMSE vs f32-dequantised {nmse(out_f32[:, sel], unstaged):.2e}")
     assert err_un <= 2e-5 and rel_l2(out_f32[:, sel], want) <= 5e-3
+    # the engine's own metric, |a - e| / max(1, |e|), against the reference that rounds nothing: outputs are O(500) here, so
+    # an f32-accumulated product is well inside the configuration's 2e-3
+    value, at, actual, expected, row_rms = reference_metric(out_f32[:, sel], unstaged)
+    print(f"config1 M={tokens}: reference metric {value:.2e} at element {at} (got {actual:.6g}, reference {expected:.6g}, row rms {row_rms:.3g})")
+    assert value <= 2e-3
     # every column: permuting the token rows permutes the output rows bit for bit (tiles hold no row state)
     perm = np.random.default_rng(1).permutation(tokens)
     out_p = tsp.dense_mm(gpu, 12, tsp.LAYOUT_GGUF, dw, gpu.upload(x[perm]), tokens, cols, rows).cpu().numpy()
@@ -467,6 +472,13 @@ def test_config3_moe_grouped_prefill(gpu, tsp, orc, synth):
           f"{max_rel_error(got, plain):.2e} (NMSE {nmse(got, plain):.2e})")
     assert rel_l2(got, staged) <= 5e-3 and nmse(got, plain) <= 2e-3
     assert max_rel_error(got, declared) <= 2e-3 and nmse(got, declared) <= 1e-7 and nmse(got, plain) <= 1e-6
+    # The engine's own metric against the reference that rounds nothing. Expert outputs are O(1e7) here (unnormalised
+    # synthetic weights through two projections), so one unit in the last place of f32 is already ~1: an element that
+    # cancels to near zero in such a row cannot meet 2e-3 of max(1, |e|) with f32 accumulation, whatever the kernel. The
+    # number is recorded; the row-scale form above is what is asserted.
+    value, at, actual, expected, row_rms = reference_metric(got, plain)
+    print(f"config3: reference metric |a-e|/max(1,|e|) = {value:.3e} at element {at} (got {actual:.8g}, reference {expected:.8g}, "
+          f"row rms {row_rms:.3g}: {abs(actual - expected) / row_rms:.2e} of the row scale)")
     # weighted combine over the routes (shared expert left out here: it is the dense GEMM of config 1 at M = 2048)
     out = gpu.mixture(y, wts_d, gpu.zeros((T, C)), gpu.zeros(T), C, S, tokens=T).cpu().numpy()
     yh, wh = y.cpu().numpy().reshape(T, S, C), wts_d.cpu().numpy()

@@ -122,7 +122,7 @@ def test_gemv_shapes(gpu, orc, synth, t, cols, rows):
     x = synth.activations_f32(1201, cols)
     want = orc.reference_gemv(t, w, cols, rows, x)
     got = gpu.gemv(t, gpu.upload(w), gpu.upload(x), cols, rows).cpu().numpy()
-    assert scaled_error(got, want) <= TOL * max(1.0, float(np.abs(want).max()) / 50) and gpu.error() == 0
+    assert scaled_error(got, want) <= TOL and gpu.error() == 0
     zero = gpu.gemv(t, gpu.upload(w), gpu.zeros(cols), cols, rows).cpu().numpy()
     assert not zero.any()  # zero input gives exactly zero output (native/tests/test_metal.cpp:41-66)
 
@@ -143,10 +143,12 @@ def test_config0_dense_q4k_gemv(gpu, tsp, orc, synth):
     # the two arms share their arithmetic: identical bits (the engine's block path is held to this too,
     # native/tests/test_block_gemv.cpp:94)
     assert np.array_equal(bits(got), bits(got_p))
-    # The configuration's bar is max scaled error 2e-3 with f32 accumulation. |y| reaches several hundred
-    # here (weights up to ~19), so f32 rounding alone is ~1e-5 absolute per partial sum.
+    # The configuration's bar is max scaled error 2e-3 with f32 accumulation. Measured: 9.2e-5, on an element of magnitude ~1
+    # in a vector whose entries reach several hundred (weights up to ~19, 2048 products): 3e-7 of the vector's scale, which
+    # is what f32 accumulation leaves. The engine's 5e-5 (native/src/main.cpp:165) is quoted on outputs of magnitude ~1 and
+    # holds at those (test_gemv_shapes, test_gemv_all_encodings_reference_fixture); here the bound asserted is 2e-4.
     print(f"config0 max scaled error {err_raw:.3e}")
-    assert err_raw <= 2e-3, err_raw
+    assert err_raw <= 2e-4, err_raw
 
 
 def test_gemv_rows_strided(gpu, orc, synth):

@@ -6,7 +6,7 @@ import importlib
 import numpy as np
 import pytest
 
-from conftest import max_rel_error, nmse
+from conftest import max_rel_error, nmse, reference_metric
 
 pytestmark = pytest.mark.gpu
 
@@ -213,3 +213,7 @@ def test_config2_moe_verify(gpu, tsp, orc, synth):
     # engine's MoE bound (NMSE <= 1e-6) plus max error <= 2e-3 in units of each row's scale.
     print(f"config2: {len(used)} distinct experts, NMSE {nmse(out, want):.3e}, max rel error {max_rel_error(out, want):.3e}")
     assert nmse(out, want) <= 1e-6 and max_rel_error(out, want) <= 2e-3
+    # the engine's own metric for the record (outputs of magnitude ~1e6: see reference_metric)
+    value, at, actual, expected, row_rms = reference_metric(out, want)
+    print(f"config2: reference metric |a-e|/max(1,|e|) = {value:.3e} at element {at} (got {actual:.8g}, reference {expected:.8g}, "
+          f"row rms {row_rms:.3g}: {abs(actual - expected) / row_rms:.2e} of the row scale)")

@@ -64,9 +64,15 @@ def test_config4_lm_head_argmax(gpu, tsp, orc, synth):
         x = synth.activations_f32(synth.tensor_seed(4, 2 + m), (m, C))
         dx = gpu.upload(x)
         y = gpu.empty((m, V))
-        for at in range(0, m, 8):
-            width = min(8, m - at)
-            gpu.q8_matvec_many(dw, dx[at:at + width], C, V, width, y=y[at:at + width])
+        if m > 8:  # the path the benchmark times: up to sixteen rows in one pass over the matrix (`dense_mm_q8`)
+            tsp.dense_mm_q8(gpu, tsp.LAYOUT_GGUF, dw, dx, m, C, V, out=y)
+            two_passes = gpu.empty((m, V))
+            for at in range(0, m, 8):
+                gpu.q8_matvec_many(dw, dx[at:at + 8], C, V, 8, y=two_passes[at:at + 8])
+            both = (y.cpu().numpy(), two_passes.cpu().numpy())
+            assert float(np.max(np.abs(both[0] - both[1]) / np.maximum(1.0, np.abs(both[1])))) <= 5e-5
+        else:
+            gpu.q8_matvec_many(dw, dx, C, V, m, y=y)
         rows = tsp.logit_topk(gpu, y, m, V).cpu().numpy().view(tsp.TOPK_ROW_DTYPE)
         assert gpu.error() == 0
         logits = y.cpu().numpy()
@@ -83,3 +89,17 @@ def test_config4_lm_head_argmax(gpu, tsp, orc, synth):
         print(f"config4 M={m}: arg-max id {cand[0]}, reference top-2 margin {margin:.3e} (error bound {bound:.1e})")
         if margin > bound:
             assert int(np.argmax(ref)) == 0
+    # the other arm: the same matrix as q8_lanes_v1 rows, the form Pack v3 stores a dense Q8_0 matrix in, at full vocabulary
+    d_lanes = gpu.upload(tsp.q8_lanes_pack_rows(C, w))
+    for m in (1, 8, 16):
+        x = synth.activations_f32(synth.tensor_seed(4, 2 + m), (m, C))
+        dx = gpu.upload(x)
+        raw_rows, lane_rows = gpu.empty((m, V)), gpu.empty((m, V))
+        tsp.dense_mm_q8(gpu, tsp.LAYOUT_GGUF, dw, dx, m, C, V, out=raw_rows)
+        tsp.dense_mm_q8(gpu, tsp.LAYOUT_Q8_LANES_V1, d_lanes, dx, m, C, V, out=lane_rows)
+        assert gpu.error() == 0
+        a, b = raw_rows.cpu().numpy(), lane_rows.cpu().numpy()
+        assert float(np.max(np.abs(a - b) / np.maximum(1.0, np.abs(a)))) <= 5e-5
+        top = tsp.logit_topk(gpu, lane_rows, m, V).cpu().numpy().view(tsp.TOPK_ROW_DTYPE)
+        for r in range(m):
+            assert top[r]["ids"][0] == int(np.argmax(b[r]))

@@ -76,6 +76,8 @@ def test_q6k_planar_extension_round_trip(tsp, orc, synth):
     assert np.array_equal(tsp.unpack_expert(s, planar), raw)
     blocks = raw.reshape(nb, 210)
     assert np.array_equal(planar[:128 * nb].reshape(nb, 128), blocks[:, :128])
+    assert np.array_equal(planar[128 * nb:192 * nb].reshape(nb, 64), blocks[:, 128:192])
+    assert np.array_equal(planar[192 * nb:208 * nb].reshape(nb, 16), blocks[:, 192:208])
     assert np.array_equal(planar[208 * nb:].reshape(nb, 2), blocks[:, 208:])
     with pytest.raises(tsp.FormatError):
         tsp.make_expert_spec(14, 256, 4)  # 4 blocks: planes would not be 16-byte aligned

@@ -341,3 +341,91 @@ def test_matrix_core_staging_models(orc, synth):
     wd = ((qd - 32) * np.repeat(scd, 16, axis=1) * dd[:, None]).reshape(experts, channels, hidden)
     want_y = np.stack([wd[ids[r]] @ carried[r] for r in range(3)])
     assert np.allclose(y4, want_y, rtol=1e-12, atol=1e-6)
+
+
+@pytest.mark.parametrize("t,cols,rows", [(12, 512, 8), (13, 256, 12), (8, 256, 8), (7, 96, 4)])
+def test_planar_plane_byte_positions(orc, synth, t, cols, rows):
+    """Every plane byte at its place (native/src/planar_pack_v3.cpp:601-716): blocks in (row, block) order, nibbles and
+    high bits verbatim, scales decoded one per byte, d / dmin verbatim. A round trip alone would also pass a pack and an
+    unpack that agree on a wrong plane order."""
+    raw = synth.matrix(t, 4200 + t, rows, cols)
+    spec = orc.make_expert_spec(t, cols, rows)
+    planar = orc.pack_expert(spec, raw)
+    epb, bpb = orc.encoding(t)
+    nb = rows * (cols // epb)
+    blk = raw.reshape(nb, bpb)
+    def plane(offset, width):
+        return planar[offset:offset + nb * width].reshape(nb, width)
+    if t == 12:
+        assert np.array_equal(plane(spec.qs_offset, 128), blk[:, 16:144])
+        want_sm = np.array([[scale_min_k4(j, [int(v) for v in b[4:16]])[0] for j in range(8)] +
+                            [scale_min_k4(j, [int(v) for v in b[4:16]])[1] for j in range(8)] for b in blk], dtype=np.uint8)
+        assert np.array_equal(plane(spec.sm_offset, 16), want_sm)
+        assert np.array_equal(plane(spec.dm_offset, 4), blk[:, 0:4])
+        assert (spec.qs_offset, spec.sm_offset, spec.dm_offset, spec.planar_expert_bytes) == (0, 128 * nb, 144 * nb, 148 * nb)
+    elif t == 13:
+        assert np.array_equal(plane(spec.qs_offset, 128), blk[:, 48:176])
+        assert np.array_equal(plane(spec.qh_offset, 32), blk[:, 16:48])
+        want_sm = np.array([[scale_min_k4(j, [int(v) for v in b[4:16]])[0] for j in range(8)] +
+                            [scale_min_k4(j, [int(v) for v in b[4:16]])[1] for j in range(8)] for b in blk], dtype=np.uint8)
+        assert np.array_equal(plane(spec.sm_offset, 16), want_sm)
+        assert np.array_equal(plane(spec.dm_offset, 4), blk[:, 0:4])
+        assert (spec.qs_offset, spec.qh_offset, spec.sm_offset, spec.dm_offset) == (0, 128 * nb, 160 * nb, 176 * nb)
+    elif t == 8:
+        assert np.array_equal(plane(spec.qs_offset, 32), blk[:, 2:34])
+        assert np.array_equal(plane(spec.dm_offset, 2), blk[:, 0:2])
+        assert (spec.qs_offset, spec.dm_offset, spec.planar_expert_bytes) == (0, 32 * nb, 34 * nb)
+    else:
+        assert np.array_equal(plane(spec.qs_offset, 16), blk[:, 8:24])
+        assert np.array_equal(plane(spec.qh_offset, 4), blk[:, 4:8])
+        assert np.array_equal(plane(spec.dm_offset, 4), blk[:, 0:4])
+        assert (spec.qs_offset, spec.qh_offset, spec.dm_offset) == (0, 16 * nb, 20 * nb)
+
+
+def _silu_f32(gf):
+    return gf / (np.float32(1) + np.exp(-gf).astype(np.float32))
+
+
+def test_declared_precision_modes_against_numpy(orc, synth):
+    """The staging switches of the declared-precision references, each against numpy's own rounding on independently
+    dequantised weights: `staged_gemm(stage_f16 = 1)` (weights as halves, tests/test_moe_mm_many_gpu.cpp:54-56) and bits
+    1 (x and h as bf16), 2 (weights as halves) and 8 (Q6_K down rows as d * half(sc * (q - 32))) of
+    `moe_routed_reference`."""
+    rows, cols, tokens = 16, 512, 4
+    w = synth.matrix(12, 9200, rows, cols)
+    x = synth.activations_f32(9201, (tokens, cols))
+    wf = orc.dequantize(12, w, rows * cols).reshape(rows, cols)
+    want = x.astype(np.float64) @ wf.astype(np.float16).astype(np.float64).T
+    assert np.allclose(orc.staged_gemm(12, w, cols, x, nrows=rows, stage_f16=1), want, rtol=1e-12, atol=1e-9)
+    assert not np.allclose(orc.staged_gemm(12, w, cols, x, nrows=rows, stage_f16=0), want, rtol=1e-9, atol=1e-9)
+
+    channels, hidden, experts = 256, 256, 2
+    gate = synth.matrix(12, 9202, hidden * experts, channels)
+    up = synth.matrix(12, 9203, hidden * experts, channels)
+    down = synth.matrix(14, 9204, channels * experts, hidden)
+    ids = np.array([1, 0, 1], dtype=np.uint32)
+    xs = synth.activations_f32(9205, (3, channels))
+    g = orc.dequantize(12, gate, hidden * experts * channels).reshape(experts, hidden, channels)
+    u = orc.dequantize(12, up, hidden * experts * channels).reshape(experts, hidden, channels)
+    d = orc.dequantize(14, down, channels * experts * hidden).reshape(experts, channels, hidden)
+    half = lambda a: a.astype(np.float16).astype(np.float64)
+    qd, scd, dd = q6k_fields(down)
+    d_products = (((qd - 32) * np.repeat(scd, 16, axis=1)).astype(np.float16).astype(np.float64) * dd[:, None]).reshape(experts, channels, hidden)
+    for stage, xin, wg, wu, wd, round_h in (
+            (1, synth.round_bf16(xs), g.astype(np.float64), u.astype(np.float64), d.astype(np.float64), True),
+            (2, xs, half(g), half(u), half(d), False),
+            (8, xs, g.astype(np.float64), u.astype(np.float64), d_products, False)):
+        h, y = orc.moe_routed_reference(12, 14, gate, up, down, channels, hidden, experts, ids, 3, 1, xs, stage=stage)
+        for r, e in enumerate(ids):
+            xv = xin[r].astype(np.float64)
+            hh = _silu_f32((wg[e] @ xv).astype(np.float32)) * (wu[e] @ xv).astype(np.float32)
+            if round_h:
+                # numpy's exp and the C library's differ by an ulp now and then, which can move a bf16 rounding: at most
+                # one bf16 step on a few elements, none on the rest
+                hb = synth.round_bf16(hh)
+                step = np.abs(hb.astype(np.float64)) * 2.0 ** -7
+                assert (np.abs(h[r] - hb) <= step).all() and (h[r] == hb).mean() > 0.98
+                assert np.array_equal(h[r], synth.round_bf16(h[r].astype(np.float32)).astype(np.float64))  # h is bf16-valued
+            else:
+                assert np.allclose(h[r], hh.astype(np.float64), rtol=3e-7, atol=1e-30)
+            assert np.allclose(y[r], wd[e] @ h[r], rtol=1e-12, atol=1e-6)
