@@ -293,7 +293,10 @@ int tsp_planar_moe_routed_m8_shared(const tsp_small_moe* moe, const tsp_shared_r
 /* include/tokspur/graph.hpp:750-753 `grouped_mm` with experts = selected = 1, broadcast (the dense case,
  * kernels/grouped_mm.metal:159-243) and 859-860 `dense_mm_q8`: out[t, r] = sum_c x[t, c] * dec(W[r, c]) for
  * `tokens` rows. Activations are used as bf16 values (carried as f16), weights enter the matrix cores as exact integer
- * factors whose block scales are applied in f32, f32 accumulation. Input rows are f32 or bf16, output rows f32 or
+ * factors whose block scales are applied in f32, f32 accumulation. The carry is exact for bf16 values of magnitude 2^-14
+ * to 65504; smaller ones lose low bits (below 2^-24: zero), and a finite input above 65504 sets TSP_ERRBIT_NONFINITE like an
+ * infinity would (the batch is refused rather than computed on a clipped value). The same holds for tsp_grouped_mm and
+ * tsp_planar_nax_grouped_moe. Input rows are f32 or bf16, output rows f32 or
  * bf16 (RNE); strides in bytes. Q4_K raw GGUF rows or planar planes, Q6_K planes. `workspace` is caller
  * owned scratch of tsp_dense_mm_workspace_bytes(tokens, columns) bytes, 16-byte aligned. */
 uint64_t tsp_dense_mm_workspace_bytes(uint32_t tokens, uint32_t columns);

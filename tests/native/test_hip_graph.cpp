@@ -478,6 +478,118 @@ void test_encode_moe_mm_many() {
     }
     release_moe_mm_many_scratch(g, scratch);
 }
+// the raw-GGUF arm of the same composition (src/moe_mm_many.cpp:214-240): three grouped products over Q4_K expert stacks in
+// GGUF rows, nothing registered; `grouped_mm` and `dense_mm` on their own; encodings the grouped product does not take are
+// refused while idle, and a refusal part-way through a batch leaves no half-encoded batch behind
+void test_encode_moe_mm_many_raw_arm() {
+    const MoeShape shape{256, 256, 6, 2};
+    const auto gate = fixture(12, shape.channels, shape.hidden, shape.experts);
+    auto up = gate;
+    for (size_t at = 0; at < up.size(); at += 144) for (size_t i = 16; i < 144; ++i) up[at + i] = uint8_t(up[at + i] * 3 + 1);
+    const auto down = fixture(12, shape.hidden, shape.channels, shape.experts);
+    const auto sg = fixture(8, shape.channels, shape.hidden, 1), sd = fixture(8, shape.hidden, shape.channels, 1);
+    const std::vector<float> router = lcg_floats(41, size_t(shape.experts) * shape.channels);
+    std::vector<float> shared_router = lcg_floats(43, shape.channels);
+    for (auto& v : shared_router) v *= 0.05f;
+    HipGraph g("unused.metallib", 256u << 20);
+    MoeWeights w{};
+    w.router = {g.upload(bytes_of(router), "router"), 0};
+    w.gate = {g.upload(bytes_of(gate), "gate"), 12};
+    w.up = {g.upload(bytes_of(up), "up"), 12};
+    w.down = {g.upload(bytes_of(down), "down"), 12};
+    w.shared_gate = {g.upload(bytes_of(sg), "shared gate"), 8};
+    w.shared_up = {g.upload(bytes_of(sg), "shared up"), 8};
+    w.shared_down = {g.upload(bytes_of(sd), "shared down"), 8};
+    w.shared_router = {g.upload(bytes_of(shared_router), "shared router"), 0};
+    g.register_q8_matrix(w.shared_gate.view, shape.channels, shape.hidden);
+    EXPECT(g.q8_matrix_count() == 1);
+    EXPECT(throws_format([&] { g.register_q8_matrix(w.shared_gate.view, shape.channels, shape.hidden); }));      // overlaps a registered matrix
+    EXPECT(throws_format([&] { g.register_q8_matrix(w.shared_down.view, shape.channels + 32, shape.hidden); }));  // byte span
+    EXPECT(!is_planar_moe(g, w, shape));
+    const uint32_t capacity = 40;
+    MoeWeights q5 = w;
+    q5.down.encoding = 13;
+    EXPECT(throws_format([&] { prepare_moe_mm_many(g, q5, shape, capacity); }));  // refused while idle, not in the middle of a batch
+    prepare_moe_mm_many(g, w, shape, capacity);
+    const uint64_t after_first = g.memory().allocations;
+    prepare_moe_mm_many(g, w, shape, capacity);  // a second layer of the same shape: nothing to do
+    EXPECT(g.memory().allocations == after_first);
+    prepare_moe_mm_many(g, w, MoeShape{512, 256, 6, 2}, capacity);  // a wider layer: the scratch grows
+    g.prepare_dense_mm(32, 256);
+    g.prepare_dense_mm(64, 512);
+    const MoeMmManyScratch scratch = allocate_moe_mm_many_scratch(g, shape, capacity);
+    const uint32_t T = 33, stride = shape.channels + 4;
+    // The grouped product carries its input rows as halves: the SwiGLU rows that feed the down product have to stay below
+    // 65504 in magnitude, which the fixture's weight scales (outputs of ~1e5 for inputs of ~1) only do for small inputs.
+    std::vector<float> x = lcg_floats(900, size_t(T) * stride);
+    for (auto& v : x) { uint32_t bad = 0; v = orc_bf16_to_f32(orc_round_bf16_bits(v * 0.0009765625f, &bad)); }
+    const GpuView dx = g.upload(bytes_of(x), "x", false), dy = g.zeros(uint64_t(T) * stride * 4, "y");
+    g.begin();
+    encode_moe_mm_many(g, w, scratch, {dx, T, shape.channels, uint64_t(stride) * 4}, {dy, T, shape.channels, uint64_t(stride) * 4}, shape, RouterMode::softmax, true);
+    (void)g.submit();
+    const auto y = read_as<float>(g, dy);
+    double worst = 0;
+    for (uint32_t t = 0; t < T; ++t) {
+        const float* xt = &x[size_t(t) * stride];
+        std::vector<double> logits(shape.experts), weights(shape.selected), out(shape.channels);
+        orc_reference_gemv(0, reinterpret_cast<const uint8_t*>(router.data()), router.size() * 4, shape.channels, shape.experts, xt, shape.channels, logits.data());
+        for (auto& v : logits) v = double(float(v));
+        std::vector<uint32_t> ids(shape.selected);
+        orc_route_reference(logits.data(), shape.experts, shape.selected, 0, 1, ids.data(), weights.data());
+        std::vector<double> h(size_t(shape.selected) * shape.hidden), yy(size_t(shape.selected) * shape.channels);
+        orc_moe_routed_reference(12, 12, gate.data(), up.data(), down.data(), shape.channels, shape.hidden, shape.experts, ids.data(), 1, shape.selected, xt,
+                                 shape.channels, 1, 0, h.data(), yy.data(), 1);
+        std::vector<double> sgv(shape.hidden), sy(shape.channels);
+        orc_reference_gemv(8, sg.data(), sg.size(), shape.channels, shape.hidden, xt, shape.channels, sgv.data());
+        std::vector<float> act(shape.hidden);
+        for (uint32_t i = 0; i < shape.hidden; ++i) { const double v = sgv[i]; act[i] = float(v / (1.0 + std::exp(-v)) * sgv[i]); }
+        orc_reference_gemv(8, sd.data(), sd.size(), shape.hidden, shape.channels, act.data(), shape.hidden, sy.data());
+        double shared_logit = 0;
+        orc_reference_gemv(0, reinterpret_cast<const uint8_t*>(shared_router.data()), shared_router.size() * 4, shape.channels, 1, xt, shape.channels, &shared_logit);
+        orc_mixture_reference(yy.data(), weights.data(), shape.selected, sy.data(), shape.channels, double(float(shared_logit)), out.data());
+        double scale = 1;
+        for (double v : out) scale = std::max(scale, std::fabs(v));
+        for (uint32_t c = 0; c < shape.channels; ++c) worst = std::max(worst, std::fabs(double(y[size_t(t) * stride + c]) - out[c]) / scale);
+    }
+    std::printf("encode_moe_mm_many raw arm T=%u: max error / row max %.3e\n", T, worst);
+    EXPECT(worst <= 2e-3);
+    // the grouped and the dense product on their own (graph.hpp:750-753), against the staged reference of one route
+    {
+        const std::vector<uint32_t> ids{3, 1, 0, 5, 2, 4};  // 3 tokens x 2
+        const GpuView dids = g.upload(bytes_of(ids), "ids"), out = g.zeros(6ull * shape.hidden * 4, "out");
+        const GpuView map = g.zeros(uint64_t(shape.experts) * 3 * 4, "map"), counts = g.zeros(shape.experts * 4, "counts"), tasks = g.zeros((2 + 2 * (6 / 32 + shape.experts)) * 4, "tasks");
+        const GpuView in3 = g.slice(dx, 0, 2ull * stride * 4 + shape.channels * 4);
+        g.begin();
+        g.grouped_mm(12, PrefillWeightLayout::gguf, w.gate.view, dids, {in3, 3, shape.channels, uint64_t(stride) * 4}, {out, 6, shape.hidden, uint64_t(shape.hidden) * 4},
+                     map, counts, tasks, shape.experts, 2, true);
+        (void)g.submit();
+        const auto got = read_as<float>(g, out);
+        std::vector<double> want(shape.hidden);
+        const size_t expert_bytes = gate.size() / shape.experts;
+        orc_reference_gemv(12, gate.data() + 5 * expert_bytes, expert_bytes, shape.channels, shape.hidden, &x[size_t(1) * stride], shape.channels, want.data());  // route 3 = token 1, expert 5
+        EXPECT(row_error(std::vector<float>(got.begin() + 3 * shape.hidden, got.begin() + 4 * shape.hidden), want) <= 2e-3);
+        const GpuView dense_out = g.zeros(3ull * shape.hidden * 4, "dense out"), one = g.slice(w.gate.view, 2 * expert_bytes, expert_bytes);
+        g.begin();
+        g.dense_mm(12, PrefillWeightLayout::gguf, one, {in3, 3, shape.channels, uint64_t(stride) * 4}, {dense_out, 3, shape.hidden, uint64_t(shape.hidden) * 4});
+        (void)g.submit();
+        const auto dense = read_as<float>(g, dense_out);
+        orc_reference_gemv(12, gate.data() + 2 * expert_bytes, expert_bytes, shape.channels, shape.hidden, &x[size_t(2) * stride], shape.channels, want.data());
+        EXPECT(row_error(std::vector<float>(dense.begin() + 2 * shape.hidden, dense.end()), want) <= 2e-3);
+    }
+    // a refusal inside the composition aborts the batch (src/moe_mm_many.cpp:282): the graph is idle again afterwards
+    {
+        MoeWeights broken = w;
+        broken.router.encoding = 99;  // no such encoding: the router projection refuses
+        g.begin();
+        EXPECT(throws_format([&] {
+            encode_moe_mm_many(g, broken, scratch, {dx, 4, shape.channels, uint64_t(stride) * 4}, {dy, 4, shape.channels, uint64_t(stride) * 4}, shape, RouterMode::softmax, true);
+        }));
+        EXPECT(throws_format([&] { g.abort(); }));  // nothing left to abort
+        g.begin();                                  // and a new batch can start
+        g.abort();
+    }
+    release_moe_mm_many_scratch(g, scratch);
+}
 }  // namespace
 
 int main() {
@@ -486,7 +598,8 @@ int main() {
                                                          {"dense_mm_q8 in both row layouts", test_dense_mm_q8_layouts},
                                                          {"encode_moe single token", test_encode_moe_single_token},
                                                          {"encode_moe_batch", test_encode_moe_batch},
-                                                         {"encode_moe_mm_many", test_encode_moe_mm_many}};
+                                                         {"encode_moe_mm_many", test_encode_moe_mm_many},
+                                                         {"encode_moe_mm_many, raw-GGUF arm; prepare twice; Q8_0 registration", test_encode_moe_mm_many_raw_arm}};
     for (const auto& [name, fn] : tests) {
         std::printf("== %s\n", name);
         std::fflush(stdout);

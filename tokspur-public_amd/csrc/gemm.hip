@@ -756,9 +756,9 @@ NaxLayout nax_layout(uint32_t tokens, uint32_t selected, uint32_t experts, uint3
 // matrix-core path keeps its h rows in, which is never smaller.
 int grouped_moe_in_eights(const tsp_grouped_moe* m, const NaxLayout& l, void* stream) {
     auto* ws = static_cast<uint8_t*>(m->workspace);
+    TSP_REQUIRE(uint64_t(8) * m->selected * m->hidden * 4 <= l.meta - l.hbuf, "planar v3 NAX scratch too small for requested batch");  // before anything is enqueued
     int rc = tsp_grouped_routes(m->ids, m->token_map, m->counts, m->experts, m->selected, m->tokens, m->error_word, stream);
     if (rc == TSP_OK) rc = tsp_grouped_tasks(m->counts, m->tasks, m->experts, m->selected, m->tokens, 32, m->error_word, stream);
-    TSP_REQUIRE(uint64_t(8) * m->selected * m->hidden * 4 <= l.meta - l.hbuf, "planar v3 NAX scratch too small for requested batch");
     for (uint32_t t0 = 0; rc == TSP_OK && t0 < m->tokens; t0 += 8) {
         tsp_small_moe c{};
         c.pair_lo = m->pair_lo; c.pair_hi = m->pair_hi; c.down = m->down;
@@ -773,8 +773,7 @@ int grouped_moe_in_eights(const tsp_grouped_moe* m, const NaxLayout& l, void* st
         c.y_stride_bytes = m->y_stride_bytes;
         c.union_meta = reinterpret_cast<uint32_t*>(ws + l.meta);
         c.error_word = m->error_word;
-        rc = tsp_planar_union_build(c.ids, c.union_meta, m->experts, m->selected, c.tokens, m->hidden, m->channels, m->error_word, stream);
-        if (rc == TSP_OK) rc = tsp_planar_moe_routed_m8(&c, stream);
+        rc = tsp_planar_moe_routed_m8(&c, stream);  // builds the chunk's union records itself
     }
     return rc;
 }

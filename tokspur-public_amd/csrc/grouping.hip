@@ -27,7 +27,7 @@ __global__ __launch_bounds__(kRouteThreads) void grouped_routes_kernel(const uin
         uint32_t slot = 0xffffffffu, matches = 0;
         if (token < tokens) {
             const uint32_t* row = ids + uint64_t(token) * selected;
-            if (selected % 2 == 0) {  // rows of an even number of ids are 8-byte aligned: half as many loads
+            if (selected % 2 == 0 && reinterpret_cast<uintptr_t>(ids) % 8 == 0) {  // 8-byte aligned rows of an even number of ids: half as many loads
                 for (uint32_t i = 0; i < selected; i += 2) {
                     const uint2 pair = *reinterpret_cast<const uint2*>(row + i);
                     if (pair.x >= experts || pair.y >= experts) bad = TSP_ERRBIT_INDEX;

@@ -53,6 +53,7 @@ struct HipGraph::Impl {
     uint64_t budget = 0, live_bytes = 0, peak_bytes = 0, allocations = 0;
     std::vector<Allocation> slots;  // never recycled
     std::vector<PlanarEntry> planar;
+    std::vector<PlanarEntry> q8;  // registered dense Q8_0 matrices: shape.kind holds the row layout
     std::thread::id thread = std::this_thread::get_id();
     hipStream_t stream = nullptr;
     hipEvent_t started = nullptr, finished = nullptr;
@@ -112,6 +113,19 @@ struct HipGraph::Impl {
         ++allocations;
         return p;
     }
+    // internal scratch kept or grown while idle (nothing in flight reads it): preparing twice, or for a second layer of
+    // another shape, is as harmless as it is in the engine, whose prepare_* calls only build pipelines (graph.mm:4468)
+    void grow(void*& scratch, uint64_t& have, uint64_t need) {
+        if (need <= have) return;
+        if (scratch) {
+            hip(hipFree(scratch), "hipFree");
+            live_bytes -= have;
+            scratch = nullptr;
+            have = 0;
+        }
+        scratch = raw(need);
+        have = need;
+    }
     static bool overlaps(const GpuView& a, const GpuView& b) {
         return a.slot == b.slot && a.offset < b.offset + b.bytes && b.offset < a.offset + a.bytes;
     }
@@ -127,6 +141,10 @@ struct HipGraph::Impl {
                 message);
     }
 };
+
+// include/tokspur/graph.hpp:433 `MetalGraph(library_path, byte_budget)`: the engine loads its compiled kernels from that
+// path. Here they are linked into libtokspur_hip.so, so the path is not opened; a caller's construction code runs unchanged.
+HipGraph::HipGraph(const std::string& library_path, uint64_t byte_budget) : HipGraph(byte_budget) { (void)library_path; }
 
 HipGraph::HipGraph(uint64_t byte_budget) : impl_(std::make_unique<Impl>()) {
     require(byte_budget > 0, "GPU graph byte budget must be positive");
@@ -196,6 +214,7 @@ void HipGraph::release(GpuView full_buffer) {
     const Allocation& a = impl_->allocation(full_buffer);
     require(full_buffer.offset == 0 && full_buffer.bytes == a.bytes, "release requires the full buffer view");
     for (const auto& e : impl_->planar) require(e.slot != full_buffer.slot, "registered planar matrices stay resident");
+    for (const auto& e : impl_->q8) require(e.slot != full_buffer.slot, "registered Q8_0 matrices stay resident");
     hip(hipFree(a.device), "hipFree");
     Allocation& slot = impl_->slots[full_buffer.slot];
     impl_->live_bytes -= slot.bytes;
@@ -247,6 +266,22 @@ void HipGraph::register_planar_matrix(GpuView matrix, PlanarMatrixShape shape) {
     impl_->planar.push_back({matrix.slot, matrix.offset, matrix.bytes, shape});
 }
 
+// include/tokspur/graph.hpp:468 `register_q8_matrix` (src/graph.mm:9001-9019): a dense Q8_0 matrix announced before the first
+// batch, in GGUF rows or q8_lanes_v1 rows (the two have the same byte span). The checks are the engine's: immutable view,
+// whole rows of 34-byte blocks, no overlap with a registered matrix.
+void HipGraph::register_q8_matrix(GpuView matrix, uint32_t columns, uint32_t rows, PrefillWeightLayout layout) {
+    impl_->idle();
+    require(!impl_->locked, "Q8_0 matrices are registered before the first batch");
+    const Allocation& a = impl_->allocation(matrix);
+    require(a.immutable, "Q8_0 matrix must be an immutable view");
+    require(layout == PrefillWeightLayout::gguf || layout == PrefillWeightLayout::q8_lanes_v1, "dense Q8_0 GEMM layout");
+    require(columns >= 32 && columns % 32 == 0 && columns <= 65536 && rows >= 1 && rows <= 1000000, "Q8_0 matrix geometry mismatch");
+    require(matrix.bytes == checked_mul(checked_mul(rows, columns / 32), 34), "Q8_0 matrix byte span mismatch");
+    for (const auto& e : impl_->q8) require(!Impl::overlaps(matrix, {impl_->owner, e.slot, e.offset, e.bytes}), "Q8_0 matrix overlaps a registered matrix");
+    impl_->q8.push_back({matrix.slot, matrix.offset, matrix.bytes, {8, uint32_t(layout), columns, rows, 1}});
+}
+uint64_t HipGraph::q8_matrix_count() const { return impl_->q8.size(); }
+
 uint64_t HipGraph::planar_matrix_count() const { return impl_->planar.size(); }
 
 std::optional<PlanarMatrixShape> HipGraph::planar_matrix_shape(GpuView matrix) const {
@@ -266,11 +301,7 @@ void HipGraph::prepare_planar_moe_v3(uint32_t gate_up_encoding, uint32_t down_en
     if (prepare_nax) {
         const uint32_t channels = (max_channels + 255) / 256 * 256, hidden = (max_hidden + 255) / 256 * 256;
         const uint64_t bytes = tsp_planar_nax_shared_workspace_bytes(max_nax_tokens, max_selected, max_experts, channels, hidden);  // room for an always-on expert's rows too
-        if (bytes > impl_->nax_workspace_bytes) {
-            require(impl_->nax_workspace == nullptr, "planar v3 NAX scratch is sized once");
-            impl_->nax_workspace = impl_->raw(bytes);
-            impl_->nax_workspace_bytes = bytes;
-        }
+        impl_->grow(impl_->nax_workspace, impl_->nax_workspace_bytes, bytes);
     }
     impl_->prepared_gate_up = gate_up_encoding;
     impl_->prepared_down = down_encoding;
@@ -280,9 +311,7 @@ void HipGraph::prepare_dense_mm(uint32_t max_tokens, uint32_t max_columns) {
     impl_->idle();
     require(max_tokens >= 1 && max_tokens <= 65536 && max_columns >= 256 && max_columns <= 65536, "dense dequant-GEMM preparation bounds mismatch");
     const uint64_t bytes = tsp_dense_mm_workspace_bytes(max_tokens, (max_columns + 255) / 256 * 256);
-    require(impl_->dense_workspace == nullptr, "dense dequant-GEMM scratch is sized once");
-    impl_->dense_workspace = impl_->raw(bytes);
-    impl_->dense_workspace_bytes = bytes;
+    impl_->grow(impl_->dense_workspace, impl_->dense_workspace_bytes, bytes);
 }
 
 // ------------------------------------------------------------------ batches
@@ -542,11 +571,12 @@ void HipGraph::planar_nax_grouped_moe(GpuView pair_lo, GpuView pair_hi, GpuView 
 void HipGraph::prepare_grouped_mm(uint32_t encoding, PrefillWeightLayout layout, uint32_t max_tokens, uint32_t max_selected, uint32_t max_experts,
                                   uint32_t max_columns) {
     impl_->idle();
-    require(encoding == 12 && layout == PrefillWeightLayout::gguf, "grouped prefill requires idle preparation and direct batches");
-    require(impl_->grouped_workspace == nullptr, "grouped prefill scratch is sized once");
+    require(grouped_mm_takes(encoding, layout), "grouped prefill requires idle preparation and direct batches");
+    require(max_tokens >= 1 && max_tokens <= 2048 && max_selected >= 1 && max_selected <= 16 && max_experts >= 1 && max_experts <= 512 &&
+                max_columns >= 256 && max_columns <= 65536,
+            "grouped prefill geometry mismatch");
     const uint64_t bytes = tsp_grouped_mm_workspace_bytes(max_tokens, max_selected, max_experts, (max_columns + 255) / 256 * 256, 0);
-    impl_->grouped_workspace = impl_->raw(bytes);
-    impl_->grouped_workspace_bytes = bytes;
+    impl_->grow(impl_->grouped_workspace, impl_->grouped_workspace_bytes, bytes);
 }
 
 void HipGraph::grouped_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView matrices, GpuView indices, GpuRowsF32 input, GpuRowsF32 output,
@@ -591,15 +621,7 @@ void HipGraph::prepare_dense_mm_q8(PrefillWeightLayout layout, uint32_t max_toke
     require(max_tokens >= 1 && max_tokens <= 65536 && max_columns >= 32 && max_columns <= 65536 && max_rows >= 1 && max_rows <= 1000000,
             "dense Q8_0 GEMM preparation bounds mismatch");
     const uint64_t bytes = tsp_dense_mm_q8_workspace_bytes(max_tokens, max_columns, max_rows);
-    if (bytes <= impl_->q8_workspace_bytes) return;
-    if (impl_->q8_workspace) {  // idle: nothing in flight reads the old scratch
-        hip(hipFree(impl_->q8_workspace), "hipFree");
-        impl_->live_bytes -= impl_->q8_workspace_bytes;
-        impl_->q8_workspace = nullptr;
-        impl_->q8_workspace_bytes = 0;
-    }
-    impl_->q8_workspace = impl_->raw(bytes);
-    impl_->q8_workspace_bytes = bytes;
+    impl_->grow(impl_->q8_workspace, impl_->q8_workspace_bytes, bytes);
 }
 
 void HipGraph::dense_mm_q8(PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output, bool) {
@@ -685,6 +707,8 @@ MoeScratch allocate_moe_scratch(HipGraph& graph, MoeShape shape) {
 void release_moe_scratch(HipGraph& graph, const MoeScratch& scratch) {
     for (const auto view : scratch.views()) graph.release(view);
 }
+
+bool grouped_mm_takes(uint32_t encoding, PrefillWeightLayout layout) { return encoding == 12 && layout == PrefillWeightLayout::gguf; }
 
 bool is_planar_moe(const HipGraph& g, const MoeWeights& w, MoeShape s) {
     const auto lo = g.planar_matrix_shape(w.gate.view);
@@ -800,6 +824,14 @@ void release_moe_mm_many_scratch(HipGraph& graph, const MoeMmManyScratch& scratc
     for (const auto view : scratch.views()) graph.release(view);
 }
 
+namespace {
+// The raw-GGUF arm runs its three grouped products on the matrix cores, which unpack Q4_K expert stacks in GGUF rows.
+void raw_arm_check(const MoeWeights& w, const MoeMmLayouts& l) {
+    for (const auto& [matrix, layout] : {std::pair{w.gate, l.gate}, std::pair{w.up, l.up}, std::pair{w.down, l.down}})
+        require(grouped_mm_takes(matrix.encoding, layout), "tiled MoE raw-GGUF experts: grouped prefill takes Q4_K expert stacks in GGUF rows");
+}
+}  // namespace
+
 void prepare_moe_mm_many(HipGraph& graph, const MoeWeights& w, MoeShape shape, uint32_t capacity, MoeMmLayouts l) {
     shape_check(shape);
     require(capacity >= 1, "tiled MoE capacity");
@@ -807,6 +839,7 @@ void prepare_moe_mm_many(HipGraph& graph, const MoeWeights& w, MoeShape shape, u
     if (is_planar_moe(graph, w, shape)) {
         graph.prepare_planar_moe_v3(w.gate.encoding, w.down.encoding, true, rows, shape.experts, shape.selected, shape.channels, shape.hidden);
     } else {
+        raw_arm_check(w, l);  // refused here, while idle, rather than in the middle of a batch
         graph.prepare_grouped_mm(w.gate.encoding, l.gate, rows, shape.selected, shape.experts, shape.channels > shape.hidden ? shape.channels : shape.hidden);
     }
     const uint32_t widest = shape.channels > shape.hidden ? shape.channels : shape.hidden;
@@ -829,6 +862,8 @@ void encode_moe_mm_many(HipGraph& g, const MoeWeights& w, const MoeMmManyScratch
         }
         return;
     }
+    const bool planar = is_planar_moe(g, w, shape);
+    if (!planar) raw_arm_check(w, l);  // before anything is enqueued
     const MoeMmManyBytes b = moe_mm_many_bytes(shape, s.capacity, true);
     const auto all = s.views();
     for (size_t i = 0; i < all.size(); ++i) require(all[i].bytes == b.views[i], "tiled MoE scratch capacity extent");
@@ -843,13 +878,14 @@ void encode_moe_mm_many(HipGraph& g, const MoeWeights& w, const MoeMmManyScratch
     std::copy(all.begin(), all.end(), write.begin() + 1);
     g.validate_disjoint(read, write);
     // the first `per_row * n` floats of a scratch view, flat or as n rows
+    try {
     const auto active = [&](GpuView v, uint64_t per_row) { return g.slice(v, 0, per_row * n * 4); };
     const auto rows = [&](GpuView v, uint32_t count, uint32_t columns) { return GpuRowsF32{g.slice(v, 0, uint64_t(count) * columns * 4), count, columns, uint64_t(columns) * 4}; };
     const GpuView logits = active(s.rows.logits, shape.experts), ids = active(s.rows.indices, shape.selected), weights = active(s.rows.weights, shape.selected);
     g.gemv_rows(w.router.encoding, w.router.view, input, {logits, n, shape.experts, uint64_t(shape.experts) * 4});
     g.prefill_route_batch(logits, ids, weights, shape.experts, shape.selected, n, mode, normalize_selected);
     const GpuRowsF32 gate = rows(s.rows.gate, n * shape.selected, shape.hidden), down_rows = rows(s.rows.down, n * shape.selected, shape.channels);
-    if (is_planar_moe(g, w, shape)) {
+    if (planar) {
         if (n <= 8) g.planar_moe_routed_m8(w.gate.view, w.up.view, w.down.view, ids, input, gate, down_rows, shape.experts, shape.selected);
         else g.planar_nax_grouped_moe(w.gate.view, w.up.view, w.down.view, ids, input, down_rows, s.token_map, s.counts, s.tasks, shape.experts, shape.selected);
     } else {
@@ -868,6 +904,10 @@ void encode_moe_mm_many(HipGraph& g, const MoeWeights& w, const MoeMmManyScratch
     g.gemv_rows(w.shared_router.encoding, w.shared_router.view, input, {shared_logit, n, 1, 4});
     g.prefill_mixture_batch(active(s.rows.down, uint64_t(shape.selected) * shape.channels), weights, active(s.rows.shared_down, shape.channels),
                             shared_logit, output, shape.selected);
+    } catch (...) {  // src/moe_mm_many.cpp:282: a refusal part-way leaves no half-encoded batch behind
+        g.abort();
+        throw;
+    }
 }
 
 }  // namespace tokspur

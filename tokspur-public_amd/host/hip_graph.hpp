@@ -84,6 +84,7 @@ static_assert(sizeof(GpuLogitTopKRow) == 528, "GpuLogitTopKRow ABI");
 class HipGraph {
 public:
     explicit HipGraph(uint64_t byte_budget);
+    HipGraph(const std::string& library_path, uint64_t byte_budget);  // graph.hpp:433; the kernels are linked in, the path is not opened
     ~HipGraph();
     HipGraph(const HipGraph&) = delete;
     HipGraph& operator=(const HipGraph&) = delete;
@@ -103,6 +104,8 @@ public:
     // ---- Pack v3 registration (idle only, before the first batch), graph.hpp:465-471
     void register_planar_matrix(GpuView matrix, PlanarMatrixShape shape);
     [[nodiscard]] uint64_t planar_matrix_count() const;
+    void register_q8_matrix(GpuView matrix, uint32_t columns, uint32_t rows, PrefillWeightLayout layout = PrefillWeightLayout::gguf);  // graph.hpp:468
+    [[nodiscard]] uint64_t q8_matrix_count() const;
     [[nodiscard]] std::optional<PlanarMatrixShape> planar_matrix_shape(GpuView matrix) const;
     void prepare_planar_moe_v3(uint32_t gate_up_encoding, uint32_t down_encoding, bool prepare_nax = true,
                                uint32_t max_nax_tokens = 2048, uint32_t max_experts = 512, uint32_t max_selected = 10,
@@ -178,6 +181,8 @@ struct MoeScratch {
 MoeScratch allocate_moe_scratch(HipGraph& graph, MoeShape shape);
 void release_moe_scratch(HipGraph& graph, const MoeScratch& scratch);
 [[nodiscard]] bool is_planar_moe(const HipGraph& graph, const MoeWeights& weights, MoeShape shape);
+// what `grouped_mm` multiplies (src/grouped_mm.cpp:9): an encoding and a row layout
+[[nodiscard]] bool grouped_mm_takes(uint32_t encoding, PrefillWeightLayout layout);
 // Encodes router GEMV -> top-k -> routed experts -> shared expert -> mixture into the caller's current batch; allocates,
 // reads and commits nothing.
 void encode_moe(HipGraph& graph, const MoeWeights& weights, const MoeScratch& scratch, GpuView input, GpuView output,
