@@ -182,7 +182,7 @@ def main():
     gu_flops = T * S * 2.0 * (2 * H) * C
     gu_bytes = nonempty * 2 * H * (C // 256) * 144 + T * C * 2 + T * S * H * 2
     gu_s = gu["avg_us"] * 1e-6
-    roofline = {"kernel": "gemm_gate_up_swiglu (routed experts of configs[3]: Q4_K planar rows -> integer f16 MFMA 32x32x16 + SwiGLU)",
+    roofline = {"kernel": "gemm_gate_up_swiglu (routed experts of configs[3]: persistent workgroups, a task's activation rows resident in registers, Q4_K planar weight tiles streamed global->LDS once per task -> integer f16 MFMA 32x32x16 + SwiGLU)",
                 "bound": "hbm", "achieved": gu_bytes / gu_s / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": gu_bytes / gu_s / 1e9 / HBM_PEAK_GBPS, "traffic": measured_traffic("gemm_gate_up_swiglu"),
                 "avg_launch_us": gu["avg_us"], "bytes_per_launch": gu_bytes, "flops_per_launch": gu_flops,
