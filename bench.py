@@ -37,6 +37,24 @@ def timed(torch, fn, steps, warmup):
     return start.elapsed_time(stop) / steps
 
 
+def timed_batches(torch, fn, batches=50, warmup=3):
+    """`batches` launches of `fn`, each bracketed by its own pair of events (the engine's BatchResult.gpu_ms, src/graph.mm:3979-3984):
+    mean, median and min in ms. The event pairs add a few microseconds of idle time per batch that the back-to-back loop of
+    `timed` does not see."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(batches)]
+    for start, stop in pairs:
+        start.record()
+        fn()
+        stop.record()
+    torch.cuda.synchronize()
+    ms = sorted(start.elapsed_time(stop) for start, stop in pairs)
+    return {"batches": batches, "mean_ms": sum(ms) / len(ms), "median_ms": ms[len(ms) // 2] if len(ms) % 2 else 0.5 * (ms[len(ms) // 2 - 1] + ms[len(ms) // 2]),
+            "min_ms": ms[0]}
+
+
 def graph_of(torch, fn, result, times=1):
     """`fn` recorded `times` times into one HIP graph (the launches of a step replayed by the driver instead of being
     issued one by one from Python), or None when capture fails or a replay does not reproduce the eager result bit for
@@ -165,10 +183,12 @@ def main():
     assert args.skip_comparison or torch.equal(out, reference_out), "the two ways of running the shared expert disagree"
     graph = None if args.no_graph else graph_of(torch, step_c3, out)
     graph_ms_step = timed(torch, graph.replay, args.steps, args.warmup) if graph is not None else None
-    if graph_ms_step is None or graph_ms_step >= eager_ms_step:
-        graph, ms_step = None, eager_ms_step  # the step is reported the way it ran fastest
-    else:
-        ms_step = graph_ms_step
+    # the step is reported the way it ran fastest; both ways are in the line
+    ms_step = eager_ms_step if graph_ms_step is None or graph_ms_step >= eager_ms_step else graph_ms_step
+    # the same step under the engine's protocol: 3 warm-up batches, then 50 batches with an event pair around each
+    batches = max(50, args.steps)
+    protocol = {"eager": timed_batches(torch, step_c3, batches, 3),
+                "graph": timed_batches(torch, graph.replay, batches, 3) if graph is not None else None}
     assert gpu.error() == 0, "device error word set during the timed region"
     counts = scratch.counts.cpu().numpy().view(np.uint32)
     nonempty = int((counts > 0).sum())
@@ -199,11 +219,52 @@ def main():
         "hbm_gbps": bytes_step / (ms_step * 1e-3) / 1e9, "hbm_frac": bytes_step / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
         "expert_loads": {"nonempty": nonempty, "min": int(counts.min()), "median": int(np.median(counts)), "max": int(counts.max())},
         "kernels_us": {k: round(v["avg_us"], 2) for k, v in prof.items()},
-        "launch": "HIP graph replay of the step's kernels" if graph is not None else "eager launches from Python",
+        "launch": "HIP graph replay of the step's kernels" if ms_step is graph_ms_step else "eager launches from Python",
         "eager_ms_per_step": eager_ms_step, "graph_ms_per_step": graph_ms_step,
+        "per_batch_events": protocol,
         "shared_expert": "rides in the routed experts' gate/up and down launches" + (
             "" if two_streams_ms_step is None else
             f" (same bits as run beside them on a second stream: {two_streams_ms_step:.3f} ms per step that way, eager)")}}
+
+    # ------------------------------------------------------------------ the whole sublayer, router projection included
+    # What encode_moe_mm_many enqueues for a chunk (src/moe_mm_many.cpp:126-283): router projection as ONE f32 GEMM
+    # (kernels/moe_router_f32_batch.metal:13) -> batch top-k -> routed experts -> shared expert as three dense Q8_0 products
+    # with SwiGLU between -> shared router -> batch mixture. The router weights are random here, so the expert loads are
+    # near uniform (the headline step draws Zipf-biased logits instead of projecting them).
+    rw = gpu.upload(synth.activations_f32(synth.tensor_seed(3, 30), (E, C)) / np.float32(np.sqrt(C)))
+    srw = gpu.upload(synth.activations_f32(synth.tensor_seed(3, 31), (1, C)) / np.float32(np.sqrt(C)))
+    q8g, q8u = gpu.upload(synth.matrix(8, synth.tensor_seed(3, 32), H, C)), gpu.upload(synth.matrix(8, synth.tensor_seed(3, 33), H, C))
+    q8d = gpu.upload(synth.matrix(8, synth.tensor_seed(3, 34), C, H))
+    lg_l, sl_l = gpu.empty((T, E)), gpu.empty(T)
+    sg_l, su_l, sd_l = gpu.empty((T, H)), gpu.empty((T, H)), gpu.empty((T, C))
+    q8ws = gpu.empty(max(capi.dense_mm_q8_workspace_bytes(T, C, H), capi.dense_mm_q8_workspace_bytes(T, H, C)), "uint8")
+    scratch_l = capi.GroupedScratch(gpu, T, S, E, C, H)
+
+    def step_sublayer():
+        gpu.router_f32_batch(rw, d_x, T, C, E, out=lg_l)
+        gpu.route(lg_l, S, 0, True, tokens=T, out=(ids, wts))
+        capi.planar_nax_grouped_moe(gpu, w, ids, d_x, T, S, scratch_l, y=y)
+        capi.dense_mm_q8_staged(gpu, capi.LAYOUT_GGUF, q8g, d_x, T, C, H, out=sg_l, workspace=q8ws)
+        capi.dense_mm_q8_staged(gpu, capi.LAYOUT_GGUF, q8u, d_x, T, C, H, out=su_l, workspace=q8ws)
+        gpu.swiglu(sg_l, su_l, out=sg_l)
+        capi.dense_mm_q8_staged(gpu, capi.LAYOUT_GGUF, q8d, sg_l, T, H, C, out=sd_l, workspace=q8ws)
+        gpu.gemv_rows(0, srw, d_x, sl_l, T, C, 1, C * 4, 4)
+        gpu.mixture(y, wts, sd_l, sl_l, C, S, tokens=T, out=out)
+
+    sub_eager = timed(torch, step_sublayer, args.steps, args.warmup)
+    sub_graph = None if args.no_graph else graph_of(torch, step_sublayer, out)
+    sub_graph_ms = timed(torch, sub_graph.replay, args.steps, args.warmup) if sub_graph is not None else None
+    sub_ms = sub_eager if sub_graph_ms is None or sub_graph_ms >= sub_eager else sub_graph_ms
+    sub_counts = scratch_l.counts.cpu().numpy().view(np.uint32)
+    configs["c3_sublayer_with_router"] = {
+        "tok_per_s": T / (sub_ms * 1e-3), "ms_per_step": sub_ms, "eager_ms_per_step": sub_eager, "graph_ms_per_step": sub_graph_ms,
+        "per_batch_events": {"eager": timed_batches(torch, step_sublayer, batches, 3),
+                             "graph": timed_batches(torch, sub_graph.replay, batches, 3) if sub_graph is not None else None},
+        "expert_loads": {"nonempty": int((sub_counts > 0).sum()), "min": int(sub_counts.min()), "median": int(np.median(sub_counts)), "max": int(sub_counts.max())},
+        "kernels_us": {k: round(v["avg_us"], 2) for k, v in profiled(capi, torch, step_sublayer, 5).items()},
+        "composition": "router f32 GEMM -> top-10 -> grouped gate/up + SwiGLU -> grouped down -> shared expert as 3 dense Q8_0 GEMMs + SwiGLU -> shared router -> mixture"}
+    assert gpu.error() == 0, "device error word set during the sublayer steps"
+    del sub_graph
 
     # ------------------------------------------------------------------ CPU baseline (rank 0, bounded sample)
     cpu = None

@@ -210,6 +210,16 @@ int tsp_route(const float* logits, uint32_t* indices, float* weights, uint32_t e
  * the same per token row; logits [tokens, experts], outputs [tokens, selected]. */
 int tsp_route_batch(const float* logits, uint32_t* indices, float* weights, uint32_t experts, uint32_t selected,
                     uint32_t tokens, uint32_t mode, int normalize_selected, uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:825 `moe_router_f32_batch` and :836 `moe_router_f32_window` (kernels/moe_router_f32_batch.metal:13-50;
+ * planner src/moe_mm_many_plan.cpp:6-26): the router projection of a whole chunk as one f32 GEMM,
+ * output[t, e] = sum_k weights[e, k] * input[t, k], both operands f32 from memory to the accumulator (f32 matrix-core
+ * multiply-accumulate, nothing narrowed). weights is [experts, columns] row-major; input and output rows lie
+ * `*_stride_bytes` apart (multiples of 16, as the engine's planner demands). Columns in multiples of 32. The engine bounds
+ * the shape to 2560 x 512 and 512 (2048 for the window) tokens; this entry point takes any shape within 65536 each way and
+ * leaves those bounds to the planner above it. TSP_ERRBIT_NONFINITE when a result is not finite. */
+int tsp_router_f32_batch(const float* weights, const float* input, uint64_t input_stride_bytes, float* output,
+                         uint64_t output_stride_bytes, uint32_t columns, uint32_t experts, uint32_t tokens,
+                         uint32_t* error_word, void* stream);
 /* include/tokspur/graph.hpp:1102 `mixture` (kernels/graph.metal:528-544; CPU: src/routing.cpp:42-60):
  * y[c] = sigmoid(shared_logit) * shared[c] + sum_r w[r] * experts[r, c], r in route order. */
 int tsp_mixture(const float* expert_outputs, const float* weights, const float* shared_output, const float* shared_logit,

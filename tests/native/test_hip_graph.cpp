@@ -7,6 +7,7 @@
 #include <cstring>
 #include <cstdlib>
 #include <functional>
+#include <limits>
 #include <string>
 #include <vector>
 
@@ -403,12 +404,13 @@ std::vector<double> cpu_moe_token_q8_shared(const MoeFixture& f, const std::vect
     return out;
 }
 
-void test_encode_moe_mm_many() {
+void encode_moe_mm_many_case(bool router_batch) {
     // planar Q4_K / Q6_K routed experts, dense Q8_0 shared expert (gate in q8_lanes_v1 rows, up and down in GGUF rows), F32 routers;
     // 70 rows take the grouped GEMM, 5 rows the routed kernels for at most eight
     const MoeFixture f = make_moe(256, 256, 8, 3);
     const uint32_t capacity = 70;
     HipGraph g(512u << 20);
+    g.configure_moe_router_f32_batch(router_batch);  // src/moe_mm_many.cpp:170-177: the chunk's router logits from one f32 GEMM
     MoeOnGraph m = upload_moe(g, f);
     const auto sg = fixture(8, f.shape.channels, f.shape.hidden, 1), sd = fixture(8, f.shape.hidden, f.shape.channels, 1);
     auto su = sg;
@@ -446,7 +448,7 @@ void test_encode_moe_mm_many() {
             for (uint32_t c = 0; c < f.shape.channels; ++c) worst = std::max(worst, std::fabs(double(y[size_t(t) * stride + c]) - want[c]) / scale);
             for (uint32_t c = f.shape.channels; c < stride; ++c) pads = pads && y[size_t(t) * stride + c] == -3.0f;
         }
-        std::printf("encode_moe_mm_many T=%u: max error / row max %.3e\n", T, worst);
+        std::printf("encode_moe_mm_many T=%u%s: max error / row max %.3e\n", T, router_batch ? ", router as one GEMM" : "", worst);
         EXPECT(worst <= 2e-3 && pads);
         g.release(dx);
         g.release(dy);
@@ -478,6 +480,86 @@ void test_encode_moe_mm_many() {
     }
     release_moe_mm_many_scratch(g, scratch);
 }
+void test_encode_moe_mm_many() { encode_moe_mm_many_case(false); }
+void test_encode_moe_mm_many_router_batch() { encode_moe_mm_many_case(true); }
+
+// native/tests/test_moe_mm_many.cpp:35-47 (the plan) and native/tests/test_moe_mm_many_gpu.cpp:194-262 (selection, preparation,
+// the 5e-5 logit bound against double sums and against the per-row GEMV, untouched padding, refusals that write nothing)
+void test_router_projection_controls() {
+    for (const uint32_t n : {1u, 2u, 3u, 8u, 31u, 32u, 33u, 511u, 512u}) {
+        const auto p = moe_router_f32_plan(2560, 512, n, 10272, 2080);
+        EXPECT(p.matrix_bytes == 5242880 && p.input_bytes == uint64_t(n - 1) * 10272 + 10240 && p.output_bytes == uint64_t(n - 1) * 2080 + 2048);
+        EXPECT(p.grid_x == 16 && p.grid_y == (n + 31) / 32 && p.args.tokens == n && p.args.reserved == 0);
+    }
+    for (const uint32_t n : {0u, 513u, std::numeric_limits<uint32_t>::max()}) EXPECT(throws_format([&] { (void)moe_router_f32_plan(2560, 512, n, 10240, 2048); }));
+    EXPECT(throws_format([] { (void)moe_router_f32_plan(2559, 512, 3, 10240, 2048); }));
+    EXPECT(throws_format([] { (void)moe_router_f32_plan(2560, 511, 3, 10240, 2048); }));
+    EXPECT(throws_format([] { (void)moe_router_f32_plan(2560, 512, 3, 10236, 2048); }));
+    EXPECT(throws_format([] { (void)moe_router_f32_plan(2560, 512, 3, 10240, 2044); }));
+    EXPECT(throws_format([] { (void)moe_router_f32_plan(2560, 512, 512, std::numeric_limits<uint64_t>::max() - 15, 2048); }));
+    EXPECT(throws_format([] { (void)moe_router_f32_plan(2560, 512, 512, 10240, std::numeric_limits<uint64_t>::max() - 15); }));
+    EXPECT(throws_format([] { (void)moe_router_f32_plan(2560, 512, 2, 256ull << 20, 2048); }));
+    // the device kernel's own limits: any multiple of 32 columns, any expert count
+    EXPECT(moe_router_f32_plan(2048, 70, 2048, 8192, 288, false).grid_x == 3);
+    EXPECT(throws_format([] { (void)moe_router_f32_plan(2040, 70, 3, 8160, 288, false); }));
+
+    HipGraph g(256u << 20);
+    EXPECT(!g.moe_router_f32_batch_enabled() && std::string(g.moe_router_f32_projection_kernel()) == "graph_quantized_gemv");
+    g.configure_moe_router_f32_batch(true);
+    EXPECT(g.moe_router_f32_batch_enabled() && std::string(g.moe_router_f32_projection_kernel()) == "graph_moe_router_f32_batch");
+    constexpr uint32_t c = 2560, e = 512, capacity = 512;
+    constexpr uint64_t xs = c * 4 + 32, ys = e * 4 + 32;
+    std::vector<float> weights(uint64_t(c) * e), input(capacity * xs / 4, -9876.25f), poison(capacity * ys / 4 + 16, -7654.25f);
+    uint32_t rng = 44;
+    for (auto& v : weights) { rng = rng * 1664525u + 1013904223u; v = float(int(rng % 1993) - 996) / 997 / 256; }
+    for (uint32_t t = 0; t < capacity; ++t)
+        for (uint32_t k = 0; k < c; ++k) { rng = rng * 1664525u + 1013904223u; input[t * xs / 4 + k] = float(int(rng % 1993) - 996) / 997; }
+    const GpuView w = g.upload(bytes_of(weights), "router"), x = g.upload(bytes_of(input), "x");
+    const GpuView y = g.upload(bytes_of(poison), "y", false), scalar = g.upload(bytes_of(poison), "scalar", false);
+    g.begin();
+    EXPECT(throws_format([&] { g.moe_router_f32_batch(w, {x, 3, c, xs}, {y, 3, e, ys}); }));  // selected but not prepared
+    g.abort();
+    EXPECT(read_as<float>(g, y) == poison);
+    g.prepare_moe_router_f32_batch();
+    EXPECT(throws_format([&] { g.configure_moe_router_f32_batch(false); }));
+    for (const uint32_t n : {3u, 33u, 512u}) {
+        const uint64_t allocations = g.memory().allocations;
+        g.begin();
+        g.gemv_rows(0, w, {x, n, c, xs}, {scalar, n, e, ys});
+        g.moe_router_f32_batch(w, {x, n, c, xs}, {y, n, e, ys});
+        const BatchResult r = g.submit();
+        EXPECT(r.dispatches == 2 && g.memory().allocations == allocations);
+        const auto got = read_as<float>(g, y), legacy = read_as<float>(g, scalar);
+        bool bound = true, pads = true;
+        for (uint32_t t = 0; t < n; ++t) {
+            for (uint32_t expert = 0; expert < e; ++expert) {
+                double sum = 0;
+                for (uint32_t k = 0; k < c; ++k) sum += double(weights[uint64_t(expert) * c + k]) * input[t * xs / 4 + k];
+                const double a = got[t * ys / 4 + expert], b = legacy[t * ys / 4 + expert], tol = 0.00005 * std::max(1.0, std::fabs(sum));
+                bound = bound && std::isfinite(a) && std::fabs(a - sum) <= tol && std::fabs(b - sum) <= tol && std::fabs(a - b) <= 0.00005 * std::max(1.0, std::fabs(b));
+            }
+            for (uint32_t k = e; k < ys / 4; ++k) pads = pads && got[t * ys / 4 + k] == -7654.25f;
+        }
+        for (size_t k = n * ys / 4; k < got.size(); ++k) pads = pads && got[k] == -7654.25f;
+        EXPECT(bound && pads);
+    }
+    const auto saved = read_as<float>(g, y);
+    const auto refused = [&](GpuRowsF32 in, GpuRowsF32 out) {
+        g.begin();
+        const bool threw = throws_format([&] { g.moe_router_f32_batch(w, in, out); });
+        g.abort();
+        return threw && read_as<float>(g, y) == saved;
+    };
+    const GpuRowsF32 in{x, 3, c, xs}, out{y, 3, e, ys};
+    GpuRowsF32 bad = out;
+    bad.rows = 2;
+    EXPECT(refused(in, bad));
+    bad = out; bad.stride_bytes = e * 4 - 4;
+    EXPECT(refused(in, bad));
+    bad = out; bad.view = x;  // immutable, and the input itself
+    EXPECT(refused(in, bad));
+}
+
 // the raw-GGUF arm of the same composition (src/moe_mm_many.cpp:214-240): three grouped products over Q4_K expert stacks in
 // GGUF rows, nothing registered; `grouped_mm` and `dense_mm` on their own; encodings the grouped product does not take are
 // refused while idle, and a refusal part-way through a batch leaves no half-encoded batch behind
@@ -599,6 +681,8 @@ int main() {
                                                          {"encode_moe single token", test_encode_moe_single_token},
                                                          {"encode_moe_batch", test_encode_moe_batch},
                                                          {"encode_moe_mm_many", test_encode_moe_mm_many},
+                                                         {"encode_moe_mm_many, router projection as one f32 GEMM", test_encode_moe_mm_many_router_batch},
+                                                         {"router projection: plan, selection, bounds, refusals", test_router_projection_controls},
                                                          {"encode_moe_mm_many, raw-GGUF arm; prepare twice; Q8_0 registration", test_encode_moe_mm_many_raw_arm}};
     for (const auto& [name, fn] : tests) {
         std::printf("== %s\n", name);

@@ -64,6 +64,91 @@ def test_route_batch_ids_bit_exact(gpu, orc, synth, tokens, experts, selected):
     assert np.allclose(w.sum(axis=1), 1.0, rtol=1e-5)
 
 
+def lcg_values(state, count):
+    """`count` draws of the 32-bit generator x -> 1664525 x + 1013904223 as float(int(x % 1993) - 996) / 997, and the state."""
+    out = np.empty(count, dtype=np.float64)
+    for i in range(count):
+        state = (state * 1664525 + 1013904223) & 0xFFFFFFFF
+        out[i] = (state % 1993) - 996
+    return (out / 997), state
+
+
+def test_router_f32_batch_reference_controls(gpu, orc, tsp):
+    """native/tests/test_moe_mm_many_gpu.cpp:194-262: dense non-binary f32 weights [512, 2560] and strided, poisoned rows;
+    every logit within 5e-5 * max(1, |sum|) of the double sum and of the per-row f32 GEMV, padding untouched, the ten
+    selected ids equal to the scalar path's and to the double route for both modes."""
+    c, e, capacity = 2560, 512, 512
+    xs, ys = c * 4 + 32, e * 4 + 32
+    w64, state = lcg_values(44, c * e)
+    weights = (w64.astype(np.float32) / np.float32(256)).reshape(e, c)
+    x64, state = lcg_values(state, capacity * c)
+    x_rows = np.full((capacity, xs // 4), -9876.25, dtype=np.float32)
+    x_rows[:, :c] = x64.astype(np.float32).reshape(capacity, c)
+    d_w, d_x = gpu.upload(weights), gpu.upload(x_rows)
+    want = x_rows[:, :c].astype(np.float64) @ weights.astype(np.float64).T
+    for n in (1, 2, 3, 8, 31, 32, 33, 511, 512):
+        y = gpu.full((capacity, ys // 4), -7654.25)
+        scalar = gpu.full((capacity, ys // 4), -7654.25)
+        gpu.router_f32_batch(d_w, d_x, n, c, e, x_stride=xs, out=y, out_stride=ys)
+        gpu.gemv_rows(0, d_w, d_x, scalar, n, c, e, xs, ys)
+        got, legacy = y.cpu().numpy(), scalar.cpu().numpy()
+        bound = 0.00005 * np.maximum(1.0, np.abs(want[:n]))
+        assert np.isfinite(got[:n, :e]).all() and (np.abs(got[:n, :e] - want[:n]) <= bound).all(), n
+        assert (np.abs(legacy[:n, :e] - want[:n]) <= bound).all() and (np.abs(got[:n, :e].astype(np.float64) - legacy[:n, :e]) <= bound).all(), n
+        assert (got[:n, e:] == -7654.25).all() and (got[n:] == -7654.25).all(), "router output row padding / inactive rows"
+        # tighter than the engine asks: f32 products and sums leave ~1e-6 of the sum of |w x|
+        scale = np.abs(x_rows[:n, :c]).astype(np.float64) @ np.abs(weights).astype(np.float64).T
+        assert (np.abs(got[:n, :e] - want[:n]) <= 2e-6 * scale).all(), n
+        compact, compact_old = gpu.upload(np.ascontiguousarray(got[:n, :e])), gpu.upload(np.ascontiguousarray(legacy[:n, :e]))
+        for mode in (0, 1):
+            for normalise in (False, True):
+                ids, wts = gpu.route(compact, 10, mode, normalise, tokens=n)
+                old_ids, old_wts = gpu.route(compact_old, 10, mode, normalise, tokens=n)
+                assert np.array_equal(u32(ids), u32(old_ids)), "router all-row selected IDs differ from actual scalar route"
+                assert np.abs(wts.cpu().numpy() - old_wts.cpu().numpy()).max() <= 0.00005
+                for t in range(0, n, max(1, n // 16)):
+                    want_ids, want_w = orc.route_reference(want[t], 10, mode, normalise)
+                    assert np.array_equal(u32(ids)[t], want_ids) and np.abs(wts.cpu().numpy()[t] - want_w).max() <= 0.00005
+    # exact ties select low ids
+    y = gpu.router_f32_batch(gpu.zeros((e, c)), d_x, 3, c, e, x_stride=xs)
+    ids, _ = gpu.route(y, 10, 0, True, tokens=3)
+    assert (u32(ids) == np.arange(10)).all() and gpu.error() == 0
+    # refusals: short stride, output over an input, odd column count
+    y = gpu.full((capacity, ys // 4), -7654.25)
+    for call in (lambda: gpu.router_f32_batch(d_w, d_x, 3, c, e, x_stride=xs, out=y, out_stride=e * 4 - 4),
+                 lambda: gpu.router_f32_batch(d_w, d_x, 3, c, e, x_stride=xs, out=d_x, out_stride=ys),
+                 lambda: gpu.router_f32_batch(d_w, d_x, 3, c, e, x_stride=xs, out=d_w, out_stride=ys),
+                 lambda: gpu.router_f32_batch(d_w, d_x, 3, c - 8, e, x_stride=xs, out=y, out_stride=ys),
+                 lambda: gpu.router_f32_batch(d_w, d_x, 0, c, e, x_stride=xs, out=y, out_stride=ys)):
+        with pytest.raises(tsp.FormatError):
+            call()
+    assert (y.cpu().numpy() == -7654.25).all(), "router refusal does not write output"
+
+
+@pytest.mark.parametrize("tokens,columns,experts", [(1, 32, 1), (33, 96, 70), (130, 160, 65), (2048, 2048, 512)])
+def test_router_f32_batch_shapes(gpu, synth, tokens, columns, experts):
+    """Ragged tiles in every direction and the configs[3] chunk; a non-finite input raises the sticky bit."""
+    w = synth.activations_f32(synth.tensor_seed(5, tokens), (experts, columns)) / np.float32(16)
+    x = synth.activations_f32(synth.tensor_seed(6, tokens), (tokens, columns))
+    pitch = (experts + 3) // 4 * 4  # output rows lie a multiple of 16 bytes apart, as the engine's planner demands
+
+    def run(rows):
+        out = gpu.full((tokens, pitch), -3.0)
+        gpu.router_f32_batch(gpu.upload(w), gpu.upload(rows), tokens, columns, experts, out=out, out_stride=pitch * 4)
+        out = out.cpu().numpy()
+        assert (out[:, experts:] == -3.0).all()
+        return np.ascontiguousarray(out[:, :experts])
+
+    got = run(x)
+    want = x.astype(np.float64) @ w.astype(np.float64).T
+    scale = np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64).T
+    assert (np.abs(got - want) <= 2e-6 * scale + 1e-30).all() and gpu.error() == 0
+    assert np.array_equal(got.view(np.uint32), run(x).view(np.uint32))
+    x[tokens // 2, columns - 1] = np.inf
+    run(x)
+    assert gpu.error() == 1
+
+
 def test_route_errors(gpu, tsp):
     logits = np.zeros(16, dtype=np.float32)
     logits[3] = np.nan

@@ -277,6 +277,14 @@ class Device:
                                     C.c_int(bool(broadcast)), self.ptr(self.err), self.stream()))
         return y
 
+    def router_f32_batch(self, weights, x, tokens, columns, experts, x_stride=None, out=None, out_stride=None):
+        """logits[t, e] = sum_k weights[e, k] * x[t, k] for a whole chunk of token rows in one f32 GEMM."""
+        out = self.empty((tokens, experts)) if out is None else out
+        check(dll().tsp_router_f32_batch(self.ptr(weights), self.ptr(x), C.c_uint64(columns * 4 if x_stride is None else x_stride),
+                                         self.ptr(out), C.c_uint64(experts * 4 if out_stride is None else out_stride), C.c_uint32(columns),
+                                         C.c_uint32(experts), C.c_uint32(tokens), self.ptr(self.err), self.stream()))
+        return out
+
     def route(self, logits, selected, mode=0, normalize=True, tokens=None, out=None):
         """logits [experts] (tokens=None: the single-row operator) or [tokens, experts]."""
         experts = logits.shape[-1]
@@ -411,6 +419,12 @@ def dense_mm_q8(dev, layout, matrix, x, tokens, columns, rows, out=None, x_strid
                                 C.c_uint64(rows * 4 if out_stride is None else out_stride), C.c_uint32(tokens), C.c_uint32(columns),
                                 C.c_uint32(rows), dev.ptr(dev.err), dev.stream()))
     return out
+
+
+def dense_mm_q8_workspace_bytes(tokens, columns, rows):
+    f = dll().tsp_dense_mm_q8_workspace_bytes
+    f.restype = C.c_uint64
+    return f(C.c_uint32(tokens), C.c_uint32(columns), C.c_uint32(rows))
 
 
 def dense_mm_q8_staged(dev, layout, matrix, x, tokens, columns, rows, out=None, x_stride=None, out_stride=None, workspace=None):

@@ -72,6 +72,7 @@ struct HipGraph::Impl {
     void* q8_workspace = nullptr;
     uint64_t q8_workspace_bytes = 0;
     uint32_t prepared_gate_up = 0, prepared_down = 0;
+    bool router_batch = false, router_batch_prepared = false;
 
     void same_thread() const { require(std::this_thread::get_id() == thread, "GPU graph used from another thread"); }
     void idle() const {
@@ -371,6 +372,34 @@ void HipGraph::gemv_rows(uint32_t encoding, GpuView matrix, GpuRowsF32 input, Gp
     check(tsp_gemv_rows(encoding, TSP_LAYOUT_GGUF, p.device(matrix), matrix.bytes, reinterpret_cast<const float*>(p.device(input.view)), input.stride_bytes,
                         reinterpret_cast<float*>(p.device(output.view, true)), output.stride_bytes, input.rows, input.columns, output.columns,
                         p.error_word, p.stream));
+}
+
+void HipGraph::configure_moe_router_f32_batch(bool enabled) {
+    auto& p = *impl_; p.idle();
+    require(!p.router_batch_prepared && !p.locked, "router FP32 batch selection is fixed before preparation or any batch");
+    p.router_batch = enabled;
+}
+bool HipGraph::moe_router_f32_batch_enabled() const { impl_->same_thread(); return impl_->router_batch; }
+const char* HipGraph::moe_router_f32_projection_kernel() const {
+    impl_->same_thread();
+    return impl_->router_batch ? moe_router_f32_kernel : "graph_quantized_gemv";
+}
+void HipGraph::prepare_moe_router_f32_batch() {
+    auto& p = *impl_; p.idle();
+    p.router_batch_prepared = true;
+}
+void HipGraph::moe_router_f32_batch(GpuView matrix, GpuRowsF32 input, GpuRowsF32 output) {
+    auto& p = *impl_; p.active();
+    require(p.router_batch && p.router_batch_prepared, "router FP32 batch requires explicit idle selection/preparation and direct batches");
+    require(input.rows == output.rows, "router FP32 batch row count mismatch");
+    const auto plan = moe_router_f32_plan(input.columns, output.columns, input.rows, input.stride_bytes, output.stride_bytes, false);
+    require(matrix.bytes == plan.matrix_bytes && input.view.bytes >= plan.input_bytes && output.view.bytes >= plan.output_bytes &&
+                matrix.offset % 4 == 0 && input.view.offset % 4 == 0 && output.view.offset % 4 == 0,
+            "router FP32 batch view extent/alignment");
+    validate_disjoint(std::array{matrix, input.view}, std::array{output.view});
+    check(tsp_router_f32_batch(reinterpret_cast<const float*>(p.device(matrix)), reinterpret_cast<const float*>(p.device(input.view)),
+                               input.stride_bytes, reinterpret_cast<float*>(p.device(output.view, true)), output.stride_bytes, input.columns,
+                               output.columns, input.rows, p.error_word, p.stream));
 }
 
 void HipGraph::prepare_q8_matvec_many(uint32_t width) {
@@ -800,6 +829,23 @@ void encode_moe_batch(HipGraph& graph, const MoeWeights& w, const MoeBatchScratc
 }
 
 // ------------------------------------------------------------------ encode_moe_mm_many
+MoeRouterF32Plan moe_router_f32_plan(uint32_t columns, uint32_t experts, uint32_t tokens, uint64_t input_stride_bytes,
+                                     uint64_t output_stride_bytes, bool engine_bounds) {
+    const bool shape_ok = engine_bounds ? (columns == 2560 && experts == 512 && tokens && tokens <= 512)
+                                        : (columns && columns % 32 == 0 && columns <= 65536 && experts && experts <= 65536 && tokens && tokens <= 65536);
+    if (!shape_ok || input_stride_bytes < uint64_t(columns) * 4 || output_stride_bytes < uint64_t(experts) * 4 || input_stride_bytes % 16 ||
+        output_stride_bytes % 16)
+        throw FormatError("bounded raw FP32 router batch geometry/stride");
+    const auto span = [](uint32_t rows, uint64_t stride, uint64_t last) {
+        if (rows > 1 && stride > (UINT64_MAX - last) / (rows - 1)) throw FormatError("bounded raw FP32 router batch span");
+        return uint64_t(rows - 1) * stride + last;
+    };
+    const uint64_t input = span(tokens, input_stride_bytes, uint64_t(columns) * 4), output = span(tokens, output_stride_bytes, uint64_t(experts) * 4);
+    if (input > (256ull << 20) || output > (256ull << 20)) throw FormatError("bounded raw FP32 router batch span");
+    return {{columns, experts, tokens, 0, input_stride_bytes, output_stride_bytes}, uint64_t(columns) * experts * 4, input, output,
+            (experts + 31) / 32, (tokens + 31) / 32};
+}
+
 MoeMmManyBytes moe_mm_many_bytes(MoeShape shape, uint32_t capacity, bool allow_nax_2k) {
     shape_check(shape);
     MoeMmManyBytes b;
@@ -842,6 +888,7 @@ void prepare_moe_mm_many(HipGraph& graph, const MoeWeights& w, MoeShape shape, u
         raw_arm_check(w, l);  // refused here, while idle, rather than in the middle of a batch
         graph.prepare_grouped_mm(w.gate.encoding, l.gate, rows, shape.selected, shape.experts, shape.channels > shape.hidden ? shape.channels : shape.hidden);
     }
+    graph.prepare_moe_router_f32_batch();  // src/moe_mm_many.cpp:50
     const uint32_t widest = shape.channels > shape.hidden ? shape.channels : shape.hidden;
     for (const auto layout : {l.shared_gate, l.shared_up, l.shared_down}) graph.prepare_dense_mm_q8(layout, rows, widest, widest);
 }
@@ -882,7 +929,11 @@ void encode_moe_mm_many(HipGraph& g, const MoeWeights& w, const MoeMmManyScratch
     const auto active = [&](GpuView v, uint64_t per_row) { return g.slice(v, 0, per_row * n * 4); };
     const auto rows = [&](GpuView v, uint32_t count, uint32_t columns) { return GpuRowsF32{g.slice(v, 0, uint64_t(count) * columns * 4), count, columns, uint64_t(columns) * 4}; };
     const GpuView logits = active(s.rows.logits, shape.experts), ids = active(s.rows.indices, shape.selected), weights = active(s.rows.weights, shape.selected);
-    g.gemv_rows(w.router.encoding, w.router.view, input, {logits, n, shape.experts, uint64_t(shape.experts) * 4});
+    // src/moe_mm_many.cpp:170-177: one f32 GEMM for the chunk when selected, else one GEMV per row
+    if (g.moe_router_f32_batch_enabled() && w.router.encoding == 0 && n > 1)
+        g.moe_router_f32_batch(w.router.view, input, {logits, n, shape.experts, uint64_t(shape.experts) * 4});
+    else
+        g.gemv_rows(w.router.encoding, w.router.view, input, {logits, n, shape.experts, uint64_t(shape.experts) * 4});
     g.prefill_route_batch(logits, ids, weights, shape.experts, shape.selected, n, mode, normalize_selected);
     const GpuRowsF32 gate = rows(s.rows.gate, n * shape.selected, shape.hidden), down_rows = rows(s.rows.down, n * shape.selected, shape.channels);
     if (planar) {

@@ -120,6 +120,13 @@ public:
     // ---- operators (between begin and submit)
     void gemv(uint32_t encoding, GpuView matrix, GpuView input, GpuView output, uint32_t columns, uint32_t rows);  // graph.hpp:730
     void gemv_rows(uint32_t encoding, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output);                         // graph.hpp:733
+    // graph.hpp:821-825: the router projection of a whole chunk as one f32 GEMM instead of one GEMV per row. Off until
+    // selected; selection and preparation happen while idle, before the first use (src/graph.mm:5701-5746).
+    void configure_moe_router_f32_batch(bool enabled);
+    [[nodiscard]] bool moe_router_f32_batch_enabled() const;
+    [[nodiscard]] const char* moe_router_f32_projection_kernel() const;
+    void prepare_moe_router_f32_batch();
+    void moe_router_f32_batch(GpuView matrix, GpuRowsF32 input, GpuRowsF32 output);
     void prepare_q8_matvec_many(uint32_t width);                                                                    // graph.hpp:744
     void q8_matvec_many(GpuView matrix, GpuView input, GpuView output, uint32_t columns, uint32_t rows, uint32_t width);
     void route(GpuView logits, GpuView indices, GpuView weights, uint32_t selected, RouterMode mode, bool normalize_selected);  // 1091
@@ -208,6 +215,22 @@ struct MoeMmLayouts {
     PrefillWeightLayout gate = PrefillWeightLayout::gguf, up = PrefillWeightLayout::gguf, down = PrefillWeightLayout::gguf;
     PrefillWeightLayout shared_gate = PrefillWeightLayout::gguf, shared_up = PrefillWeightLayout::gguf, shared_down = PrefillWeightLayout::gguf;
 };
+// include/tokspur/moe_mm_many.hpp:11-25 and src/moe_mm_many_plan.cpp:6-14. With `engine_bounds` the plan refuses what the
+// engine refuses (2560 columns, 512 experts, at most 512 rows); without, what the device kernel cannot take (columns not in
+// multiples of 32, more than 65536 either way). Strides are byte counts, multiples of 16.
+struct MoeRouterF32Args {
+    uint32_t columns, experts, tokens, reserved;
+    uint64_t input_stride_bytes, output_stride_bytes;
+};
+static_assert(sizeof(MoeRouterF32Args) == 32, "router FP32 argument ABI");
+struct MoeRouterF32Plan {
+    MoeRouterF32Args args;
+    uint64_t matrix_bytes, input_bytes, output_bytes;
+    uint32_t grid_x, grid_y;  // 32-wide tiles of experts and of rows, as the engine counts them
+};
+inline constexpr const char* moe_router_f32_kernel = "graph_moe_router_f32_batch";
+MoeRouterF32Plan moe_router_f32_plan(uint32_t columns, uint32_t experts, uint32_t tokens, uint64_t input_stride_bytes,
+                                     uint64_t output_stride_bytes, bool engine_bounds = true);
 struct MoeMmManyBytes {
     std::array<uint64_t, 13> views{};
     uint64_t total = 0;
