@@ -11,7 +11,9 @@
 #include <string>
 #include <vector>
 
+#include "gguf_writer.hpp"
 #include "hip_graph.hpp"
+#include "pack_v3.hpp"
 #include "tokspur_hip.h"
 #include "tokspur_oracle.h"
 
@@ -382,7 +384,7 @@ void test_encode_moe_batch() {
 }
 // CPU composition of the whole sublayer for one token with a dense Q8_0 shared expert (src/moe_mm_many.cpp:126-283 order)
 std::vector<double> cpu_moe_token_q8_shared(const MoeFixture& f, const std::vector<uint8_t>& sg, const std::vector<uint8_t>& su, const std::vector<uint8_t>& sd,
-                                            const float* x) {
+                                            const float* x, uint32_t gate_up_type = 12, uint32_t down_type = 14) {
     const MoeShape s = f.shape;
     std::vector<double> logits(s.experts), weights(s.selected), out(s.channels);
     orc_reference_gemv(0, reinterpret_cast<const uint8_t*>(f.router.data()), f.router.size() * 4, s.channels, s.experts, x, s.channels, logits.data());
@@ -390,8 +392,8 @@ std::vector<double> cpu_moe_token_q8_shared(const MoeFixture& f, const std::vect
     std::vector<uint32_t> ids(s.selected);
     orc_route_reference(logits.data(), s.experts, s.selected, 0, 1, ids.data(), weights.data());
     std::vector<double> h(size_t(s.selected) * s.hidden), y(size_t(s.selected) * s.channels);
-    orc_moe_routed_reference(12, 14, f.gate.data(), f.up.data(), f.down.data(), s.channels, s.hidden, s.experts, ids.data(), 1, s.selected, x, s.channels, 1, 0,
-                             h.data(), y.data(), 1);
+    orc_moe_routed_reference(gate_up_type, down_type, f.gate.data(), f.up.data(), f.down.data(), s.channels, s.hidden, s.experts, ids.data(), 1, s.selected, x,
+                             s.channels, 1, 0, h.data(), y.data(), 1);
     std::vector<double> g(s.hidden), u(s.hidden), sy(s.channels);
     orc_reference_gemv(8, sg.data(), sg.size(), s.channels, s.hidden, x, s.channels, g.data());
     orc_reference_gemv(8, su.data(), su.size(), s.channels, s.hidden, x, s.channels, u.data());
@@ -560,6 +562,81 @@ void test_router_projection_controls() {
     EXPECT(refused(in, bad));
 }
 
+// A block of an adopted Pack v3 file on the graph: synthetic shards on disk -> build_block_pack_v3 -> adopt_block_pack_v3 (full
+// authentication) -> upload_moe_block_v3 registers the co-located Q4_K halves and the Q5_1 down planes as they lie in the file ->
+// encode_moe_mm_many runs on them, the shared expert's Q8_0 matrices coming from the pack in q8_lanes_v1 rows.
+void test_pack_v3_block_on_graph() {
+    using gguf_writer::TensorSpec;
+    MoeFixture f{{256, 256, 4, 2}};
+    f.gate = fixture(12, 256, 256, 4);
+    f.up = f.gate;
+    for (size_t at = 0; at < f.up.size(); at += 144) for (size_t i = 16; i < 144; ++i) f.up[at + i] ^= 0x5a;
+    f.down = fixture(7, 256, 256, 4);
+    f.router = lcg_floats(31, size_t(4) * 256);
+    f.shared_router = lcg_floats(37, 256);
+    for (auto& v : f.shared_router) v *= 0.05f;
+    const auto sg = fixture(8, 256, 256, 1), sd = fixture(8, 256, 256, 1);
+    auto su = sg;
+    for (size_t at = 0; at < su.size(); at += 34) for (size_t i = 2; i < 34; ++i) su[at + i] = uint8_t(su[at + i] * 5 + 3);
+    const auto raw = [](const std::vector<float>& v) { std::vector<uint8_t> b(v.size() * 4); std::memcpy(b.data(), v.data(), b.size()); return b; };
+    const std::vector<TensorSpec> specs{{"blk.0.ffn_down_exps.weight", 7, {256, 256, 4}, f.down},      {"blk.0.ffn_down_shexp.weight", 8, {256, 256}, sd},
+                                        {"blk.0.ffn_gate_exps.weight", 12, {256, 256, 4}, f.gate},     {"blk.0.ffn_gate_inp.weight", 0, {256, 4}, raw(f.router)},
+                                        {"blk.0.ffn_gate_inp_shexp.weight", 0, {256}, raw(f.shared_router)}, {"blk.0.ffn_gate_shexp.weight", 8, {256, 256}, sg},
+                                        {"blk.0.ffn_up_exps.weight", 12, {256, 256, 4}, f.up},         {"blk.0.ffn_up_shexp.weight", 8, {256, 256}, su}};
+    gguf_writer::TempDir dir("tokspur_pack_v3_gpu");
+    gguf_writer::write_file(dir.path / "source.gguf", gguf_writer::shard_bytes("qwen35moe", specs));
+    const auto source = std::make_shared<const ModelFiles>(std::vector<std::filesystem::path>{dir.path / "source.gguf"});
+    const auto pack_path = dir.path / "tokspur-pack-v3-blk0.asa.gguf";
+    const auto built = planar_v3::build_block_pack_v3(source, nullptr, 0, pack_path, 2, 1 << 20);
+    EXPECT(built.tensors.size() == 8);
+    const planar_v3::AdoptedPackV3 pack = planar_v3::adopt_block_pack_v3(source, nullptr, 0, pack_path, 2, derived_pack::default_chunk_bytes, 3);
+    EXPECT(pack.plan.tensors.size() == 8 && pack.authentication_workers == 3);
+
+    HipGraph g(512u << 20);
+    const planar_v3::PackMoeBlockV3 block = planar_v3::upload_moe_block_v3(g, pack, 0);
+    EXPECT(block.channels == 256 && block.hidden == 256 && block.experts == 4 && g.planar_matrix_count() == 3);
+    EXPECT(block.gate.encoding == 12 && block.up.encoding == 12 && block.down.encoding == 7);
+    EXPECT(throws_format([&] { (void)planar_v3::upload_moe_block_v3(g, pack, 5); }));
+    MoeWeights w{};
+    const auto from_pack = [&](const char* name) { return g.upload(pack.model->tensor_bytes(name), name); };
+    w.router = {from_pack("blk.0.ffn_gate_inp.weight"), 0};
+    w.shared_router = {from_pack("blk.0.ffn_gate_inp_shexp.weight"), 0};
+    w.gate = block.gate; w.up = block.up; w.down = block.down;
+    w.shared_gate = {from_pack("blk.0.ffn_gate_shexp.weight"), 8};
+    w.shared_up = {from_pack("blk.0.ffn_up_shexp.weight"), 8};
+    w.shared_down = {from_pack("blk.0.ffn_down_shexp.weight"), 8};
+    MoeMmLayouts layouts;  // dense Q8_0 matrices lie in the pack in q8_lanes_v1 rows
+    layouts.shared_gate = layouts.shared_up = layouts.shared_down = PrefillWeightLayout::q8_lanes_v1;
+    for (const auto& t : pack.plan.tensors)
+        if (t.name.find("shexp.weight") != std::string::npos && t.type == 8) EXPECT(t.kind == planar_v3::PlanarKind::q8_lanes_v1);
+    EXPECT(is_planar_moe(g, w, f.shape));
+    const uint32_t capacity = 70;
+    g.configure_moe_router_f32_batch(true);
+    prepare_moe_mm_many(g, w, f.shape, capacity, layouts);
+    const MoeMmManyScratch scratch = allocate_moe_mm_many_scratch(g, f.shape, capacity);
+    for (const uint32_t T : {70u, 5u}) {
+        std::vector<float> x = lcg_floats(900 + T, size_t(T) * 256);
+        for (auto& v : x) { uint32_t bad = 0; v = orc_bf16_to_f32(orc_round_bf16_bits(v, &bad)); }
+        const GpuView dx = g.upload(bytes_of(x), "x", false), dy = g.zeros(uint64_t(T) * 256 * 4, "y");
+        g.begin();
+        encode_moe_mm_many(g, w, scratch, {dx, T, 256, 1024}, {dy, T, 256, 1024}, f.shape, RouterMode::softmax, true, layouts);
+        (void)g.submit();
+        const auto y = read_as<float>(g, dy);
+        double worst = 0;
+        for (uint32_t t = 0; t < T; ++t) {
+            const auto want = cpu_moe_token_q8_shared(f, sg, su, sd, &x[size_t(t) * 256], 12, 7);
+            double scale = 1;
+            for (double v : want) scale = std::max(scale, std::fabs(v));
+            for (uint32_t c = 0; c < 256; ++c) worst = std::max(worst, std::fabs(double(y[size_t(t) * 256 + c]) - want[c]) / scale);
+        }
+        std::printf("encode_moe_mm_many on an adopted pack v3 block, T=%u: max error / row max %.3e\n", T, worst);
+        EXPECT(worst <= 2e-3);
+        g.release(dx);
+        g.release(dy);
+    }
+    release_moe_mm_many_scratch(g, scratch);
+}
+
 // the raw-GGUF arm of the same composition (src/moe_mm_many.cpp:214-240): three grouped products over Q4_K expert stacks in
 // GGUF rows, nothing registered; `grouped_mm` and `dense_mm` on their own; encodings the grouped product does not take are
 // refused while idle, and a refusal part-way through a batch leaves no half-encoded batch behind
@@ -683,6 +760,7 @@ int main() {
                                                          {"encode_moe_mm_many", test_encode_moe_mm_many},
                                                          {"encode_moe_mm_many, router projection as one f32 GEMM", test_encode_moe_mm_many_router_batch},
                                                          {"router projection: plan, selection, bounds, refusals", test_router_projection_controls},
+                                                         {"pack v3: build, adopt, upload a block, encode_moe_mm_many on it", test_pack_v3_block_on_graph},
                                                          {"encode_moe_mm_many, raw-GGUF arm; prepare twice; Q8_0 registration", test_encode_moe_mm_many_raw_arm}};
     for (const auto& [name, fn] : tests) {
         std::printf("== %s\n", name);

@@ -53,10 +53,11 @@ def build(verbose=False, jobs=8):
 
 
 def build_host():
-    """The C++ host class (tokspur::HipGraph) over the C ABI: host/hip_graph.cpp -> libtokspur_graph.so."""
+    """The C++ host side over the C ABI (tokspur::HipGraph, the GGUF reader and the Pack v3 builder / adopter): host/*.cpp -> libtokspur_graph.so."""
     root = os.path.dirname(HERE)
-    cmd = ["hipcc", "-std=c++20", "-O2", "-fPIC", "-shared", "-Wall", os.path.join(HERE, "host", "hip_graph.cpp"),
-           "-I", os.path.join(root, "include"), "-L", HERE, "-ltokspur_hip", "-Wl,-rpath,$ORIGIN", "-o", HOST_LIB]
+    host = os.path.join(HERE, "host")
+    cmd = ["hipcc", "-std=c++20", "-O2", "-fPIC", "-shared", "-Wall", "-pthread"] + sorted(os.path.join(host, f) for f in os.listdir(host) if f.endswith(".cpp")) + [
+        "-I", os.path.join(root, "include"), "-L", HERE, "-ltokspur_hip", "-Wl,-rpath,$ORIGIN", "-o", HOST_LIB]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if proc.returncode:
         raise RuntimeError(f"host library build failed:\n{proc.stdout}")
