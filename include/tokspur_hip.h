@@ -52,6 +52,7 @@ extern "C" {
 /* Row layouts of a dense matrix (include/tokspur/grouped_mm.hpp:6; planar = one Pack v3 expert). */
 #define TSP_LAYOUT_GGUF 0u
 #define TSP_LAYOUT_Q8_LANES_V1 1u
+#define TSP_LAYOUT_Q51_LANES_V1 2u
 #define TSP_LAYOUT_PLANAR_V3 3u
 
 /* Pack v3 planar kinds (include/tokspur/planar_pack_v3.hpp:29-40). Kind 10 is this library's
@@ -121,6 +122,12 @@ int tsp_pack_coloc_half(const tsp_planar_spec* spec, const uint8_t* gate_gguf, c
 int tsp_q8_lanes_quant_offset(uint32_t columns, uint32_t block, uint32_t index, uint64_t* offset);
 int tsp_q8_lanes_pack_rows(uint32_t columns, const uint8_t* original, uint8_t* packed, uint64_t bytes);
 int tsp_q8_lanes_unpack_rows(uint32_t columns, const uint8_t* packed, uint8_t* original, uint64_t bytes);
+
+/* The same for Q5_1 rows (`q51_lanes_v1`): [8-byte block heads d, m, qh x blocks][runs of 16 blocks, 256 B: quant byte i of the
+ * run's blocks side by side]; index < 16. */
+int tsp_q51_lanes_quant_offset(uint32_t columns, uint32_t block, uint32_t index, uint64_t* offset);
+int tsp_q51_lanes_pack_rows(uint32_t columns, const uint8_t* original, uint8_t* packed, uint64_t bytes);
+int tsp_q51_lanes_unpack_rows(uint32_t columns, const uint8_t* packed, uint8_t* original, uint64_t bytes);
 
 /* ------------------------------------------------------------------ host: planners */
 
@@ -317,9 +324,14 @@ int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matrix, uint64_
 
 /* include/tokspur/graph.hpp:750-753 `grouped_mm` (src/graph.mm:4534-4606; kernels/grouped_mm.metal:159-243; route and task
  * preparation kernels/grouped_mpp.metal:12-64): for every route rid = t*selected + slot, output[rid, :] = W[ids[rid]] * x, with x the
- * token's row (broadcast) or row rid of the input. `matrices` is a raw GGUF stack [experts][rows][row bytes] (Q4_K here); token_map,
- * counts and tasks (tile 32) are outputs with the engine's layouts. Activations are used as bf16 values, weights as exact integer
- * factors with f32 block scales, f32 accumulation. workspace: tsp_grouped_mm_workspace_bytes(...) bytes, 256-byte aligned. */
+ * token's row (broadcast) or row rid of the input. `matrices` is an expert stack [experts][rows][row bytes]; token_map, counts and
+ * tasks (tile 32) are outputs with the engine's layouts. Encodings and layouts as src/grouped_mm.cpp:8-12: Q4_K, Q5_K, Q5_1 and
+ * Q8_0 in GGUF rows, Q8_0 in q8_lanes_v1 rows, Q5_1 in q51_lanes_v1 rows (640 columns, more than one expert).
+ *   Q4_K: activations are used as bf16 values, weights as exact integer factors with f32 block scales, f32 accumulation;
+ *   workspace: tsp_grouped_mm_workspace_bytes(...) bytes, 256-byte aligned.
+ *   The others: every weight decoded in f32 and rounded once to half, every activation rounded once to half, f32
+ *   accumulation on the matrix cores (the engine's staging, kernels/grouped_mm.metal:205-216); strides in multiples of 16
+ *   bytes and 16-byte aligned input, as its planner demands; the workspace is not touched. */
 uint64_t tsp_grouped_mm_workspace_bytes(uint32_t tokens, uint32_t selected, uint32_t experts, uint32_t columns, int broadcast);
 int tsp_grouped_mm(uint32_t encoding, uint32_t layout, const void* matrices, uint64_t matrices_bytes, const uint32_t* ids,
                    const float* input, uint64_t input_stride_bytes, float* output, uint64_t output_stride_bytes, uint32_t* token_map,

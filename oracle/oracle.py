@@ -164,6 +164,24 @@ class _Lib:
         _check(self._f("q8_lanes_unpack_rows")(C.c_uint32(columns), _p(packed, _u8p), _p(out, _u8p), C.c_uint64(packed.size)))
         return out
 
+    # ---- q51 lanes ----
+    def q51_lanes_quant_offset(self, columns, block, index):
+        o = C.c_uint64()
+        _check(self._f("q51_lanes_quant_offset")(C.c_uint32(columns), C.c_uint32(block), C.c_uint32(index), C.byref(o)))
+        return o.value
+
+    def q51_lanes_pack_rows(self, columns, original):
+        original = _u8(original)
+        out = np.empty_like(original)
+        _check(self._f("q51_lanes_pack_rows")(C.c_uint32(columns), _p(original, _u8p), _p(out, _u8p), C.c_uint64(original.size)))
+        return out
+
+    def q51_lanes_unpack_rows(self, columns, packed):
+        packed = _u8(packed)
+        out = np.empty_like(packed)
+        _check(self._f("q51_lanes_unpack_rows")(C.c_uint32(columns), _p(packed, _u8p), _p(out, _u8p), C.c_uint64(packed.size)))
+        return out
+
     # ---- top-k ----
     def logit_topk_row(self, logits):
         logits = np.ascontiguousarray(logits, dtype=np.float32)

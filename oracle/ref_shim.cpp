@@ -106,6 +106,22 @@ int ref_q8_lanes_unpack_rows(uint32_t columns, const uint8_t* packed, uint8_t* o
     });
 }
 
+int ref_q51_lanes_quant_offset(uint32_t columns, uint32_t block, uint32_t index, uint64_t* offset) {
+    return guarded([&] { *offset = lanes::packed_quant_offset(lanes::row_layout(7, columns), block, index); });
+}
+int ref_q51_lanes_pack_rows(uint32_t columns, const uint8_t* original, uint8_t* packed, uint64_t nbytes) {
+    return guarded([&] {
+        lanes::pack_rows(lanes::row_layout(7, columns), bytes(original, nbytes),
+                         std::span<std::byte>(reinterpret_cast<std::byte*>(packed), size_t(nbytes)));
+    });
+}
+int ref_q51_lanes_unpack_rows(uint32_t columns, const uint8_t* packed, uint8_t* original, uint64_t nbytes) {
+    return guarded([&] {
+        lanes::unpack_rows(lanes::row_layout(7, columns), bytes(packed, nbytes),
+                           std::span<std::byte>(reinterpret_cast<std::byte*>(original), size_t(nbytes)));
+    });
+}
+
 int ref_logit_topk_row(const float* logits, uint64_t n, void* out528) {
     return guarded([&] {
         const auto row = cpu_logit_topk_row(std::span<const float>(logits, size_t(n)));

@@ -568,6 +568,45 @@ int orc_q8_lanes_unpack_rows(uint32_t columns, const uint8_t* packed, uint8_t* o
     return q8_lanes_rows(columns, packed, original, bytes, 0);
 }
 
+/* src/expert_lanes.cpp:60-119, type 7: [8-byte heads (d, m, qh) x blocks][runs of 16 blocks x 256 B]. */
+int orc_q51_lanes_quant_offset(uint32_t columns, uint32_t block, uint32_t index, uint64_t* offset) {
+    REQUIRE(columns && columns % 32 == 0 && columns <= 65536);
+    const uint32_t blocks = columns / 32;
+    REQUIRE(block < blocks && index < 16);
+    const uint32_t run = block / 16;
+    const uint32_t remaining = blocks - run * 16;
+    const uint32_t width = remaining < 16 ? remaining : 16;
+    *offset = (uint64_t)blocks * 8 + (uint64_t)run * 256 + (uint64_t)index * width + block % 16;
+    return ORC_OK;
+}
+
+static int q51_lanes_rows(uint32_t columns, const uint8_t* in, uint8_t* out, uint64_t bytes, int pack) {
+    REQUIRE(columns && columns % 32 == 0 && columns <= 65536);
+    const uint32_t blocks = columns / 32;
+    const uint64_t row_bytes = (uint64_t)blocks * 24;
+    REQUIRE(bytes && bytes % row_bytes == 0);
+    for (uint64_t row = 0; row < bytes; row += row_bytes) {
+        const uint8_t* src = in + row; uint8_t* dst = out + row;
+        for (uint32_t b = 0; b < blocks; ++b) {
+            if (pack) memcpy(dst + (uint64_t)b * 8, src + (uint64_t)b * 24, 8);
+            else memcpy(dst + (uint64_t)b * 24, src + (uint64_t)b * 8, 8);
+            for (uint32_t i = 0; i < 16; ++i) {
+                uint64_t at;
+                orc_q51_lanes_quant_offset(columns, b, i, &at);
+                if (pack) dst[at] = src[(uint64_t)b * 24 + 8 + i];
+                else dst[(uint64_t)b * 24 + 8 + i] = src[at];
+            }
+        }
+    }
+    return ORC_OK;
+}
+int orc_q51_lanes_pack_rows(uint32_t columns, const uint8_t* original, uint8_t* packed, uint64_t bytes) {
+    return q51_lanes_rows(columns, original, packed, bytes, 1);
+}
+int orc_q51_lanes_unpack_rows(uint32_t columns, const uint8_t* packed, uint8_t* original, uint64_t bytes) {
+    return q51_lanes_rows(columns, packed, original, bytes, 0);
+}
+
 /* ------------------------------------------------------------------------- */
 /* kernels/grouped_mpp.metal:12-37 — per expert, stable compaction over token order. */
 int orc_grouped_routes(const uint32_t* ids, uint32_t experts, uint32_t selected, uint32_t tokens,

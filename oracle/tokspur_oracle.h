@@ -19,7 +19,7 @@
  *   sigmoid/silu        closed-form points; _ref
  *   pack v3             pack_sm16 vs closed form; round trip; planar dequant
  *                       == GGUF dequant to the bit
- *   q8 lanes            bijection + closed-form offset; _ref
+ *   q8 / q51 lanes      bijection + closed-form offset; _ref
  *   grouped routes/tasks  brute force on tiny inputs + invariants
  *   union metadata      row-major specification cases (T=1..8 x S=1..16)
  *   logit top-k         sort-based brute force; _ref
@@ -98,6 +98,10 @@ int orc_pack_coloc_half(const orc_planar_spec* s, const uint8_t* gate_gguf, cons
 int orc_q8_lanes_quant_offset(uint32_t columns, uint32_t block, uint32_t index, uint64_t* offset);
 int orc_q8_lanes_pack_rows(uint32_t columns, const uint8_t* original, uint8_t* packed, uint64_t bytes);
 int orc_q8_lanes_unpack_rows(uint32_t columns, const uint8_t* packed, uint8_t* original, uint64_t bytes);
+/* ---- q51_lanes_v1 row layout: src/expert_lanes.cpp:60-119 (type 7) ---- */
+int orc_q51_lanes_quant_offset(uint32_t columns, uint32_t block, uint32_t index, uint64_t* offset);
+int orc_q51_lanes_pack_rows(uint32_t columns, const uint8_t* original, uint8_t* packed, uint64_t bytes);
+int orc_q51_lanes_unpack_rows(uint32_t columns, const uint8_t* packed, uint8_t* original, uint64_t bytes);
 
 /* ---- expert permutation + prefix-sum offsets: kernels/grouped_mpp.metal:12-64 ---- */
 /* error |= 4 on id >= experts, duplicate expert within one token, off > bound, sum != T*S. */

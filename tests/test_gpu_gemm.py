@@ -158,7 +158,65 @@ def test_grouped_mm_raw_q4k(gpu, tsp, orc, synth, tokens, selected, experts, bro
     assert np.array_equal(scratch["counts"].cpu().numpy().view(np.uint32), want_counts)
     assert np.array_equal(scratch["tasks"].cpu().numpy().view(np.uint32), orc.grouped_tasks(want_counts, experts, selected, tokens, 32)[0])
     with pytest.raises(tsp.FormatError):
-        tsp.grouped_mm(gpu, 8, gpu.upload(w), gpu.upload(ids), gpu.upload(x), cols, rows, experts, selected, tokens, broadcast)
+        tsp.grouped_mm(gpu, 14, gpu.upload(w), gpu.upload(ids), gpu.upload(x), cols, rows, experts, selected, tokens, broadcast)
+
+
+@pytest.mark.parametrize("broadcast", [True, False])
+@pytest.mark.parametrize("encoding,layout,cols", [(8, 0, 544), (8, 1, 544), (8, 1, 1024), (7, 0, 640), (7, 2, 640), (13, 0, 512)])
+def test_grouped_mm_staged_kinds(gpu, tsp, orc, synth, encoding, layout, cols, broadcast):
+    """`grouped_mm` in the engine's other encodings and row layouts (src/grouped_mm.cpp:8-12): Q8_0 and Q5_1 in GGUF rows and in their
+    lane layouts, Q5_K in GGUF rows. Weights and activations are staged as halves (kernels/grouped_mm.metal:205-216), so the result
+    is compared with the reference whose weights are rounded to half, on inputs that are half values already."""
+    rows, experts, selected, tokens = 200, 5, 2, 70  # 200 rows: a ragged last tile of 128; 70 tokens: tasks of 32 routes and tails
+    w = synth.matrix(encoding, 2700 + encoding, rows * experts, cols)
+    stored = w
+    if layout == 1:
+        stored = tsp.q8_lanes_pack_rows(cols, w)
+    elif layout == 2:
+        stored = tsp.q51_lanes_pack_rows(cols, w)
+    rng = np.random.default_rng(cols + encoding)
+    ids = np.stack([rng.permutation(experts)[:selected] for _ in range(tokens)]).astype(np.uint32).reshape(-1)
+    ids[: 40 * selected : selected] = 3  # one expert with more than 32 routes
+    for t in range(40):
+        if ids[t * selected + 1] == 3:
+            ids[t * selected + 1] = 4
+    routes = tokens * selected
+    in_rows = tokens if broadcast else routes
+    x = synth.activations_f32(2701 + cols, (in_rows, cols + 4)).astype(np.float16).astype(np.float32)
+    out = gpu.full((routes, rows + 4), -9.0)
+    got, scratch = tsp.grouped_mm(gpu, encoding, gpu.upload(stored), gpu.upload(ids), gpu.upload(x), cols, rows, experts, selected, tokens, broadcast,
+                                  out=out, x_stride=(cols + 4) * 4, out_stride=(rows + 4) * 4, layout=layout)
+    got = got.cpu().numpy()
+    assert gpu.error() == 0 and (got[:, rows:] == -9.0).all()
+    per_expert = w.size // experts
+    worst_staged = worst_plain = 0.0
+    for e in range(experts):
+        mine = np.nonzero(ids == e)[0]
+        if mine.size == 0:
+            continue
+        xr = x[mine // selected if broadcast else mine, :cols]
+        staged = orc.staged_gemm(encoding, w[e * per_expert:(e + 1) * per_expert], cols, xr, nrows=rows, stage_f16=True)
+        plain = orc.staged_gemm(encoding, w[e * per_expert:(e + 1) * per_expert], cols, xr, nrows=rows, stage_f16=False)
+        for j, rid in enumerate(mine):
+            worst_staged = max(worst_staged, max_rel_error(got[rid, :rows], staged[j]))
+            worst_plain = max(worst_plain, max_rel_error(got[rid, :rows], plain[j]))
+    print(f"grouped_mm encoding {encoding} layout {layout}: vs half-staged reference {worst_staged:.2e}, vs unrounded {worst_plain:.2e}")
+    assert worst_staged <= 1e-4 and worst_plain <= 2e-3
+    want_map, want_counts, _ = orc.grouped_routes(ids, experts, selected, tokens)
+    assert np.array_equal(scratch["counts"].cpu().numpy().view(np.uint32), want_counts)
+    assert np.array_equal(scratch["tasks"].cpu().numpy().view(np.uint32), orc.grouped_tasks(want_counts, experts, selected, tokens, 32)[0])
+    tm = scratch["token_map"].cpu().numpy().view(np.uint32).reshape(experts, tokens)
+    for e in range(experts):
+        assert np.array_equal(tm[e, :want_counts[e]], want_map.reshape(experts, tokens)[e, :want_counts[e]])
+    # a bad id sets the sticky index bit and writes nothing for that route; layouts that do not fit the encoding are refused
+    poisoned = ids.copy()
+    poisoned[5] = experts + 2
+    tsp.grouped_mm(gpu, encoding, gpu.upload(stored), gpu.upload(poisoned), gpu.upload(x), cols, rows, experts, selected, tokens, broadcast,
+                   x_stride=(cols + 4) * 4, layout=layout)
+    assert gpu.error() & 4
+    with pytest.raises(tsp.FormatError):
+        tsp.grouped_mm(gpu, encoding, gpu.upload(stored), gpu.upload(ids), gpu.upload(x), cols, rows, experts, selected, tokens, broadcast,
+                       x_stride=(cols + 4) * 4, layout=2 if encoding == 8 else 1)
 
 
 # ---------------------------------------------------------------------------------- grouped MoE

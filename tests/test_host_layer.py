@@ -111,6 +111,21 @@ def test_q8_lanes_matches_oracle(tsp, orc, synth, cols):
             assert tsp.q8_lanes_quant_offset(cols, b, i) == orc.q8_lanes_quant_offset(cols, b, i)
 
 
+@pytest.mark.parametrize("cols", [32, 640, 2048, 544])
+def test_q51_lanes_matches_oracle(tsp, orc, synth, cols):
+    raw = synth.matrix(7, 72, 3, cols)
+    packed = tsp.q51_lanes_pack_rows(cols, raw)
+    assert np.array_equal(packed, orc.q51_lanes_pack_rows(cols, raw))
+    assert np.array_equal(tsp.q51_lanes_unpack_rows(cols, packed), raw)
+    for b in (0, cols // 32 - 1):
+        for i in (0, 15):
+            assert tsp.q51_lanes_quant_offset(cols, b, i) == orc.q51_lanes_quant_offset(cols, b, i)
+    with pytest.raises(tsp.FormatError):
+        tsp.q51_lanes_quant_offset(cols, 0, 16)
+    with pytest.raises(tsp.FormatError):
+        tsp.q51_lanes_pack_rows(cols, raw[:-1])
+
+
 def test_planners_match_oracle(tsp, orc):
     from oracle.oracle import FormatError as OracleRefusal
     rng = np.random.default_rng(9)

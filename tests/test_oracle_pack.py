@@ -97,6 +97,28 @@ def test_q8_lanes_layout(cpu, synth, cols):
     assert seen == set(range(blocks * 2, blocks * 34))
 
 
+@pytest.mark.parametrize("cols", [32, 640, 2048, 544])
+def test_q51_lanes_layout(cpu, synth, cols):
+    # native/src/expert_lanes.cpp:75-95: 8-byte heads (d, m, qh) first, then runs of 16 blocks x 256 B, byte = index*width + block%16.
+    blocks = cols // 32
+    rows = 3
+    raw = synth.matrix(7, 71, rows, cols)
+    packed = cpu.q51_lanes_pack_rows(cols, raw)
+    assert np.array_equal(cpu.q51_lanes_unpack_rows(cols, packed), raw)
+    seen = set()
+    for b in range(blocks):
+        run, width = b // 16, min(16, blocks - (b // 16) * 16)
+        for i in range(16):
+            at = cpu.q51_lanes_quant_offset(cols, b, i)
+            assert at == blocks * 8 + run * 256 + i * width + b % 16
+            seen.add(at)
+            assert packed[at] == raw[b * 24 + 8 + i]
+        assert np.array_equal(packed[8 * b:8 * b + 8], raw[b * 24:b * 24 + 8])
+    assert seen == set(range(blocks * 8, blocks * 24))
+    # the second row starts a whole row later
+    assert np.array_equal(packed[blocks * 24:blocks * 24 + 8], raw[blocks * 24:blocks * 24 + 8])
+
+
 def brute_routes(ids, experts, selected, tokens):
     token_map = {}
     counts = []

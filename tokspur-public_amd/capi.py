@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(HERE, "libtokspur_hip.so")
 
 OK, ERR_FORMAT, ERR_HIP = 0, 1, 2
 ERRBIT_NONFINITE, ERRBIT_INDEX = 1, 4
-LAYOUT_GGUF, LAYOUT_Q8_LANES_V1, LAYOUT_PLANAR_V3 = 0, 1, 3
+LAYOUT_GGUF, LAYOUT_Q8_LANES_V1, LAYOUT_Q51_LANES_V1, LAYOUT_PLANAR_V3 = 0, 1, 2, 3
 u8p = C.POINTER(C.c_uint8)
 
 
@@ -137,6 +137,26 @@ def q8_lanes_pack_rows(columns, original):
     original = _np_u8(original)
     out = np.empty_like(original)
     check(dll().tsp_q8_lanes_pack_rows(C.c_uint32(columns), original.ctypes.data_as(u8p), out.ctypes.data_as(u8p), C.c_uint64(original.size)))
+    return out
+
+
+def q51_lanes_quant_offset(columns, block, index):
+    o = C.c_uint64()
+    check(dll().tsp_q51_lanes_quant_offset(C.c_uint32(columns), C.c_uint32(block), C.c_uint32(index), C.byref(o)))
+    return o.value
+
+
+def q51_lanes_pack_rows(columns, original):
+    original = _np_u8(original)
+    out = np.empty_like(original)
+    check(dll().tsp_q51_lanes_pack_rows(C.c_uint32(columns), original.ctypes.data_as(u8p), out.ctypes.data_as(u8p), C.c_uint64(original.size)))
+    return out
+
+
+def q51_lanes_unpack_rows(columns, packed):
+    packed = _np_u8(packed)
+    out = np.empty_like(packed)
+    check(dll().tsp_q51_lanes_unpack_rows(C.c_uint32(columns), packed.ctypes.data_as(u8p), out.ctypes.data_as(u8p), C.c_uint64(packed.size)))
     return out
 
 
@@ -447,8 +467,8 @@ def dense_mm_workspace_bytes(tokens, columns):
 
 
 def grouped_mm(dev, encoding, matrices, ids, x, columns, rows, experts, selected, tokens, broadcast, out=None, scratch=None,
-               x_stride=None, out_stride=None):
-    """Raw-GGUF grouped dequant-GEMM (`grouped_mm`): out[rid] = W[ids[rid]] x (x per token when broadcast, else per route)."""
+               x_stride=None, out_stride=None, layout=LAYOUT_GGUF):
+    """Grouped dequant-GEMM over expert stacks (`grouped_mm`): out[rid] = W[ids[rid]] x (x per token when broadcast, else per route)."""
     f = dll().tsp_grouped_mm_workspace_bytes
     f.restype = C.c_uint64
     routes = tokens * selected
@@ -457,7 +477,7 @@ def grouped_mm(dev, encoding, matrices, ids, x, columns, rows, experts, selected
         scratch = {"token_map": dev.zeros(experts * tokens, "int32"), "counts": dev.zeros(experts, "int32"),
                    "tasks": dev.zeros(2 + 2 * (routes // 32 + experts), "int32"),
                    "workspace": dev.empty(f(C.c_uint32(tokens), C.c_uint32(selected), C.c_uint32(experts), C.c_uint32(columns), C.c_int(bool(broadcast))), "uint8")}
-    check(dll().tsp_grouped_mm(C.c_uint32(encoding), C.c_uint32(LAYOUT_GGUF), dev.ptr(matrices), C.c_uint64(dev.nbytes(matrices)), dev.ptr(ids),
+    check(dll().tsp_grouped_mm(C.c_uint32(encoding), C.c_uint32(layout), dev.ptr(matrices), C.c_uint64(dev.nbytes(matrices)), dev.ptr(ids),
                                dev.ptr(x), C.c_uint64(columns * 4 if x_stride is None else x_stride), dev.ptr(out),
                                C.c_uint64(rows * 4 if out_stride is None else out_stride), dev.ptr(scratch["token_map"]), dev.ptr(scratch["counts"]),
                                dev.ptr(scratch["tasks"]), C.c_uint32(columns), C.c_uint32(rows), C.c_uint32(experts), C.c_uint32(selected),

@@ -25,6 +25,7 @@
 //   * For gate/up the two column tiles of a wave are the gate rows and the up rows of the same 32 hidden
 //     units, so SwiGLU is an element-wise epilogue on accumulator registers.
 #include "gate_up_resident.hpp"
+#include "grouped_staged.hpp"
 #include "grouping_device.hpp"
 #include "mfma_quant.hpp"
 
@@ -693,7 +694,37 @@ extern "C" int tsp_grouped_mm(uint32_t encoding, uint32_t layout, const void* ma
                               uint32_t* token_map, uint32_t* counts, uint32_t* tasks, uint32_t columns, uint32_t rows, uint32_t experts,
                               uint32_t selected, uint32_t tokens, int broadcast, void* workspace, uint64_t workspace_bytes,
                               uint32_t* error_word, void* stream) {
-    TSP_REQUIRE(encoding == 12 && layout == TSP_LAYOUT_GGUF, "grouped dequant-GEMM on the matrix cores takes raw GGUF Q4_K expert stacks");
+    if (grouped_staged_takes(encoding, layout)) {
+        // src/grouped_mm.cpp:24-47: the planner's geometry and byte spans decide; the routes, counts and 32-route tasks are written for
+        // the caller as in the Q4_K arm, and the staged kernel reads that task list itself (the workspace is not used)
+        tsp_grouped_mm_plan_t plan;
+        const int planned = tsp_grouped_mm_plan(encoding, layout, columns, rows, experts, selected, tokens, input_stride_bytes, output_stride_bytes,
+                                                broadcast, 1, &plan);
+        if (planned != TSP_OK) return planned;
+        TSP_REQUIRE(matrices && ids && input && output && token_map && counts && tasks && error_word, "null device pointer");
+        TSP_REQUIRE(matrices_bytes == plan.matrix_bytes && plan.args.expert_stride_bytes < (1ull << 32), "grouped prefill matrix byte span mismatch");
+        TSP_REQUIRE(reinterpret_cast<uintptr_t>(matrices) % 16 == 0 && reinterpret_cast<uintptr_t>(input) % 16 == 0 && reinterpret_cast<uintptr_t>(output) % 4 == 0,
+                    "grouped prefill buffer span or alignment is invalid");
+        const void* ins[] = {matrices, ids, input};
+        const uint64_t in_bytes[] = {matrices_bytes, plan.indices_bytes, plan.input_bytes};
+        const void* outs[] = {output, token_map, counts, tasks};
+        const uint64_t out_bytes[] = {plan.output_bytes, plan.token_map_bytes, plan.counts_bytes, plan.tasks_bytes};
+        for (int o = 0; o < 4; ++o) {
+            for (int i = 0; i < 3; ++i) TSP_REQUIRE(!ranges_overlap(outs[o], out_bytes[o], ins[i], in_bytes[i]), "grouped prefill outputs overlap inputs");
+            for (int q = 0; q < o; ++q) TSP_REQUIRE(!ranges_overlap(outs[o], out_bytes[o], outs[q], out_bytes[q]), "grouped prefill outputs overlap each other");
+        }
+        int rc = tsp_grouped_routes(ids, token_map, counts, experts, selected, tokens, error_word, stream);
+        if (rc == TSP_OK) rc = tsp_grouped_tasks(counts, tasks, experts, selected, tokens, 32, error_word, stream);
+        if (rc != TSP_OK) return rc;
+        GroupedStagedArgs g{};
+        g.matrices = static_cast<const uint8_t*>(matrices); g.input = input; g.output = output;
+        g.expert_stride = plan.args.expert_stride_bytes; g.input_stride = input_stride_bytes; g.output_stride = output_stride_bytes;
+        g.columns = columns; g.rows = rows; g.row_bytes = plan.args.row_bytes; g.experts = experts; g.selected = selected; g.tokens = tokens;
+        g.broadcast = broadcast ? 1 : 0; g.maximum_tasks = plan.args.maximum_tasks;
+        g.ids = ids; g.token_map = token_map; g.counts = counts; g.tasks = tasks; g.error_word = error_word;
+        return launch_grouped_staged(encoding, layout, g, static_cast<hipStream_t>(stream));
+    }
+    TSP_REQUIRE(encoding == 12 && layout == TSP_LAYOUT_GGUF, "grouped dequant-GEMM takes Q4_K, Q5_K, Q5_1 and Q8_0 expert stacks in GGUF rows, Q8_0 in q8_lanes_v1 and Q5_1 in q51_lanes_v1 rows");
     TSP_REQUIRE(columns && columns <= 65536 && columns % 256 == 0 && rows && rows <= 32768 && experts >= 1 && experts <= 512 &&
                     selected >= 1 && selected <= 16 && selected <= experts && tokens >= 1 && tokens <= 2048,
                 "grouped prefill geometry mismatch");

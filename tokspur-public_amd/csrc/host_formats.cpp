@@ -218,6 +218,47 @@ int tsp_q8_lanes_unpack_rows(uint32_t columns, const uint8_t* packed, uint8_t* o
     return q8_lanes_move(columns, packed, original, bytes, false);
 }
 
+int tsp_q51_lanes_quant_offset(uint32_t columns, uint32_t block, uint32_t index, uint64_t* offset) {
+    TSP_REQUIRE(columns && columns % 32 == 0 && columns <= 65536, "Q5_1 lane layout needs whole 32-element blocks");
+    const uint32_t blocks = columns / 32;
+    TSP_REQUIRE(block < blocks && index < 16, "lane layout block/quant bound");
+    const uint32_t run = block / 16, width = std::min(16u, blocks - run * 16);
+    *offset = uint64_t(blocks) * 8 + uint64_t(run) * 256 + uint64_t(index) * width + block % 16;
+    return TSP_OK;
+}
+
+namespace {
+int q51_lanes_move(uint32_t columns, const uint8_t* in, uint8_t* out, uint64_t bytes, bool pack) {
+    TSP_REQUIRE(columns && columns % 32 == 0 && columns <= 65536, "Q5_1 lane layout needs whole 32-element blocks");
+    const uint32_t blocks = columns / 32;
+    const uint64_t row_bytes = uint64_t(blocks) * 24;
+    TSP_REQUIRE(bytes && bytes % row_bytes == 0, "lane layout needs whole rows");
+    TSP_REQUIRE(!ranges_overlap(in, bytes, out, bytes), "lane layout input and output overlap");
+    for (uint64_t row = 0; row < bytes; row += row_bytes) {
+        const uint8_t* src = in + row; uint8_t* dst = out + row;
+        for (uint32_t b = 0; b < blocks; ++b) {
+            const uint32_t run = b / 16, width = std::min(16u, blocks - run * 16);
+            const uint64_t base = uint64_t(blocks) * 8 + uint64_t(run) * 256 + b % 16;
+            if (pack) {
+                std::memcpy(dst + 8 * b, src + 24 * b, 8);
+                for (uint32_t i = 0; i < 16; ++i) dst[base + uint64_t(i) * width] = src[24 * b + 8 + i];
+            } else {
+                std::memcpy(dst + 24 * b, src + 8 * b, 8);
+                for (uint32_t i = 0; i < 16; ++i) dst[24 * b + 8 + i] = src[base + uint64_t(i) * width];
+            }
+        }
+    }
+    return TSP_OK;
+}
+}  // namespace
+
+int tsp_q51_lanes_pack_rows(uint32_t columns, const uint8_t* original, uint8_t* packed, uint64_t bytes) {
+    return q51_lanes_move(columns, original, packed, bytes, true);
+}
+int tsp_q51_lanes_unpack_rows(uint32_t columns, const uint8_t* packed, uint8_t* original, uint64_t bytes) {
+    return q51_lanes_move(columns, packed, original, bytes, false);
+}
+
 // ---------------------------------------------------------------- planners
 
 namespace {

@@ -602,7 +602,7 @@ void HipGraph::prepare_grouped_mm(uint32_t encoding, PrefillWeightLayout layout,
     impl_->idle();
     require(grouped_mm_takes(encoding, layout), "grouped prefill requires idle preparation and direct batches");
     require(max_tokens >= 1 && max_tokens <= 2048 && max_selected >= 1 && max_selected <= 16 && max_experts >= 1 && max_experts <= 512 &&
-                max_columns >= 256 && max_columns <= 65536,
+                max_columns >= 32 && max_columns <= 65536,
             "grouped prefill geometry mismatch");
     const uint64_t bytes = tsp_grouped_mm_workspace_bytes(max_tokens, max_selected, max_experts, (max_columns + 255) / 256 * 256, 0);
     impl_->grow(impl_->grouped_workspace, impl_->grouped_workspace_bytes, bytes);
@@ -737,7 +737,11 @@ void release_moe_scratch(HipGraph& graph, const MoeScratch& scratch) {
     for (const auto view : scratch.views()) graph.release(view);
 }
 
-bool grouped_mm_takes(uint32_t encoding, PrefillWeightLayout layout) { return encoding == 12 && layout == PrefillWeightLayout::gguf; }
+// src/grouped_mm.cpp:8-12 `layout_check`
+bool grouped_mm_takes(uint32_t encoding, PrefillWeightLayout layout) {
+    if (layout == PrefillWeightLayout::gguf) return encoding == 7 || encoding == 8 || encoding == 12 || encoding == 13;
+    return (layout == PrefillWeightLayout::q8_lanes_v1 && encoding == 8) || (layout == PrefillWeightLayout::q51_lanes_v1 && encoding == 7);
+}
 
 bool is_planar_moe(const HipGraph& g, const MoeWeights& w, MoeShape s) {
     const auto lo = g.planar_matrix_shape(w.gate.view);
@@ -871,10 +875,10 @@ void release_moe_mm_many_scratch(HipGraph& graph, const MoeMmManyScratch& scratc
 }
 
 namespace {
-// The raw-GGUF arm runs its three grouped products on the matrix cores, which unpack Q4_K expert stacks in GGUF rows.
+// The raw-GGUF arm runs three grouped products: each takes what `grouped_mm` takes (Q4_K, Q5_K, Q5_1, Q8_0 rows and the two lane layouts).
 void raw_arm_check(const MoeWeights& w, const MoeMmLayouts& l) {
     for (const auto& [matrix, layout] : {std::pair{w.gate, l.gate}, std::pair{w.up, l.up}, std::pair{w.down, l.down}})
-        require(grouped_mm_takes(matrix.encoding, layout), "tiled MoE raw-GGUF experts: grouped prefill takes Q4_K expert stacks in GGUF rows");
+        require(grouped_mm_takes(matrix.encoding, layout), "grouped mm layout/encoding mismatch");
 }
 }  // namespace
 
