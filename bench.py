@@ -317,6 +317,20 @@ def main():
             fl = 2.0 * m * C * 8192
             configs[f"c1_dense_gemm_m{m}"] = {"tok_per_s": m / (ms * 1e-3), "ms": ms, "tflops": fl / (ms * 1e-3) / 1e12,
                                               "mfma_frac": fl / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS}
+        # config 3 with the engine's own down kind: Q4_K co-located gate/up (the same tensors) and Q8_0 planes down (kind 9), whose
+        # weights the down kernel decodes to halves on the fly
+        down8 = synth.matrix(8, synth.tensor_seed(3, 13), C * E, H)
+        w8 = capi.PlanarMoeWeights(gpu, 12, 8, C, H, E, gate, up, down8)
+        del down8
+
+        def routed_q8_down():
+            capi.planar_nax_grouped_moe(gpu, w8, ids, d_x, T, S, scratch, y=y)
+
+        gpu.route(d_logits, S, 0, True, tokens=T, out=(ids, wts))  # the headline's routes again (the sublayer drew its own)
+        ms = timed(torch, routed_q8_down, k2, 2)
+        configs["c3_routed_q4k_gate_up_q8_down"] = {"ms": ms, "tok_per_s": T / (ms * 1e-3),
+                                                    "kernels_us": {k: round(v["avg_us"], 2) for k, v in profiled(capi, torch, routed_q8_down, 5).items()}}
+        del w8
         # config 0: dense Q4_K GEMV over a rotation of distinct weight copies (> 512 MB) so every read comes from HBM
         w0 = synth.matrix(12, synth.tensor_seed(0, 1), 4096, C)
         x0, y0 = gpu.upload(synth.activations_f32(synth.tensor_seed(0, 2), C)), gpu.empty(4096)

@@ -838,10 +838,10 @@ static void* moe_worker(void* arg) {
         for (uint32_t r = 0; r < j->hidden; ++r) {
             double dg = 0, du = 0;
             if (orc_dequantize(j->gu_type, j->gate + ((uint64_t)e * j->hidden + r) * gu_row, gu_row, wrow, j->channels)) goto done;
-            if (j->stage_bf16 & 2) for (uint32_t c = 0; c < j->channels; ++c) wrow[c] = orc_round_f16(wrow[c]);
+            if (j->stage_bf16 & (2 | 16)) for (uint32_t c = 0; c < j->channels; ++c) wrow[c] = orc_round_f16(wrow[c]);
             for (uint32_t c = 0; c < j->channels; ++c) dg += (double)wrow[c] * xs[c];
             if (orc_dequantize(j->gu_type, j->up + ((uint64_t)e * j->hidden + r) * gu_row, gu_row, wrow, j->channels)) goto done;
-            if (j->stage_bf16 & 2) for (uint32_t c = 0; c < j->channels; ++c) wrow[c] = orc_round_f16(wrow[c]);
+            if (j->stage_bf16 & (2 | 16)) for (uint32_t c = 0; c < j->channels; ++c) wrow[c] = orc_round_f16(wrow[c]);
             for (uint32_t c = 0; c < j->channels; ++c) du += (double)wrow[c] * xs[c];
             if (j->silu_f32) h[r] = silu_f32((float)dg) * (float)du;
             else { double s; orc_stable_silu(dg, &s); h[r] = s * du; }
@@ -852,7 +852,7 @@ static void* moe_worker(void* arg) {
         if (j->down && j->down_out) for (uint32_t r = 0; r < j->channels; ++r) {
             double dd = 0;
             if (orc_dequantize(j->dn_type, j->down + ((uint64_t)e * j->channels + r) * dn_row, dn_row, wrow, j->hidden)) goto done;
-            if (j->stage_bf16 & 2) for (uint32_t c = 0; c < j->hidden; ++c) wrow[c] = orc_round_f16(wrow[c]);
+            if (j->stage_bf16 & (2 | 32)) for (uint32_t c = 0; c < j->hidden; ++c) wrow[c] = orc_round_f16(wrow[c]);
             if ((j->stage_bf16 & 8) && j->dn_type == 14) stage_q6k_products(j->down + ((uint64_t)e * j->channels + r) * dn_row, wrow, j->hidden);
             for (uint32_t c = 0; c < j->hidden; ++c) dd += (double)wrow[c] * h[c];
             j->down_out[(uint64_t)rid * j->channels + r] = dd;

@@ -169,7 +169,8 @@ float orc_round_f16(float v);
  * other types unchanged).
  * `stage` in orc_moe_routed_reference: bit 0 = activations and h as bf16 (kernels/planar_moe_v3.metal:82-94,
  * 2406-2483), bit 1 = weights as half, bit 2 = activations as bf16 and h as 256 * half(h / 256), bit 3 = Q6_K
- * down rows staged as under stage_f16 = 2. Bits 2 and 3 describe the HIP kernels, not the reference. */
+ * down rows staged as under stage_f16 = 2, bit 4 = gate and up weights as half, bit 5 = down weights as half (bit 1 for one
+ * product only). Bits 2 to 5 describe the HIP kernels, not the reference. */
 int orc_staged_gemm(uint32_t type, const uint8_t* matrix, uint32_t columns, const uint32_t* rows_sel, uint32_t nsel,
                     const float* x, uint64_t x_stride_floats, uint32_t tokens, int stage_f16, double* out, uint32_t threads);
 

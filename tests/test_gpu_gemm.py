@@ -427,35 +427,49 @@ def test_grouped_moe_exact_when_products_fit_half(gpu, tsp, orc, synth):
     assert max_rel_error(y, carried) <= 2e-3 and nmse(y, carried) <= 1e-7 and nmse(y, plain) <= 1e-6
 
 
-@pytest.mark.parametrize("gu_type,dn_type", [(13, 7), (8, 8), (12, 8), (13, 14)])
-def test_grouped_moe_other_planar_kinds(gpu, tsp, orc, synth, gu_type, dn_type):
-    """The planar kinds of include/tokspur/moe.hpp:27-29 that the matrix-core kernels do not unpack (Q5_K / Q8_0 gate and
-    up, Q5_1 / Q8_0 down) go through the grouped entry point as well, eight tokens at a time on the f32 kernels: same
-    token_map / counts / tasks, expert_down rows within the GEMV bound of the unrounded reference."""
-    channels, hidden, experts, selected, n = 256, 256, 6, 3, 29
+@pytest.mark.parametrize("gu_type,dn_type,channels,hidden", [(13, 7, 256, 256), (8, 8, 256, 256), (12, 8, 256, 256), (13, 14, 256, 256), (12, 7, 512, 160),
+                                                             (8, 7, 96, 64), (8, 14, 160, 256)])
+def test_grouped_moe_other_planar_kinds(gpu, tsp, orc, synth, gu_type, dn_type, channels, hidden):
+    """The planar kinds of include/tokspur/moe.hpp:27-29 beside Q4_K gate/up and Q6_K down (Q5_K / Q8_0 gate and up, Q5_1 / Q8_0
+    down) run on the matrix cores as well, their weights decoded to halves on the fly; any gate/up kind combines with any down
+    kind. Same token_map / counts / tasks; expert_down rows against the reference with the declared staging: activations as
+    bf16 values, h as 256 * half(h / 256), weights of the staged kinds rounded to half (Q4_K / Q6_K keep their integer factors)."""
+    experts, selected, n = 6, 3, 75  # an expert with more than 64 routes, one with more than 32, ragged tails
     gate = synth.matrix(gu_type, 3301, hidden * experts, channels)
     up = synth.matrix(gu_type, 3302, hidden * experts, channels)
     down = synth.matrix(dn_type, 3303, channels * experts, hidden)
     w = tsp.PlanarMoeWeights(gpu, gu_type, dn_type, channels, hidden, experts, gate, up, down)
     rng = np.random.default_rng(11)
-    ids = np.stack([rng.permutation(experts)[:selected] for _ in range(n)]).astype(np.uint32).reshape(-1)
-    x = synth.activations_f32(3304, (n, channels))
+    ids = np.stack([rng.permutation(experts)[:selected] for _ in range(n)]).astype(np.uint32)
+    for t in range(70):  # expert 0 in slot 0 of seventy tokens
+        row = ids[t]
+        if 0 in row[1:]:
+            row[list(row).index(0)] = row[0]
+        row[0] = 0
+    ids = ids.reshape(-1)
+    x = synth.round_bf16(synth.activations_f32(3304, (n, channels)))
     scratch = tsp.GroupedScratch(gpu, n, selected, experts, channels, hidden)
     y = tsp.planar_nax_grouped_moe(gpu, w, gpu.upload(ids), gpu.upload(x), n, selected, scratch).cpu().numpy()
     assert gpu.error() == 0
     want_map, want_counts, _ = orc.grouped_routes(ids, experts, selected, n)
     counts = scratch.counts.cpu().numpy().view(np.uint32)
-    assert np.array_equal(counts, want_counts)
+    assert np.array_equal(counts, want_counts) and counts[0] >= 70
     tm = scratch.token_map.cpu().numpy().view(np.uint32).reshape(experts, n)
     for e in range(experts):
         assert np.array_equal(tm[e, :counts[e]], want_map.reshape(experts, n)[e, :counts[e]])
     assert np.array_equal(scratch.tasks.cpu().numpy().view(np.uint32), orc.grouped_tasks(want_counts, experts, selected, n, 32)[0])
-    # Q6_K down rows take the matrix-core GEMV for at most eight rows, whose integer products above 2048 lose their lowest bit
-    # (stage bit 3 of the reference restates that); every other kind is decoded and accumulated in f32
-    _, want = orc.moe_routed_reference(gu_type, dn_type, gate, up, down, channels, hidden, experts, ids, n, selected, x,
-                                       stage=8 if dn_type == 14 else 0, threads=8)
+    # stage bits of the reference restatement: 4 = activations as bf16 and h as 256 * half(h / 256), 16 / 32 = gate and up / down
+    # weights as halves (the kinds decoded on the fly; Q4_K and Q6_K keep their integer factors), 8 = Q6_K integer products
+    # above 2048 lose their lowest bit on the matrix cores
+    stage = 4 | (0 if gu_type == 12 else 16) | (8 if dn_type == 14 else 32)
+    _, want = orc.moe_routed_reference(gu_type, dn_type, gate, up, down, channels, hidden, experts, ids, n, selected, x, stage=stage, threads=8)
     _, plain = orc.moe_routed_reference(gu_type, dn_type, gate, up, down, channels, hidden, experts, ids, n, selected, x, stage=0, threads=8)
-    assert max_rel_error(y, want) <= 5e-5 and nmse(y, want) <= 1e-10 and max_rel_error(y, plain) <= 2e-3 and nmse(y, plain) <= 1e-6
+    print(f"planar kinds ({gu_type}, {dn_type}) {channels}x{hidden}: vs declared staging {max_rel_error(y, want):.2e} (NMSE {nmse(y, want):.2e}), "
+          f"vs unrounded {max_rel_error(y, plain):.2e} (NMSE {nmse(y, plain):.2e})")
+    # against the unrounded reference the half staging of the weights shows (2^-11 per weight, twice over the two products)
+    assert max_rel_error(y, want) <= 1e-3 and nmse(y, want) <= 1e-9 and max_rel_error(y, plain) <= 1e-2 and nmse(y, plain) <= 1e-5
+    again = tsp.planar_nax_grouped_moe(gpu, w, gpu.upload(ids), gpu.upload(x), n, selected, scratch).cpu().numpy()
+    assert np.array_equal(y.view(np.uint32), again.view(np.uint32))
 
 
 def test_grouped_moe_sticky_errors(gpu, tsp, synth):

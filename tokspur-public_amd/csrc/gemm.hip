@@ -27,6 +27,7 @@
 #include "gate_up_resident.hpp"
 #include "grouped_staged.hpp"
 #include "grouping_device.hpp"
+#include "planar_staged.hpp"
 #include "mfma_quant.hpp"
 
 #include <type_traits>
@@ -832,10 +833,14 @@ extern "C" int tsp_planar_nax_grouped_moe_shared(const tsp_grouped_moe* m, const
 namespace {
 int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void* stream) {
     TSP_REQUIRE(m, "null grouped MoE description");
-    const bool matrix_cores = m->gate_kind == TSP_KIND_Q4K_COLOC_GATE && m->up_kind == TSP_KIND_Q4K_COLOC_UP && m->down_kind == TSP_KIND_Q6K_PLANAR_X;
+    const bool fast_gate_up = m->gate_kind == TSP_KIND_Q4K_COLOC_GATE && m->up_kind == TSP_KIND_Q4K_COLOC_UP;
+    const bool fast_down = m->down_kind == TSP_KIND_Q6K_PLANAR_X;
+    const bool matrix_cores = (fast_gate_up || planar_staged_gate_up_takes(m->gate_kind, m->up_kind)) && (fast_down || planar_staged_down_takes(m->down_kind));
+    // columns of the K kinds come in super-blocks of 256, those of Q5_1 / Q8_0 in blocks of 32; hidden units in multiples of 32
+    const uint32_t channel_step = (m->gate_kind == TSP_KIND_Q8_COLOC_GATE) ? 32u : 256u, hidden_step = fast_down ? 256u : 32u;
     TSP_REQUIRE(m->tokens >= 1 && m->tokens <= 2048 && m->selected >= 1 && m->selected <= 16 && m->selected <= m->experts &&
-                    m->experts >= 2 && m->experts <= 512 && m->experts % 2 == 0 && m->channels % 256 == 0 && m->hidden % 256 == 0 &&
-                    m->channels <= 65536 && m->hidden <= 65536,
+                    m->experts >= 2 && m->experts <= 512 && m->experts % 2 == 0 && m->channels && m->hidden && m->channels % channel_step == 0 &&
+                    m->hidden % hidden_step == 0 && m->channels <= 65536 && m->hidden <= 65536,
                 "planar v3 NAX grouped MoE shape or stride mismatch");
     TSP_REQUIRE(m->x_stride_bytes >= uint64_t(m->channels) * 4 && m->x_stride_bytes % 4 == 0 &&
                     m->y_stride_bytes >= uint64_t(m->channels) * 4 && m->y_stride_bytes % 4 == 0,
@@ -843,7 +848,7 @@ int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void*
     TSP_REQUIRE(m->pair_lo && m->pair_hi && m->down && m->ids && m->x && m->y && m->token_map && m->counts && m->tasks &&
                     m->workspace && m->error_word,
                 "null device pointer");
-    TSP_REQUIRE(!shared || matrix_cores, "the always-on expert rides only with Q4_K co-located gate/up and Q6_K planes down");
+    TSP_REQUIRE(!shared || (fast_gate_up && fast_down), "the always-on expert rides only with Q4_K co-located gate/up and Q6_K planes down");
     if (!matrix_cores) {
         const NaxLayout lay = nax_layout(m->tokens, m->selected, m->experts, m->channels, m->hidden);
         TSP_REQUIRE(m->workspace_bytes >= lay.total && reinterpret_cast<uintptr_t>(m->workspace) % 256 == 0,
@@ -851,8 +856,10 @@ int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void*
         return grouped_moe_in_eights(m, lay, stream);  // kinds, spans and overlaps are checked per chunk
     }
     tsp_planar_spec gu, dn;
-    int rc = tsp_make_expert_spec(12, m->channels, m->hidden, &gu);
-    if (rc == TSP_OK) rc = tsp_make_expert_spec(14, m->hidden, m->channels, &dn);
+    const uint32_t gate_up_type = fast_gate_up ? 12u : m->gate_kind == TSP_KIND_Q5K_COLOC_GATE ? 13u : 8u;
+    const uint32_t down_type = fast_down ? 14u : m->down_kind == TSP_KIND_Q51_PLANAR ? 7u : 8u;
+    int rc = tsp_make_expert_spec(gate_up_type, m->channels, m->hidden, &gu);
+    if (rc == TSP_OK) rc = tsp_make_expert_spec(down_type, m->hidden, m->channels, &dn);
     if (rc != TSP_OK) return rc;
     TSP_REQUIRE(gu.planar_expert_bytes < (1ull << 32) && dn.planar_expert_bytes < (1ull << 32),
                 "planar v3 grouped MoE addresses weight rows with 32-bit offsets: one expert must be under 4 GiB");
@@ -900,9 +907,17 @@ int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void*
     auto* hbuf = reinterpret_cast<_Float16*>(ws + l.hbuf);
 
     rc = tsp_grouped_routes(m->ids, m->token_map, m->counts, m->experts, m->selected, m->tokens, m->error_word, stream);
+    // only the Q4_K gate/up kernels want the activation sums and the column order that goes with them
     if (rc == TSP_OK) rc = lists_and_rows(TaskLists{m->counts, m->tasks, 32, task_list, kTaskRows, m->experts, m->selected, m->tokens, shared != nullptr, reinterpret_cast<uint32_t*>(ws + l.classes)}, m->x,
-                                          m->x_stride_bytes, xh, sx, m->tokens, m->channels, m->error_word, s);
+                                          m->x_stride_bytes, xh, fast_gate_up ? sx : nullptr, m->tokens, m->channels, m->error_word, s);
     if (rc != TSP_OK) return rc;
+
+    PlanarStagedArgs staged{};
+    staged.xh = xh; staged.pair_lo = static_cast<const uint8_t*>(m->pair_lo); staged.pair_hi = static_cast<const uint8_t*>(m->pair_hi);
+    staged.down = static_cast<const uint8_t*>(m->down); staged.spec = gu; staged.down_spec = dn;
+    staged.channels = m->channels; staged.hidden = m->hidden; staged.experts = m->experts; staged.selected = m->selected; staged.tokens = m->tokens;
+    staged.task_list = task_list; staged.task_slots = l.bound; staged.counts = m->counts; staged.token_map = m->token_map; staged.ids = m->ids;
+    staged.hbuf = hbuf; staged.y = m->y; staged.y_stride = m->y_stride_bytes; staged.error_word = m->error_word;
 
     GemmArgs g{};
     g.a = xh; g.a_stride = m->channels; g.sx = sx; g.w0 = static_cast<const uint8_t*>(m->pair_lo); g.w1 = static_cast<const uint8_t*>(m->pair_hi);
@@ -910,7 +925,9 @@ int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void*
     g.tokens = m->tokens; g.selected = m->selected; g.n = m->hidden; g.k = m->channels; g.out = hbuf; g.out_scale = 1.0f;
     g.error_word = m->error_word;
     if (shared) { g.shared_w0 = static_cast<const uint8_t*>(shared->gate); g.shared_w1 = static_cast<const uint8_t*>(shared->up); }
-    if (resident_gate_up_takes(m->channels, m->hidden)) {
+    if (!fast_gate_up) {
+        rc = launch_planar_staged_gate_up(staged, s);
+    } else if (resident_gate_up_takes(m->channels, m->hidden)) {
         ResidentGateUpArgs r{};
         r.xh = xh; r.sx = sx; r.pair_lo = g.w0; r.pair_hi = g.w1; r.shared_gate = g.shared_w0; r.shared_up = g.shared_w1; r.spec = gu;
         r.experts = m->experts; r.tokens = m->tokens; r.selected = m->selected; r.hidden = m->hidden;
@@ -921,6 +938,7 @@ int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void*
         rc = launch<B_Q4K_PLANAR, EPI_SWIGLU, ROWS_GATHER_TOKENS>(g, (m->hidden + 127) / 128, l.bound, s);
     }
     if (rc != TSP_OK) return rc;
+    if (!fast_down) return launch_planar_staged_down(staged, s);
 
     GemmArgs d{};
     d.a = hbuf; d.a_stride = m->hidden; d.w0 = static_cast<const uint8_t*>(m->down); d.spec = dn; d.experts = m->experts;
