@@ -239,6 +239,30 @@ int tsp_mixture_batch(const float* expert_outputs, const float* weights, const f
 /* include/tokspur/graph.hpp:990 `swiglu` (kernels/graph.metal:312-326): out = silu(gate*scale) * up. */
 int tsp_swiglu(const float* gate, const float* up, float* output, uint64_t count, float scale, uint32_t* error_word, void* stream);
 
+/* ------------------------------------------------------------------ device: the f32 operators around the sublayer */
+
+/* include/tokspur/graph.hpp:983 `rms` (src/graph.mm:7399-7409; kernels/graph.metal:222-247): independent groups of `group_width`
+ * values, out = x * rsqrt(mean(x^2) + epsilon) * gain; `gains` holds one gain per element, or `group_width` gains shared by
+ * every group (shared_gains). A non-finite sum or result sets TSP_ERRBIT_NONFINITE and is not stored. */
+int tsp_rms(const float* input, const float* gains, float* output, uint64_t count, uint32_t group_width, int shared_gains, float epsilon,
+            uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:984 `rms_sigmoid_gate` (kernels/graph.metal:249-282): the same times sigmoid(gate), in one pass. */
+int tsp_rms_sigmoid_gate(const float* input, const float* gains, const float* gate, float* output, uint64_t count, uint32_t group_width,
+                         int shared_gains, float epsilon, uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:985 `activate` (kernels/graph.metal:284-300): out = f(scale * x), kind 0 identity, 1 SiLU, 2 sigmoid,
+ * 3 softplus (include/tokspur/graph.hpp:134 `Activation`); may run in place. */
+int tsp_activate(const float* input, float* output, uint64_t count, uint32_t kind, float scale, uint32_t* error_word, void* stream);
+/* include/tokspur/graph.hpp:986 `multiply` (kernels/graph.metal:302-311): out = x * gate, or x * sigmoid(gate). */
+int tsp_multiply(const float* input, const float* gate, float* output, uint64_t count, int sigmoid_gate, uint32_t* error_word, void* stream);
+/* `residual_read` (src/graph.mm:7715-7725; kernels/graph.metal:330-351): output[c] = mean over branches of
+ * normalized[b, c] * sigmoid(scores[b, c]); scales[b] = 2 sigmoid(inject[b] / branches). At most 64 branches of 65536 channels. */
+int tsp_residual_read(const float* normalized, const float* scores, const float* inject, float* output, float* scales, uint32_t branches,
+                      uint32_t channels, uint32_t* error_word, void* stream);
+/* `residual_write` (src/graph.mm:7726-7734; kernels/graph.metal:353-361): output[b, c] = streams[b, c] + scales[b] * input[c];
+ * output may be the streams themselves. */
+int tsp_residual_write(const float* streams, const float* input, const float* scales, float* output, uint32_t branches, uint32_t channels,
+                       uint32_t* error_word, void* stream);
+
 /* ------------------------------------------------------------------ device: expert permutation */
 
 /* kernels/grouped_mpp.metal:12-37 `graph_grouped_routes` (encoded inside `grouped_mm`, src/graph.mm:4571,

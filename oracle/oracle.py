@@ -126,6 +126,30 @@ class _Lib:
     def stable_softplus(self, v):
         return self._scalar("stable_softplus", v)
 
+    # ---- operators around the sublayer ----
+    def group_rms_reference(self, x, gains, group_width, epsilon):
+        x = np.ascontiguousarray(x, dtype=np.float64).reshape(-1)
+        gains = np.ascontiguousarray(gains, dtype=np.float64).reshape(-1)
+        out = np.empty_like(x)
+        _check(self._f("group_rms_reference")(_p(x, _f64p), _p(gains, _f64p), C.c_uint64(x.size), C.c_uint64(group_width), C.c_double(epsilon), _p(out, _f64p)))
+        return out
+
+    def gated_residual_reference(self, streams, gains, down, up, inject, branches, channels, rank, epsilon):
+        arrays = [np.ascontiguousarray(a, dtype=np.float64).reshape(-1) for a in (streams, gains, down, up, inject)]
+        read, scales = np.empty(channels, dtype=np.float64), np.empty(branches, dtype=np.float64)
+        _check(self._f("gated_residual_reference")(*[_p(a, _f64p) for a in arrays], C.c_uint64(branches), C.c_uint64(channels), C.c_uint64(rank),
+                                                   C.c_double(epsilon), _p(read, _f64p), _p(scales, _f64p)))
+        return read, scales
+
+    def residual_write_reference(self, streams, output, scales):
+        streams = np.ascontiguousarray(streams, dtype=np.float64).reshape(-1)
+        output = np.ascontiguousarray(output, dtype=np.float64).reshape(-1)
+        scales = np.ascontiguousarray(scales, dtype=np.float64).reshape(-1)
+        result = np.empty_like(streams)
+        _check(self._f("residual_write_reference")(_p(streams, _f64p), _p(output, _f64p), _p(scales, _f64p), C.c_uint64(scales.size), C.c_uint64(output.size),
+                                                   _p(result, _f64p)))
+        return result
+
     # ---- routing ----
     def route_reference(self, logits, selected, mode=0, normalize=True):
         logits = np.ascontiguousarray(logits, dtype=np.float64)

@@ -69,6 +69,30 @@ int ref_q8_many_chunks(uint32_t rows, uint32_t* chunks) { return guarded([&] { *
 int ref_stable_sigmoid(double v, double* out) { return guarded([&] { *out = stable_sigmoid(v); }); }
 int ref_stable_silu(double v, double* out) { return guarded([&] { *out = stable_silu(v); }); }
 int ref_stable_softplus(double v, double* out) { return guarded([&] { *out = stable_softplus(v); }); }
+int ref_group_rms_reference(const double* input, const double* gains, uint64_t count, uint64_t group_width, double epsilon, double* output) {
+    return guarded([&] {
+        const auto r = group_rms_reference(std::span<const double>(input, size_t(count)), std::span<const double>(gains, size_t(count)), size_t(group_width), epsilon);
+        std::copy(r.begin(), r.end(), output);
+    });
+}
+int ref_gated_residual_reference(const double* streams, const double* gains, const double* down, const double* up, const double* inject,
+                                 uint64_t branches, uint64_t channels, uint64_t rank, double epsilon, double* read, double* write_scales) {
+    return guarded([&] {
+        const size_t width = size_t(branches * channels);
+        const auto r = gated_residual_reference(std::span<const double>(streams, width), std::span<const double>(gains, width),
+                                                std::span<const double>(down, width * size_t(rank)), std::span<const double>(up, width * size_t(rank)),
+                                                std::span<const double>(inject, width * size_t(branches)), size_t(branches), size_t(channels), size_t(rank), epsilon);
+        std::copy(r.input.begin(), r.input.end(), read);
+        std::copy(r.write_scales.begin(), r.write_scales.end(), write_scales);
+    });
+}
+int ref_residual_write_reference(const double* streams, const double* output, const double* scales, uint64_t branches, uint64_t channels, double* result) {
+    return guarded([&] {
+        const auto r = residual_write_reference(std::span<const double>(streams, size_t(branches * channels)), std::span<const double>(output, size_t(channels)),
+                                                std::span<const double>(scales, size_t(branches)));
+        std::copy(r.begin(), r.end(), result);
+    });
+}
 
 int ref_route_reference(const double* logits, uint64_t count, uint64_t selected, uint32_t mode, int normalize,
                         uint32_t* ids, double* weights) {

@@ -257,6 +257,74 @@ int orc_stable_softplus(double v, double* out) {
 }
 
 /* ------------------------------------------------------------------------- */
+/* src/operators.cpp:42-58 — independent groups, double accumulation, gains per element. */
+int orc_group_rms_reference(const double* input, const double* gains, uint64_t count, uint64_t group_width,
+                            double epsilon, double* output) {
+    REQUIRE(group_width && count && count % group_width == 0 && isfinite(epsilon) && epsilon > 0);
+    for (uint64_t i = 0; i < count; ++i) REQUIRE(isfinite(input[i]) && isfinite(gains[i]));
+    for (uint64_t group = 0; group < count; group += group_width) {
+        double squared = 0;
+        for (uint64_t i = 0; i < group_width; ++i) squared += input[group + i] * input[group + i];
+        REQUIRE(isfinite(squared));
+        const double inverse = 1 / sqrt(squared / (double)group_width + epsilon);
+        for (uint64_t i = 0; i < group_width; ++i) output[group + i] = input[group + i] * inverse * gains[group + i];
+    }
+    for (uint64_t i = 0; i < count; ++i) REQUIRE(isfinite(output[i]));
+    return ORC_OK;
+}
+
+/* src/operators.cpp:60-84 — streams [branch, channel]; down [rank, width], up [width, rank], inject [branches, width],
+ * width = branches * channels: normalise, bottleneck = silu(down n / branches), scores = up bottleneck,
+ * read[c] = mean_b n[b, c] sigmoid(scores[b, c]), write_scales[b] = 2 sigmoid((inject n)[b] / branches). */
+int orc_gated_residual_reference(const double* streams, const double* gains, const double* down, const double* up,
+                                 const double* inject, uint64_t branches, uint64_t channels, uint64_t rank, double epsilon,
+                                 double* read, double* write_scales) {
+    REQUIRE(branches && channels && rank);
+    const uint64_t width = branches * channels;
+    double* normalized = (double*)malloc(width * sizeof(double));
+    double* bottleneck = (double*)malloc(rank * sizeof(double));
+    REQUIRE(normalized && bottleneck);
+    int rc = orc_group_rms_reference(streams, gains, width, channels, epsilon, normalized);
+    if (rc == ORC_OK) {
+        for (uint64_t r = 0; r < rank && rc == ORC_OK; ++r) {
+            double sum = 0;
+            for (uint64_t i = 0; i < width; ++i) sum += down[r * width + i] * normalized[i];
+            rc = orc_stable_silu(sum / (double)branches, &bottleneck[r]);
+        }
+    }
+    for (uint64_t c = 0; c < channels; ++c) read[c] = 0;
+    for (uint64_t b = 0; b < branches && rc == ORC_OK; ++b) {
+        double scale = 0, gate;
+        for (uint64_t i = 0; i < width; ++i) scale += inject[b * width + i] * normalized[i];
+        rc = orc_stable_sigmoid(scale / (double)branches, &gate);
+        write_scales[b] = 2 * gate;
+        for (uint64_t c = 0; c < channels && rc == ORC_OK; ++c) {
+            const uint64_t at = b * channels + c;
+            double score = 0;
+            for (uint64_t r = 0; r < rank; ++r) score += up[at * rank + r] * bottleneck[r];
+            rc = orc_stable_sigmoid(score, &gate);
+            read[c] += normalized[at] * gate / (double)branches;
+        }
+    }
+    free(normalized);
+    free(bottleneck);
+    return rc;
+}
+
+/* src/operators.cpp:86-96 */
+int orc_residual_write_reference(const double* streams, const double* output, const double* scales, uint64_t branches,
+                                 uint64_t channels, double* result) {
+    REQUIRE(branches && channels);
+    for (uint64_t b = 0; b < branches; ++b)
+        for (uint64_t c = 0; c < channels; ++c) {
+            const double v = streams[b * channels + c] + scales[b] * output[c];
+            REQUIRE(isfinite(v));
+            result[b * channels + c] = v;
+        }
+    return ORC_OK;
+}
+
+/* ------------------------------------------------------------------------- */
 /* src/routing.cpp:11-40 — top-k by (logit desc, id asc); softmax / sigmoid weights. */
 static double route_activate(const double* logits, uint32_t index, double maximum, uint32_t mode, int normalize) {
     double a, b;

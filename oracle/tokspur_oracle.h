@@ -64,6 +64,14 @@ int orc_reference_q8_many(const uint8_t* matrix, uint64_t nbytes, const float* i
 int orc_stable_sigmoid(double v, double* out);
 int orc_stable_silu(double v, double* out);
 int orc_stable_softplus(double v, double* out);
+/* src/operators.cpp:42-96: grouped RMS with effective gains, the gated-residual read (write scales included) and write. */
+int orc_group_rms_reference(const double* input, const double* gains, uint64_t count, uint64_t group_width,
+                            double epsilon, double* output);
+int orc_gated_residual_reference(const double* streams, const double* gains, const double* down, const double* up,
+                                 const double* inject, uint64_t branches, uint64_t channels, uint64_t rank, double epsilon,
+                                 double* read, double* write_scales);
+int orc_residual_write_reference(const double* streams, const double* output, const double* scales, uint64_t branches,
+                                 uint64_t channels, double* result);
 
 /* ---- router / mixture: src/routing.cpp:11-60 ---- */
 int orc_route_reference(const double* logits, uint64_t count, uint64_t selected, uint32_t mode,

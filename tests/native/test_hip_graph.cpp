@@ -2,6 +2,7 @@
 // tests/test_planar_pack_v3.cpp): build weights with the tests' LCG fixture, run the operators through the graph
 // class, compare with the CPU reference, and check the lifecycle and error contract (idle / encoding phases,
 // ledger, budget, sticky error word, no allocation while encoding, canaries).
+#include <array>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -637,6 +638,55 @@ void test_pack_v3_block_on_graph() {
     release_moe_mm_many_scratch(g, scratch);
 }
 
+// native/tests/test_graph.cpp:113-141 `residual_cases` through the graph class: rms -> F32 GEMV -> SiLU in place -> two F32 GEMVs ->
+// residual_read -> residual_write, seven operators in one batch with a partial commit in the middle, 5e-5 scaled error
+void test_residual_streams_and_partial_commit() {
+    HipGraph g(64u << 20);
+    for (const auto& shape : {std::array<uint32_t, 3>{1, 7, 3}, std::array<uint32_t, 3>{4, 9, 5}, std::array<uint32_t, 3>{3, 257, 16}, std::array<uint32_t, 3>{4, 2560, 320}}) {
+        const uint32_t branches = shape[0], channels = shape[1], rank = shape[2], width = branches * channels;
+        auto streams = lcg_floats(11 + channels, width), gains = lcg_floats(12 + channels, width);
+        for (auto& v : gains) v = 1 + 0.1f * v;
+        auto down = lcg_floats(13 + channels, size_t(width) * rank), up = lcg_floats(14 + channels, size_t(rank) * width), inject = lcg_floats(15 + channels, size_t(width) * branches);
+        for (auto* m : {&down, &up, &inject}) for (auto& v : *m) v *= 0.01f;
+        const float epsilon = 1e-6f;
+        const auto real = [](const std::vector<float>& v) { return std::vector<double>(v.begin(), v.end()); };
+        std::vector<double> want_read(channels), want_scales(branches), want_written(width);
+        EXPECT(orc_gated_residual_reference(real(streams).data(), real(gains).data(), real(down).data(), real(up).data(), real(inject).data(), branches, channels, rank,
+                                            epsilon, want_read.data(), want_scales.data()) == 0);
+        EXPECT(orc_residual_write_reference(real(streams).data(), want_read.data(), want_scales.data(), branches, channels, want_written.data()) == 0);
+        const GpuView stream = g.upload(bytes_of(streams), "streams"), gain = g.upload(bytes_of(gains), "gains"), w_down = g.upload(bytes_of(down), "down");
+        const GpuView w_up = g.upload(bytes_of(up), "up"), w_inject = g.upload(bytes_of(inject), "inject");
+        const GpuView normalized = g.zeros(width * 4, "normalized"), bottleneck = g.zeros(rank * 4, "bottleneck"), scores = g.zeros(width * 4, "scores");
+        const GpuView logits = g.zeros(branches * 4, "inject logits"), scales = g.zeros(branches * 4, "scales"), output = g.zeros(channels * 4, "output");
+        const GpuView written = g.zeros(width * 4, "written");
+        const uint64_t allocations = g.memory().allocations;
+        g.begin();
+        EXPECT(!g.commit_partial());  // nothing encoded yet
+        g.rms(stream, gain, normalized, channels, epsilon);
+        g.gemv(0, w_down, normalized, bottleneck, width, rank);
+        g.activate(bottleneck, bottleneck, Activation::silu, 1.0f / float(branches));
+        EXPECT(g.commit_partial());
+        g.gemv(0, w_up, bottleneck, scores, rank, width);
+        g.gemv(0, w_inject, normalized, logits, width, branches);
+        g.residual_read(normalized, scores, logits, output, scales, branches, channels);
+        g.residual_write(stream, output, scales, written);
+        const BatchResult r = g.submit();
+        EXPECT(r.dispatches == 7 && g.memory().allocations == allocations);
+        EXPECT(scaled_error(read_as<float>(g, output), want_read) <= 5e-5 && scaled_error(read_as<float>(g, scales), want_scales) <= 5e-5);
+        EXPECT(scaled_error(read_as<float>(g, written), want_written) <= 5e-5 && read_as<float>(g, stream) == streams);
+        // refusals: a group width that does not divide, a zero epsilon, an output over its input, a gate of another size
+        g.begin();
+        EXPECT(throws_format([&] { g.rms(stream, gain, normalized, channels + 1, epsilon); }));
+        EXPECT(throws_format([&] { g.rms(stream, gain, normalized, channels, 0.0f); }));
+        EXPECT(throws_format([&] { g.rms(stream, gain, stream, channels, epsilon); }));  // immutable, and its own input
+        EXPECT(throws_format([&] { g.rms_sigmoid_gate(stream, gain, output, normalized, channels, epsilon); }) || width == channels);
+        EXPECT(throws_format([&] { g.multiply(normalized, output, scores); }) || width == channels);
+        EXPECT(throws_format([&] { g.residual_read(normalized, scores, logits, output, scales, branches + 1, channels); }));
+        g.abort();
+        for (const GpuView v : {stream, gain, w_down, w_up, w_inject, normalized, bottleneck, scores, logits, scales, output, written}) g.release(v);
+    }
+}
+
 // the raw-GGUF arm of the same composition (src/moe_mm_many.cpp:214-240): three grouped products over Q4_K expert stacks in
 // GGUF rows, nothing registered; `grouped_mm` and `dense_mm` on their own; encodings the grouped product does not take are
 // refused while idle, and a refusal part-way through a batch leaves no half-encoded batch behind
@@ -761,6 +811,7 @@ int main() {
                                                          {"encode_moe_mm_many, router projection as one f32 GEMM", test_encode_moe_mm_many_router_batch},
                                                          {"router projection: plan, selection, bounds, refusals", test_router_projection_controls},
                                                          {"pack v3: build, adopt, upload a block, encode_moe_mm_many on it", test_pack_v3_block_on_graph},
+                                                         {"RMS, activation, residual streams; partial commit", test_residual_streams_and_partial_commit},
                                                          {"encode_moe_mm_many, raw-GGUF arm; prepare twice; Q8_0 registration", test_encode_moe_mm_many_raw_arm}};
     for (const auto& [name, fn] : tests) {
         std::printf("== %s\n", name);

@@ -1,5 +1,7 @@
 """GPU parity for the router (ids bit-exact), the expert permutation and prefix-sum offsets
 (bit-exact), the T <= 8 union records (bit-exact), and the mixture / SwiGLU operators."""
+import math
+
 import numpy as np
 import pytest
 
@@ -266,3 +268,86 @@ def test_swiglu(gpu, tsp, orc):
     bad[5] = np.nan
     gpu.swiglu(gpu.upload(bad), gpu.upload(u))
     assert gpu.error() == tsp.ERRBIT_NONFINITE
+
+
+# ---------------------------------------------------------------------------------- RMS, activations, residual streams
+
+def scaled(got, want):
+    return float(np.max(np.abs(np.asarray(got, dtype=np.float64) - want) / np.maximum(1.0, np.abs(want))))
+
+
+@pytest.mark.parametrize("branches,channels,rank", [(1, 7, 3), (4, 9, 5), (3, 257, 16), (4, 2560, 320)])
+def test_gated_residual_composition(gpu, orc, branches, channels, rank):
+    """native/tests/test_graph.cpp:113-141: rms -> F32 GEMV -> SiLU(x / branches) in place -> two F32 GEMVs -> residual_read ->
+    residual_write against gated_residual_reference / residual_write_reference, 5e-5 scaled error; the streams stay untouched."""
+    rng = np.random.default_rng(branches * 1000 + channels)
+    width = branches * channels
+    streams = rng.uniform(-1, 1, width).astype(np.float32)
+    gains = (1 + rng.uniform(-0.1, 0.1, width)).astype(np.float32)
+    down = rng.uniform(-0.01, 0.01, (rank, width)).astype(np.float32)
+    up = rng.uniform(-0.01, 0.01, (width, rank)).astype(np.float32)
+    inject = rng.uniform(-0.01, 0.01, (branches, width)).astype(np.float32)
+    epsilon = 1e-6
+    want_read, want_scales = orc.gated_residual_reference(streams, gains, down, up, inject, branches, channels, rank, np.float32(epsilon))
+    d_streams = gpu.upload(streams)
+    normalized = gpu.rms(d_streams, gpu.upload(gains), channels, epsilon)
+    bottleneck = gpu.gemv(0, gpu.upload(down), normalized, width, rank)
+    gpu.activate(bottleneck, 1, 1.0 / branches, out=bottleneck)
+    scores = gpu.gemv(0, gpu.upload(up), bottleneck, rank, width)
+    logits = gpu.gemv(0, gpu.upload(inject), normalized, width, branches)
+    read, scales = gpu.residual_read(normalized, scores, logits, branches, channels)
+    written = gpu.residual_write(d_streams, read, scales, branches, channels)
+    assert gpu.error() == 0
+    assert scaled(read.cpu().numpy(), want_read) <= 5e-5 and scaled(scales.cpu().numpy(), want_scales) <= 5e-5
+    assert scaled(written.cpu().numpy(), orc.residual_write_reference(streams, want_read, want_scales)) <= 5e-5
+    assert np.array_equal(d_streams.cpu().numpy(), streams)
+    # the streams updated in place give the same bits
+    gpu.residual_write(d_streams, read, scales, branches, channels, out=d_streams)
+    assert np.array_equal(d_streams.cpu().numpy().view(np.uint32), written.cpu().numpy().view(np.uint32))
+
+
+def test_rms_activate_multiply(gpu, orc, tsp):
+    rng = np.random.default_rng(77)
+    for groups, width, shared in ((1, 1, False), (5, 128, True), (48, 128, True), (7, 333, False), (3, 65536, True)):
+        x = rng.normal(size=groups * width).astype(np.float32)
+        gains = rng.normal(size=width if shared else groups * width).astype(np.float32)
+        gate = rng.normal(size=groups * width).astype(np.float32) * 3
+        full_gains = np.tile(gains, groups) if shared else gains
+        want = orc.group_rms_reference(x, full_gains, width, np.float32(1e-6))
+        got = gpu.rms(gpu.upload(x), gpu.upload(gains), width, 1e-6).cpu().numpy()
+        assert scaled(got, want) <= 5e-5, (groups, width)
+        gated = gpu.rms(gpu.upload(x), gpu.upload(gains), width, 1e-6, gate=gpu.upload(gate)).cpu().numpy()
+        assert scaled(gated, want / (1 + np.exp(-gate.astype(np.float64)))) <= 5e-5
+        # the fused form is the composition of rms and multiply(sigmoid_gate) (kernels/graph.metal:249)
+        two_step = gpu.multiply(gpu.upload(got), gpu.upload(gate), True).cpu().numpy()
+        assert np.abs(gated - two_step).max() <= 1e-6 * max(1.0, np.abs(gated).max())
+    x = np.concatenate([rng.normal(size=1000) * 10, [0.0, -0.0, 88.0, -88.0, 1e-30, -104.0, 30.0, -30.0]]).astype(np.float32)
+    x64 = x.astype(np.float64)
+    for kind, f in ((0, lambda v: v), (1, lambda v: v / (1 + np.exp(-v))), (2, lambda v: 1 / (1 + np.exp(-v))), (3, lambda v: np.maximum(v, 0) + np.log1p(np.exp(-np.abs(v))))):
+        for scale in (1.0, 0.25):
+            got = gpu.activate(gpu.upload(x), kind, scale).cpu().numpy()
+            assert scaled(got, f(x64 * np.float32(scale))) <= 5e-5, kind
+    # softplus keeps its tiny tail where 1 + e^-|x| rounds to 1
+    tail = gpu.activate(gpu.upload(np.array([-30.0, -80.0], dtype=np.float32)), 3).cpu().numpy()
+    assert tail[0] > 0 and abs(tail[0] / math.exp(-30.0) - 1) < 1e-5 and tail[1] > 0
+    y = gpu.multiply(gpu.upload(x), gpu.upload(x[::-1].copy())).cpu().numpy()
+    assert np.array_equal(y, x * x[::-1])
+    assert gpu.error() == 0
+    # error contract: a non-finite input raises the flag and leaves its destination alone; refusals on the host
+    bad = x.copy()
+    bad[3] = np.inf
+    out = gpu.full(bad.size, -5.0)
+    gpu.activate(gpu.upload(bad), 2, out=out)
+    assert gpu.error() == 1 and out.cpu().numpy()[3] == -5.0 and out.cpu().numpy()[4] != -5.0
+    out = gpu.full(bad.size, -5.0)
+    gpu.multiply(gpu.upload(x), gpu.upload(bad), out=out)
+    assert gpu.error() == 1 and out.cpu().numpy()[3] == -5.0
+    big = np.full(64, 3e38, dtype=np.float32)
+    out = gpu.full(64, -5.0)
+    gpu.rms(gpu.upload(big), gpu.upload(np.ones(64, dtype=np.float32)), 64, 1e-6, out=out)
+    assert gpu.error() == 1 and (out.cpu().numpy() == -5.0).all()
+    d = gpu.upload(x)
+    for call in (lambda: gpu.rms(d, d, 11, 1e-6), lambda: gpu.rms(d, d, 8, 0.0), lambda: gpu.rms(d, d, 8, float("nan")), lambda: gpu.rms(d, d, 8, 1e-6, out=d),
+                 lambda: gpu.activate(d, 4), lambda: gpu.activate(d, 1, float("inf")), lambda: gpu.residual_read(d, d, d, 65, 4), lambda: gpu.residual_write(d, d, d, 2, 70000)):
+        with pytest.raises(tsp.FormatError):
+            call()

@@ -91,6 +91,40 @@ def test_scalar_operators(cpu):
         assert abs(cpu.stable_softplus(x) - cpu.stable_softplus(-x) - x) < 1e-12
 
 
+def test_rms_and_residual_goldens(cpu):
+    # native/tests/test_operators.cpp:35-59: the scalar gated-residual case worked by hand, and two RMS groups.
+    a, b = 2 / math.sqrt(5.0), 6 / math.sqrt(10.0)
+    projected = (0.25 * a - 0.5 * b) / 2
+    hidden = projected / (1 + math.exp(-projected))
+    expected = (a / (1 + math.exp(-0.3 * hidden)) + b / (1 + math.exp(0.7 * hidden))) / 2
+    read, scales = cpu.gated_residual_reference([2, 3], [1, 2], [0.25, -0.5], [0.3, -0.7], [0.1, 0.2, -0.5, 0.7], 2, 1, 1, 1.0)
+    assert abs(read[0] - expected) < 1e-15
+    assert abs(scales[0] - 2 / (1 + math.exp(-(0.1 * a + 0.2 * b) / 2))) < 1e-15
+    assert abs(scales[1] - 2 / (1 + math.exp(-(-0.5 * a + 0.7 * b) / 2))) < 1e-15
+    written = cpu.residual_write_reference([2, 3], read, scales)
+    assert abs(written[0] - (2 + read[0] * scales[0])) < 1e-15 and abs(written[1] - (3 + read[0] * scales[1])) < 1e-15
+    normalized = cpu.group_rms_reference([3, 4, 0, 2], [1, 1, 1, 1], 2, 0.5)
+    assert abs(normalized[0] - 3 / math.sqrt(13.0)) < 1e-15 and abs(normalized[3] - 2 / math.sqrt(2.5)) < 1e-15
+    from oracle.oracle import FormatError
+    for bad in (lambda: cpu.group_rms_reference([3, 4, 0, 2], [1, 1, 1, 1], 3, 1e-6), lambda: cpu.group_rms_reference([3, 4, 0, 2], [1, 1, 1, 1], 2, 0.0)):
+        with pytest.raises(FormatError):
+            bad()
+    # against plain numpy on a wider case: three branches, rank 4
+    rng = np.random.default_rng(5)
+    branches, channels, rank = 3, 17, 4
+    width = branches * channels
+    streams, gains = rng.normal(size=width), 1 + 0.1 * rng.normal(size=width)
+    down, up, inject = 0.1 * rng.normal(size=(rank, width)), 0.1 * rng.normal(size=(width, rank)), 0.1 * rng.normal(size=(branches, width))
+    n = (streams.reshape(branches, channels) / np.sqrt((streams.reshape(branches, channels) ** 2).mean(axis=1, keepdims=True) + 1e-6)).reshape(-1) * gains
+    assert np.allclose(cpu.group_rms_reference(streams, gains, channels, 1e-6), n, rtol=1e-14)
+    z = down @ n / branches
+    bottleneck = z / (1 + np.exp(-z))
+    scores = 1 / (1 + np.exp(-(up @ bottleneck)))
+    read, scales = cpu.gated_residual_reference(streams, gains, down, up, inject, branches, channels, rank, 1e-6)
+    assert np.allclose(read, (n * scores).reshape(branches, channels).mean(axis=0), rtol=1e-13)
+    assert np.allclose(scales, 2 / (1 + np.exp(-(inject @ n) / branches)), rtol=1e-13)
+
+
 def test_oracle_equals_reference_routing(orc, ref):
     rng = np.random.default_rng(3)
     for _ in range(200):

@@ -332,6 +332,39 @@ class Device:
                                self.ptr(self.err), self.stream()))
         return out
 
+    def rms(self, x, gains, group_width, epsilon, gate=None, out=None):
+        out = self.empty(x.shape) if out is None else out
+        shared = int(gains.numel() == group_width and x.numel() != group_width)
+        if gate is None:
+            check(dll().tsp_rms(self.ptr(x), self.ptr(gains), self.ptr(out), C.c_uint64(x.numel()), C.c_uint32(group_width), C.c_int(shared),
+                                C.c_float(epsilon), self.ptr(self.err), self.stream()))
+        else:
+            check(dll().tsp_rms_sigmoid_gate(self.ptr(x), self.ptr(gains), self.ptr(gate), self.ptr(out), C.c_uint64(x.numel()), C.c_uint32(group_width),
+                                             C.c_int(shared), C.c_float(epsilon), self.ptr(self.err), self.stream()))
+        return out
+
+    def activate(self, x, kind, scale=1.0, out=None):
+        out = self.empty(x.shape) if out is None else out
+        check(dll().tsp_activate(self.ptr(x), self.ptr(out), C.c_uint64(x.numel()), C.c_uint32(kind), C.c_float(scale), self.ptr(self.err), self.stream()))
+        return out
+
+    def multiply(self, x, gate, sigmoid_gate=False, out=None):
+        out = self.empty(x.shape) if out is None else out
+        check(dll().tsp_multiply(self.ptr(x), self.ptr(gate), self.ptr(out), C.c_uint64(x.numel()), C.c_int(bool(sigmoid_gate)), self.ptr(self.err), self.stream()))
+        return out
+
+    def residual_read(self, normalized, scores, inject, branches, channels):
+        out, scales = self.empty(channels), self.empty(branches)
+        check(dll().tsp_residual_read(self.ptr(normalized), self.ptr(scores), self.ptr(inject), self.ptr(out), self.ptr(scales), C.c_uint32(branches),
+                                      C.c_uint32(channels), self.ptr(self.err), self.stream()))
+        return out, scales
+
+    def residual_write(self, streams, x, scales, branches, channels, out=None):
+        out = self.empty(streams.shape) if out is None else out
+        check(dll().tsp_residual_write(self.ptr(streams), self.ptr(x), self.ptr(scales), self.ptr(out), C.c_uint32(branches), C.c_uint32(channels),
+                                       self.ptr(self.err), self.stream()))
+        return out
+
     def grouped_routes(self, ids, experts, selected, tokens, fill=0xDEADBEEF):
         token_map = self.full((experts, tokens), np.int32(np.uint32(fill).view(np.int32)), "int32")
         counts = self.zeros(experts, "int32")

@@ -1,6 +1,8 @@
 // tokspur::HipGraph over the C ABI of include/tokspur_hip.h. See hip_graph.hpp for the contract.
 #include "hip_graph.hpp"
 
+#include <cmath>
+
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -372,6 +374,77 @@ void HipGraph::gemv_rows(uint32_t encoding, GpuView matrix, GpuRowsF32 input, Gp
     check(tsp_gemv_rows(encoding, TSP_LAYOUT_GGUF, p.device(matrix), matrix.bytes, reinterpret_cast<const float*>(p.device(input.view)), input.stride_bytes,
                         reinterpret_cast<float*>(p.device(output.view, true)), output.stride_bytes, input.rows, input.columns, output.columns,
                         p.error_word, p.stream));
+}
+
+namespace {
+uint64_t floats(const GpuView& v) {
+    require(v.bytes % 4 == 0 && v.bytes / 4 <= 0xffffffffull, "graph float view byte span");
+    return v.bytes / 4;
+}
+}  // namespace
+
+bool HipGraph::commit_partial() {
+    auto& p = *impl_;
+    p.same_thread();
+    require(p.encoding, "GPU graph operator outside begin/submit");
+    return p.dispatches != 0;
+}
+
+void HipGraph::rms(GpuView input, GpuView gains, GpuView output, uint32_t group_width, float epsilon) {
+    auto& p = *impl_; p.active();
+    const uint64_t count = floats(input);
+    require(group_width && count % group_width == 0 && group_width <= 65536 && floats(output) == count &&
+                (floats(gains) == count || floats(gains) == group_width) && std::isfinite(epsilon) && epsilon > 0,
+            "graph RMS shape/epsilon mismatch");
+    validate_disjoint(std::array{input, gains}, std::array{output});
+    check(tsp_rms(reinterpret_cast<const float*>(p.device(input)), reinterpret_cast<const float*>(p.device(gains)), reinterpret_cast<float*>(p.device(output, true)),
+                  count, group_width, gains.bytes == uint64_t(group_width) * 4 && count != group_width, epsilon, p.error_word, p.stream));
+}
+void HipGraph::rms_sigmoid_gate(GpuView input, GpuView gains, GpuView gate, GpuView output, uint32_t group_width, float epsilon) {
+    auto& p = *impl_; p.active();
+    const uint64_t count = floats(input);
+    require(group_width && count % group_width == 0 && group_width <= 65536 && floats(gate) == count && floats(output) == count &&
+                (floats(gains) == count || floats(gains) == group_width) && std::isfinite(epsilon) && epsilon > 0,
+            "graph RMS sigmoid gate shape/epsilon mismatch");
+    validate_disjoint(std::array{input, gains, gate}, std::array{output});
+    check(tsp_rms_sigmoid_gate(reinterpret_cast<const float*>(p.device(input)), reinterpret_cast<const float*>(p.device(gains)),
+                               reinterpret_cast<const float*>(p.device(gate)), reinterpret_cast<float*>(p.device(output, true)), count, group_width,
+                               gains.bytes == uint64_t(group_width) * 4 && count != group_width, epsilon, p.error_word, p.stream));
+}
+void HipGraph::activate(GpuView input, GpuView output, Activation kind, float scale) {
+    auto& p = *impl_; p.active();
+    const uint64_t count = floats(input);
+    require(floats(output) == count && uint32_t(kind) <= 3 && std::isfinite(scale), "graph activation shape/mode mismatch");
+    // the output may be the input itself, not a view that merely overlaps it: the C ABI refuses that
+    check(tsp_activate(reinterpret_cast<const float*>(p.device(input)), reinterpret_cast<float*>(p.device(output, true)), count, uint32_t(kind), scale,
+                       p.error_word, p.stream));
+}
+void HipGraph::multiply(GpuView input, GpuView gate, GpuView output, bool sigmoid_gate) {
+    auto& p = *impl_; p.active();
+    const uint64_t count = floats(input);
+    require(floats(gate) == count && floats(output) == count, "graph multiplication shape mismatch");
+    check(tsp_multiply(reinterpret_cast<const float*>(p.device(input)), reinterpret_cast<const float*>(p.device(gate)),
+                       reinterpret_cast<float*>(p.device(output, true)), count, sigmoid_gate, p.error_word, p.stream));
+}
+void HipGraph::residual_read(GpuView normalized, GpuView scores, GpuView inject, GpuView output, GpuView scales, uint32_t branches, uint32_t channels) {
+    auto& p = *impl_; p.active();
+    require(branches && branches <= 64 && channels && channels <= 65536 && floats(normalized) == checked_mul(branches, channels) &&
+                floats(scores) == floats(normalized) && floats(inject) == branches && floats(output) == channels && floats(scales) == branches,
+            "graph residual-read shape mismatch");
+    validate_disjoint(std::array{normalized, scores, inject}, std::array{output, scales});
+    check(tsp_residual_read(reinterpret_cast<const float*>(p.device(normalized)), reinterpret_cast<const float*>(p.device(scores)),
+                            reinterpret_cast<const float*>(p.device(inject)), reinterpret_cast<float*>(p.device(output, true)),
+                            reinterpret_cast<float*>(p.device(scales, true)), branches, channels, p.error_word, p.stream));
+}
+void HipGraph::residual_write(GpuView streams, GpuView input, GpuView scales, GpuView destination) {
+    auto& p = *impl_; p.active();
+    const uint64_t channels = floats(input), branches = floats(scales);
+    require(branches && branches <= 64 && channels && channels <= 65536 && floats(streams) == checked_mul(branches, channels) && floats(destination) == floats(streams),
+            "graph residual-write shape mismatch");
+    validate_disjoint(std::array{input, scales}, std::array{destination});
+    check(tsp_residual_write(reinterpret_cast<const float*>(p.device(streams)), reinterpret_cast<const float*>(p.device(input)),
+                             reinterpret_cast<const float*>(p.device(scales)), reinterpret_cast<float*>(p.device(destination, true)), uint32_t(branches),
+                             uint32_t(channels), p.error_word, p.stream));
 }
 
 void HipGraph::configure_moe_router_f32_batch(bool enabled) {

@@ -68,6 +68,7 @@ struct BatchResult {
     double gpu_ms = 0;
 };
 // include/tokspur/routing.hpp:10, include/tokspur/grouped_mm.hpp:6 (+ the Pack v3 planes as layout 3)
+enum class Activation : uint32_t { identity, silu, sigmoid, softplus };  // include/tokspur/graph.hpp:134
 enum class RouterMode : uint32_t { softmax, sigmoid };
 enum class PrefillWeightLayout : uint32_t { gguf = 0, q8_lanes_v1 = 1, q51_lanes_v1 = 2, planar_v3 = 3 };
 // include/tokspur/sampling.hpp:21-29
@@ -116,6 +117,10 @@ public:
     void begin();
     void abort();
     [[nodiscard]] BatchResult submit();
+    // graph.hpp:715-716: hands what is encoded so far to the GPU without waiting and continues the same batch. Operators are
+    // launched on the graph's stream as they are encoded, so there is nothing left to hand over: true for a batch with
+    // operators in it, false (and no change) for an empty one. submit() and abort() wait for every part.
+    bool commit_partial();
 
     // ---- operators (between begin and submit)
     void gemv(uint32_t encoding, GpuView matrix, GpuView input, GpuView output, uint32_t columns, uint32_t rows);  // graph.hpp:730
@@ -134,6 +139,13 @@ public:
                              uint32_t tokens, RouterMode mode, bool normalize_selected);                             // graph.hpp:852
     void routed_gemv(uint32_t encoding, GpuView matrices, GpuView indices, GpuView input, GpuView output, uint32_t columns,
                      uint32_t rows, uint32_t experts, bool broadcast_input);                                         // graph.hpp:1093
+    // the f32 operators either side of the sublayer, graph.hpp:983-986 and src/graph.mm:7715-7734
+    void rms(GpuView input, GpuView effective_gains, GpuView output, uint32_t group_width, float epsilon);
+    void rms_sigmoid_gate(GpuView input, GpuView effective_gains, GpuView gate, GpuView output, uint32_t group_width, float epsilon);
+    void activate(GpuView input, GpuView output, Activation kind, float scale = 1);
+    void multiply(GpuView input, GpuView gate, GpuView output, bool sigmoid_gate = false);
+    void residual_read(GpuView normalized, GpuView scores, GpuView inject, GpuView output, GpuView scales, uint32_t branches, uint32_t channels);
+    void residual_write(GpuView streams, GpuView input, GpuView scales, GpuView destination);
     void swiglu(GpuView gate, GpuView up, GpuView output, float scale = 1);                                          // graph.hpp:990
     void mixture(GpuView expert_outputs, GpuView weights, GpuView shared_output, GpuView shared_logit, GpuView output);  // 1102
     void prefill_mixture_batch(GpuView experts, GpuView weights, GpuView shared, GpuView shared_logit, GpuRowsF32 output,
