@@ -419,9 +419,13 @@ def main():
                                        "two_streams_us": None if two_streams_ms is None else two_streams_ms * 1e3}
         state["i"] = 0
         configs["c2_moe_verify_t8"]["kernels_us"] = {k: round(v["avg_us"], 2) for k, v in profiled(capi, torch, step_c2, 8).items()}
-        # config 4: Q8_0 LM head, vocab 151936 x 2048, raw GGUF rows; M = 16 goes through the dense Q8_0 GEMM entry point (one pass, K halves summed)
+        # config 4: Q8_0 LM head, vocab 151936 x 2048, both arms: raw GGUF rows and the same matrix as q8_lanes_v1 rows. M = 16 goes
+        # through the dense Q8_0 GEMM entry point (raw rows: one pass, K halves summed; lanes rows: two passes of eight)
         V = 151936
-        w4 = gpu.upload(synth.matrix(8, synth.tensor_seed(4, 1), V, C))
+        w4_host = synth.matrix(8, synth.tensor_seed(4, 1), V, C)
+        w4 = gpu.upload(w4_host)
+        w4_lanes = gpu.upload(capi.q8_lanes_pack_rows(C, w4_host))
+        del w4_host
         for m in (1, 4, 8, 16):
             x4 = gpu.upload(synth.activations_f32(synth.tensor_seed(4, 2 + m), (m, C)))
             y4 = gpu.empty((m, V))
@@ -442,6 +446,16 @@ def main():
                 capi.logit_topk(gpu, y4, m, V, scratch=tk_scratch, out=tk_rows)
 
             configs[f"c4_lm_head_q8_m{m}"]["us_with_top64"] = timed(torch, lm_head_argmax, k2, 2) * 1e3
+            y4_lanes = gpu.empty((m, V))
+
+            def lm_head_lanes():
+                capi.dense_mm_q8(gpu, capi.LAYOUT_Q8_LANES_V1, w4_lanes, x4, m, C, V, out=y4_lanes)
+
+            lanes_ms = timed(torch, lm_head_lanes, k2, 2)
+            lm_head()
+            both = (y4.cpu().numpy(), y4_lanes.cpu().numpy())
+            assert float(np.max(np.abs(both[0] - both[1]) / np.maximum(1.0, np.abs(both[0])))) <= 5e-5, "the two row layouts disagree (config 4)"
+            configs[f"c4_lm_head_q8_m{m}"].update({"lanes_us": lanes_ms * 1e3, "lanes_hbm_frac": b4 / (lanes_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS})
         assert gpu.error() == 0, "device error word set during the secondary configurations"
 
     line = {

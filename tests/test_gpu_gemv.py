@@ -220,7 +220,7 @@ def test_gemv_refusals(gpu, tsp, synth):
 # ---------------------------------------------------------------------------------- Q8 many rows
 
 @pytest.mark.parametrize("tokens,cols,rows", [(1, 64, 5), (19, 512, 160), (40, 2048, 96), (9, 1024, 64), (13, 2048, 1000), (16, 2048, 2084),
-                                              (27, 1024, 132)])
+                                              (27, 1024, 132), (8, 1536, 77), (3, 512, 16)])
 def test_dense_mm_q8(gpu, tsp, orc, synth, tokens, cols, rows):
     # graph.hpp:860 `dense_mm_q8`: a dense Q8_0 matrix times f32 rows, GGUF rows and q8_lanes_v1 rows; rows back to back
     # (width groups 8, 4, 2, 1; nine or more GGUF rows of 1024 / 2048 columns go up to sixteen at a time, each half of the

@@ -180,6 +180,8 @@ extern "C" int tsp_q8_matvec_many(uint32_t layout, const void* matrix, uint64_t 
     const Q8Args a{static_cast<const uint8_t*>(matrix), x, y, columns, rows, error_word};
     const auto s = static_cast<hipStream_t>(stream);
     if (layout == TSP_LAYOUT_GGUF && q8_mfma_supported(matrix, x, columns, rows)) return q8_mfma(matrix, x, y, columns, rows, width, error_word, s);
+    if (layout == TSP_LAYOUT_Q8_LANES_V1 && q8_lanes_mfma_supported(matrix, x, columns, rows))
+        return q8_lanes_mfma(matrix, x, y, columns, rows, width, error_word, s);
     switch (width) {
     case 1: return launch<1>(layout, a, s);
     case 2: return launch<2>(layout, a, s);

@@ -64,6 +64,75 @@ __global__ void clear_rows(float4* out, uint64_t count4) {
     if (i < count4) out[i] = float4{0, 0, 0, 0};
 }
 
+// The token rows of a workgroup, [kRows, K] from column k0 on, in chunks of eight columns: chunk i = tid + j * kThreads is columns
+// 8 (i % (K / 8)) .. + 7 of row i / (K / 8). kRows * K / 8 <= 2048 = kMine * kThreads for K <= 2048 (8 rows) or 1024 (16 rows).
+constexpr uint32_t kMine = 4;
+
+template <int kRows>
+__device__ __forceinline__ void request_token_rows(const Q8MfmaArgs& a, uint32_t K, uint32_t k0, float4 (&xv)[kMine][2]) {
+    const uint32_t chunks = K / 8;
+#pragma unroll
+    for (uint32_t j = 0; j < kMine; ++j) {
+        const uint32_t i = threadIdx.x + j * kThreads, r = i / chunks, c = i % chunks;
+        xv[j][0] = xv[j][1] = float4{0, 0, 0, 0};
+        if (i < kRows * chunks && r < a.m) {
+            const float4* src = reinterpret_cast<const float4*>(a.x + uint64_t(r) * a.columns + k0 + c * 8);
+            xv[j][0] = src[0];
+            xv[j][1] = src[1];
+        }
+    }
+}
+
+// Largest magnitude of the workgroup's rows -> power-of-two scale -> hi + lo halves in LDS, the 16-byte chunks of a row swizzled
+// by the row's index (chunk c of row r sits at c ^ r). Returns the factor that undoes the scale; ends with a barrier.
+template <int kRows>
+__device__ __forceinline__ float stage_token_rows(const float4 (&xv)[kMine][2], uint32_t K, _Float16* a_hi, _Float16* a_lo, float* wave_max,
+                                                  uint32_t& bad) {
+    const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave, chunks = K / 8;
+    float biggest = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < kMine; ++j) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float4 v = xv[j][h];
+            if (nonfinite(v.x) || nonfinite(v.y) || nonfinite(v.z) || nonfinite(v.w)) bad = TSP_ERRBIT_NONFINITE;
+            biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+        }
+    }
+    biggest = wave_largest(biggest);
+    if (lane == 0) wave_max[wave] = biggest;
+    __syncthreads();
+    biggest = wave_max[0];
+#pragma unroll
+    for (uint32_t w = 1; w < kWaves; ++w) biggest = fmaxf(biggest, wave_max[w]);
+    float scale = 1.0f, inv_scale = 1.0f;
+    if (biggest > 0 && !nonfinite(biggest)) {
+        const int e = int((__float_as_uint(biggest) >> 23) & 0xffu) - 127;
+        int shift = 13 - e;
+        shift = shift > 100 ? 100 : shift < -100 ? -100 : shift;
+        scale = __uint_as_float(uint32_t(127 + shift) << 23);
+        inv_scale = __uint_as_float(uint32_t(127 - shift) << 23);
+    }
+#pragma unroll
+    for (uint32_t j = 0; j < kMine; ++j) {
+        const uint32_t i = tid + j * kThreads, r = i / chunks, c = i % chunks;
+        if (i >= kRows * chunks) break;
+        const float v[8] = {xv[j][0].x, xv[j][0].y, xv[j][0].z, xv[j][0].w, xv[j][1].x, xv[j][1].y, xv[j][1].z, xv[j][1].w};
+        f16x8 hi, lo;  // zeros for the rows past a.m
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float sv = v[e] * scale;
+            hi[e] = _Float16(sv);
+            lo[e] = _Float16(sv - float(hi[e]));
+        }
+        const uint32_t at = (r * chunks + (c ^ r)) * 8;
+        *reinterpret_cast<f16x8*>(a_hi + at) = hi;
+        *reinterpret_cast<f16x8*>(a_lo + at) = lo;
+    }
+    __syncthreads();
+    return inv_scale;
+}
+
 // DEPTH = (tile, group) items whose bytes are on their way while one is multiplied (1, 2 or 4; it divides the number of groups
 // of a workgroup). ROWS = token rows staged (8: all of K per workgroup; 16: half of K per workgroup, sums added into y).
 template <int DEPTH, int ROWS>
@@ -87,21 +156,10 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     uint8_t* const tile = lds + 2 * kRows * K * 2 + wave * kTileBytes;
 
     // ---- the token rows: this lane's 16-byte chunks are requested first (they come from cache and return first), then the
-    // wave's first weight bytes, and only then the arithmetic: largest magnitude -> power-of-two scale -> hi/lo halves,
-    // 16-byte chunks swizzled by row. The weights travel while the rows are staged.
-    constexpr uint32_t kMine = 4;  // chunks per lane: kRows * K / 8 <= 2048 = 4 * kThreads for K <= 2048 (8 rows) or 1024 (16 rows)
+    // wave's first weight bytes, and only then the arithmetic. The weights travel while the rows are staged.
     uint32_t bad = 0;
     float4 xv[kMine][2];
-#pragma unroll
-    for (uint32_t j = 0; j < kMine; ++j) {
-        const uint32_t i = tid + j * kThreads, r = i / chunks, c = i % chunks;
-        xv[j][0] = xv[j][1] = float4{0, 0, 0, 0};
-        if (i < kRows * chunks && r < a.m) {
-            const float4* src = reinterpret_cast<const float4*>(a.x + uint64_t(r) * a.columns + k0 + c * 8);
-            xv[j][0] = src[0];
-            xv[j][1] = src[1];
-        }
-    }
+    request_token_rows<kRows>(a, K, k0, xv);
     // chunk `id` of a group tile: row id / 17 of the wave's 32, bytes (id % 17) * 16 of that row's 272. The byte offsets from
     // the tile's first row and the group's first byte never change, so a request is a uniform address plus a lane offset.
     uint32_t chunk_at[kStageLoads];
@@ -150,47 +208,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
         }
     }
     __builtin_amdgcn_sched_barrier(0);  // every request above is out before the first wait below
-    float biggest = 0;
-#pragma unroll
-    for (uint32_t j = 0; j < kMine; ++j) {
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const float4 v = xv[j][h];
-            if (nonfinite(v.x) || nonfinite(v.y) || nonfinite(v.z) || nonfinite(v.w)) bad = TSP_ERRBIT_NONFINITE;
-            biggest = fmaxf(biggest, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
-        }
-    }
-    biggest = wave_largest(biggest);
-    if (lane == 0) wave_max[wave] = biggest;
-    __syncthreads();
-    biggest = wave_max[0];
-#pragma unroll
-    for (uint32_t w = 1; w < kWaves; ++w) biggest = fmaxf(biggest, wave_max[w]);
-    float scale = 1.0f, inv_scale = 1.0f;
-    if (biggest > 0 && !nonfinite(biggest)) {
-        const int e = int((__float_as_uint(biggest) >> 23) & 0xffu) - 127;
-        int shift = 13 - e;
-        shift = shift > 100 ? 100 : shift < -100 ? -100 : shift;
-        scale = __uint_as_float(uint32_t(127 + shift) << 23);
-        inv_scale = __uint_as_float(uint32_t(127 - shift) << 23);
-    }
-#pragma unroll
-    for (uint32_t j = 0; j < kMine; ++j) {
-        const uint32_t i = tid + j * kThreads, r = i / chunks, c = i % chunks;
-        if (i >= kRows * chunks) break;
-        const float v[8] = {xv[j][0].x, xv[j][0].y, xv[j][0].z, xv[j][0].w, xv[j][1].x, xv[j][1].y, xv[j][1].z, xv[j][1].w};
-        f16x8 hi, lo;  // zeros for the rows past a.m
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float sv = v[e] * scale;
-            hi[e] = _Float16(sv);
-            lo[e] = _Float16(sv - float(hi[e]));
-        }
-        const uint32_t at = (r * chunks + (c ^ r)) * 8;
-        *reinterpret_cast<f16x8*>(a_hi + at) = hi;
-        *reinterpret_cast<f16x8*>(a_lo + at) = lo;
-    }
-    __syncthreads();
+    const float inv_scale = stage_token_rows<kRows>(xv, K, a_hi, a_lo, wave_max, bad);
 
     // The activation chunk of block B of group g, columns 8 kq .. 8 kq + 7, is chunk g * 32 + B * 4 + kq of row `arow`, kept at
     // position chunk ^ arow. arow < kRows only flips the low bits, which B % kVariants and kq decide: the lane keeps one
@@ -298,6 +316,180 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     publish_error(bad, a.error_word);
 }
 
+// ---- q8_lanes_v1 rows: [f16 scale x blocks][runs of 16 blocks x 512 B: quant i of the run's sixteen blocks side by side].
+// The unit of work is 16 weight rows x one run (512 columns): per row 32 bytes of scales and 512 bytes of quants, both whole
+// 16-byte chunks at 16-byte aligned offsets when the row has a multiple of 16 blocks. A wave parks the 34 chunks of each row
+// in its LDS tile at a row stride of 560 bytes (140 dwords = 12 mod 64 banks: the sixteen rows that a quarter-wave reads one
+// 16-byte chunk of land in 64 different banks). A lane (n, kq) then reads the eight chunks of quants 8 kq .. 8 kq + 7 of row n,
+// which hold those quants for all sixteen blocks, and turns each 4 x 4 byte square (4 quants x 4 blocks) into the four dwords
+// "4 quants of one block" with two rounds of byte permutes: four permutes per block and lane. From there on a block is what it
+// is for raw rows: exact halves, one 16x16x32 MFMA step for the lo and one for the hi halves of the token rows, and the
+// block's scale times the f32 result.
+constexpr uint32_t kRunBlocks = 16, kRunChunks = 2 + 32;  // 32 B of scales + 512 B of quants per row and run
+constexpr uint32_t kLaneRows = 16, kLaneStride = 560, kLaneTileBytes = kLaneRows * kLaneStride;  // 8 960 B per wave
+constexpr uint32_t kLaneLoads = (kLaneRows * kRunChunks + kWave - 1) / kWave;  // 9 chunk loads per lane and run (the last half used)
+
+template <int DEPTH>
+__global__ __launch_bounds__(kThreads, 1) void q8_lanes_mfma_kernel(Q8MfmaArgs a) {
+    constexpr int kRows = 8;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [hi plane][lo plane][8 weight tiles]
+    __shared__ float wave_max[kWaves];
+    __shared__ uint32_t next_tile;
+
+    const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const uint32_t n16 = lane % 16, kq = lane / 16;
+    const uint32_t K = a.columns, chunks = K / 8, blocks = K / 32, runs = blocks / kRunBlocks, row_bytes = blocks * 34;
+    const uint32_t tiles = (a.rows + kLaneRows - 1) / kLaneRows;
+    if (tid == 0) next_tile = uint32_t(uint64_t(tiles) * blockIdx.x / gridDim.x);
+    __syncthreads();
+    _Float16* const a_hi = reinterpret_cast<_Float16*>(lds);
+    _Float16* const a_lo = a_hi + kRows * K;
+    uint8_t* const tile = lds + 2 * kRows * K * 2 + wave * kLaneTileBytes;
+
+    uint32_t bad = 0;
+    float4 xv[kMine][2];
+    request_token_rows<kRows>(a, K, 0, xv);
+
+    // chunk `id` of a tile: row id / 34 of the wave's 16, piece id % 34 of that row's run: pieces 0 and 1 are the run's scales
+    // (32 bytes per run from the row's start), pieces 2 .. 33 its quants (512 bytes per run after all the scales).
+    auto piece_at = [&](uint32_t row, uint32_t piece, uint32_t run) {
+        return row * row_bytes + (piece < 2 ? run * 32 + piece * 16 : 2 * blocks + run * 512 + (piece - 2) * 16);
+    };
+    uint32_t chunk_at[kLaneLoads], chunk_step[kLaneLoads];  // byte offset at run 0 and bytes per run
+#pragma unroll
+    for (uint32_t t = 0; t < kLaneLoads; ++t) {
+        uint32_t id = t * kWave + lane;
+        id = id < kLaneRows * kRunChunks ? id : kLaneRows * kRunChunks - 1;  // the tail lanes repeat the last chunk
+        chunk_at[t] = piece_at(id / kRunChunks, id % kRunChunks, 0);
+        chunk_step[t] = id % kRunChunks < 2 ? 32 : 512;
+    }
+    uint2 stage[DEPTH][kLaneLoads][2];
+    auto fetch_run = [&](uint32_t row0, uint32_t run, auto set_tag) {
+        constexpr int SET = decltype(set_tag)::value;
+        const uint8_t* from = a.matrix + uint64_t(row0) * row_bytes;  // uniform
+        const bool whole = row0 + kLaneRows <= a.rows;               // uniform
+#pragma unroll
+        for (uint32_t t = 0; t < kLaneLoads; ++t) {
+            uint32_t at = chunk_at[t] + run * chunk_step[t];
+            if (!whole) {  // the matrix's last tile: rows past the end repeat the last row
+                uint32_t id = t * kWave + lane;
+                id = id < kLaneRows * kRunChunks ? id : kLaneRows * kRunChunks - 1;
+                const uint32_t row = row0 + id / kRunChunks < a.rows ? id / kRunChunks : a.rows - 1 - row0;
+                at = piece_at(row, id % kRunChunks, run);
+            }
+            const uint4 v = *reinterpret_cast<const uint4*>(from + at);
+            stage[SET][t][0] = uint2{v.x, v.y};
+            stage[SET][t][1] = uint2{v.z, v.w};
+        }
+    };
+    const uint32_t share_end = uint32_t(uint64_t(tiles) * (blockIdx.x + 1) / gridDim.x);
+    auto take_tile = [&]() {
+        uint32_t t = 0;
+        if (lane == 0) t = atomicAdd(&next_tile, 1u);
+        return uint32_t(__builtin_amdgcn_readfirstlane(int(t)));
+    };
+    uint32_t t = take_tile(), t_next = take_tile();
+    if (t < share_end) {
+        fetch_run(t * kLaneRows, 0, std::integral_constant<int, 0>{});
+        if constexpr (DEPTH >= 2) fetch_run(t * kLaneRows, 1, std::integral_constant<int, 1 % DEPTH>{});
+    }
+    __builtin_amdgcn_sched_barrier(0);  // every request above is out before the first wait below
+    const float inv_scale = stage_token_rows<kRows>(xv, K, a_hi, a_lo, wave_max, bad);
+
+    // the activation chunk of block B of run g, columns 8 kq .. 8 kq + 7: chunk g * 64 + B * 4 + kq of row `arow`, kept at
+    // chunk ^ arow; arow < 8 flips the three low bits, which B % 2 and kq decide
+    const uint32_t arow = n16 & (kRows - 1);
+    uint32_t a_at[2];
+#pragma unroll
+    for (uint32_t v = 0; v < 2; ++v) a_at[v] = (arow * chunks + ((v * 4 + kq) ^ arow)) * 8;
+    auto store_run = [&](auto set_tag) {
+        constexpr int SET = decltype(set_tag)::value;
+#pragma unroll
+        for (uint32_t t = 0; t < kLaneLoads; ++t) {
+            uint32_t id = t * kWave + lane;
+            id = id < kLaneRows * kRunChunks ? id : kLaneRows * kRunChunks - 1;
+            uint8_t* at = tile + (id / kRunChunks) * kLaneStride + (id % kRunChunks) * 16;
+            *reinterpret_cast<uint4*>(at) = uint4{stage[SET][t][0].x, stage[SET][t][0].y, stage[SET][t][1].x, stage[SET][t][1].y};
+        }
+    };
+
+    for (; t < share_end; t = t_next, t_next = take_tile()) {
+        const uint32_t row0 = t * kLaneRows;
+        float acc[4] = {0, 0, 0, 0};  // token row 4 kq + v
+        auto item = [&](uint32_t g, auto set_tag) {
+            store_run(set_tag);  // the previous item's reads were issued before this point; LDS serves a wave in order
+            const uint32_t ahead = g + DEPTH;
+            const bool wraps = ahead >= runs;
+            // past the workgroup's share: ask again for the run at hand (its lines are in cache), nothing new comes from memory
+            const bool more = t_next < share_end;
+            const uint32_t following = wraps && more ? t_next : t;
+            const uint32_t run = !wraps ? ahead : more ? ahead - runs : g;
+            fetch_run(following * kLaneRows, run, set_tag);
+            const uint8_t* mine = tile + n16 * kLaneStride;
+            const uint4 s0 = *reinterpret_cast<const uint4*>(mine), s1 = *reinterpret_cast<const uint4*>(mine + 16);
+            const uint32_t scales[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};  // two f16 scales per dword
+            uint4 q[8];  // q[j]: quant 8 kq + j of the run's sixteen blocks, one byte per block
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[j] = *reinterpret_cast<const uint4*>(mine + 32 + (8 * kq + j) * 16);
+            auto quad = [&](auto m_tag) {  // blocks 4 M .. 4 M + 3 of the run
+                constexpr int M = decltype(m_tag)::value;
+                uint32_t d[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) d[j] = M == 0 ? q[j].x : M == 1 ? q[j].y : M == 2 ? q[j].z : q[j].w;
+                // byte b of d[j] = quant j of block 4 M + b. First round: pairs of quants interleaved, for blocks 0, 1 (lo) and 2, 3 (hi)
+                uint32_t lo[4], hi[4];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    lo[p] = __builtin_amdgcn_perm(d[2 * p + 1], d[2 * p], 0x05010400u);
+                    hi[p] = __builtin_amdgcn_perm(d[2 * p + 1], d[2 * p], 0x07030602u);
+                }
+                // second round: w[b][0] = quants 0 .. 3 and w[b][1] = quants 4 .. 7 of block 4 M + b
+                uint32_t w[4][2];
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    w[0][half] = __builtin_amdgcn_perm(lo[2 * half + 1], lo[2 * half], 0x05040100u);
+                    w[1][half] = __builtin_amdgcn_perm(lo[2 * half + 1], lo[2 * half], 0x07060302u);
+                    w[2][half] = __builtin_amdgcn_perm(hi[2 * half + 1], hi[2 * half], 0x05040100u);
+                    w[3][half] = __builtin_amdgcn_perm(hi[2 * half + 1], hi[2 * half], 0x07060302u);
+                }
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    constexpr int kBase = 4 * M;
+                    const int B = kBase + b;
+                    const f16x8 b_frag = quants8(w[b][0], w[b][1]);
+                    const float scale_d = half_bits_to_float((scales[B / 2] >> (16 * (B % 2))) & 0xffffu);
+                    const uint32_t at = a_at[B % 2] + (g * 64 + (B / 2) * 8) * 8;  // columns g * 512 + B * 32 + 8 kq of the lane's token row
+                    const f16x8 ah = *reinterpret_cast<const f16x8*>(a_hi + at), al = *reinterpret_cast<const f16x8*>(a_lo + at);
+                    const f32x4 zero{};
+                    const f32x4 part_lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, b_frag, zero, 0, 0, 0);
+                    const f32x4 part = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, b_frag, part_lo, 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[v] = __builtin_fmaf(scale_d, part[v], acc[v]);
+                }
+            };
+            quad(std::integral_constant<int, 0>{});
+            quad(std::integral_constant<int, 1>{});
+            quad(std::integral_constant<int, 2>{});
+            quad(std::integral_constant<int, 3>{});
+        };
+        for (uint32_t g = 0; g < runs; g += DEPTH) {  // the host picks a DEPTH that divides the number of runs
+            item(g, std::integral_constant<int, 0>{});
+            if constexpr (DEPTH >= 2) item(g + 1, std::integral_constant<int, 1 % DEPTH>{});
+        }
+        const uint32_t r = row0 + n16;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const uint32_t m = 4 * kq + v;  // lanes with kq >= 2 hold repeats of rows 0 .. 7
+            if (m < kRows && m < a.m && r < a.rows) {
+                const float val = acc[v] * inv_scale;
+                if (nonfinite(val)) bad = TSP_ERRBIT_NONFINITE;
+                a.y[uint64_t(m) * a.rows + r] = val;
+            }
+        }
+    }
+    publish_error(bad, a.error_word);
+}
+
 }  // namespace
 
 namespace tsp {
@@ -343,6 +535,33 @@ int q8_mfma(const void* matrix, const float* x, float* y, uint32_t columns, uint
     if ((columns / 256) % 2 == 0) TSP_LAUNCH("q8_mfma", s, q8_mfma_kernel<2, 8><<<grid, kThreads, lds_bytes, s>>>(a));
     else TSP_LAUNCH("q8_mfma", s, q8_mfma_kernel<1, 8><<<grid, kThreads, lds_bytes, s>>>(a));
     return launch_status("q8_mfma");
+}
+
+bool q8_lanes_mfma_supported(const void* matrix, const float* x, uint32_t columns, uint32_t rows) {
+    return columns % 512 == 0 && columns <= 2048 && rows >= 16 && reinterpret_cast<uintptr_t>(matrix) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(x) % 16 == 0;
+}
+
+int q8_lanes_mfma(const void* matrix, const float* x, float* y, uint32_t columns, uint32_t rows, uint32_t width, uint32_t* error_word,
+                  hipStream_t s) {
+    const Q8MfmaArgs a{static_cast<const uint8_t*>(matrix), x, y, columns, rows, width, error_word};
+    const uint32_t lds_bytes = 2 * 8 * columns * 2 + kWaves * kLaneTileBytes;
+    static std::atomic<uint64_t> raised{0};
+    static int units_of[64] = {};
+    int device = 0;
+    if (first_use_on_device(raised, &device)) {
+        const int most = int(2 * 8 * 2048 * 2 + kWaves * kLaneTileBytes);
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_lanes_mfma_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_lanes_mfma_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        TSP_HIP(hipDeviceGetAttribute(&units_of[device], hipDeviceAttributeMultiprocessorCount, device));
+    }
+    const int compute_units = units_of[device];
+    const uint32_t tiles = (rows + kLaneRows - 1) / kLaneRows;
+    uint32_t grid = uint32_t(compute_units > 0 ? compute_units : 256);
+    if (grid * kWaves > tiles) grid = (tiles + kWaves - 1) / kWaves;
+    if ((columns / 512) % 2 == 0) TSP_LAUNCH("q8_lanes_mfma", s, q8_lanes_mfma_kernel<2><<<grid, kThreads, lds_bytes, s>>>(a));
+    else TSP_LAUNCH("q8_lanes_mfma", s, q8_lanes_mfma_kernel<1><<<grid, kThreads, lds_bytes, s>>>(a));
+    return launch_status("q8_lanes_mfma");
 }
 
 }  // namespace tsp
