@@ -15,7 +15,8 @@
 // aligned dword reads and a byte funnel shift. The next group of 8 blocks is in flight while the current one is multiplied.
 //
 // Workgroups are persistent (one per compute unit, 8 waves): the activations are staged once per workgroup, which owns
-// a contiguous share of the matrix's 32-row tiles; its waves take tiles from that share through a counter in LDS. A
+// every n-th of the matrix's 32-row tiles (n workgroups: at any moment the grid reads one stretch of the matrix, 1 us
+// faster at 151 936 x 2048 than a contiguous share per workgroup); its waves take the workgroup's tiles through a counter in LDS. A
 // lane asks for its share of the token rows first and for its wave's first weight bytes second, and stages the rows
 // while the weights travel. Every address inside the loop is a uniform base plus a lane offset fixed before the loop.
 //
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
     const uint32_t K = a.columns / KSPLIT, chunks = K / 8, groups = K / 256, row_bytes = a.columns / 32 * 34;
     const uint32_t k0 = (blockIdx.x % KSPLIT) * K, g0 = k0 / 256;
     const uint32_t sharer = blockIdx.x / KSPLIT, sharers = gridDim.x / KSPLIT;  // the host launches a multiple of KSPLIT
-    if (tid == 0) next_tile = uint32_t(uint64_t((a.rows + 31) / 32) * sharer / sharers);
+    if (tid == 0) next_tile = 0;
     __syncthreads();  // the tile counter is set before any wave takes from it
     _Float16* const a_hi = reinterpret_cast<_Float16*>(lds);
     _Float16* const a_lo = a_hi + kRows * K;
@@ -188,15 +189,14 @@ __global__ __launch_bounds__(kThreads, 1) void q8_mfma_kernel(Q8MfmaArgs a) {
             stage[SET][t][1] = uint2{v.z, v.w};
         }
     };
-    // Each workgroup owns a contiguous share of the 32-row tiles and its waves take the next free tile of that share from
+    // Workgroup b of n owns tiles b, b + n, b + 2 n, ... and its waves take the next free one of them from
     // a counter in LDS (which wave computes a tile does not change the result). The bytes of the next (tile, group) item
     // are requested before the current one is multiplied, so a wave always holds its next tile index one step ahead.
-    const uint32_t tiles = (a.rows + 31) / 32;
-    const uint32_t share_end = uint32_t(uint64_t(tiles) * (sharer + 1) / sharers);
+    const uint32_t share_end = (a.rows + 31) / 32;
     auto take_tile = [&]() {
         uint32_t t = 0;
         if (lane == 0) t = atomicAdd(&next_tile, 1u);
-        return uint32_t(__builtin_amdgcn_readfirstlane(int(t)));
+        return uint32_t(__builtin_amdgcn_readfirstlane(int(t))) * sharers + sharer;
     };
     uint32_t t = take_tile(), t_next = take_tile();
     if (t < share_end) {
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_lanes_mfma_kernel(Q8MfmaArgs a
     const uint32_t n16 = lane % 16, kq = lane / 16;
     const uint32_t K = a.columns, chunks = K / 8, blocks = K / 32, runs = blocks / kRunBlocks, row_bytes = blocks * 34;
     const uint32_t tiles = (a.rows + kLaneRows - 1) / kLaneRows;
-    if (tid == 0) next_tile = uint32_t(uint64_t(tiles) * blockIdx.x / gridDim.x);
+    if (tid == 0) next_tile = 0;
     __syncthreads();
     _Float16* const a_hi = reinterpret_cast<_Float16*>(lds);
     _Float16* const a_lo = a_hi + kRows * K;
@@ -382,11 +382,11 @@ __global__ __launch_bounds__(kThreads, 1) void q8_lanes_mfma_kernel(Q8MfmaArgs a
             stage[SET][t][1] = uint2{v.z, v.w};
         }
     };
-    const uint32_t share_end = uint32_t(uint64_t(tiles) * (blockIdx.x + 1) / gridDim.x);
+    const uint32_t share_end = tiles;
     auto take_tile = [&]() {
         uint32_t t = 0;
         if (lane == 0) t = atomicAdd(&next_tile, 1u);
-        return uint32_t(__builtin_amdgcn_readfirstlane(int(t)));
+        return uint32_t(__builtin_amdgcn_readfirstlane(int(t))) * gridDim.x + blockIdx.x;
     };
     uint32_t t = take_tile(), t_next = take_tile();
     if (t < share_end) {
