@@ -1,0 +1,287 @@
+// Grouped down GEMM for 512-column Q6_K experts (planes ql / qh / sc / d), the task's h rows resident in registers.
+//
+// The companion of the activation-resident gate/up kernel, built the same way around the stream of expert weights:
+//
+//   * One persistent workgroup of eight waves per CU takes an equal contiguous share of the launch's (task, 128 output
+//     channels) items, in task order; consecutive shares go to workgroups of one XCD.
+//   * K = 512 is two super-blocks. Wave w multiplies super-block w / 4 of the 32 output channels w % 4 of the item: its A
+//     operands, the task's <= 64 rows of h (halves of h / 256, by task slot) in those 256 columns, are loaded once per task
+//     into registers (64 or 128 VGPRs) and stay there while the expert's 2048 weight rows stream past.
+//   * A weight tile (32 rows x one super-block: 4 KB of low nibbles, 2 KB of high bit pairs, 512 B of sub-scales, the
+//     rows' d) comes global -> LDS directly into a wave-private ring of two stages, requested two tiles ahead by a cursor
+//     that runs across task boundaries. Nothing but these requests and the tile's stores uses the vector memory counter
+//     inside the loop, so every wait is an exact count.
+//   * The two waves that hold the two super-blocks of the same channels exchange the halves of their 32 x 32 f32 sums
+//     through LDS (one LDS-only barrier per 32 rows) and each finishes 16 rows: out = fma(d1, sum1, d0 * sum0) * scale,
+//     the order and the roundings of a sequential pass over the two super-blocks, whichever wave computes it.
+//   * Every lane stores, always: a row past the task's end repeats the task's first row, operands and destination alike
+//     (the same values to the same address), so the number of stores in flight is a constant too.
+#include "down_resident.hpp"
+#include "mfma_quant.hpp"
+
+#include <type_traits>
+
+using namespace tsp;
+
+namespace {
+
+constexpr int kWaves = 8, kThreads = kWaves * kWave;
+constexpr int kTaskRows = 64;
+// a stage: [32 rows x 128 B low nibbles][32 x 64 B high bits][32 x 16 B sub-scales][128 B of d: 32 rows x 2 super-blocks][pad]
+constexpr int kQlAt = 0, kQhAt = 4096, kScAt = 6144, kDAt = 6656, kStageBytes = 7168;
+constexpr int kStages = 2;
+constexpr int kTileLoads = 7;               // direct-to-LDS requests per tile and wave
+constexpr int kExchangeBytes = 2048;        // what a wave hands its partner per 32 rows: eight accumulators per lane
+constexpr int kPhaseBytes = kWaves * kExchangeBytes;
+
+struct TaskInfo { uint32_t expert, start, nrows; bool shared, ok; };
+
+__device__ __forceinline__ TaskInfo resolve_task(const ResidentDownArgs& a, uint32_t task) {
+    TaskInfo t;
+    t.expert = a.tasks[2 + 2 * task];
+    t.start = a.tasks[3 + 2 * task];
+    t.shared = a.shared_down != nullptr && t.expert == a.experts;
+    const uint32_t count = t.shared ? a.tokens : t.expert < a.experts ? a.counts[t.expert] : 0;
+    t.ok = (t.expert < a.experts || t.shared) && count <= a.tokens && t.start < count;
+    t.nrows = t.ok ? (count - t.start < kTaskRows ? count - t.start : kTaskRows) : 0;
+    if (!t.ok) { t.expert = 0; t.start = 0; t.shared = false; }  // addresses stay inside the tensors; its rows go to the spill row
+    return t;
+}
+
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void down_resident_kernel(ResidentDownArgs a) {
+    // LDS: [2 phases][8 waves][2 KB exchange] | [2 tasks][64 destination rows] | [8 waves][2 stages][7 KB weight tile]
+    constexpr int kRowsAt = 2 * kPhaseBytes, kStagesAt = kRowsAt + 2 * kTaskRows * 4;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kStagesAt + kWaves * kStages * kStageBytes];
+    uint32_t* const dst_rows = reinterpret_cast<uint32_t*>(lds_raw + kRowsAt);
+
+    const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const uint32_t kh = wave / 4, nq = wave % 4;  // super-block, channel tile of the item
+    constexpr uint32_t bpr = 2;                   // 512 columns
+    const uint32_t units = a.channels / 128;
+
+    const uint32_t bound = a.task_slots;
+    const uint32_t listed = a.tasks[0];
+    if (listed > bound || a.tasks[1] != a.tokens * a.selected || a.classes[0] + a.classes[1] != listed) {
+        if (tid == 0 && blockIdx.x == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+        return;
+    }
+    const uint32_t groups = gridDim.x, share = (blockIdx.x % 8) * (groups / 8) + blockIdx.x / 8;
+
+    uint8_t* const my_stage = lds_raw + kStagesAt + wave * (kStages * kStageBytes);
+    const uint32_t my_stage_lds = __builtin_amdgcn_readfirstlane(lds_address(my_stage));
+
+    // ---- per-lane parts of the request addresses, from the first byte of the expert (the per-tile parts are uniform)
+    // low nibbles: request q covers rows 8q .. 8q+7 of the tile, eight lanes per row (one 128-byte line: the row's super-block
+    // kh); lane l sits at 16-byte slot l % 8 of its row in LDS and fetches chunk (l % 8) ^ (row % 8)
+    const uint32_t ql_lane = uint32_t(a.spec.qs_offset) + (lane / 8) * (bpr * 128) + kh * 128 + (((lane % 8) ^ ((lane / 8) & 7)) * 16);
+    // high bits: request q covers rows 16q .. 16q+15, four lanes per row (64 bytes); slot l % 4 holds chunk (l % 4) ^ ((row / 4) % 4)
+    const uint32_t qh_lane = uint32_t(a.spec.qh_offset) + (lane / 4) * (bpr * 64) + kh * 64 + (((lane % 4) ^ ((lane / 16) & 3)) * 16);
+    // lanes 0..31: the sixteen sub-scales of row l; lanes 32..39: the 128 bytes of d of the tile's rows; the rest repeat lane 39
+    const uint32_t tail = lane < 40 ? lane - 32 : 7;
+    const uint32_t hdr_lane = lane < 32 ? uint32_t(a.spec.sm_offset) + lane * (bpr * 16) + kh * 16 : uint32_t(a.spec.dm_offset) + tail * 16;
+    const uint32_t hdr_tile_step = lane < 32 ? 32 * bpr * 16 : 32 * bpr * 2;
+
+    auto weight_base = [&](const TaskInfo& t) {
+        return t.shared ? a.shared_down : a.down + uint64_t(t.expert) * a.spec.planar_expert_bytes;
+    };
+    auto request_tile = [&](const uint8_t* base, uint32_t unit, uint32_t stage_offset) {  // base: one expert (under 4 GiB), uniform
+        const uint32_t tile = unit * 4 + nq;
+        const uint8_t* ql = base + uint64_t(tile) * (32 * bpr * 128);
+        const uint8_t* qh = base + uint64_t(tile) * (32 * bpr * 64);
+        const uint32_t dst = my_stage_lds + stage_offset;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) load_to_lds_16(ql + q * (8 * bpr * 128), ql_lane, dst + kQlAt + q * 1024);
+#pragma unroll
+        for (int q = 0; q < 2; ++q) load_to_lds_16(qh + q * (16 * bpr * 64), qh_lane, dst + kQhAt + q * 1024);
+        load_to_lds_16(base, hdr_lane + tile * hdr_tile_step, dst + kScAt);
+    };
+
+    uint32_t bad = 0, phase = 0, parity = 0;
+
+    auto pass = [&](auto mt_tag) {
+        constexpr int MT = decltype(mt_tag)::value;
+        const uint32_t of_kind = a.classes[MT - 1];
+        const uint32_t* list = a.classes + 2 + (MT - 1) * bound;
+        const uint32_t items = of_kind * units;
+        const uint32_t it0 = uint32_t(uint64_t(items) * share / groups), it1 = uint32_t(uint64_t(items) * (share + 1) / groups);
+        if (it0 >= it1) return;
+        const uint32_t k0 = it0 / units, k1 = (it1 - 1) / units;  // first and last position in the kind's list
+        auto first_unit = [&](uint32_t k) { return k == k0 ? it0 % units : 0; };
+        auto end_unit = [&](uint32_t k) { return k == k1 ? (it1 - 1) % units + 1 : units; };
+        auto task_at = [&](uint32_t k) { const uint32_t t = list[k]; return t < listed ? t : 0; };
+
+        f16x8 A[MT][16];  // h fragments: [row tile][section * 8 + quarter * 2 + fragment]
+        // ---- the request cursor runs two tiles ahead of the arithmetic: (list position, unit)
+        uint32_t rk = k0, runit = first_unit(k0), rstage = 0;
+        bool rdone = false;
+        const uint8_t* rbase = weight_base(resolve_task(a, task_at(k0)));
+        auto request_next = [&]() {  // past the end of the share the last tile is requested again (unused)
+            request_tile(rbase, runit, rstage);
+            rstage = rstage + kStageBytes == kStages * kStageBytes ? 0 : rstage + kStageBytes;
+            if (rdone) return;
+            if (runit + 1 < end_unit(rk)) { ++runit; return; }
+            if (rk == k1) { rdone = true; return; }
+            ++rk;
+            runit = 0;
+            rbase = weight_base(resolve_task(a, task_at(rk)));
+        };
+        request_next();
+        request_next();
+        uint32_t stage = 0;  // byte offset of the stage the next tile sits in
+
+        TaskInfo cur{};
+        uint8_t* out_base = nullptr;  // the rows the task's results go to, and their stride
+        uint64_t out_stride = 0;
+        auto load_rows = [&](uint32_t k) {  // the task at list position k: destination rows into LDS, this wave's 256 columns of its h rows into registers
+            const uint32_t task = task_at(k);
+            cur = resolve_task(a, task);
+            if (!cur.ok && tid == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+            out_base = reinterpret_cast<uint8_t*>(cur.shared ? a.shared_y : a.y);
+            out_stride = cur.shared ? a.shared_y_stride : a.y_stride;
+            const uint32_t n = lane % 32, khalf = lane / 32;
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                const uint32_t r = i * 32 + n, rr = r < cur.nrows ? r : 0;  // a row past the end repeats the first
+                const _Float16* row = a.hbuf + (uint64_t(task) * kTaskRows + rr) * (bpr * 256) + kh * 256 + khalf * 16;
+#pragma unroll
+                for (int t = 0; t < 16; ++t) A[i][t] = *reinterpret_cast<const f16x8*>(row + (t / 8) * 128 + ((t / 2) % 4) * 32 + (t % 2) * 8);
+            }
+            // lane l looks up where task row l goes: the route (or, for the always-on expert, the token) of row l
+            parity ^= 1;
+            const uint32_t rr = lane < cur.nrows ? lane : 0;
+            uint32_t dst;
+            if (cur.shared) {
+                dst = cur.start + rr;
+            } else {
+                const uint32_t rid = a.token_map[uint64_t(cur.expert) * a.tokens + cur.start + rr];
+                const bool ok = rid < a.tokens * a.selected && a.ids[rid < a.tokens * a.selected ? rid : 0] == cur.expert;
+                if (!ok && cur.ok) bad |= TSP_ERRBIT_INDEX;
+                dst = ok ? rid : 0xffffffffu;
+            }
+            if (!cur.ok) dst = 0xffffffffu;
+            dst_rows[parity * kTaskRows + lane] = dst;  // every wave keeps the table for itself: all eight write the same 64 words
+            // The rows are needed at once. Naming every fragment as an operand here makes the compiler wait for their loads now:
+            // left to itself it waits at the fragments' first uses inside the tile loop, in every pass of the loop, with counts
+            // that know nothing of the requests in flight and so drain them tile after tile.
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int t = 0; t < 16; ++t) asm volatile("" : "+v"(A[i][t]));
+        };
+
+        auto tile = [&](uint32_t unit) {
+            // wait for the tile's seven requests, which went out in the tile before last, ahead of that tile's stores: younger than
+            // they are those stores, the seven requests of the other stage and the stores of the tile before (everything
+            // completes in issue order; at a task's first tiles nothing older than the task's rows is outstanding at all)
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((kStages - 1) * kTileLoads + 16 * MT) : "memory");
+            uint32_t lane_now = lane;
+            if constexpr (MT == 2) asm volatile("" : "+v"(lane_now));  // lane-derived addresses are derived again per tile, not kept
+            const uint32_t n = lane_now % 32, khalf = (lane_now / 32) & 1;  // & 1: the compiler must see that khalf picks no sub-scale word
+            const uint8_t* st = my_stage + stage;
+            RawQ6 raw[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                raw[s].la = *reinterpret_cast<const u32x4*>(st + kQlAt + n * 128 + (((4 * s + khalf) ^ (n & 7)) * 16));
+                raw[s].lb = *reinterpret_cast<const u32x4*>(st + kQlAt + n * 128 + (((4 * s + 2 + khalf) ^ (n & 7)) * 16));
+                raw[s].qh = *reinterpret_cast<const u32x4*>(st + kQhAt + n * 64 + (((2 * s + khalf) ^ ((n >> 2) & 3)) * 16));
+            }
+            const uint4 sc = *reinterpret_cast<const uint4*>(st + kScAt + n * 16);
+            const uint32_t dd = *reinterpret_cast<const uint32_t*>(st + kDAt + n * 4);  // d of super-blocks 0 and 1 of row n
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            request_next();  // the stage is free again: the tile two ahead goes there
+            stage = stage + kStageBytes == kStages * kStageBytes ? 0 : stage + kStageBytes;
+            raw[0].sc[0] = sc.x; raw[0].sc[1] = sc.y; raw[1].sc[0] = sc.z; raw[1].sc[1] = sc.w;
+            const float d0 = half_bits_to_float(dd & 0xffffu), d1 = half_bits_to_float(dd >> 16);
+
+            f32x16 blk[MT];
+            auto quarter = [&](auto s_tag, auto q_tag) {
+                constexpr int S = decltype(s_tag)::value, Q = decltype(q_tag)::value;
+                f16x8 f[2];
+                frags_q6k<Q>(raw[S], khalf, f);
+#pragma unroll
+                for (int ff = 0; ff < 2; ++ff)
+#pragma unroll
+                    for (int i = 0; i < MT; ++i) {
+                        if (S == 0 && Q == 0 && ff == 0) {
+                            const f32x16 zero{};
+                            blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][0], f[0], zero, 0, 0, 0);
+                        } else {
+                            blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][S * 8 + Q * 2 + ff], f[ff], blk[i], 0, 0, 0);
+                        }
+                    }
+            };
+            quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+            quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
+            quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 2>{});
+            quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 3>{});
+            quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+            quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{});
+            quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{});
+            quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 3>{});
+
+            // Accumulator v of a 32 x 32 tile is row 8 (v / 4) + 4 khalf + v % 4, column n. The wave of super-block 0 finishes
+            // rows 0..15 (v < 8), its partner rows 16..31: each hands over the eight sums of the other's rows.
+            const uint32_t partner = wave ^ 4;
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                uint8_t* out = lds_raw + (phase & 1) * kPhaseBytes + wave * kExchangeBytes + lane_now * 16;
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    f32x4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = kh == 0 ? blk[i][8 + 4 * c + e] : blk[i][4 * c + e];
+                    *reinterpret_cast<f32x4*>(out + c * 1024) = v;
+                }
+                lds_barrier();
+                const uint8_t* in = lds_raw + (phase & 1) * kPhaseBytes + partner * kExchangeBytes + lane_now * 16;
+                ++phase;
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    const f32x4 theirs = *reinterpret_cast<const f32x4*>(in + c * 1024);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float mine = kh == 0 ? blk[i][4 * c + e] : blk[i][8 + 4 * c + e];
+                        const float sum0 = kh == 0 ? mine : theirs[e], sum1 = kh == 0 ? theirs[e] : mine;
+                        const float val = __builtin_fmaf(d1, sum1, d0 * sum0) * a.out_scale;
+                        if (nonfinite(val)) bad |= TSP_ERRBIT_NONFINITE;
+                        const uint32_t r = i * 32 + 16 * kh + 8 * c + 4 * khalf + e;
+                        const uint32_t dst = dst_rows[parity * kTaskRows + (r < cur.nrows ? r : 0)];
+                        float* row = dst == 0xffffffffu ? a.spill : reinterpret_cast<float*>(out_base + uint64_t(dst) * out_stride);
+                        row[(unit * 4 + nq) * 32 + n] = val;
+                    }
+                }
+            }
+        };
+
+        for (uint32_t k = k0; k <= k1; ++k) {
+            load_rows(k);
+            const uint32_t u1 = end_unit(k);
+            for (uint32_t unit = first_unit(k); unit < u1; ++unit) tile(unit);
+        }
+        wait_all_loads();  // the last requests fetched tiles nobody reads: they must have landed before the stages are reused or given away
+    };
+    pass(std::integral_constant<int, 2>{});
+    pass(std::integral_constant<int, 1>{});
+    publish_error(bad, a.error_word);
+}
+
+}  // namespace
+
+namespace tsp {
+
+bool resident_down_takes(uint32_t channels, uint32_t hidden) { return hidden == 512 && channels % 128 == 0 && channels >= 128; }
+
+int launch_resident_down(const ResidentDownArgs& a, hipStream_t s) {
+    static std::atomic<uint64_t> seen{0};
+    static int cus[64];
+    int device = 0;
+    if (first_use_on_device(seen, &device) || cus[device] == 0) {
+        int n = 0;
+        TSP_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device));
+        cus[device] = n >= 8 ? n / 8 * 8 : 8;
+    }
+    TSP_LAUNCH("gemm_down", s, down_resident_kernel<<<cus[device], kThreads, 0, s>>>(a));
+    return launch_status("down_resident");
+}
+
+}  // namespace tsp

@@ -179,6 +179,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                 for (int t = 0; t < 16; ++t) A[i][t] = *reinterpret_cast<const f16x8*>(row + (t / 4) * 64 + ((t / 2) % 2) * 32 + (t % 2) * 8);
                 sxA[i] = *reinterpret_cast<const f16x8*>(a.sx + (uint64_t(token[i]) * bpr + wave) * 16 + khalf * 8);
             }
+            // The rows are needed at once. Naming every fragment as an operand here makes the compiler wait for their loads now:
+            // left to itself it waits at the fragments' first uses inside the tile loop, in every pass of the loop, with counts
+            // that know nothing of the requests in flight and so drain them tile after tile.
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+#pragma unroll
+                for (int t = 0; t < 16; ++t) asm volatile("" : "+v"(A[i][t]));
+                asm volatile("" : "+v"(sxA[i]));
+            }
         };
 
         // ---- one tile: unpack, multiply, add the eight waves' partial results up, and for an up tile apply SwiGLU and store
