@@ -15,7 +15,10 @@
 //     through LDS (one LDS-only barrier per 32 rows) and each finishes 16 rows: out = fma(d1, sum1, d0 * sum0) * scale,
 //     the order and the roundings of a sequential pass over the two super-blocks, whichever wave computes it.
 //   * Every lane stores, always: a row past the task's end repeats the task's first row, operands and destination alike
-//     (the same values to the same address), so the number of stores in flight is a constant too.
+//     (the same values to the same address), so the number of stores in flight is a constant too. Where a lane's sixteen
+//     results go is worked out once per task (32-bit offsets from the output's first byte, a table in LDS), the share's
+//     tasks are looked up once per pass (a table in LDS), and the routes are those the gate/up product of the same call
+//     has already checked against the expert: inside the tile loop nothing is read from memory but weights.
 #include "down_resident.hpp"
 #include "mfma_quant.hpp"
 
@@ -33,6 +36,7 @@ constexpr int kStages = 2;
 constexpr int kTileLoads = 7;               // direct-to-LDS requests per tile and wave
 constexpr int kExchangeBytes = 2048;        // what a wave hands its partner per 32 rows: eight accumulators per lane
 constexpr int kPhaseBytes = kWaves * kExchangeBytes;
+constexpr uint32_t kInfoSlots = 32;         // tasks of a workgroup's share kept in LDS
 
 struct TaskInfo { uint32_t expert, start, nrows; bool shared, ok; };
 
@@ -49,10 +53,11 @@ __device__ __forceinline__ TaskInfo resolve_task(const ResidentDownArgs& a, uint
 }
 
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void down_resident_kernel(ResidentDownArgs a) {
-    // LDS: [2 phases][8 waves][2 KB exchange] | [2 tasks][64 destination rows] | [8 waves][2 stages][7 KB weight tile]
-    constexpr int kRowsAt = 2 * kPhaseBytes, kStagesAt = kRowsAt + 2 * kTaskRows * 4;
+    // LDS: [2 phases][8 waves][2 KB exchange] | [2 passes][32 tasks of the share] | [2 tasks][64 row offsets] | [8 waves][2 stages][7 KB weight tile]
+    constexpr int kInfoAt = 2 * kPhaseBytes, kRowsAt = kInfoAt + 2 * kInfoSlots * 16, kStagesAt = kRowsAt + 2 * kTaskRows * 4;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kStagesAt + kWaves * kStages * kStageBytes];
-    uint32_t* const dst_rows = reinterpret_cast<uint32_t*>(lds_raw + kRowsAt);
+    uint4* const info_tables = reinterpret_cast<uint4*>(lds_raw + kInfoAt);
+    uint32_t* const row_at = reinterpret_cast<uint32_t*>(lds_raw + kRowsAt);
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const uint32_t kh = wave / 4, nq = wave % 4;  // super-block, channel tile of the item
@@ -81,9 +86,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const uint32_t hdr_lane = lane < 32 ? uint32_t(a.spec.sm_offset) + lane * (bpr * 16) + kh * 16 : uint32_t(a.spec.dm_offset) + tail * 16;
     const uint32_t hdr_tile_step = lane < 32 ? 32 * bpr * 16 : 32 * bpr * 2;
 
-    auto weight_base = [&](const TaskInfo& t) {
-        return t.shared ? a.shared_down : a.down + uint64_t(t.expert) * a.spec.planar_expert_bytes;
-    };
     auto request_tile = [&](const uint8_t* base, uint32_t unit, uint32_t stage_offset) {  // base: one expert (under 4 GiB), uniform
         const uint32_t tile = unit * 4 + nq;
         const uint8_t* ql = base + uint64_t(tile) * (32 * bpr * 128);
@@ -97,6 +99,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     };
 
     uint32_t bad = 0, phase = 0, parity = 0;
+    uint32_t biggest = 0;  // the largest result's bits without the sign: anything not finite shows at the end
+    const float s256 = a.out_scale;
 
     auto pass = [&](auto mt_tag) {
         constexpr int MT = decltype(mt_tag)::value;
@@ -108,13 +112,41 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         const uint32_t k0 = it0 / units, k1 = (it1 - 1) / units;  // first and last position in the kind's list
         auto first_unit = [&](uint32_t k) { return k == k0 ? it0 % units : 0; };
         auto end_unit = [&](uint32_t k) { return k == k1 ? (it1 - 1) % units + 1 : units; };
-        auto task_at = [&](uint32_t k) { const uint32_t t = list[k]; return t < listed ? t : 0; };
 
-        f16x8 A[MT][16];  // h fragments: [row tile][section * 8 + quarter * 2 + fragment]
+        // ---- the share's tasks, looked up once: (task, expert, first row, rows | shared << 8 | ok << 9) per list position, in
+        // LDS. Every wave writes the whole table for itself (the same words), so nothing inside the tile loop reads task lists
+        // from memory: a vector load there would have the compiler drain the requests in flight before it goes on.
+        uint4* const info = info_tables + (MT - 1) * kInfoSlots;  // a table per pass: a wave may start the second pass while others finish the first
+        if (lane < kInfoSlots && k0 + lane <= k1) {
+            const uint32_t listed_task = list[k0 + lane], task = listed_task < listed ? listed_task : 0;
+            const TaskInfo t = resolve_task(a, task);
+            if (!t.ok) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+            info[lane] = uint4{task, t.expert, t.start, t.nrows | (t.shared ? 256u : 0u) | (t.ok ? 512u : 0u)};
+        }
+        struct Info { uint32_t task, expert, start, nrows; bool shared, ok; };
+        auto info_at = [&](uint32_t k) {  // uniform
+            uint4 v;
+            if (k - k0 < kInfoSlots) {
+                v = info[k - k0];
+            } else {  // a share of more tasks than the table holds: the slow way
+                const uint32_t listed_task = list[k], task = listed_task < listed ? listed_task : 0;
+                const TaskInfo t = resolve_task(a, task);
+                v = uint4{task, t.expert, t.start, t.nrows | (t.shared ? 256u : 0u) | (t.ok ? 512u : 0u)};
+            }
+            Info r;
+            r.task = __builtin_amdgcn_readfirstlane(v.x); r.expert = __builtin_amdgcn_readfirstlane(v.y);
+            r.start = __builtin_amdgcn_readfirstlane(v.z);
+            const uint32_t w = __builtin_amdgcn_readfirstlane(v.w);
+            r.nrows = w & 255u; r.shared = (w & 256u) != 0; r.ok = (w & 512u) != 0;
+            return r;
+        };
+        auto weight_base_of = [&](const Info& t) { return t.shared ? a.shared_down : a.down + uint64_t(t.expert) * a.spec.planar_expert_bytes; };
+
+        f16x8 A[MT][16];        // h fragments: [row tile][section * 8 + quarter * 2 + fragment]
         // ---- the request cursor runs two tiles ahead of the arithmetic: (list position, unit)
         uint32_t rk = k0, runit = first_unit(k0), rstage = 0;
         bool rdone = false;
-        const uint8_t* rbase = weight_base(resolve_task(a, task_at(k0)));
+        const uint8_t* rbase = weight_base_of(info_at(k0));
         auto request_next = [&]() {  // past the end of the share the last tile is requested again (unused)
             request_tile(rbase, runit, rstage);
             rstage = rstage + kStageBytes == kStages * kStageBytes ? 0 : rstage + kStageBytes;
@@ -123,43 +155,40 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             if (rk == k1) { rdone = true; return; }
             ++rk;
             runit = 0;
-            rbase = weight_base(resolve_task(a, task_at(rk)));
+            rbase = weight_base_of(info_at(rk));
         };
         request_next();
         request_next();
         uint32_t stage = 0;  // byte offset of the stage the next tile sits in
 
-        TaskInfo cur{};
-        uint8_t* out_base = nullptr;  // the rows the task's results go to, and their stride
-        uint64_t out_stride = 0;
-        auto load_rows = [&](uint32_t k) {  // the task at list position k: destination rows into LDS, this wave's 256 columns of its h rows into registers
-            const uint32_t task = task_at(k);
-            cur = resolve_task(a, task);
-            if (!cur.ok && tid == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+        uint8_t* out_base = nullptr;  // the rows the task's results go to
+        auto load_rows = [&](uint32_t k) {  // the task at list position k: this wave's 256 columns of its h rows, and where its results go
+            const Info cur = info_at(k);
             out_base = reinterpret_cast<uint8_t*>(cur.shared ? a.shared_y : a.y);
-            out_stride = cur.shared ? a.shared_y_stride : a.y_stride;
+            const uint32_t out_stride = uint32_t(cur.shared ? a.shared_y_stride : a.y_stride);
             const uint32_t n = lane % 32, khalf = lane / 32;
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
                 const uint32_t r = i * 32 + n, rr = r < cur.nrows ? r : 0;  // a row past the end repeats the first
-                const _Float16* row = a.hbuf + (uint64_t(task) * kTaskRows + rr) * (bpr * 256) + kh * 256 + khalf * 16;
+                const _Float16* row = a.hbuf + (uint64_t(cur.task) * kTaskRows + rr) * (bpr * 256) + kh * 256 + khalf * 16;
 #pragma unroll
                 for (int t = 0; t < 16; ++t) A[i][t] = *reinterpret_cast<const f16x8*>(row + (t / 8) * 128 + ((t / 2) % 4) * 32 + (t % 2) * 8);
             }
-            // lane l looks up where task row l goes: the route (or, for the always-on expert, the token) of row l
-            parity ^= 1;
+            // Lane l looks up where task row l goes: its route (for the always-on expert its token). The gate/up product of
+            // the same call has checked every route against the expert; here the index only has to stay inside the output.
             const uint32_t rr = lane < cur.nrows ? lane : 0;
             uint32_t dst;
             if (cur.shared) {
                 dst = cur.start + rr;
             } else {
-                const uint32_t rid = a.token_map[uint64_t(cur.expert) * a.tokens + cur.start + rr];
-                const bool ok = rid < a.tokens * a.selected && a.ids[rid < a.tokens * a.selected ? rid : 0] == cur.expert;
-                if (!ok && cur.ok) bad |= TSP_ERRBIT_INDEX;
-                dst = ok ? rid : 0xffffffffu;
+                dst = a.token_map[uint64_t(cur.expert) * a.tokens + cur.start + rr];
+                if (dst >= a.tokens * a.selected) { if (cur.ok) bad |= TSP_ERRBIT_INDEX; dst = 0; }
             }
-            if (!cur.ok) dst = 0xffffffffu;
-            dst_rows[parity * kTaskRows + lane] = dst;  // every wave keeps the table for itself: all eight write the same 64 words
+            if (!cur.ok) dst = 0;  // a task that does not check out is flagged; the batch is refused whatever lands in row 0
+            // where the 64 task rows go, as byte offsets from the output's first byte: a table per wave (all eight write the same
+            // words, each reads its own), two of them in turn because a wave may be a task ahead of its partner's last reads
+            parity ^= 1;
+            row_at[parity * kTaskRows + lane] = dst * out_stride;  // a row past the end has looked up the first row's
             // The rows are needed at once. Naming every fragment as an operand here makes the compiler wait for their loads now:
             // left to itself it waits at the fragments' first uses inside the tile loop, in every pass of the loop, with counts
             // that know nothing of the requests in flight and so drain them tile after tile.
@@ -191,7 +220,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             request_next();  // the stage is free again: the tile two ahead goes there
             stage = stage + kStageBytes == kStages * kStageBytes ? 0 : stage + kStageBytes;
             raw[0].sc[0] = sc.x; raw[0].sc[1] = sc.y; raw[1].sc[0] = sc.z; raw[1].sc[1] = sc.w;
-            const float d0 = half_bits_to_float(dd & 0xffffu), d1 = half_bits_to_float(dd >> 16);
+            // the output scale is a power of two: folded into d it changes no rounding
+            const float d0 = half_bits_to_float(dd & 0xffffu) * s256, d1 = half_bits_to_float(dd >> 16) * s256;
 
             f32x16 blk[MT];
             auto quarter = [&](auto s_tag, auto q_tag) {
@@ -220,37 +250,46 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 3>{});
 
             // Accumulator v of a 32 x 32 tile is row 8 (v / 4) + 4 khalf + v % 4, column n. The wave of super-block 0 finishes
-            // rows 0..15 (v < 8), its partner rows 16..31: each hands over the eight sums of the other's rows.
-            const uint32_t partner = wave ^ 4;
+            // rows 0..15 (v < 8), its partner rows 16..31: each hands over the eight sums of the other's rows. Which of the two a
+            // wave is, is a scalar: one branch per tile instead of a select per value.
+            uint8_t* const tile_base = out_base + (unit * 4 + nq) * 128;  // uniform
+            auto finish = [&](auto kh_tag) {
+                constexpr int KH = decltype(kh_tag)::value;
 #pragma unroll
-            for (int i = 0; i < MT; ++i) {
-                uint8_t* out = lds_raw + (phase & 1) * kPhaseBytes + wave * kExchangeBytes + lane_now * 16;
+                for (int i = 0; i < MT; ++i) {
+                    uint8_t* out = lds_raw + (phase & 1) * kPhaseBytes + wave * kExchangeBytes + lane_now * 16;
 #pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    f32x4 v;
+                    for (int c = 0; c < 2; ++c) {
+                        f32x4 v;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = kh == 0 ? blk[i][8 + 4 * c + e] : blk[i][4 * c + e];
-                    *reinterpret_cast<f32x4*>(out + c * 1024) = v;
-                }
-                lds_barrier();
-                const uint8_t* in = lds_raw + (phase & 1) * kPhaseBytes + partner * kExchangeBytes + lane_now * 16;
-                ++phase;
+                        for (int e = 0; e < 4; ++e) v[e] = blk[i][8 * (1 - KH) + 4 * c + e];
+                        *reinterpret_cast<f32x4*>(out + c * 1024) = v;
+                    }
+                    lds_barrier();
+                    const uint8_t* in = lds_raw + (phase & 1) * kPhaseBytes + (wave ^ 4) * kExchangeBytes + lane_now * 16;
+                    ++phase;
 #pragma unroll
-                for (int c = 0; c < 2; ++c) {
-                    const f32x4 theirs = *reinterpret_cast<const f32x4*>(in + c * 1024);
+                    for (int c = 0; c < 2; ++c) {
+                        const f32x4 theirs = *reinterpret_cast<const f32x4*>(in + c * 1024);
+                        // accumulator 4 c + e of the wave's half of the row tile is task row 32 i + 16 KH + 8 c + 4 khalf + e
+                        const u32x4 to = *reinterpret_cast<const u32x4*>(&row_at[parity * kTaskRows + i * 32 + 16 * KH + 8 * c + 4 * khalf]);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float mine = kh == 0 ? blk[i][4 * c + e] : blk[i][8 + 4 * c + e];
-                        const float sum0 = kh == 0 ? mine : theirs[e], sum1 = kh == 0 ? theirs[e] : mine;
-                        const float val = __builtin_fmaf(d1, sum1, d0 * sum0) * a.out_scale;
-                        if (nonfinite(val)) bad |= TSP_ERRBIT_NONFINITE;
-                        const uint32_t r = i * 32 + 16 * kh + 8 * c + 4 * khalf + e;
-                        const uint32_t dst = dst_rows[parity * kTaskRows + (r < cur.nrows ? r : 0)];
-                        float* row = dst == 0xffffffffu ? a.spill : reinterpret_cast<float*>(out_base + uint64_t(dst) * out_stride);
-                        row[(unit * 4 + nq) * 32 + n] = val;
+                        for (int e = 0; e < 4; ++e) {
+                            const float mine = blk[i][8 * KH + 4 * c + e];
+                            const float sum0 = KH == 0 ? mine : theirs[e], sum1 = KH == 0 ? theirs[e] : mine;
+                            const float val = __builtin_fmaf(d1, sum1, d0 * sum0);
+                            const uint32_t magnitude = __float_as_uint(val) & 0x7fffffffu;
+                            biggest = biggest > magnitude ? biggest : magnitude;
+                            // uniform base + 32-bit lane offset, spelled out: the compiler would form 64-bit addresses
+                            const uint32_t at = to[e] + n * 4;
+                            uint8_t* const base = tile_base;
+                            asm volatile("global_store_dword %0, %1, %2" ::"v"(at), "v"(val), "s"(base) : "memory");
+                        }
                     }
                 }
-            }
+            };
+            if (kh == 0) finish(std::integral_constant<int, 0>{});
+            else finish(std::integral_constant<int, 1>{});
         };
 
         for (uint32_t k = k0; k <= k1; ++k) {
@@ -262,6 +301,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     };
     pass(std::integral_constant<int, 2>{});
     pass(std::integral_constant<int, 1>{});
+    if (biggest >= 0x7f800000u) bad |= TSP_ERRBIT_NONFINITE;
     publish_error(bad, a.error_word);
 }
 

@@ -16,12 +16,11 @@ struct ResidentDownArgs {
     const uint32_t* token_map;
     const uint32_t* ids;
     uint32_t task_slots;
-    float* y;                    // [tokens * selected] rows by route, y_stride bytes apart
+    float* y;                    // [tokens * selected] rows by route, y_stride bytes apart; the whole output spans less than 4 GiB
     uint64_t y_stride;
     float* shared_y;             // the always-on expert's rows by token
     uint64_t shared_y_stride;
     float out_scale;             // 256: undoes the 2^-8 that h carries
-    float* spill;                // `channels` floats that take the rows of a task whose list entry or routes do not check out
     uint32_t* error_word;
 };
 
