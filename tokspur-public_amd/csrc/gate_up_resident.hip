@@ -41,6 +41,7 @@ constexpr int kStages = 2;
 constexpr int kPartialBytes = 4096;        // one wave's 32 x 32 f32 partial tile
 constexpr int kPhaseBytes = kWaves * kPartialBytes;
 constexpr int kTileLoads = 5;              // direct-to-LDS requests per tile and wave
+constexpr uint32_t kInfoSlots = 32;        // tasks of a workgroup's share kept in LDS, per pass
 
 struct TaskInfo { uint32_t expert, start, nrows; bool shared, ok; };
 
@@ -57,9 +58,10 @@ __device__ __forceinline__ TaskInfo resolve_task(const ResidentGateUpArgs& a, ui
 }
 
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gate_up_resident_kernel(ResidentGateUpArgs a) {
-    // LDS: [2 phases][8 waves][4 KB partial tile] | [8 waves][2 stages][5 KB weight tile]
-    constexpr int kStagesAt = 2 * kPhaseBytes;
+    // LDS: [2 phases][8 waves][4 KB partial tile] | [2 passes][32 tasks of the share] | [8 waves][2 stages][5 KB weight tile]
+    constexpr int kInfoAt = 2 * kPhaseBytes, kStagesAt = kInfoAt + 2 * kInfoSlots * 16;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kStagesAt + kWaves * kStages * kStageBytes];
+    uint4* const info_tables = reinterpret_cast<uint4*>(lds_raw + kInfoAt);
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const uint32_t n = lane % 32, khalf = lane / 32;
@@ -88,7 +90,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                                         : uint32_t(a.spec.dm_offset) + (lane - 32) * (bpr * 4) + (wave / 4) * 16;
     const uint32_t hdr_unit_step = lane < 32 ? 32 * bpr * 16 : 32 * bpr * 4;
 
-    auto weight_bases = [&](const TaskInfo& t, const uint8_t*& gate, const uint8_t*& up) {
+    struct Info { uint32_t task, expert, start, nrows; bool shared, ok; };
+    auto weight_bases = [&](const Info& t, const uint8_t*& gate, const uint8_t*& up) {
         if (t.shared) { gate = a.shared_gate; up = a.shared_up; return; }
         const uint32_t half_e = a.experts / 2;
         const uint8_t* pair = (t.expert < half_e ? a.pair_lo : a.pair_hi) + uint64_t(t.expert < half_e ? t.expert : t.expert - half_e) * 2 * a.spec.planar_expert_bytes;
@@ -104,6 +107,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     };
 
     uint32_t bad = 0, phase = 0;
+    uint32_t biggest = 0;  // the largest carried half's bits without the sign: anything not finite shows at the end
     const Q4Consts q4c = q4_consts();
     const Q4ScaleConsts q4s = q4_scale_consts();
 
@@ -120,7 +124,30 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         const uint32_t k0 = it0 / units, k1 = (it1 - 1) / units;  // first and last position in the kind's list
         auto first_unit = [&](uint32_t k) { return k == k0 ? it0 % units : 0; };
         auto end_unit = [&](uint32_t k) { return k == k1 ? (it1 - 1) % units + 1 : units; };
-        auto task_at = [&](uint32_t k) { const uint32_t t = list[k]; return t < listed ? t : 0; };
+        // ---- the share's tasks, looked up once: (task, expert, first row, rows | shared << 8 | ok << 9) per list position, in
+        // LDS. Every wave writes the whole table for itself (the same words), so nothing inside the tile loop reads task lists
+        // from memory: a vector load there would have the compiler drain the requests in flight before it goes on. A table per
+        // pass: a wave may start the second pass while others finish the first.
+        uint4* const info = info_tables + (MT - 1) * kInfoSlots;
+        auto packed_info = [&](uint32_t k) {
+            const uint32_t listed_task = list[k], task = listed_task < listed ? listed_task : 0;
+            const TaskInfo t = resolve_task(a, task);
+            return uint4{task, t.expert, t.start, t.nrows | (t.shared ? 256u : 0u) | (t.ok ? 512u : 0u)};
+        };
+        if (lane < kInfoSlots && k0 + lane <= k1) {
+            const uint4 v = packed_info(k0 + lane);
+            if (!(v.w & 512u)) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+            info[lane] = v;
+        }
+        auto info_at = [&](uint32_t k) {  // uniform
+            const uint4 v = k - k0 < kInfoSlots ? info[k - k0] : packed_info(k);  // a share of more tasks than the table holds: the slow way
+            Info r;
+            r.task = __builtin_amdgcn_readfirstlane(v.x); r.expert = __builtin_amdgcn_readfirstlane(v.y);
+            r.start = __builtin_amdgcn_readfirstlane(v.z);
+            const uint32_t w = __builtin_amdgcn_readfirstlane(v.w);
+            r.nrows = w & 255u; r.shared = (w & 256u) != 0; r.ok = (w & 512u) != 0;
+            return r;
+        };
 
         f16x8 A[MT][16];   // activation fragments: [row tile][k16 step of the super-block]
         f16x8 sxA[MT];     // activation sums (k-half 0: the eight sub-block sums' high halves, k-half 1: the residuals)
@@ -128,7 +155,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         uint32_t rk = k0, runit = first_unit(k0), rj = 0, rstage = 0;
         bool rdone = false;
         const uint8_t *rgate, *rup;
-        weight_bases(resolve_task(a, task_at(k0)), rgate, rup);
+        weight_bases(info_at(k0), rgate, rup);
         auto request_next = [&]() {  // past the end of the share the last tile is requested again (unused)
             request_tile(rj == 0 ? rgate : rup, runit, rstage);
             rstage = rstage + kStageBytes == kStages * kStageBytes ? 0 : rstage + kStageBytes;
@@ -139,46 +166,42 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             ++rk;
             rj = 0;
             runit = 0;
-            weight_bases(resolve_task(a, task_at(rk)), rgate, rup);
+            weight_bases(info_at(rk), rgate, rup);
         };
         request_next();
         request_next();
         uint32_t stage = 0;  // byte offset of the stage the next tile sits in
 
         uint32_t task = 0;
-        TaskInfo cur{};
         auto load_rows = [&](uint32_t k) {  // the task at list position k: its activation rows, this wave's 256 columns of them, into registers
-            task = task_at(k);
-            cur = resolve_task(a, task);
-            if (!cur.ok && tid == 0) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
-            // first every row's token (two dependent look-ups), then all the row loads at once
-            uint32_t token[MT];
+            const Info cur = info_at(k);
+            task = cur.task;
+            // every row's route first, then, side by side, the route's expert (checked against the task's) and the row of the
+            // route's token: two round trips, not three
+            uint32_t rid[MT], token[MT];
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
                 const uint32_t r = i * 32 + n, rr = r < cur.nrows ? r : 0;
-                token[i] = cur.shared ? cur.start + rr : a.token_map[uint64_t(cur.expert) * a.tokens + cur.start + rr];
+                rid[i] = cur.shared ? 0 : a.token_map[uint64_t(cur.expert) * a.tokens + cur.start + rr];
+                token[i] = cur.shared ? cur.start + rr : rid[i] / a.selected;
+                // A row past the task's end repeats its first row, and a route outside the batch stands in for token 0 (the batch is
+                // refused): their h lands in slots of the task's 64 that nobody reads. So every lane stores, every wave issues the
+                // same number of stores per unit, and the waits below can count them.
+                if (!cur.shared && rid[i] >= a.tokens * a.selected) { rid[i] = 0; token[i] = 0; if (cur.ok) bad |= TSP_ERRBIT_INDEX; }
+                if (!cur.ok) token[i] = 0;
             }
+            uint32_t owner[MT];
 #pragma unroll
             for (int i = 0; i < MT; ++i) {
-                bool ok = true;
-                if (!cur.shared) {
-                    const uint32_t rid = token[i];
-                    ok = rid < a.tokens * a.selected && a.ids[rid < a.tokens * a.selected ? rid : 0] == cur.expert;
-                    token[i] = ok ? rid / a.selected : 0;
-                }
-                // A row past the task's end repeats its first row and a row whose route does not check out stands in for token
-                // 0: their h lands in slots of the task's 64 that nobody reads, or the batch is refused. So every lane stores,
-                // every wave issues the same number of stores per unit, and the waits below can count them.
-                if (!cur.ok) { token[i] = 0; ok = false; }
-                if (!ok && cur.ok) bad |= TSP_ERRBIT_INDEX;
-            }
-#pragma unroll
-            for (int i = 0; i < MT; ++i) {
+                owner[i] = cur.shared ? cur.expert : a.ids[rid[i]];
                 const _Float16* row = a.xh + uint64_t(token[i]) * (bpr * 256) + wave * 256 + khalf * 16;
 #pragma unroll
                 for (int t = 0; t < 16; ++t) A[i][t] = *reinterpret_cast<const f16x8*>(row + (t / 4) * 64 + ((t / 2) % 2) * 32 + (t % 2) * 8);
                 sxA[i] = *reinterpret_cast<const f16x8*>(a.sx + (uint64_t(token[i]) * bpr + wave) * 16 + khalf * 8);
             }
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                if (owner[i] != cur.expert && cur.ok) bad |= TSP_ERRBIT_INDEX;  // a route that is not the expert's: the batch is refused
             // The rows are needed at once. Naming every fragment as an operand here makes the compiler wait for their loads now:
             // left to itself it waits at the fragments' first uses inside the tile loop, in every pass of the loop, with counts
             // that know nothing of the requests in flight and so drain them tile after tile.
@@ -277,10 +300,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                         const uint32_t r = i * 32 + 4 * wave + 2 * (lane_now % 2) + e;
                         const float g = gate_sum[i][e], u = up_sum[e];
                         const float h = (g * sigmoid_fast(g)) * u;
-                        // h travels to the down GEMM as the half nearest to h * 2^-8
+                        // h travels to the down GEMM as the half nearest to h * 2^-8. A gate or up sum that is not finite, or a
+                        // product too large for a half, leaves an infinity or a NaN here, and only here is it looked for.
                         const _Float16 carried = _Float16(h * 0.00390625f);
-                        if (nonfinite(g) || nonfinite(u) || nonfinite(h) || (__builtin_bit_cast(uint16_t, carried) & 0x7c00u) == 0x7c00u) bad |= TSP_ERRBIT_NONFINITE;
-                        a.hbuf[(uint64_t(task) * kTaskRows + r) * a.hidden + unit * 32 + lane_now / 2] = carried;
+                        const uint32_t bits = __builtin_bit_cast(uint16_t, carried), magnitude = bits & 0x7fffu;
+                        biggest = biggest > magnitude ? biggest : magnitude;
+                        // uniform base (the task's slots, the unit's columns) + 32-bit lane offset, spelled out: the compiler would
+                        // form a 64-bit address per store
+                        const uint32_t at = (r * a.hidden + lane_now / 2) * 2;
+                        const _Float16* const base = a.hbuf + (uint64_t(task) * kTaskRows) * a.hidden + unit * 32;
+                        asm volatile("global_store_short %0, %1, %2" ::"v"(at), "v"(bits), "s"(base) : "memory");
                     }
                 }
             }
@@ -298,6 +327,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     };
     pass(std::integral_constant<int, 2>{});
     pass(std::integral_constant<int, 1>{});
+    if (biggest >= 0x7c00u) bad |= TSP_ERRBIT_NONFINITE;
     publish_error(bad, a.error_word);
 }
 
