@@ -357,6 +357,72 @@ def test_grouped_moe_2048_columns(gpu, tsp, orc, synth, n, hidden, experts, sele
         assert gpu.error() == 0 and np.array_equal(clean.view(np.uint32), y.view(np.uint32))
 
 
+@pytest.mark.parametrize("n,channels,experts,selected", [(1, 256, 4, 2), (33, 768, 6, 3), (96, 256, 8, 4), (300, 256, 4, 2), (700, 256, 2, 1),
+                                                         (130, 1024, 8, 2)])
+def test_grouped_moe_512_hidden_units(gpu, tsp, orc, synth, n, channels, experts, selected):
+    """Experts of 512 hidden units take the down kernel that keeps a task's h rows in registers and streams the Q6_K tiles
+    past them (two waves per tile, one per super-block): empty experts, tasks of 1..32 and 33..64 rows, experts of several
+    tasks, fewer items than workgroups and more, gate/up kernels that leave the unused slots of a task unwritten (widths
+    other than 2048), rows with padding (canaries stay), the always-on expert riding along (the routed rows' bits must
+    not change, its rows must equal a separate call's bits), sticky errors, against the CPU composition at the kernels'
+    declared precision."""
+    hidden = 512
+    gate = synth.matrix(12, 3501, hidden * experts, channels)
+    up = synth.matrix(12, 3502, hidden * experts, channels)
+    down = synth.matrix(14, 3503, channels * experts, hidden)
+    w = tsp.PlanarMoeWeights(gpu, 12, 14, channels, hidden, experts, gate, up, down)
+    ids = reference_ids(n, selected, experts).reshape(n, selected)
+    for t in range(n):  # each token's experts distinct; expert 1 stays empty when there are more than four
+        seen = set()
+        for s in range(selected):
+            e = int(ids[t, s])
+            while e in seen or (experts > 4 and e == 1):
+                e = (e + 1) % experts
+            seen.add(e)
+            ids[t, s] = e
+    ids = ids.reshape(-1)
+    x = synth.round_bf16(synth.activations_f32(3504 + n, (n, channels)))
+    d_ids, d_x = gpu.upload(ids), gpu.upload(x)
+    scratch = tsp.GroupedScratch(gpu, n, selected, experts, channels, hidden)
+    padded = gpu.full((n * selected, channels + 4), -6.0)
+    tsp.planar_nax_grouped_moe(gpu, w, d_ids, d_x, n, selected, scratch, y=padded, y_stride=(channels + 4) * 4)
+    assert gpu.error() == 0
+    got = padded.cpu().numpy()
+    assert (got[:, channels:] == -6.0).all()
+    y = np.ascontiguousarray(got[:, :channels])
+    _, declared = orc.moe_routed_reference(12, 14, gate, up, down, channels, hidden, experts, ids, n, selected, x, stage=12, threads=8)
+    _, plain = orc.moe_routed_reference(12, 14, gate, up, down, channels, hidden, experts, ids, n, selected, x, stage=0, threads=8)
+    scale = np.maximum(1.0, np.sqrt((declared ** 2).mean(axis=1, keepdims=True)))
+    err = np.abs(y - declared) / np.maximum(scale, np.abs(declared))
+    assert float(np.median(err)) <= 2e-5 and float(err.max()) <= 4e-3 and nmse(y, declared) <= 1e-7 and nmse(y, plain) <= 1e-5
+    again = tsp.planar_nax_grouped_moe(gpu, w, d_ids, d_x, n, selected, scratch).cpu().numpy()
+    assert np.array_equal(again.view(np.uint32), y.view(np.uint32))  # packed rows, the same bits
+    sg, su, sd = synth.matrix(12, 3505, hidden, channels), synth.matrix(12, 3506, hidden, channels), synth.matrix(14, 3507, channels, hidden)
+    shared = tsp.PlanarSharedExpert(gpu, channels, hidden, sg, su, sd)
+    riding = tsp.GroupedScratch(gpu, n, selected, experts, channels, hidden, with_shared=True)
+    y2, ys = tsp.planar_nax_grouped_moe(gpu, w, d_ids, d_x, n, selected, riding, shared=shared)
+    assert gpu.error() == 0
+    assert np.array_equal(y2.cpu().numpy().view(np.uint32), y.view(np.uint32))
+    alone = tsp.PlanarMoeWeights(gpu, 12, 14, channels, hidden, 2, np.concatenate([sg, sg]), np.concatenate([su, su]), np.concatenate([sd, sd]))
+    separate = tsp.planar_nax_grouped_moe(gpu, alone, gpu.upload(np.zeros(n, dtype=np.uint32)), d_x, n, 1,
+                                          tsp.GroupedScratch(gpu, n, 1, 2, channels, hidden)).cpu().numpy()
+    assert np.array_equal(ys.cpu().numpy().view(np.uint32), separate.view(np.uint32))
+    _, want_s = orc.moe_routed_reference(12, 14, sg, su, sd, channels, hidden, 1, np.zeros(n, dtype=np.uint32), n, 1, x, stage=12, threads=8)
+    assert max_rel_error(separate, want_s) <= 4e-3 and nmse(separate, want_s) <= 1e-7
+    if n >= 33 and selected >= 2:
+        for poison in ([0, 0], [0, experts + 3]):
+            broken = ids.copy()
+            broken[10 * selected:10 * selected + 2] = poison
+            tsp.planar_nax_grouped_moe(gpu, w, gpu.upload(broken), d_x, n, selected, scratch)
+            assert gpu.error() & tsp.ERRBIT_INDEX
+        nan = x.copy()
+        nan[5, channels - 3] = np.nan
+        tsp.planar_nax_grouped_moe(gpu, w, d_ids, gpu.upload(nan), n, selected, scratch)
+        assert gpu.error() & tsp.ERRBIT_NONFINITE
+        clean = tsp.planar_nax_grouped_moe(gpu, w, d_ids, d_x, n, selected, scratch).cpu().numpy()
+        assert gpu.error() == 0 and np.array_equal(clean.view(np.uint32), y.view(np.uint32))
+
+
 @pytest.mark.parametrize("n", [1, 33, 70, 200])
 def test_grouped_moe_with_always_on_expert(gpu, tsp, orc, synth, n):
     """The layer's always-on expert riding in the grouped launches (every token is a row of it): the routed rows are the
