@@ -394,11 +394,12 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
                 return *reinterpret_cast<const u32x4*>(my_w + wbuf * 4096 + ((j * 32 + col) * 4 + ((2 * p2 + khalf) ^ ((col >> 1) & 3))) * 16);
             };
             const Q4Consts q4c = q4_consts();
-            HdrQ4 hdr[2], hdr_next[2];
+            HdrQ4 hdr[2];
+            RawHdrQ4 hdr_next[2];  // requested at P == 2, decoded at the end of P == 3: nothing touches the bytes while they travel
     #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                hdr[j] = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, 0);
-                hdr_next[j] = hdr[j];
+                hdr_next[j] = fetch_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, 0);
+                hdr[j] = decode_hdr_q4k<BKIND>(hdr_next[j]);
             }
             fetch_w_all(0);
             store_w(0);
@@ -419,7 +420,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
                 if (P == 0 || P == 2) fetch_w_all(step / 2 + 1);
                 if (P == 2) {
     #pragma unroll
-                    for (int j = 0; j < 2; ++j) hdr_next[j] = load_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, b + 1 < bpr ? b + 1 : b);
+                    for (int j = 0; j < 2; ++j) hdr_next[j] = fetch_hdr_q4k<BKIND>(wbase[j], a.spec, wrow[j], bpr, b + 1 < bpr ? b + 1 : b);
                 }
                 const u32x4 raw0 = read_w(wbuf, 0, P & 1), raw1 = read_w(wbuf, 1, P & 1);
                 f16x8 f0[2], f1[2];
@@ -446,7 +447,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kernel(GemmArgs a) {  // two work
                 }
                 if (P == 1) store_sx((b + 1) & 1);  // read at P == 3 of the next super-block; the buffer was last read at P == 3 of the one before
                 if (P == 1 || P == 3) store_w(wbuf ^ 1);  // read again two barriers from now; this buffer was last read a step ago
-                if (P == 3) { hdr[0] = hdr_next[0]; hdr[1] = hdr_next[1]; }
+                if (P == 3) { hdr[0] = decode_hdr_q4k<BKIND>(hdr_next[0]); hdr[1] = decode_hdr_q4k<BKIND>(hdr_next[1]); }
             };
             wait_all_loads();  // slabs 0 and 1 (the stores above already waited for younger loads)
             for (uint32_t b = 0; b < bpr; ++b) {

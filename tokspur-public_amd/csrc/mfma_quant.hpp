@@ -68,17 +68,34 @@ __device__ __forceinline__ f16x8 scaled8_q6(uint32_t c0, uint32_t c1, f16x2 sc, 
 // ---------------------------------------------------------------- Q4_K operands
 struct HdrQ4 { uint32_t sc[2], mn[2]; float d, dmin; };  // eight 6-bit scales and minima, one per byte
 
+// The header of super-block b of a row, as loaded: for planes the 16 bytes of scales and minima and the word holding d and dmin,
+// for GGUF rows the block's first 16 bytes (d, dmin, the 12 packed bytes). Kept apart from its decoding so that a kernel
+// can request a header a step ahead and touch the bytes only when it needs them: any arithmetic on a loaded register makes
+// the compiler wait for the load on the spot, and with it for every request issued before it.
+struct RawHdrQ4 { uint4 words; uint32_t dm; };
+
 template <int BKIND>
-__device__ __forceinline__ HdrQ4 load_hdr_q4k(const uint8_t* base, const tsp_planar_spec& s, uint64_t row, uint32_t bpr, uint32_t b) {
+__device__ __forceinline__ RawHdrQ4 fetch_hdr_q4k(const uint8_t* base, const tsp_planar_spec& s, uint64_t row, uint32_t bpr, uint32_t b) {
     const uint64_t blk = row * bpr + b;
+    RawHdrQ4 r;
+    if constexpr (BKIND == B_Q4K_PLANAR) {
+        r.words = *reinterpret_cast<const uint4*>(base + s.sm_offset + blk * 16);
+        r.dm = *reinterpret_cast<const uint32_t*>(base + s.dm_offset + blk * 4);
+    } else {
+        r.words = *reinterpret_cast<const uint4*>(base + blk * 144);
+        r.dm = 0;
+    }
+    return r;
+}
+
+template <int BKIND>
+__device__ __forceinline__ HdrQ4 decode_hdr_q4k(const RawHdrQ4& r) {
     HdrQ4 h;
     if constexpr (BKIND == B_Q4K_PLANAR) {
-        const uint4 sm = *reinterpret_cast<const uint4*>(base + s.sm_offset + blk * 16);
-        const uint32_t dm = *reinterpret_cast<const uint32_t*>(base + s.dm_offset + blk * 4);
-        h.sc[0] = sm.x; h.sc[1] = sm.y; h.mn[0] = sm.z; h.mn[1] = sm.w;
-        h.d = half_bits_to_float(dm & 0xffffu); h.dmin = half_bits_to_float(dm >> 16);
+        h.sc[0] = r.words.x; h.sc[1] = r.words.y; h.mn[0] = r.words.z; h.mn[1] = r.words.w;
+        h.d = half_bits_to_float(r.dm & 0xffffu); h.dmin = half_bits_to_float(r.dm >> 16);
     } else {
-        const uint4 g = *reinterpret_cast<const uint4*>(base + blk * 144);
+        const uint4 g = r.words;
         h.d = half_bits_to_float(g.x & 0xffffu); h.dmin = half_bits_to_float(g.x >> 16);
         // 12 packed bytes -> one byte per value: sub-blocks 0..3 are the low six bits of bytes 0..7, sub-blocks
         // 4..7 take four bits from bytes 8..11 and two from the top of bytes 0..7
@@ -88,6 +105,11 @@ __device__ __forceinline__ HdrQ4 load_hdr_q4k(const uint8_t* base, const tsp_pla
         h.mn[1] = ((g.w >> 4) & 0x0f0f0f0fu) | ((g.z >> 2) & 0x30303030u);
     }
     return h;
+}
+
+template <int BKIND>
+__device__ __forceinline__ HdrQ4 load_hdr_q4k(const uint8_t* base, const tsp_planar_spec& s, uint64_t row, uint32_t bpr, uint32_t b) {
+    return decode_hdr_q4k<BKIND>(fetch_hdr_q4k<BKIND>(base, s, row, bpr, b));
 }
 
 // Fragments of pair P: bytes 16h..16h+15 of the 32-byte pair; low nibbles (HI = 0) are sub-block 2P, high nibbles
