@@ -21,7 +21,7 @@
 //   * A wave issues at most one instruction every four cycles and two waves share a SIMD, so what a wave executes per
 //     tile is kept short: unpacking is one mask-or and one packed multiply-add per pair of weights, scales are set up two
 //     sub-blocks at a time, the sigmoid uses the hardware exponential and reciprocal, every lane stores (rows a task
-//     does not have land in slots nobody reads), and the tasks of at most 32 rows run in a loop of their own that keeps
+//     does not have repeat its first row, value and slot alike), and the tasks of at most 32 rows run in a loop of their own that keeps
 //     every address in registers. Measured with the arithmetic, the requests or the barrier taken out in turn, no single
 //     one of them bounds the kernel: what is left is the chain of latencies of one tile (arrival, LDS, matrix results,
 //     barrier, sum) at two waves per SIMD.
@@ -172,10 +172,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         request_next();
         uint32_t stage = 0;  // byte offset of the stage the next tile sits in
 
-        uint32_t task = 0;
+        uint32_t task = 0, task_rows = 0;
         auto load_rows = [&](uint32_t k) {  // the task at list position k: its activation rows, this wave's 256 columns of them, into registers
             const Info cur = info_at(k);
             task = cur.task;
+            task_rows = cur.nrows;
             // every row's route first, then, side by side, the route's expert (checked against the task's) and the row of the
             // route's token: two round trips, not three
             uint32_t rid[MT], token[MT];
@@ -184,9 +185,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                 const uint32_t r = i * 32 + n, rr = r < cur.nrows ? r : 0;
                 rid[i] = cur.shared ? 0 : a.token_map[uint64_t(cur.expert) * a.tokens + cur.start + rr];
                 token[i] = cur.shared ? cur.start + rr : rid[i] / a.selected;
-                // A row past the task's end repeats its first row, and a route outside the batch stands in for token 0 (the batch is
-                // refused): their h lands in slots of the task's 64 that nobody reads. So every lane stores, every wave issues the
-                // same number of stores per unit, and the waits below can count them.
+                // A row past the task's end repeats its first row (and stores what it computes, the first row's h, to the first
+                // row's slot), and a route outside the batch stands in for token 0 (the batch is refused). So every lane stores,
+                // every wave issues the same number of stores per unit, and the waits below can count them.
                 if (!cur.shared && rid[i] >= a.tokens * a.selected) { rid[i] = 0; token[i] = 0; if (cur.ok) bad |= TSP_ERRBIT_INDEX; }
                 if (!cur.ok) token[i] = 0;
             }
@@ -307,7 +308,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                         biggest = biggest > magnitude ? biggest : magnitude;
                         // uniform base (the task's slots, the unit's columns) + 32-bit lane offset, spelled out: the compiler would
                         // form a 64-bit address per store
-                        const uint32_t at = (r * a.hidden + lane_now / 2) * 2;
+                        // a row past the task's end has multiplied the first row's activations: the same bits, stored to the first
+                        // row's slot, so that the slots nobody reads cost no traffic (and every lane still stores)
+                        const uint32_t at = ((r < task_rows ? r : 0) * a.hidden + lane_now / 2) * 2;
                         const _Float16* const base = a.hbuf + (uint64_t(task) * kTaskRows) * a.hidden + unit * 32;
                         asm volatile("global_store_short %0, %1, %2" ::"v"(at), "v"(bits), "s"(base) : "memory");
                     }
