@@ -1,4 +1,5 @@
-// Grouped down GEMM for 512-column Q6_K experts (planes ql / qh / sc / d), the task's h rows resident in registers.
+// Grouped down GEMM for 512-column experts in Q6_K planes (ql / qh / sc / d) or Q8_0 planes (quants / d), the task's h rows
+// resident in registers.
 //
 // The companion of the activation-resident gate/up kernel, built the same way around the stream of expert weights:
 //
@@ -30,10 +31,18 @@ namespace {
 
 constexpr int kWaves = 8, kThreads = kWaves * kWave;
 constexpr int kTaskRows = 64;
-// a stage: [32 rows x 128 B low nibbles][32 x 64 B high bits][32 x 16 B sub-scales][128 B of d: 32 rows x 2 super-blocks][pad]
-constexpr int kQlAt = 0, kQhAt = 4096, kScAt = 6144, kDAt = 6656, kStageBytes = 7168;
+// A stage holds one tile, 32 weight rows x one super-block (256 columns):
+//   Q6_K planes: [32 rows x 128 B low nibbles][32 x 64 B high bits][32 x 16 B sub-scales][128 B of d: 32 rows x 2 super-blocks][pad]
+//   Q8_0 planes: [32 rows x 256 B quants][32 x 16 B of d: eight blocks]
+constexpr int kQ6 = 14, kQ8 = 8;  // the planes' source types
+constexpr int kQlAt = 0, kQhAt = 4096, kScAt = 6144, kDAt = 6656;
+constexpr int kQ8dAt = 8192;
+template <int KIND> constexpr int kStageBytes = KIND == kQ6 ? 7168 : 8704;
+template <int KIND> constexpr int kTileLoads = KIND == kQ6 ? 7 : 9;  // direct-to-LDS requests per tile and wave
+// Q6_K exchanges through two buffers in turn (one barrier per exchange); the larger Q8_0 stages leave room for one buffer,
+// which a second barrier hands back
+template <int KIND> constexpr int kPhases = KIND == kQ6 ? 2 : 1;
 constexpr int kStages = 2;
-constexpr int kTileLoads = 7;               // direct-to-LDS requests per tile and wave
 constexpr int kExchangeBytes = 2048;        // what a wave hands its partner per 32 rows: eight accumulators per lane
 constexpr int kPhaseBytes = kWaves * kExchangeBytes;
 constexpr uint32_t kInfoSlots = 32;         // tasks of a workgroup's share kept in LDS
@@ -52,10 +61,13 @@ __device__ __forceinline__ TaskInfo resolve_task(const ResidentDownArgs& a, uint
     return t;
 }
 
+template <int KIND>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void down_resident_kernel(ResidentDownArgs a) {
-    // LDS: [2 phases][8 waves][2 KB exchange] | [2 passes][32 tasks of the share] | [2 tasks][64 row offsets] | [8 waves][2 stages][7 KB weight tile]
-    constexpr int kInfoAt = 2 * kPhaseBytes, kRowsAt = kInfoAt + 2 * kInfoSlots * 16, kStagesAt = kRowsAt + 2 * kTaskRows * 4;
+    // LDS: [1 or 2 phases][8 waves][2 KB exchange] | [2 passes][32 tasks of the share] | [2 tasks][64 row offsets] | [8 waves][2 stages][weight tile]
+    constexpr int kStageBytes = ::kStageBytes<KIND>, kTileLoads = ::kTileLoads<KIND>, kPhases = ::kPhases<KIND>;
+    constexpr int kInfoAt = kPhases * kPhaseBytes, kRowsAt = kInfoAt + 2 * kInfoSlots * 16, kStagesAt = kRowsAt + 2 * kTaskRows * 4;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kStagesAt + kWaves * kStages * kStageBytes];
+    static_assert(sizeof(lds_raw) <= 160 * 1024, "one workgroup per compute unit");
     uint4* const info_tables = reinterpret_cast<uint4*>(lds_raw + kInfoAt);
     uint32_t* const row_at = reinterpret_cast<uint32_t*>(lds_raw + kRowsAt);
 
@@ -76,8 +88,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const uint32_t my_stage_lds = __builtin_amdgcn_readfirstlane(lds_address(my_stage));
 
     // ---- per-lane parts of the request addresses, from the first byte of the expert (the per-tile parts are uniform)
-    // low nibbles: request q covers rows 8q .. 8q+7 of the tile, eight lanes per row (one 128-byte line: the row's super-block
-    // kh); lane l sits at 16-byte slot l % 8 of its row in LDS and fetches chunk (l % 8) ^ (row % 8)
+    // Q6_K low nibbles: request q covers rows 8q .. 8q+7 of the tile, eight lanes per row (one 128-byte line: the row's
+    // super-block kh); lane l sits at 16-byte slot l % 8 of its row in LDS and fetches chunk (l % 8) ^ (row % 8)
     const uint32_t ql_lane = uint32_t(a.spec.qs_offset) + (lane / 8) * (bpr * 128) + kh * 128 + (((lane % 8) ^ ((lane / 8) & 7)) * 16);
     // high bits: request q covers rows 16q .. 16q+15, four lanes per row (64 bytes); slot l % 4 holds chunk (l % 4) ^ ((row / 4) % 4)
     const uint32_t qh_lane = uint32_t(a.spec.qh_offset) + (lane / 4) * (bpr * 64) + kh * 64 + (((lane % 4) ^ ((lane / 16) & 3)) * 16);
@@ -85,17 +97,31 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const uint32_t tail = lane < 40 ? lane - 32 : 7;
     const uint32_t hdr_lane = lane < 32 ? uint32_t(a.spec.sm_offset) + lane * (bpr * 16) + kh * 16 : uint32_t(a.spec.dm_offset) + tail * 16;
     const uint32_t hdr_tile_step = lane < 32 ? 32 * bpr * 16 : 32 * bpr * 2;
+    // Q8_0 quants: a row is 16 blocks x 32 bytes; request q covers rows 4q .. 4q+3, sixteen lanes per row (the 256 bytes of the
+    // row's super-block kh); slot l % 16 of row r holds chunk (l % 16) ^ (r % 16), and r % 16 = (l / 16) | (4q % 16), so request q
+    // flips bits 2..3 of the chunk index of request 0: an exclusive or with (4q % 16) << 4 on the byte offset, whose bits 4..7
+    // are the chunk's alone (row stride 512, super-block 256)
+    const uint32_t q8_lane = (lane / 16) * 512 + kh * 256 + (((lane % 16) ^ (lane / 16)) * 16);
+    // d: lanes 0..31 fetch the 16 bytes holding the eight d of row l's super-block kh; lanes 32..63 sit out
+    const uint32_t q8d_lane = uint32_t(a.spec.dm_offset) + (lane % 32) * 32 + kh * 16;
 
     auto request_tile = [&](const uint8_t* base, uint32_t unit, uint32_t stage_offset) {  // base: one expert (under 4 GiB), uniform
         const uint32_t tile = unit * 4 + nq;
-        const uint8_t* ql = base + uint64_t(tile) * (32 * bpr * 128);
-        const uint8_t* qh = base + uint64_t(tile) * (32 * bpr * 64);
         const uint32_t dst = my_stage_lds + stage_offset;
+        if constexpr (KIND == kQ6) {
+            const uint8_t* ql = base + uint64_t(tile) * (32 * bpr * 128);
+            const uint8_t* qh = base + uint64_t(tile) * (32 * bpr * 64);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) load_to_lds_16(ql + q * (8 * bpr * 128), ql_lane, dst + kQlAt + q * 1024);
+            for (int q = 0; q < 4; ++q) load_to_lds_16(ql + q * (8 * bpr * 128), ql_lane, dst + kQlAt + q * 1024);
 #pragma unroll
-        for (int q = 0; q < 2; ++q) load_to_lds_16(qh + q * (16 * bpr * 64), qh_lane, dst + kQhAt + q * 1024);
-        load_to_lds_16(base, hdr_lane + tile * hdr_tile_step, dst + kScAt);
+            for (int q = 0; q < 2; ++q) load_to_lds_16(qh + q * (16 * bpr * 64), qh_lane, dst + kQhAt + q * 1024);
+            load_to_lds_16(base, hdr_lane + tile * hdr_tile_step, dst + kScAt);
+        } else {
+            const uint8_t* qs = base + a.spec.qs_offset + uint64_t(tile) * (32 * 512);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) load_to_lds_16(qs + q * (4 * 512), q8_lane ^ (((4 * q) & 15) << 4), dst + q * 1024);
+            if (lane < 32) load_to_lds_16(base, q8d_lane + tile * (32 * 32), dst + kQ8dAt);  // one request of the wave, half its lanes
+        }
     };
 
     uint32_t bad = 0, phase = 0, parity = 0;
@@ -172,7 +198,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                 const uint32_t r = i * 32 + n, rr = r < cur.nrows ? r : 0;  // a row past the end repeats the first
                 const _Float16* row = a.hbuf + (uint64_t(cur.task) * kTaskRows + rr) * (bpr * 256) + kh * 256 + khalf * 16;
 #pragma unroll
-                for (int t = 0; t < 16; ++t) A[i][t] = *reinterpret_cast<const f16x8*>(row + (t / 8) * 128 + ((t / 2) % 4) * 32 + (t % 2) * 8);
+                for (int t = 0; t < 16; ++t) {
+                    // Q6_K: section t / 8, quarter (t / 2) % 4, fragment t % 2; Q8_0: block t / 2, fragment t % 2. Either way a
+                    // lane's k-half takes sixteen consecutive columns of every 32.
+                    if constexpr (KIND == kQ6) A[i][t] = *reinterpret_cast<const f16x8*>(row + (t / 8) * 128 + ((t / 2) % 4) * 32 + (t % 2) * 8);
+                    else A[i][t] = *reinterpret_cast<const f16x8*>(row + (t / 2) * 32 + (t % 2) * 8);
+                }
             }
             // Lane l looks up where task row l goes: its route (for the always-on expert its token). The gate/up product of
             // the same call has checked every route against the expert; here the index only has to stay inside the output.
@@ -207,47 +238,84 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             if constexpr (MT == 2) asm volatile("" : "+v"(lane_now));  // lane-derived addresses are derived again per tile, not kept
             const uint32_t n = lane_now % 32, khalf = (lane_now / 32) & 1;  // & 1: the compiler must see that khalf picks no sub-scale word
             const uint8_t* st = my_stage + stage;
-            RawQ6 raw[2];
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                raw[s].la = *reinterpret_cast<const u32x4*>(st + kQlAt + n * 128 + (((4 * s + khalf) ^ (n & 7)) * 16));
-                raw[s].lb = *reinterpret_cast<const u32x4*>(st + kQlAt + n * 128 + (((4 * s + 2 + khalf) ^ (n & 7)) * 16));
-                raw[s].qh = *reinterpret_cast<const u32x4*>(st + kQhAt + n * 64 + (((2 * s + khalf) ^ ((n >> 2) & 3)) * 16));
-            }
-            const uint4 sc = *reinterpret_cast<const uint4*>(st + kScAt + n * 16);
-            const uint32_t dd = *reinterpret_cast<const uint32_t*>(st + kDAt + n * 4);  // d of super-blocks 0 and 1 of row n
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            request_next();  // the stage is free again: the tile two ahead goes there
-            stage = stage + kStageBytes == kStages * kStageBytes ? 0 : stage + kStageBytes;
-            raw[0].sc[0] = sc.x; raw[0].sc[1] = sc.y; raw[1].sc[0] = sc.z; raw[1].sc[1] = sc.w;
-            // the output scale is a power of two: folded into d it changes no rounding
-            const float d0 = half_bits_to_float(dd & 0xffffu) * s256, d1 = half_bits_to_float(dd >> 16) * s256;
-
             f32x16 blk[MT];
-            auto quarter = [&](auto s_tag, auto q_tag) {
-                constexpr int S = decltype(s_tag)::value, Q = decltype(q_tag)::value;
-                f16x8 f[2];
-                frags_q6k<Q>(raw[S], khalf, f);
+            float d0 = 0, d1 = 0;
+            if constexpr (KIND == kQ6) {
+                RawQ6 raw[2];
 #pragma unroll
-                for (int ff = 0; ff < 2; ++ff)
+                for (int s = 0; s < 2; ++s) {
+                    raw[s].la = *reinterpret_cast<const u32x4*>(st + kQlAt + n * 128 + (((4 * s + khalf) ^ (n & 7)) * 16));
+                    raw[s].lb = *reinterpret_cast<const u32x4*>(st + kQlAt + n * 128 + (((4 * s + 2 + khalf) ^ (n & 7)) * 16));
+                    raw[s].qh = *reinterpret_cast<const u32x4*>(st + kQhAt + n * 64 + (((2 * s + khalf) ^ ((n >> 2) & 3)) * 16));
+                }
+                const uint4 sc = *reinterpret_cast<const uint4*>(st + kScAt + n * 16);
+                const uint32_t dd = *reinterpret_cast<const uint32_t*>(st + kDAt + n * 4);  // d of super-blocks 0 and 1 of row n
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                request_next();  // the stage is free again: the tile two ahead goes there
+                raw[0].sc[0] = sc.x; raw[0].sc[1] = sc.y; raw[1].sc[0] = sc.z; raw[1].sc[1] = sc.w;
+                // the output scale is a power of two: folded into d it changes no rounding
+                d0 = half_bits_to_float(dd & 0xffffu) * s256;
+                d1 = half_bits_to_float(dd >> 16) * s256;
+                auto quarter = [&](auto s_tag, auto q_tag) {
+                    constexpr int S = decltype(s_tag)::value, Q = decltype(q_tag)::value;
+                    f16x8 f[2];
+                    frags_q6k<Q>(raw[S], khalf, f);
 #pragma unroll
-                    for (int i = 0; i < MT; ++i) {
-                        if (S == 0 && Q == 0 && ff == 0) {
-                            const f32x16 zero{};
-                            blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][0], f[0], zero, 0, 0, 0);
-                        } else {
-                            blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][S * 8 + Q * 2 + ff], f[ff], blk[i], 0, 0, 0);
+                    for (int ff = 0; ff < 2; ++ff)
+#pragma unroll
+                        for (int i = 0; i < MT; ++i) {
+                            if (S == 0 && Q == 0 && ff == 0) {
+                                const f32x16 zero{};
+                                blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][0], f[0], zero, 0, 0, 0);
+                            } else {
+                                blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][S * 8 + Q * 2 + ff], f[ff], blk[i], 0, 0, 0);
+                            }
                         }
+                };
+                quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+                quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
+                quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 2>{});
+                quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 3>{});
+                quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+                quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{});
+                quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{});
+                quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 3>{});
+            } else {
+                // Q8_0: sixteen quants of row n per block (the lane's k-half of the block's 32) and the row's eight d. A weight
+                // is the half nearest to d * q, the engine's arithmetic for this kind: q is exact as a half and so is d, so one
+                // packed half multiply rounds once, as the f32 product rounded to half does.
+                u32x4 q[8];
+#pragma unroll
+                for (int b = 0; b < 8; ++b) q[b] = *reinterpret_cast<const u32x4*>(st + n * 256 + (((2 * b + khalf) ^ (n & 15)) * 16));
+                const u32x4 dd = *reinterpret_cast<const u32x4*>(st + kQ8dAt + n * 16);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                request_next();  // the stage is free again: the tile two ahead goes there
+#pragma unroll
+                for (int b = 0; b < 8; ++b) {
+                    const uint32_t pair = dd[b / 2];
+                    const f16x2 d2 = as_h2(b % 2 ? __builtin_amdgcn_perm(pair, pair, 0x07060706u) : __builtin_amdgcn_perm(pair, pair, 0x05040504u));
+                    f16x8 f[2];
+#pragma unroll
+                    for (int ff = 0; ff < 2; ++ff) {
+                        const f16x8 whole = quants8(q[b][2 * ff], q[b][2 * ff + 1]);
+                        const f16x2 p0 = f16x2{whole[0], whole[1]} * d2, p1 = f16x2{whole[2], whole[3]} * d2;
+                        const f16x2 p2 = f16x2{whole[4], whole[5]} * d2, p3 = f16x2{whole[6], whole[7]} * d2;
+                        f[ff] = f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
                     }
-            };
-            quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
-            quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
-            quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 2>{});
-            quarter(std::integral_constant<int, 0>{}, std::integral_constant<int, 3>{});
-            quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
-            quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{});
-            quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{});
-            quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 3>{});
+#pragma unroll
+                    for (int ff = 0; ff < 2; ++ff)
+#pragma unroll
+                        for (int i = 0; i < MT; ++i) {
+                            if (b == 0 && ff == 0) {
+                                const f32x16 zero{};
+                                blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][0], f[0], zero, 0, 0, 0);
+                            } else {
+                                blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][b * 2 + ff], f[ff], blk[i], 0, 0, 0);
+                            }
+                        }
+                }
+            }
+            stage = stage + kStageBytes == kStages * kStageBytes ? 0 : stage + kStageBytes;
 
             // Accumulator v of a 32 x 32 tile is row 8 (v / 4) + 4 khalf + v % 4, column n. The wave of super-block 0 finishes
             // rows 0..15 (v < 8), its partner rows 16..31: each hands over the eight sums of the other's rows. Which of the two a
@@ -257,7 +325,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                 constexpr int KH = decltype(kh_tag)::value;
 #pragma unroll
                 for (int i = 0; i < MT; ++i) {
-                    uint8_t* out = lds_raw + (phase & 1) * kPhaseBytes + wave * kExchangeBytes + lane_now * 16;
+                    uint8_t* out = lds_raw + (phase % kPhases) * kPhaseBytes + wave * kExchangeBytes + lane_now * 16;
 #pragma unroll
                     for (int c = 0; c < 2; ++c) {
                         f32x4 v;
@@ -266,18 +334,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                         *reinterpret_cast<f32x4*>(out + c * 1024) = v;
                     }
                     lds_barrier();
-                    const uint8_t* in = lds_raw + (phase & 1) * kPhaseBytes + (wave ^ 4) * kExchangeBytes + lane_now * 16;
+                    const uint8_t* in = lds_raw + (phase % kPhases) * kPhaseBytes + (wave ^ 4) * kExchangeBytes + lane_now * 16;
                     ++phase;
+                    f32x4 theirs[2];
+#pragma unroll
+                    for (int c = 0; c < 2; ++c) theirs[c] = *reinterpret_cast<const f32x4*>(in + c * 1024);
+                    if constexpr (kPhases == 1) lds_barrier();  // both have read: the one buffer may be written again
 #pragma unroll
                     for (int c = 0; c < 2; ++c) {
-                        const f32x4 theirs = *reinterpret_cast<const f32x4*>(in + c * 1024);
                         // accumulator 4 c + e of the wave's half of the row tile is task row 32 i + 16 KH + 8 c + 4 khalf + e
                         const u32x4 to = *reinterpret_cast<const u32x4*>(&row_at[parity * kTaskRows + i * 32 + 16 * KH + 8 * c + 4 * khalf]);
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             const float mine = blk[i][8 * KH + 4 * c + e];
-                            const float sum0 = KH == 0 ? mine : theirs[e], sum1 = KH == 0 ? theirs[e] : mine;
-                            const float val = __builtin_fmaf(d1, sum1, d0 * sum0);
+                            const float sum0 = KH == 0 ? mine : theirs[c][e], sum1 = KH == 0 ? theirs[c][e] : mine;
+                            // Q6_K: the integer sums of the two super-blocks times their d, in the order of a sequential pass;
+                            // Q8_0: the weights carried their d, the two halves of K just add
+                            const float val = KIND == kQ6 ? __builtin_fmaf(d1, sum1, d0 * sum0) : (sum0 + sum1) * s256;
                             const uint32_t magnitude = __float_as_uint(val) & 0x7fffffffu;
                             biggest = biggest > magnitude ? biggest : magnitude;
                             // uniform base + 32-bit lane offset, spelled out: the compiler would form 64-bit addresses
@@ -309,7 +382,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 
 namespace tsp {
 
-bool resident_down_takes(uint32_t channels, uint32_t hidden) { return hidden == 512 && channels % 128 == 0 && channels >= 128; }
+bool resident_down_takes(uint32_t source_type, uint32_t channels, uint32_t hidden) {
+    return (source_type == kQ6 || source_type == kQ8) && hidden == 512 && channels % 128 == 0 && channels >= 128;
+}
 
 int launch_resident_down(const ResidentDownArgs& a, hipStream_t s) {
     static std::atomic<uint64_t> seen{0};
@@ -320,7 +395,8 @@ int launch_resident_down(const ResidentDownArgs& a, hipStream_t s) {
         TSP_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device));
         cus[device] = n >= 8 ? n / 8 * 8 : 8;
     }
-    TSP_LAUNCH("gemm_down", s, down_resident_kernel<<<cus[device], kThreads, 0, s>>>(a));
+    if (a.spec.source_type == kQ6) TSP_LAUNCH("gemm_down", s, down_resident_kernel<kQ6><<<cus[device], kThreads, 0, s>>>(a));
+    else TSP_LAUNCH("gemm_down", s, down_resident_kernel<kQ8><<<cus[device], kThreads, 0, s>>>(a));
     return launch_status("down_resident");
 }
 

@@ -940,6 +940,17 @@ int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void*
         rc = launch<B_Q4K_PLANAR, EPI_SWIGLU, ROWS_GATHER_TOKENS>(g, (m->hidden + 127) / 128, l.bound, s);
     }
     if (rc != TSP_OK) return rc;
+    const uint64_t shared_span = shared ? uint64_t(m->tokens) * shared->y_stride_bytes : 0;
+    if (resident_down_takes(down_type, m->channels, m->hidden) && uint64_t(routes) * m->y_stride_bytes < (1ull << 32) && shared_span < (1ull << 32)) {
+        ResidentDownArgs r{};
+        r.hbuf = hbuf; r.down = static_cast<const uint8_t*>(m->down); r.shared_down = shared ? static_cast<const uint8_t*>(shared->down) : nullptr;
+        r.spec = dn; r.experts = m->experts; r.tokens = m->tokens; r.selected = m->selected;
+        r.channels = m->channels; r.tasks = task_list; r.classes = reinterpret_cast<const uint32_t*>(ws + l.classes); r.counts = m->counts;
+        r.token_map = m->token_map; r.ids = m->ids; r.task_slots = l.bound; r.y = static_cast<float*>(m->y); r.y_stride = m->y_stride_bytes;
+        r.shared_y = shared ? static_cast<float*>(shared->y) : nullptr; r.shared_y_stride = shared ? shared->y_stride_bytes : 0;
+        r.out_scale = 256.0f; r.error_word = m->error_word;
+        return launch_resident_down(r, s);
+    }
     if (!fast_down) return launch_planar_staged_down(staged, s);
 
     GemmArgs d{};
@@ -948,16 +959,6 @@ int grouped_moe(const tsp_grouped_moe* m, const tsp_shared_expert* shared, void*
     d.n = m->channels; d.k = m->hidden; d.out = m->y; d.out_stride = m->y_stride_bytes; d.out_scale = 256.0f;  // undo the 2^-8 carried by h
     d.error_word = m->error_word;
     if (shared) { d.shared_w0 = static_cast<const uint8_t*>(shared->down); d.shared_out = shared->y; d.shared_out_stride = shared->y_stride_bytes; }
-    const uint64_t shared_span = shared ? uint64_t(m->tokens) * shared->y_stride_bytes : 0;
-    if (resident_down_takes(m->channels, m->hidden) && uint64_t(routes) * m->y_stride_bytes < (1ull << 32) && shared_span < (1ull << 32)) {
-        ResidentDownArgs r{};
-        r.hbuf = hbuf; r.down = d.w0; r.shared_down = d.shared_w0; r.spec = dn; r.experts = m->experts; r.tokens = m->tokens; r.selected = m->selected;
-        r.channels = m->channels; r.tasks = task_list; r.classes = reinterpret_cast<const uint32_t*>(ws + l.classes); r.counts = m->counts;
-        r.token_map = m->token_map; r.ids = m->ids; r.task_slots = l.bound; r.y = static_cast<float*>(m->y); r.y_stride = m->y_stride_bytes;
-        r.shared_y = shared ? static_cast<float*>(shared->y) : nullptr; r.shared_y_stride = shared ? shared->y_stride_bytes : 0;
-        r.out_scale = 256.0f; r.error_word = m->error_word;
-        return launch_resident_down(r, s);
-    }
     return launch<B_Q6K_PLANAR, EPI_F32, ROWS_TASK_SLOTS>(d, (m->channels + 255) / 256, l.bound, s);
 }
 }  // namespace

@@ -65,6 +65,16 @@ __device__ __forceinline__ f16x8 scaled8_q6(uint32_t c0, uint32_t c1, f16x2 sc, 
     return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
 }
 
+// Eight int8 quants (two dwords) as exact halves: q ^ 0x80 = q + 128 in 0..255, 0x6400 | u = 1024 + u, minus 1152.
+__device__ __forceinline__ f16x8 quants8(uint32_t w0, uint32_t w1) {
+    constexpr uint32_t K = 0x64646464u;
+    const uint32_t u0 = w0 ^ 0x80808080u, u1 = w1 ^ 0x80808080u;
+    const f16x2 off = splat(-1152.0f);
+    const f16x2 p0 = as_h2(spread01(u0, K)) + off, p1 = as_h2(spread23(u0, K)) + off;
+    const f16x2 p2 = as_h2(spread01(u1, K)) + off, p3 = as_h2(spread23(u1, K)) + off;
+    return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+}
+
 // ---------------------------------------------------------------- Q4_K operands
 struct HdrQ4 { uint32_t sc[2], mn[2]; float d, dmin; };  // eight 6-bit scales and minima, one per byte
 
