@@ -495,7 +495,7 @@ def test_grouped_moe_exact_when_products_fit_half(gpu, tsp, orc, synth):
 
 @pytest.mark.parametrize("gu_type,dn_type,channels,hidden", [(13, 7, 256, 256), (8, 8, 256, 256), (12, 8, 256, 256), (13, 14, 256, 256), (12, 7, 512, 160),
                                                              (8, 7, 96, 64), (8, 14, 160, 256), (12, 8, 256, 512), (8, 8, 384, 512),
-                                                             (13, 8, 2048, 512), (12, 7, 256, 512)])
+                                                             (13, 8, 2048, 512), (12, 7, 256, 512), (8, 7, 768, 512)])
 def test_grouped_moe_other_planar_kinds(gpu, tsp, orc, synth, gu_type, dn_type, channels, hidden):
     """The planar kinds of include/tokspur/moe.hpp:27-29 beside Q4_K gate/up and Q6_K down (Q5_K / Q8_0 gate and up, Q5_1 / Q8_0
     down) run on the matrix cores as well, their weights decoded to halves on the fly; any gate/up kind combines with any down

@@ -1,5 +1,5 @@
-// Grouped down GEMM for 512-column experts in Q6_K planes (ql / qh / sc / d) or Q8_0 planes (quants / d), the task's h rows
-// resident in registers.
+// Grouped down GEMM for 512-column experts in Q6_K planes (ql / qh / sc / d), Q8_0 planes (quants / d) or Q5_1 planes
+// (nibbles / fifth bits / d, m), the task's h rows resident in registers.
 //
 // The companion of the activation-resident gate/up kernel, built the same way around the stream of expert weights:
 //
@@ -34,14 +34,16 @@ constexpr int kTaskRows = 64;
 // A stage holds one tile, 32 weight rows x one super-block (256 columns):
 //   Q6_K planes: [32 rows x 128 B low nibbles][32 x 64 B high bits][32 x 16 B sub-scales][128 B of d: 32 rows x 2 super-blocks][pad]
 //   Q8_0 planes: [32 rows x 256 B quants][32 x 16 B of d: eight blocks]
-constexpr int kQ6 = 14, kQ8 = 8;  // the planes' source types
+//   Q5_1 planes: [32 rows x 128 B nibbles][32 x 32 B fifth bits: eight blocks][32 x 32 B of d, m: eight blocks]
+constexpr int kQ6 = 14, kQ8 = 8, kQ51 = 7;  // the planes' source types
 constexpr int kQlAt = 0, kQhAt = 4096, kScAt = 6144, kDAt = 6656;
 constexpr int kQ8dAt = 8192;
-template <int KIND> constexpr int kStageBytes = KIND == kQ6 ? 7168 : 8704;
-template <int KIND> constexpr int kTileLoads = KIND == kQ6 ? 7 : 9;  // direct-to-LDS requests per tile and wave
+constexpr int kQ51hAt = 4096, kQ51dAt = 5120;
+template <int KIND> constexpr int kStageBytes = KIND == kQ6 ? 7168 : KIND == kQ8 ? 8704 : 6144;
+template <int KIND> constexpr int kTileLoads = KIND == kQ6 ? 7 : KIND == kQ8 ? 9 : 6;  // direct-to-LDS requests per tile and wave
 // Q6_K exchanges through two buffers in turn (one barrier per exchange); the larger Q8_0 stages leave room for one buffer,
 // which a second barrier hands back
-template <int KIND> constexpr int kPhases = KIND == kQ6 ? 2 : 1;
+template <int KIND> constexpr int kPhases = KIND == kQ8 ? 1 : 2;
 constexpr int kStages = 2;
 constexpr int kExchangeBytes = 2048;        // what a wave hands its partner per 32 rows: eight accumulators per lane
 constexpr int kPhaseBytes = kWaves * kExchangeBytes;
@@ -104,6 +106,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const uint32_t q8_lane = (lane / 16) * 512 + kh * 256 + (((lane % 16) ^ (lane / 16)) * 16);
     // d: lanes 0..31 fetch the 16 bytes holding the eight d of row l's super-block kh; lanes 32..63 sit out
     const uint32_t q8d_lane = uint32_t(a.spec.dm_offset) + (lane % 32) * 32 + kh * 16;
+    // Q5_1: the nibbles of a row's super-block are one 128-byte line, requested like the Q6_K low nibbles (ql_lane: row stride 256
+    // either way); fifth bits and (d, m) are 4 bytes per block, 32 bytes per row and super-block: two lanes per row
+    const uint32_t q51_lane = (lane / 2) * 64 + kh * 32 + (lane % 2) * 16;
 
     auto request_tile = [&](const uint8_t* base, uint32_t unit, uint32_t stage_offset) {  // base: one expert (under 4 GiB), uniform
         const uint32_t tile = unit * 4 + nq;
@@ -116,11 +121,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
             for (int q = 0; q < 2; ++q) load_to_lds_16(qh + q * (16 * bpr * 64), qh_lane, dst + kQhAt + q * 1024);
             load_to_lds_16(base, hdr_lane + tile * hdr_tile_step, dst + kScAt);
-        } else {
+        } else if constexpr (KIND == kQ8) {
             const uint8_t* qs = base + a.spec.qs_offset + uint64_t(tile) * (32 * 512);
 #pragma unroll
             for (int q = 0; q < 8; ++q) load_to_lds_16(qs + q * (4 * 512), q8_lane ^ (((4 * q) & 15) << 4), dst + q * 1024);
             if (lane < 32) load_to_lds_16(base, q8d_lane + tile * (32 * 32), dst + kQ8dAt);  // one request of the wave, half its lanes
+        } else {
+            const uint8_t* qs = base + uint64_t(tile) * (32 * 256);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) load_to_lds_16(qs + q * (8 * 256), ql_lane, dst + q * 1024);
+            load_to_lds_16(base + a.spec.qh_offset + uint64_t(tile) * (32 * 64), q51_lane, dst + kQ51hAt);
+            load_to_lds_16(base + a.spec.dm_offset + uint64_t(tile) * (32 * 64), q51_lane, dst + kQ51dAt);
         }
     };
 
@@ -199,7 +210,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                 const _Float16* row = a.hbuf + (uint64_t(cur.task) * kTaskRows + rr) * (bpr * 256) + kh * 256 + khalf * 16;
 #pragma unroll
                 for (int t = 0; t < 16; ++t) {
-                    // Q6_K: section t / 8, quarter (t / 2) % 4, fragment t % 2; Q8_0: block t / 2, fragment t % 2. Either way a
+                    // Q6_K: section t / 8, quarter (t / 2) % 4, fragment t % 2; Q8_0, Q5_1: block t / 2, fragment t % 2. Either way a
                     // lane's k-half takes sixteen consecutive columns of every 32.
                     if constexpr (KIND == kQ6) A[i][t] = *reinterpret_cast<const f16x8*>(row + (t / 8) * 128 + ((t / 2) % 4) * 32 + (t % 2) * 8);
                     else A[i][t] = *reinterpret_cast<const f16x8*>(row + (t / 2) * 32 + (t % 2) * 8);
@@ -280,6 +291,56 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                 quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{});
                 quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{});
                 quarter(std::integral_constant<int, 1>{}, std::integral_constant<int, 3>{});
+            } else if constexpr (KIND == kQ51) {
+                // Q5_1: element e of a block is nibble e % 16 (low for e < 16, high above) of byte e % 16 with bit e of the
+                // block's fifth-bit word on top; the lane's k-half takes elements 16 khalf .. 16 khalf + 15. A weight is the
+                // half nearest to d * q + m: q exact as a half, one packed fused multiply-add, one rounding (the f32
+                // evaluation rounds the sum to f32 first, which can move the half only when that sum sits on a tie).
+                u32x4 q[8];
+#pragma unroll
+                for (int b = 0; b < 8; ++b) q[b] = *reinterpret_cast<const u32x4*>(st + n * 128 + ((b ^ (n & 7)) * 16));
+                u32x4 fifth[2], dm[2];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    fifth[h] = *reinterpret_cast<const u32x4*>(st + kQ51hAt + n * 32 + h * 16);
+                    dm[h] = *reinterpret_cast<const u32x4*>(st + kQ51dAt + n * 32 + h * 16);
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                request_next();  // the stage is free again: the tile two ahead goes there
+#pragma unroll
+                for (int b = 0; b < 8; ++b) {
+                    const uint32_t pair = dm[b / 4][b % 4];  // d in the low half, m in the high half
+                    const f16x2 d2 = as_h2(__builtin_amdgcn_perm(pair, pair, 0x05040504u)), m2 = as_h2(__builtin_amdgcn_perm(pair, pair, 0x07060706u));
+                    const uint32_t bits = fifth[b / 4][b % 4] >> (16 * khalf);
+                    const f16x2 off = splat(-1024.0f);
+                    f16x8 f[2];
+#pragma unroll
+                    for (int ff = 0; ff < 2; ++ff) {
+                        f16x2 p[4];
+#pragma unroll
+                        for (int j = 0; j < 2; ++j) {
+                            const int w = 2 * ff + j;  // bytes 4 w .. 4 w + 3 of the block: elements 16 khalf + 4 w .. + 3
+                            const uint32_t nibbles = (q[b][w] >> (4 * khalf)) & 0x0f0f0f0fu;
+                            // bits 4 w .. 4 w + 3 of the fifth-bit half-word to bit 0 of four bytes: no two partial products share a bit
+                            const uint32_t four = ((bits >> (4 * w)) & 15u) * 0x00204081u & 0x01010101u;
+                            const uint32_t codes = nibbles | (four << 4);
+                            p[2 * j] = fma2(as_h2(spread01(codes, 0x64646464u)) + off, d2, m2);
+                            p[2 * j + 1] = fma2(as_h2(spread23(codes, 0x64646464u)) + off, d2, m2);
+                        }
+                        f[ff] = f16x8{p[0][0], p[0][1], p[1][0], p[1][1], p[2][0], p[2][1], p[3][0], p[3][1]};
+                    }
+#pragma unroll
+                    for (int ff = 0; ff < 2; ++ff)
+#pragma unroll
+                        for (int i = 0; i < MT; ++i) {
+                            if (b == 0 && ff == 0) {
+                                const f32x16 zero{};
+                                blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][0], f[0], zero, 0, 0, 0);
+                            } else {
+                                blk[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[i][b * 2 + ff], f[ff], blk[i], 0, 0, 0);
+                            }
+                        }
+                }
             } else {
                 // Q8_0: sixteen quants of row n per block (the lane's k-half of the block's 32) and the row's eight d. A weight
                 // is the half nearest to d * q, the engine's arithmetic for this kind: q is exact as a half and so is d, so one
@@ -349,7 +410,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                             const float mine = blk[i][8 * KH + 4 * c + e];
                             const float sum0 = KH == 0 ? mine : theirs[c][e], sum1 = KH == 0 ? theirs[c][e] : mine;
                             // Q6_K: the integer sums of the two super-blocks times their d, in the order of a sequential pass;
-                            // Q8_0: the weights carried their d, the two halves of K just add
+                            // Q8_0, Q5_1: the weights carried their scales, the two halves of K just add
                             const float val = KIND == kQ6 ? __builtin_fmaf(d1, sum1, d0 * sum0) : (sum0 + sum1) * s256;
                             const uint32_t magnitude = __float_as_uint(val) & 0x7fffffffu;
                             biggest = biggest > magnitude ? biggest : magnitude;
@@ -383,7 +444,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 namespace tsp {
 
 bool resident_down_takes(uint32_t source_type, uint32_t channels, uint32_t hidden) {
-    return (source_type == kQ6 || source_type == kQ8) && hidden == 512 && channels % 128 == 0 && channels >= 128;
+    return (source_type == kQ6 || source_type == kQ8 || source_type == kQ51) && hidden == 512 && channels % 128 == 0 && channels >= 128;
 }
 
 int launch_resident_down(const ResidentDownArgs& a, hipStream_t s) {
@@ -396,7 +457,8 @@ int launch_resident_down(const ResidentDownArgs& a, hipStream_t s) {
         cus[device] = n >= 8 ? n / 8 * 8 : 8;
     }
     if (a.spec.source_type == kQ6) TSP_LAUNCH("gemm_down", s, down_resident_kernel<kQ6><<<cus[device], kThreads, 0, s>>>(a));
-    else TSP_LAUNCH("gemm_down", s, down_resident_kernel<kQ8><<<cus[device], kThreads, 0, s>>>(a));
+    else if (a.spec.source_type == kQ8) TSP_LAUNCH("gemm_down", s, down_resident_kernel<kQ8><<<cus[device], kThreads, 0, s>>>(a));
+    else TSP_LAUNCH("gemm_down", s, down_resident_kernel<kQ51><<<cus[device], kThreads, 0, s>>>(a));
     return launch_status("down_resident");
 }
 

@@ -6,7 +6,7 @@ namespace tsp {
 
 struct ResidentDownArgs {
     const _Float16* hbuf;        // [task_slots * 64][512]: SwiGLU output rows by task slot, as halves of h / 256
-    const uint8_t* down;         // Q6_K planes (ql / qh / sub-scales / d) or Q8_0 planes (quants / d) per expert, `channels` rows of 512 columns
+    const uint8_t* down;         // Q6_K planes (ql / qh / sub-scales / d), Q8_0 planes (quants / d) or Q5_1 planes (nibbles / fifth bits / d, m) per expert, `channels` rows of 512 columns
     const uint8_t* shared_down;  // an always-on expert whose tasks carry expert id == experts (null: none)
     tsp_planar_spec spec;        // one expert
     uint32_t experts, tokens, selected, channels;
@@ -24,7 +24,7 @@ struct ResidentDownArgs {
     uint32_t* error_word;
 };
 
-bool resident_down_takes(uint32_t source_type, uint32_t channels, uint32_t hidden);  // source_type: 14 (Q6_K planes) or 8 (Q8_0 planes)
+bool resident_down_takes(uint32_t source_type, uint32_t channels, uint32_t hidden);  // source_type: 14 (Q6_K planes), 8 (Q8_0 planes) or 7 (Q5_1 planes)
 int launch_resident_down(const ResidentDownArgs& args, hipStream_t stream);
 
 }  // namespace tsp
