@@ -22,6 +22,7 @@
 //     has already checked against the expert: inside the tile loop nothing is read from memory but weights.
 #include "down_resident.hpp"
 #include "mfma_quant.hpp"
+#include "resident_tasks.hpp"
 
 #include <type_traits>
 
@@ -47,21 +48,7 @@ template <int KIND> constexpr int kPhases = KIND == kQ8 ? 1 : 2;
 constexpr int kStages = 2;
 constexpr int kExchangeBytes = 2048;        // what a wave hands its partner per 32 rows: eight accumulators per lane
 constexpr int kPhaseBytes = kWaves * kExchangeBytes;
-constexpr uint32_t kInfoSlots = 32;         // tasks of a workgroup's share kept in LDS
-
-struct TaskInfo { uint32_t expert, start, nrows; bool shared, ok; };
-
-__device__ __forceinline__ TaskInfo resolve_task(const ResidentDownArgs& a, uint32_t task) {
-    TaskInfo t;
-    t.expert = a.tasks[2 + 2 * task];
-    t.start = a.tasks[3 + 2 * task];
-    t.shared = a.shared_down != nullptr && t.expert == a.experts;
-    const uint32_t count = t.shared ? a.tokens : t.expert < a.experts ? a.counts[t.expert] : 0;
-    t.ok = (t.expert < a.experts || t.shared) && count <= a.tokens && t.start < count;
-    t.nrows = t.ok ? (count - t.start < kTaskRows ? count - t.start : kTaskRows) : 0;
-    if (!t.ok) { t.expert = 0; t.start = 0; t.shared = false; }  // addresses stay inside the tensors; its rows go to the spill row
-    return t;
-}
+constexpr uint32_t kInfoSlots = kResidentInfoSlots;
 
 template <int KIND>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void down_resident_kernel(ResidentDownArgs a) {
@@ -154,28 +141,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         // LDS. Every wave writes the whole table for itself (the same words), so nothing inside the tile loop reads task lists
         // from memory: a vector load there would have the compiler drain the requests in flight before it goes on.
         uint4* const info = info_tables + (MT - 1) * kInfoSlots;  // a table per pass: a wave may start the second pass while others finish the first
+        auto resolve = [&](uint32_t k) { return resolve_resident_task(a.tasks, a.counts, list[k], listed, a.experts, a.tokens, a.shared_down != nullptr); };
         if (lane < kInfoSlots && k0 + lane <= k1) {
-            const uint32_t listed_task = list[k0 + lane], task = listed_task < listed ? listed_task : 0;
-            const TaskInfo t = resolve_task(a, task);
+            const ResidentTask t = resolve(k0 + lane);
             if (!t.ok) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
-            info[lane] = uint4{task, t.expert, t.start, t.nrows | (t.shared ? 256u : 0u) | (t.ok ? 512u : 0u)};
+            info[lane] = pack_resident_task(t);
         }
-        struct Info { uint32_t task, expert, start, nrows; bool shared, ok; };
-        auto info_at = [&](uint32_t k) {  // uniform
-            uint4 v;
-            if (k - k0 < kInfoSlots) {
-                v = info[k - k0];
-            } else {  // a share of more tasks than the table holds: the slow way
-                const uint32_t listed_task = list[k], task = listed_task < listed ? listed_task : 0;
-                const TaskInfo t = resolve_task(a, task);
-                v = uint4{task, t.expert, t.start, t.nrows | (t.shared ? 256u : 0u) | (t.ok ? 512u : 0u)};
-            }
-            Info r;
-            r.task = __builtin_amdgcn_readfirstlane(v.x); r.expert = __builtin_amdgcn_readfirstlane(v.y);
-            r.start = __builtin_amdgcn_readfirstlane(v.z);
-            const uint32_t w = __builtin_amdgcn_readfirstlane(v.w);
-            r.nrows = w & 255u; r.shared = (w & 256u) != 0; r.ok = (w & 512u) != 0;
-            return r;
+        using Info = ResidentTask;
+        auto info_at = [&](uint32_t k) {  // uniform; a share of more tasks than the table holds resolves the rest the slow way
+            return unpack_resident_task(k - k0 < kInfoSlots ? info[k - k0] : pack_resident_task(resolve(k)));
         };
         auto weight_base_of = [&](const Info& t) { return t.shared ? a.shared_down : a.down + uint64_t(t.expert) * a.spec.planar_expert_bytes; };
 

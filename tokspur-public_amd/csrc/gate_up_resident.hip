@@ -27,6 +27,7 @@
 //     barrier, sum) at two waves per SIMD.
 #include "gate_up_resident.hpp"
 #include "mfma_quant.hpp"
+#include "resident_tasks.hpp"
 
 #include <type_traits>
 
@@ -41,21 +42,7 @@ constexpr int kStages = 2;
 constexpr int kPartialBytes = 4096;        // one wave's 32 x 32 f32 partial tile
 constexpr int kPhaseBytes = kWaves * kPartialBytes;
 constexpr int kTileLoads = 5;              // direct-to-LDS requests per tile and wave
-constexpr uint32_t kInfoSlots = 32;        // tasks of a workgroup's share kept in LDS, per pass
-
-struct TaskInfo { uint32_t expert, start, nrows; bool shared, ok; };
-
-__device__ __forceinline__ TaskInfo resolve_task(const ResidentGateUpArgs& a, uint32_t task) {
-    TaskInfo t;
-    t.expert = a.tasks[2 + 2 * task];
-    t.start = a.tasks[3 + 2 * task];
-    t.shared = a.shared_gate != nullptr && t.expert == a.experts;
-    const uint32_t count = t.shared ? a.tokens : t.expert < a.experts ? a.counts[t.expert] : 0;
-    t.ok = (t.expert < a.experts || t.shared) && count <= a.tokens && t.start < count;
-    t.nrows = t.ok ? (count - t.start < kTaskRows ? count - t.start : kTaskRows) : 0;
-    if (!t.ok) { t.expert = 0; t.start = 0; t.shared = false; }  // addresses stay inside the tensors; nothing of it is stored
-    return t;
-}
+constexpr uint32_t kInfoSlots = kResidentInfoSlots;
 
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gate_up_resident_kernel(ResidentGateUpArgs a) {
     // LDS: [2 phases][8 waves][4 KB partial tile] | [2 passes][32 tasks of the share] | [8 waves][2 stages][5 KB weight tile]
@@ -90,7 +77,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
                                         : uint32_t(a.spec.dm_offset) + (lane - 32) * (bpr * 4) + (wave / 4) * 16;
     const uint32_t hdr_unit_step = lane < 32 ? 32 * bpr * 16 : 32 * bpr * 4;
 
-    struct Info { uint32_t task, expert, start, nrows; bool shared, ok; };
+    using Info = ResidentTask;
     auto weight_bases = [&](const Info& t, const uint8_t*& gate, const uint8_t*& up) {
         if (t.shared) { gate = a.shared_gate; up = a.shared_up; return; }
         const uint32_t half_e = a.experts / 2;
@@ -129,24 +116,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         // from memory: a vector load there would have the compiler drain the requests in flight before it goes on. A table per
         // pass: a wave may start the second pass while others finish the first.
         uint4* const info = info_tables + (MT - 1) * kInfoSlots;
-        auto packed_info = [&](uint32_t k) {
-            const uint32_t listed_task = list[k], task = listed_task < listed ? listed_task : 0;
-            const TaskInfo t = resolve_task(a, task);
-            return uint4{task, t.expert, t.start, t.nrows | (t.shared ? 256u : 0u) | (t.ok ? 512u : 0u)};
-        };
+        auto resolve = [&](uint32_t k) { return resolve_resident_task(a.tasks, a.counts, list[k], listed, a.experts, a.tokens, a.shared_gate != nullptr); };
         if (lane < kInfoSlots && k0 + lane <= k1) {
-            const uint4 v = packed_info(k0 + lane);
-            if (!(v.w & 512u)) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
-            info[lane] = v;
+            const ResidentTask t = resolve(k0 + lane);
+            if (!t.ok) atomicOr(a.error_word, TSP_ERRBIT_INDEX);
+            info[lane] = pack_resident_task(t);
         }
-        auto info_at = [&](uint32_t k) {  // uniform
-            const uint4 v = k - k0 < kInfoSlots ? info[k - k0] : packed_info(k);  // a share of more tasks than the table holds: the slow way
-            Info r;
-            r.task = __builtin_amdgcn_readfirstlane(v.x); r.expert = __builtin_amdgcn_readfirstlane(v.y);
-            r.start = __builtin_amdgcn_readfirstlane(v.z);
-            const uint32_t w = __builtin_amdgcn_readfirstlane(v.w);
-            r.nrows = w & 255u; r.shared = (w & 256u) != 0; r.ok = (w & 512u) != 0;
-            return r;
+        auto info_at = [&](uint32_t k) {  // uniform; a share of more tasks than the table holds resolves the rest the slow way
+            return unpack_resident_task(k - k0 < kInfoSlots ? info[k - k0] : pack_resident_task(resolve(k)));
         };
 
         f16x8 A[MT][16];   // activation fragments: [row tile][k16 step of the super-block]
