@@ -86,14 +86,59 @@ template <int BPR, bool PLANAR>
 __global__ __launch_bounds__(256) void gemv_q4k(GemvArgs a) {
     constexpr int LPR = 4 * BPR;        // lanes per row
     constexpr int RPS = kWave / LPR;    // rows per wave step
-    __shared__ float xs[BPR * 256];
+    __shared__ __attribute__((aligned(16))) float xs[BPR * 256];
     const uint8_t* w; const float* x; float* y;
     if (!resolve(a, w, x, y)) return;
-    for (uint32_t i = threadIdx.x; i < BPR * 256; i += blockDim.x) xs[i] = x[i];
-    __syncthreads();
-
     const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const uint32_t pair = lane % 4, blk_in_row = (lane / 4) % BPR, row_in_step = lane / LPR;
+    const uint32_t steps = (a.rows + RPS - 1) / RPS;
+    const uint32_t waves = gridDim.x * (blockDim.x / kWave);
+
+    // The bytes of one step as they come from memory: nothing is computed on them until they are needed, so that a step's
+    // requests can be in flight while something else happens (the activations being staged, the step before being summed).
+    struct Raw { uint4 q0, q1, hdr; uint32_t sc, mn, dm; };
+    auto fetch = [&](uint32_t step) {
+        const uint32_t row = step * RPS + row_in_step;
+        const uint64_t blk = uint64_t(row < a.rows ? row : a.rows - 1) * BPR + blk_in_row;
+        Raw r{};
+        if constexpr (PLANAR) {
+            const uint8_t* qs = w + a.spec.qs_offset + blk * 128 + pair * 32;
+            r.q0 = *reinterpret_cast<const uint4*>(qs);
+            r.q1 = *reinterpret_cast<const uint4*>(qs + 16);
+            const uint8_t* sm = w + a.spec.sm_offset + blk * 16 + pair * 2;
+            r.sc = *reinterpret_cast<const uint16_t*>(sm);
+            r.mn = *reinterpret_cast<const uint16_t*>(sm + 8);
+            r.dm = *reinterpret_cast<const uint32_t*>(w + a.spec.dm_offset + blk * 4);
+        } else {
+            const uint8_t* block = w + blk * 144;
+            r.hdr = *reinterpret_cast<const uint4*>(block);
+            r.q0 = *reinterpret_cast<const uint4*>(block + 16 + pair * 32);
+            r.q1 = *reinterpret_cast<const uint4*>(block + 32 + pair * 32);
+        }
+        return r;
+    };
+
+    // The activations are asked for first (a few cached kilobytes: they come back first), the wave's first weight bytes right
+    // behind them; the activations are staged and summed while the weights travel.
+    constexpr uint32_t kQuads = BPR * 64;                // float4 in a row of activations
+    constexpr uint32_t kMine = (kQuads + 255) / 256;     // per thread: 1 (K = 512, half the threads) .. 16 (K = 4096)
+    float4 xv[kMine];
+    const bool x_quads = reinterpret_cast<uintptr_t>(x) % 16 == 0;  // else a row that only floats align
+#pragma unroll
+    for (uint32_t j = 0; j < kMine; ++j) {
+        const uint32_t quad = threadIdx.x + j * 256;
+        if (kQuads % 256 == 0 || quad < kQuads) {
+            if (x_quads) xv[j] = reinterpret_cast<const float4*>(x)[quad];
+            else xv[j] = make_float4(x[4 * quad], x[4 * quad + 1], x[4 * quad + 2], x[4 * quad + 3]);
+        }
+    }
+    uint32_t step = blockIdx.x * (blockDim.x / kWave) + wave;
+    Raw cur = fetch(step < steps ? step : 0);
+#pragma unroll
+    for (uint32_t j = 0; j < kMine; ++j)
+        if (kQuads % 256 == 0 || threadIdx.x + j * 256 < kQuads) reinterpret_cast<float4*>(xs)[threadIdx.x + j * 256] = xv[j];
+    __syncthreads();
+
     float xa[32], xb[32];
     float sxa = 0, sxb = 0;
     {
@@ -104,29 +149,18 @@ __global__ __launch_bounds__(256) void gemv_q4k(GemvArgs a) {
         for (int i = 0; i < 32; ++i) { xb[i] = src[32 + i]; sxb += xb[i]; }
     }
 
-    const uint32_t steps = (a.rows + RPS - 1) / RPS;
-    const uint32_t waves = gridDim.x * (blockDim.x / kWave);
-    for (uint32_t step = blockIdx.x * (blockDim.x / kWave) + wave; step < steps; step += waves) {
+    for (; step < steps; step += waves) {
         const uint32_t row = step * RPS + row_in_step;
         const bool live = row < a.rows;
-        const uint64_t blk = uint64_t(live ? row : a.rows - 1) * BPR + blk_in_row;
-        uint4 q0, q1;
+        const Raw now = cur;
+        cur = fetch(step + waves < steps ? step + waves : step);  // the next step's bytes travel while this one is summed
         float d, dmin;
         uint32_t sc_a, sc_b, mn_a, mn_b;
         if constexpr (PLANAR) {
-            const uint8_t* qs = w + a.spec.qs_offset + blk * 128 + pair * 32;
-            q0 = *reinterpret_cast<const uint4*>(qs);
-            q1 = *reinterpret_cast<const uint4*>(qs + 16);
-            const uint8_t* sm = w + a.spec.sm_offset + blk * 16 + pair * 2;
-            const uint32_t sc = *reinterpret_cast<const uint16_t*>(sm), mn = *reinterpret_cast<const uint16_t*>(sm + 8);
-            const uint32_t dm = *reinterpret_cast<const uint32_t*>(w + a.spec.dm_offset + blk * 4);
-            sc_a = sc & 0xffu; sc_b = sc >> 8; mn_a = mn & 0xffu; mn_b = mn >> 8;
-            d = half_bits_to_float(dm & 0xffffu); dmin = half_bits_to_float(dm >> 16);
+            sc_a = now.sc & 0xffu; sc_b = now.sc >> 8; mn_a = now.mn & 0xffu; mn_b = now.mn >> 8;
+            d = half_bits_to_float(now.dm & 0xffffu); dmin = half_bits_to_float(now.dm >> 16);
         } else {
-            const uint8_t* block = w + blk * 144;
-            const uint4 hdr = *reinterpret_cast<const uint4*>(block);
-            q0 = *reinterpret_cast<const uint4*>(block + 16 + pair * 32);
-            q1 = *reinterpret_cast<const uint4*>(block + 32 + pair * 32);
+            const uint4 hdr = now.hdr;
             d = half_bits_to_float(hdr.x & 0xffffu); dmin = half_bits_to_float(hdr.x >> 16);
             // sub-blocks 2*pair and 2*pair+1: byte j = (2*pair) & 3 (and j+1) of the three header words
             const uint32_t sh = (pair & 1u) * 16u;
@@ -140,7 +174,7 @@ __global__ __launch_bounds__(256) void gemv_q4k(GemvArgs a) {
                 mn_b = ((e2 >> 12) & 15u) | (((m2 >> 14) & 3u) << 4);
             }
         }
-        const uint32_t words[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+        const uint32_t words[8] = {now.q0.x, now.q0.y, now.q0.z, now.q0.w, now.q1.x, now.q1.y, now.q1.z, now.q1.w};
         float dot_a0 = 0, dot_a1 = 0, dot_b0 = 0, dot_b1 = 0;
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
