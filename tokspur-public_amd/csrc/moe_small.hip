@@ -10,6 +10,7 @@
 // and the up row of the same hidden unit, so SwiGLU needs one cross-lane move), and Q6_K planes
 // for the down projection. Every other planar encoding goes through the generic arm.
 #include "decode.hpp"
+#include "record_resident.hpp"
 #include "skinny.hpp"
 
 using namespace tsp;
@@ -421,8 +422,10 @@ SkinnyMoe skinny_view(const SmallMoeArgs& a, const tsp_shared_rows* shared = nul
 
 int launch_gate_up(const SmallMoeArgs& a, hipStream_t s, const tsp_shared_rows* shared = nullptr) {
     const uint32_t records = record_slots(a);
-    if (skinny_moe_supported(a.gu.source_type, a.dn.source_type, a.channels, a.hidden, a.x, a.x_stride, a.h, a.h_stride, false))
-        return skinny_moe_gate_up(skinny_view(a, shared), s);
+    if (skinny_moe_supported(a.gu.source_type, a.dn.source_type, a.channels, a.hidden, a.x, a.x_stride, a.h, a.h_stride, false)) {
+        const SkinnyMoe view = skinny_view(a, shared);
+        return skinny_moe_gate_up(view, s);
+    }
     TSP_REQUIRE(!shared, "the always-on expert rides only on the matrix-core small-row kernels");
     const bool x_aligned = reinterpret_cast<uintptr_t>(a.x) % 16 == 0 && a.x_stride % 16 == 0;
     if (a.gu.source_type == 12 && x_aligned && (a.channels == 512 || a.channels == 1024 || a.channels == 2048)) {
@@ -451,8 +454,10 @@ int launch_gate_up(const SmallMoeArgs& a, hipStream_t s, const tsp_shared_rows* 
 
 int launch_down(const SmallMoeArgs& a, hipStream_t s, const tsp_shared_rows* shared = nullptr) {
     const uint32_t records = record_slots(a);
-    if (a.dn.source_type == 14 && a.hidden % 256 == 0 && a.hidden <= 2048 && reinterpret_cast<uintptr_t>(a.h) % 16 == 0 && a.h_stride % 16 == 0)
-        return skinny_moe_down(skinny_view(a, shared), s);
+    if (a.dn.source_type == 14 && a.hidden % 256 == 0 && a.hidden <= 2048 && reinterpret_cast<uintptr_t>(a.h) % 16 == 0 && a.h_stride % 16 == 0) {
+        const SkinnyMoe view = skinny_view(a, shared);
+        return skinny_moe_down(view, s);
+    }
     TSP_REQUIRE(!shared, "the always-on expert rides only on the matrix-core small-row kernels");
     const bool h_aligned = reinterpret_cast<uintptr_t>(a.h) % 16 == 0 && a.h_stride % 16 == 0;
     if (a.dn.source_type == 14 && h_aligned && (a.hidden == 256 || a.hidden == 512 || a.hidden == 1024)) {
