@@ -424,7 +424,7 @@ int launch_gate_up(const SmallMoeArgs& a, hipStream_t s, const tsp_shared_rows* 
     const uint32_t records = record_slots(a);
     if (skinny_moe_supported(a.gu.source_type, a.dn.source_type, a.channels, a.hidden, a.x, a.x_stride, a.h, a.h_stride, false)) {
         const SkinnyMoe view = skinny_view(a, shared);
-        return skinny_moe_gate_up(view, s);
+        return record_gate_up_takes(view) ? launch_record_gate_up(view, s) : skinny_moe_gate_up(view, s);
     }
     TSP_REQUIRE(!shared, "the always-on expert rides only on the matrix-core small-row kernels");
     const bool x_aligned = reinterpret_cast<uintptr_t>(a.x) % 16 == 0 && a.x_stride % 16 == 0;
