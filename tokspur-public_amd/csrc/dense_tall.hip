@@ -1,0 +1,238 @@
+// Dense Q4_K GEMM for a thousand and more activation rows: out[m, n] = sum_k x[m, k] * half(dec(W[n, k])), f32 accumulation.
+//
+// With this many rows the product is bound by the matrix cores, provided the weights are not unpacked over and over: the
+// 64-row tiles of the general kernel (gemm.hip) unpack every weight once per 64 activation rows, and at 2048 rows spend
+// eight vector instructions per MFMA doing so. Here a workgroup of eight waves owns a 256 x 256 output tile, a wave 128
+// activation rows x 64 weight rows (four row tiles x two column tiles: 128 accumulator registers), so a weight is unpacked
+// once per 128 rows and a step of 64 columns is 32 MFMAs against ~180 vector instructions per wave.
+//
+//   * Arithmetic: the engine's for this path. A weight is its f32 value d * sc * q - dmin * mn rounded once to half (one
+//     v_cvt_f32_ubyte and one mixed-precision fused multiply-add per weight, exact in f32 before the rounding); activations
+//     are the bf16 values carried as halves; products accumulate in f32 on v_mfma_f32_32x32x16_f16.
+//   * Activations: 256 rows x 128 bytes per step go global -> LDS directly, two steps ahead, into a ring of three slabs
+//     shared by the eight waves (16-byte chunk c of row r at position c ^ (r % 8)); one LDS-only barrier per step.
+//   * Weights: the step's 32 bytes of nibbles of the tile's 256 rows (8 KB, ring of four) and, once per super-block, the
+//     rows' 16 header bytes (d, dmin, packed scales and minima; ring of two) travel the same way. Every request in the
+//     loop is unconditional and issued by every thread (rows past the matrix's end repeat its last row), so each wave
+//     waits with an exact count.
+//   * Workgroups are dealt to the XCDs in runs of consecutive tiles, column tiles fastest: the workgroups of one XCD
+//     share a slab of activation rows in its L2 and read every weight byte once.
+#include "dense_tall.hpp"
+
+#include <type_traits>
+
+#include "mfma_quant.hpp"
+
+using namespace tsp;
+
+namespace {
+
+// A pointer that is the same in every lane, moved to scalar registers (the base operand of a direct-to-LDS request has to be one).
+__device__ __forceinline__ const uint8_t* uniform_pointer(const uint8_t* p) {
+    const uint64_t bits = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(bits))), hi = uint32_t(__builtin_amdgcn_readfirstlane(uint32_t(bits >> 32)));
+    return reinterpret_cast<const uint8_t*>(uint64_t(hi) << 32 | lo);
+}
+
+// Byte N of a word as a float: one v_cvt_f32_ubyteN.
+template <int N>
+__device__ __forceinline__ float byte_as_float(uint32_t word) { return float((word >> (8 * N)) & 0xffu); }
+
+constexpr int kWavesT = 8, kThreadsT = kWavesT * kWave;
+constexpr int kTileM = 256, kTileN = 256, kStepK = 64;
+constexpr int kSlabBytes = kTileM * kStepK * 2, kSlabs = 3;
+constexpr int kQsBytes = kTileN * 32, kQsStages = 4;
+constexpr int kHdrBytes = kTileN * 16, kHdrStages = 2;
+constexpr int kQsAt = kSlabs * kSlabBytes, kHdrAt = kQsAt + kQsStages * kQsBytes;
+
+__global__ __launch_bounds__(kThreadsT) __attribute__((amdgpu_waves_per_eu(2, 2))) void dense_tall_kernel(DenseTallArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kHdrAt + kHdrStages * kHdrBytes];
+    static_assert(sizeof(lds_raw) <= 160 * 1024, "one workgroup per compute unit");
+
+    const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const uint32_t col = lane % 32, khalf = (lane / 32) & 1;
+    const uint32_t wm = wave / 4, wn = wave % 4;  // the wave's 128 activation rows and 64 weight rows of the tile
+
+    // ---- the workgroup's tile: XCD x (workgroup id % 8) takes the x-th run of consecutive tiles
+    const uint32_t n_tiles = (a.n + kTileN - 1) / kTileN, m_tiles = (a.m + kTileM - 1) / kTileM;
+    const uint32_t tiles = n_tiles * m_tiles, per_xcd = (tiles + 7) / 8;
+    const uint32_t logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (blockIdx.x / 8 >= per_xcd || logical >= tiles) return;
+    const uint32_t m0 = (logical / n_tiles) * kTileM, n0 = (logical % n_tiles) * kTileN;
+    const uint32_t bpr = a.k / 256, steps = a.k / kStepK;
+    const uint32_t row_bytes = bpr * 144;
+
+    // ---- per-thread parts of the request addresses (the per-step parts are uniform)
+    // activations: request i of thread t fills 16-byte position t + 512 i of the slab = slot t % 8 of row t / 8 + 64 i, with
+    // chunk (t % 8) ^ (row % 8) of that row
+    uint32_t a_lane[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t r = tid / 8 + 64 * i, row = m0 + r < a.m ? m0 + r : a.m - 1;
+        a_lane[i] = (row * a.a_stride + (((tid % 8) ^ (r & 7)) * 8)) * 2;
+    }
+    // nibbles: thread t fills position t of the stage = slot t % 2 of weight row t / 2, with chunk (t % 2) ^ ((row / 8) % 2) of the
+    // step's 32 bytes of that row; headers: position t % 256 = weight row t % 256 (the two halves of the workgroup fetch the same)
+    const uint32_t q_r = tid / 2, q_row = n0 + q_r < a.n ? n0 + q_r : a.n - 1;
+    const uint32_t q_lane = q_row * row_bytes + (((tid % 2) ^ ((q_r >> 3) & 1)) * 16);
+    const uint32_t h_r = tid % 256, h_row = n0 + h_r < a.n ? n0 + h_r : a.n - 1;
+    const uint32_t h_lane = h_row * row_bytes;
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds_raw));
+    const uint32_t my_slab = lds0 + wave * 1024, my_qs = lds0 + kQsAt + wave * 1024, my_hdr = lds0 + kHdrAt + (wave % 4) * 1024;
+    auto request = [&](uint32_t step) {  // steps past the end ask for the last step again (nobody reads it)
+        step = step < steps ? step : steps - 1;
+        const uint32_t b = step / 4, pair = step % 4;
+        const uint8_t* a_base = uniform_pointer(reinterpret_cast<const uint8_t*>(a.a) + uint64_t(step) * (kStepK * 2));
+        const uint32_t slab = my_slab + (step % kSlabs) * kSlabBytes;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load_to_lds_16(a_base, a_lane[i], slab + i * 8192);
+        load_to_lds_16(a.w + uint64_t(b) * 144 + 16 + pair * 32, q_lane, my_qs + (step % kQsStages) * kQsBytes);
+        if (pair == 0) load_to_lds_16(a.w + uint64_t(b) * 144, h_lane, my_hdr + (b % kHdrStages) * kHdrBytes);
+    };
+
+    f32x16 acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    // fragment reads: lane (col, khalf) takes chunk 4 hi + 2 khalf + ff of activation row col (+ 32 i) and the k-half's 16 bytes of
+    // the nibbles of weight row col (+ 32 j)
+    const uint32_t a_row_at = (wm * 128 + col) * 128, a_swz = col & 7;
+    uint32_t q_at[2], hdr_at[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t r = wn * 64 + j * 32 + col;
+        q_at[j] = kQsAt + r * 32 + ((khalf ^ ((r >> 3) & 1)) * 16);
+        hdr_at[j] = kHdrAt + r * 16;
+    }
+
+    float d[2], dmin[2];
+    uint32_t sc[2][2], mn[2][2];  // eight scales and eight minima per weight row, one per byte
+    auto step_fn = [&](uint32_t step, auto p_tag) {
+        constexpr int P = decltype(p_tag)::value;  // the pair of sub-blocks of the super-block: step % 4
+        // Wait for this thread's requests of the step (issued two steps ago); younger than those are the requests of the
+        // next step: four slabs pieces, the nibbles, and at the last pair the next super-block's headers. Then the
+        // barrier: every thread's pieces have landed, and every wave has left the buffers that the next requests overwrite.
+        lds_barrier_after_loads<P == 3 ? 6 : 5>();
+        request(step + 2);
+        const uint8_t* slab = lds_raw + (step % kSlabs) * kSlabBytes;
+        const uint8_t* qs = lds_raw + (step % kQsStages) * kQsBytes;
+        if constexpr (P == 0) {
+            const uint8_t* hdr = lds_raw + ((step / 4) % kHdrStages) * kHdrBytes;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                RawHdrQ4 raw;
+                raw.words = *reinterpret_cast<const uint4*>(hdr + hdr_at[j]);
+                raw.dm = 0;
+                const HdrQ4 h = decode_hdr_q4k<B_Q4K_RAW>(raw);
+                d[j] = h.d; dmin[j] = h.dmin;
+                sc[j][0] = h.sc[0]; sc[j][1] = h.sc[1]; mn[j][0] = h.mn[0]; mn[j][1] = h.mn[1];
+            }
+        }
+        // the lane's 16 bytes of the pair, per column tile: low nibbles are sub-block 2 P, high nibbles sub-block 2 P + 1
+        uint32_t nib[2][2][4];  // [column tile][low, high][word]: four codes per word, one per byte
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const u32x4 raw = *reinterpret_cast<const u32x4*>(qs + q_at[j]);
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                nib[j][0][w] = raw[w] & 0x0f0f0f0fu;
+                nib[j][1][w] = (raw[w] >> 4) & 0x0f0f0f0fu;
+                // kept as they are: left to itself the compiler digs every code out of the raw word again, a bit-field extract per weight
+                asm volatile("" : "+v"(nib[j][0][w]), "+v"(nib[j][1][w]));
+            }
+        }
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi) {
+            // sub-block 2 P + hi; weight = half(d * sc * q - dmin * mn), the f32 value rounded once
+            float scale[2], offset[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t s4 = sc[j][P / 2], m4 = mn[j][P / 2];
+                const float s8 = (P % 2) * 2 + hi == 0 ? byte_as_float<0>(s4) : (P % 2) * 2 + hi == 1 ? byte_as_float<1>(s4)
+                               : (P % 2) * 2 + hi == 2 ? byte_as_float<2>(s4) : byte_as_float<3>(s4);
+                const float m8 = (P % 2) * 2 + hi == 0 ? byte_as_float<0>(m4) : (P % 2) * 2 + hi == 1 ? byte_as_float<1>(m4)
+                               : (P % 2) * 2 + hi == 2 ? byte_as_float<2>(m4) : byte_as_float<3>(m4);
+                scale[j] = d[j] * s8;
+                offset[j] = -(dmin[j] * m8);
+            }
+#pragma unroll
+            for (int ff = 0; ff < 2; ++ff) {
+                f16x8 b[2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const uint32_t w0 = nib[j][hi][2 * ff], w1 = nib[j][hi][2 * ff + 1];
+                    b[j][0] = _Float16(__builtin_fmaf(byte_as_float<0>(w0), scale[j], offset[j]));
+                    b[j][1] = _Float16(__builtin_fmaf(byte_as_float<1>(w0), scale[j], offset[j]));
+                    b[j][2] = _Float16(__builtin_fmaf(byte_as_float<2>(w0), scale[j], offset[j]));
+                    b[j][3] = _Float16(__builtin_fmaf(byte_as_float<3>(w0), scale[j], offset[j]));
+                    b[j][4] = _Float16(__builtin_fmaf(byte_as_float<0>(w1), scale[j], offset[j]));
+                    b[j][5] = _Float16(__builtin_fmaf(byte_as_float<1>(w1), scale[j], offset[j]));
+                    b[j][6] = _Float16(__builtin_fmaf(byte_as_float<2>(w1), scale[j], offset[j]));
+                    b[j][7] = _Float16(__builtin_fmaf(byte_as_float<3>(w1), scale[j], offset[j]));
+                }
+                const uint32_t chunk = ((4 * hi + 2 * khalf + ff) ^ a_swz) * 16;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const f16x8 af = *reinterpret_cast<const f16x8*>(slab + a_row_at + i * (32 * 128) + chunk);
+                    acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b[0], acc[i][0], 0, 0, 0);
+                    acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b[1], acc[i][1], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    request(0);
+    request(1);
+    for (uint32_t b = 0; b < bpr; ++b) {
+        step_fn(b * 4 + 0, std::integral_constant<int, 0>{});
+        step_fn(b * 4 + 1, std::integral_constant<int, 1>{});
+        step_fn(b * 4 + 2, std::integral_constant<int, 2>{});
+        step_fn(b * 4 + 3, std::integral_constant<int, 3>{});
+    }
+    wait_all_loads();  // the last steps requested buffers that nobody reads: they must have landed before the LDS is given away
+
+    // ---- epilogue. Accumulator v of tile (i, j): row 32 i + 8 (v / 4) + 4 khalf + v % 4 of the wave's 128, weight row col of column tile j
+    uint32_t biggest = 0;  // the largest result's bits without the sign: anything not finite shows at the end
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const uint32_t row = m0 + wm * 128 + i * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
+            if (row >= a.m) continue;
+            uint8_t* orow = static_cast<uint8_t*>(a.out) + uint64_t(row) * a.out_stride;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t n = n0 + wn * 64 + j * 32 + col;
+                if (n >= a.n) continue;
+                const float val = acc[i][j][v];
+                const uint32_t vb = __float_as_uint(val), magnitude = vb & 0x7fffffffu;
+                biggest = biggest > magnitude ? biggest : magnitude;
+                if (a.out_bf16) reinterpret_cast<uint16_t*>(orow)[n] = uint16_t((vb + 0x7fffu + ((vb >> 16) & 1u)) >> 16);
+                else reinterpret_cast<float*>(orow)[n] = val;
+            }
+        }
+    }
+    publish_error(biggest >= 0x7f800000u ? uint32_t(TSP_ERRBIT_NONFINITE) : 0u, a.error_word);
+}
+
+}  // namespace
+
+namespace tsp {
+
+bool dense_tall_takes(uint32_t tokens, uint32_t rows, uint32_t columns, uint64_t matrix_bytes) {
+    return tokens >= 1024 && rows >= kTileN && columns % 256 == 0 && columns >= 256 && matrix_bytes < (1ull << 32) &&
+           uint64_t(tokens) * columns * 2 < (1ull << 32);
+}
+
+int launch_dense_tall(const DenseTallArgs& a, hipStream_t s) {
+    const uint32_t tiles = ((a.n + kTileN - 1) / kTileN) * ((a.m + kTileM - 1) / kTileM);
+    const uint32_t groups = (tiles + 7) / 8 * 8;
+    TSP_LAUNCH("gemm_dense_tall", s, dense_tall_kernel<<<groups, kThreadsT, 0, s>>>(a));
+    return launch_status("dense_tall");
+}
+
+}  // namespace tsp

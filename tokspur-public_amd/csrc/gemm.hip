@@ -24,6 +24,7 @@
 //     two and three steps ahead, into a ring of four slabs; one LDS-only barrier per K step.
 //   * For gate/up the two column tiles of a wave are the gate rows and the up rows of the same 32 hidden
 //     units, so SwiGLU is an element-wise epilogue on accumulator registers.
+#include "dense_tall.hpp"
 #include "down_resident.hpp"
 #include "gate_up_resident.hpp"
 #include "grouped_staged.hpp"
@@ -660,6 +661,15 @@ extern "C" int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matr
     const auto s = static_cast<hipStream_t>(stream);
     auto* xh = static_cast<_Float16*>(workspace);
     auto* sx = reinterpret_cast<_Float16*>(static_cast<uint8_t*>(workspace) + align256(uint64_t(tokens) * columns * 2));
+    if (encoding == 12 && layout == TSP_LAYOUT_GGUF && dense_tall_takes(tokens, rows, columns, matrix_bytes)) {
+        // a thousand rows and more: 256 x 256 tiles, weights rounded once to half (the engine's arithmetic for this product)
+        int rc = convert_rows(input, input_stride_bytes, input_is_bf16, xh, nullptr, tokens, columns, error_word, s);
+        if (rc != TSP_OK) return rc;
+        DenseTallArgs t{};
+        t.a = xh; t.a_stride = columns; t.w = static_cast<const uint8_t*>(matrix); t.m = tokens; t.n = rows; t.k = columns;
+        t.out = output; t.out_stride = output_stride_bytes; t.out_bf16 = output_is_bf16; t.error_word = error_word;
+        return launch_dense_tall(t, s);
+    }
     int rc = convert_rows(input, input_stride_bytes, input_is_bf16, xh, encoding == 12 ? sx : nullptr, tokens, columns, error_word, s);
     if (rc != TSP_OK) return rc;
     a.a = xh; a.a_stride = columns; a.sx = sx; a.w0 = static_cast<const uint8_t*>(matrix); a.experts = 1;
