@@ -38,20 +38,22 @@ __device__ __forceinline__ const uint8_t* uniform_pointer(const uint8_t* p) {
 template <int N>
 __device__ __forceinline__ float byte_as_float(uint32_t word) { return float((word >> (8 * N)) & 0xffu); }
 
-constexpr int kWavesT = 8, kThreadsT = kWavesT * kWave;
-constexpr int kTileM = 256, kTileN = 256, kStepK = 64;
-constexpr int kSlabBytes = kTileM * kStepK * 2, kSlabs = 3;
-constexpr int kQsBytes = kTileN * 32, kQsStages = 4;
+constexpr int kTileN = 256, kStepK = 64, kRing = 3;
+constexpr int kQsBytes = kTileN * 32;
 constexpr int kHdrBytes = kTileN * 16, kHdrStages = 2;
-constexpr int kQsAt = kSlabs * kSlabBytes, kHdrAt = kQsAt + kQsStages * kQsBytes;
 
-__global__ __launch_bounds__(kThreadsT) __attribute__((amdgpu_waves_per_eu(2, 2))) void dense_tall_kernel(DenseTallArgs a) {
+// WM: the workgroup's waves along the activation rows, 128 rows each (4 WM waves, a tile of 128 WM x 256).
+template <int WM>
+__global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))) void dense_tall_kernel(DenseTallArgs a) {
+    constexpr int kThreadsT = 256 * WM, kTileM = 128 * WM;
+    constexpr int kSlabBytes = kTileM * kStepK * 2;
+    constexpr int kQsAt = kRing * kSlabBytes, kHdrAt = kQsAt + kRing * kQsBytes;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kHdrAt + kHdrStages * kHdrBytes];
-    static_assert(sizeof(lds_raw) <= 160 * 1024, "one workgroup per compute unit");
+    static_assert(sizeof(lds_raw) * (2 / WM) <= 160 * 1024, "two waves per SIMD: one workgroup of eight waves or two of four per compute unit");
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const uint32_t col = lane % 32, khalf = (lane / 32) & 1;
-    const uint32_t wm = wave / 4, wn = wave % 4;  // the wave's 128 activation rows and 64 weight rows of the tile
+    const uint32_t wm = wave / 4, wn = wave % 4;  // the wave's 128 activation rows and 64 weight rows of the tile (wm < WM)
 
     // ---- the workgroup's tile: XCD x (workgroup id % 8) takes the x-th run of consecutive tiles
     const uint32_t n_tiles = (a.n + kTileN - 1) / kTileN, m_tiles = (a.m + kTileM - 1) / kTileM;
@@ -63,18 +65,24 @@ __global__ __launch_bounds__(kThreadsT) __attribute__((amdgpu_waves_per_eu(2, 2)
     const uint32_t row_bytes = bpr * 144;
 
     // ---- per-thread parts of the request addresses (the per-step parts are uniform)
-    // activations: request i of thread t fills 16-byte position t + 512 i of the slab = slot t % 8 of row t / 8 + 64 i, with
-    // chunk (t % 8) ^ (row % 8) of that row
+    // activations: request i of thread t fills 16-byte position t + T i of the slab (T threads) = slot t % 8 of row (t + T i) / 8,
+    // with chunk (t % 8) ^ (row % 8) of that row
     uint32_t a_lane[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const uint32_t r = tid / 8 + 64 * i, row = m0 + r < a.m ? m0 + r : a.m - 1;
+        const uint32_t r = (tid + kThreadsT * i) / 8, row = m0 + r < a.m ? m0 + r : a.m - 1;
         a_lane[i] = (row * a.a_stride + (((tid % 8) ^ (r & 7)) * 8)) * 2;
     }
-    // nibbles: thread t fills position t of the stage = slot t % 2 of weight row t / 2, with chunk (t % 2) ^ ((row / 8) % 2) of the
-    // step's 32 bytes of that row; headers: position t % 256 = weight row t % 256 (the two halves of the workgroup fetch the same)
-    const uint32_t q_r = tid / 2, q_row = n0 + q_r < a.n ? n0 + q_r : a.n - 1;
-    const uint32_t q_lane = q_row * row_bytes + (((tid % 2) ^ ((q_r >> 3) & 1)) * 16);
+    // nibbles: request q of thread t fills position u = t + T q of the stage = slot u % 2 of weight row u / 2, with chunk
+    // (u % 2) ^ ((row / 8) % 2) of the step's 32 bytes of that row; headers: position t % 256 = weight row t % 256 (with eight
+    // waves the two halves of the workgroup fetch the same)
+    constexpr int QN = 2 / WM;
+    uint32_t q_lane[QN];
+#pragma unroll
+    for (int q = 0; q < QN; ++q) {
+        const uint32_t u = tid + kThreadsT * q, q_r = u / 2, q_row = n0 + q_r < a.n ? n0 + q_r : a.n - 1;
+        q_lane[q] = q_row * row_bytes + (((u % 2) ^ ((q_r >> 3) & 1)) * 16);
+    }
     const uint32_t h_r = tid % 256, h_row = n0 + h_r < a.n ? n0 + h_r : a.n - 1;
     const uint32_t h_lane = h_row * row_bytes;
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds_raw));
@@ -83,10 +91,11 @@ __global__ __launch_bounds__(kThreadsT) __attribute__((amdgpu_waves_per_eu(2, 2)
         step = step < steps ? step : steps - 1;
         const uint32_t b = step / 4, pair = step % 4;
         const uint8_t* a_base = uniform_pointer(reinterpret_cast<const uint8_t*>(a.a) + uint64_t(step) * (kStepK * 2));
-        const uint32_t slab = my_slab + (step % kSlabs) * kSlabBytes;
+        const uint32_t slab = my_slab + (step % kRing) * kSlabBytes;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_to_lds_16(a_base, a_lane[i], slab + i * 8192);
-        load_to_lds_16(a.w + uint64_t(b) * 144 + 16 + pair * 32, q_lane, my_qs + (step % kQsStages) * kQsBytes);
+        for (int i = 0; i < 4; ++i) load_to_lds_16(a_base, a_lane[i], slab + i * (kThreadsT * 16));
+#pragma unroll
+        for (int q = 0; q < QN; ++q) load_to_lds_16(a.w + uint64_t(b) * 144 + 16 + pair * 32, q_lane[q], my_qs + (step % kRing) * kQsBytes + q * (kThreadsT * 16));
         if (pair == 0) load_to_lds_16(a.w + uint64_t(b) * 144, h_lane, my_hdr + (b % kHdrStages) * kHdrBytes);
     };
 
@@ -114,12 +123,12 @@ __global__ __launch_bounds__(kThreadsT) __attribute__((amdgpu_waves_per_eu(2, 2)
     auto step_fn = [&](uint32_t step, auto p_tag) {
         constexpr int P = decltype(p_tag)::value;  // the pair of sub-blocks of the super-block: step % 4
         // Wait for this thread's requests of the step (issued two steps ago); younger than those are the requests of the
-        // next step: four slabs pieces, the nibbles, and at the last pair the next super-block's headers. Then the
+        // next step: four slab pieces, the nibbles, and at the last pair the next super-block's headers. Then the
         // barrier: every thread's pieces have landed, and every wave has left the buffers that the next requests overwrite.
-        lds_barrier_after_loads<P == 3 ? 6 : 5>();
+        lds_barrier_after_loads<4 + QN + (P == 3 ? 1 : 0)>();
         request(step + 2);
-        const uint8_t* slab = lds_raw + (step % kSlabs) * kSlabBytes;
-        const uint8_t* qs = lds_raw + (step % kQsStages) * kQsBytes;
+        const uint8_t* slab = lds_raw + (step % kRing) * kSlabBytes;
+        const uint8_t* qs = lds_raw + (step % kRing) * kQsBytes;
         if constexpr (P == 0) {
             const uint8_t* hdr = lds_raw + ((step / 4) % kHdrStages) * kHdrBytes;
 #pragma unroll
@@ -145,42 +154,51 @@ __global__ __launch_bounds__(kThreadsT) __attribute__((amdgpu_waves_per_eu(2, 2)
                 asm volatile("" : "+v"(nib[j][0][w]), "+v"(nib[j][1][w]));
             }
         }
+        // The four k16 groups of the step, (low, high nibbles) x (first, second eight columns of the lane's sixteen). The
+        // activation fragments of a group are read one group ahead, so that their LDS latency passes behind the unpacking
+        // of the weights; left to itself the compiler reads them two at a time right before the MFMAs that use them.
+        auto read_a = [&](int g, f16x8 (&af)[4]) {
+            const uint32_t chunk = ((4 * (g / 2) + 2 * khalf + (g % 2)) ^ a_swz) * 16;
 #pragma unroll
-        for (int hi = 0; hi < 2; ++hi) {
-            // sub-block 2 P + hi; weight = half(d * sc * q - dmin * mn), the f32 value rounded once
-            float scale[2], offset[2];
+            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const f16x8*>(slab + a_row_at + i * (32 * 128) + chunk);
+        };
+        f16x8 af[2][4];
+        read_a(0, af[0]);
+        float scale[2], offset[2];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const uint32_t s4 = sc[j][P / 2], m4 = mn[j][P / 2];
-                const float s8 = (P % 2) * 2 + hi == 0 ? byte_as_float<0>(s4) : (P % 2) * 2 + hi == 1 ? byte_as_float<1>(s4)
-                               : (P % 2) * 2 + hi == 2 ? byte_as_float<2>(s4) : byte_as_float<3>(s4);
-                const float m8 = (P % 2) * 2 + hi == 0 ? byte_as_float<0>(m4) : (P % 2) * 2 + hi == 1 ? byte_as_float<1>(m4)
-                               : (P % 2) * 2 + hi == 2 ? byte_as_float<2>(m4) : byte_as_float<3>(m4);
-                scale[j] = d[j] * s8;
-                offset[j] = -(dmin[j] * m8);
-            }
-#pragma unroll
-            for (int ff = 0; ff < 2; ++ff) {
-                f16x8 b[2];
+        for (int g = 0; g < 4; ++g) {
+            const int hi = g / 2, ff = g % 2;
+            if (g < 3) read_a(g + 1, af[(g + 1) % 2]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (ff == 0) {
+                // sub-block 2 P + hi; weight = half(d * sc * q - dmin * mn), the f32 value rounded once
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
-                    const uint32_t w0 = nib[j][hi][2 * ff], w1 = nib[j][hi][2 * ff + 1];
-                    b[j][0] = _Float16(__builtin_fmaf(byte_as_float<0>(w0), scale[j], offset[j]));
-                    b[j][1] = _Float16(__builtin_fmaf(byte_as_float<1>(w0), scale[j], offset[j]));
-                    b[j][2] = _Float16(__builtin_fmaf(byte_as_float<2>(w0), scale[j], offset[j]));
-                    b[j][3] = _Float16(__builtin_fmaf(byte_as_float<3>(w0), scale[j], offset[j]));
-                    b[j][4] = _Float16(__builtin_fmaf(byte_as_float<0>(w1), scale[j], offset[j]));
-                    b[j][5] = _Float16(__builtin_fmaf(byte_as_float<1>(w1), scale[j], offset[j]));
-                    b[j][6] = _Float16(__builtin_fmaf(byte_as_float<2>(w1), scale[j], offset[j]));
-                    b[j][7] = _Float16(__builtin_fmaf(byte_as_float<3>(w1), scale[j], offset[j]));
+                    const uint32_t s4 = sc[j][P / 2], m4 = mn[j][P / 2];
+                    constexpr int B = (P % 2) * 2;
+                    const float s8 = hi == 0 ? byte_as_float<B>(s4) : byte_as_float<B + 1>(s4);
+                    const float m8 = hi == 0 ? byte_as_float<B>(m4) : byte_as_float<B + 1>(m4);
+                    scale[j] = d[j] * s8;
+                    offset[j] = -(dmin[j] * m8);
                 }
-                const uint32_t chunk = ((4 * hi + 2 * khalf + ff) ^ a_swz) * 16;
+            }
+            f16x8 b[2];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const f16x8 af = *reinterpret_cast<const f16x8*>(slab + a_row_at + i * (32 * 128) + chunk);
-                    acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b[0], acc[i][0], 0, 0, 0);
-                    acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, b[1], acc[i][1], 0, 0, 0);
-                }
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t w0 = nib[j][hi][2 * ff], w1 = nib[j][hi][2 * ff + 1];
+                b[j][0] = _Float16(__builtin_fmaf(byte_as_float<0>(w0), scale[j], offset[j]));
+                b[j][1] = _Float16(__builtin_fmaf(byte_as_float<1>(w0), scale[j], offset[j]));
+                b[j][2] = _Float16(__builtin_fmaf(byte_as_float<2>(w0), scale[j], offset[j]));
+                b[j][3] = _Float16(__builtin_fmaf(byte_as_float<3>(w0), scale[j], offset[j]));
+                b[j][4] = _Float16(__builtin_fmaf(byte_as_float<0>(w1), scale[j], offset[j]));
+                b[j][5] = _Float16(__builtin_fmaf(byte_as_float<1>(w1), scale[j], offset[j]));
+                b[j][6] = _Float16(__builtin_fmaf(byte_as_float<2>(w1), scale[j], offset[j]));
+                b[j][7] = _Float16(__builtin_fmaf(byte_as_float<3>(w1), scale[j], offset[j]));
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[g % 2][i], b[0], acc[i][0], 0, 0, 0);
+                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[g % 2][i], b[1], acc[i][1], 0, 0, 0);
             }
         }
     };
@@ -197,22 +215,79 @@ __global__ __launch_bounds__(kThreadsT) __attribute__((amdgpu_waves_per_eu(2, 2)
 
     // ---- epilogue. Accumulator v of tile (i, j): row 32 i + 8 (v / 4) + 4 khalf + v % 4 of the wave's 128, weight row col of column tile j
     uint32_t biggest = 0;  // the largest result's bits without the sign: anything not finite shows at the end
+    const uint32_t wave_m0 = m0 + wm * 128, wave_n0 = n0 + wn * 64;
+    const bool whole = wave_n0 + 64 <= a.n && reinterpret_cast<uintptr_t>(a.out) % 16 == 0 && a.out_stride % 16 == 0;  // uniform
+    __syncthreads();  // every wave has left the rings, and every request into them has landed: the LDS is the epilogue's
+    if (whole) {
+        // The wave's 128 x 64 results go out as whole 16-byte pieces, eight lanes to a row's 64 columns, after a turn through
+        // LDS that the wave has to itself (16 KB: all four row tiles as bf16, or two at a time as f32; a row pitch of 16 bytes
+        // more than the row keeps the column-wise writes and the row-wise reads off each other's banks). A lane storing
+        // its own 2- or 4-byte results one by one, 128 stores, took a fifth of the kernel's time.
+        uint8_t* const mine = lds_raw + wave * (16 * 1024 + 2048);
+        static_assert((kThreadsT / kWave) * (16 * 1024 + 2048) <= int(sizeof(lds_raw)));
+        auto pass = [&](auto bf16_tag, int first_tile) {
+            constexpr bool BF16 = decltype(bf16_tag)::value;
+            constexpr int kTiles = BF16 ? 4 : 2, kElem = BF16 ? 2 : 4, kPitch = 64 * kElem + 16;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+            for (int t = 0; t < kTiles; ++t) {
+                const int i = first_tile + t;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const uint32_t row = m0 + wm * 128 + i * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
-            if (row >= a.m) continue;
-            uint8_t* orow = static_cast<uint8_t*>(a.out) + uint64_t(row) * a.out_stride;
+                for (int v = 0; v < 16; ++v) {
+                    const uint32_t r = t * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const uint32_t n = n0 + wn * 64 + j * 32 + col;
-                if (n >= a.n) continue;
-                const float val = acc[i][j][v];
-                const uint32_t vb = __float_as_uint(val), magnitude = vb & 0x7fffffffu;
-                biggest = biggest > magnitude ? biggest : magnitude;
-                if (a.out_bf16) reinterpret_cast<uint16_t*>(orow)[n] = uint16_t((vb + 0x7fffu + ((vb >> 16) & 1u)) >> 16);
-                else reinterpret_cast<float*>(orow)[n] = val;
+                    for (int j = 0; j < 2; ++j) {
+                        const float val = acc[i][j][v];
+                        const uint32_t vb = __float_as_uint(val), magnitude = vb & 0x7fffffffu;
+                        biggest = biggest > magnitude ? biggest : magnitude;
+                        uint8_t* at = mine + r * kPitch + (j * 32 + col) * kElem;
+                        if constexpr (BF16) *reinterpret_cast<uint16_t*>(at) = uint16_t((vb + 0x7fffu + ((vb >> 16) & 1u)) >> 16);
+                        else *reinterpret_cast<float*>(at) = val;
+                    }
+                }
+            }
+            // written and read back by this wave only: LDS serves a wave's requests in order
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            constexpr int kPieces = 64 * kElem / 16;                    // 16-byte pieces per row
+            constexpr int kRounds = kTiles * 32 * kPieces / kWave;      // pieces per lane
+#pragma unroll
+            for (int q = 0; q < kRounds; ++q) {
+                const uint32_t c = q * kWave + lane, r = c / kPieces, piece = c % kPieces;
+                const uint4 data = *reinterpret_cast<const uint4*>(mine + r * kPitch + piece * 16);
+                const uint32_t row = wave_m0 + first_tile * 32 + r;
+                if (row < a.m)
+                    *reinterpret_cast<uint4*>(static_cast<uint8_t*>(a.out) + uint64_t(row) * a.out_stride + uint64_t(wave_n0) * kElem + piece * 16) = data;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        };
+        if (a.out_bf16) {
+            pass(std::true_type{}, 0);
+        } else {
+            pass(std::false_type{}, 0);
+            pass(std::false_type{}, 2);
+        }
+    } else {
+        // a ragged column tile or rows that 16 bytes do not align: element by element
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const uint32_t row = wave_m0 + i * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
+                if (row >= a.m) continue;
+                uint8_t* orow = static_cast<uint8_t*>(a.out) + uint64_t(row) * a.out_stride;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const uint32_t n = wave_n0 + j * 32 + col;
+                    if (n >= a.n) continue;
+                    const float val = acc[i][j][v];
+                    const uint32_t vb = __float_as_uint(val), magnitude = vb & 0x7fffffffu;
+                    biggest = biggest > magnitude ? biggest : magnitude;
+                    if (a.out_bf16) reinterpret_cast<uint16_t*>(orow)[n] = uint16_t((vb + 0x7fffu + ((vb >> 16) & 1u)) >> 16);
+                    else reinterpret_cast<float*>(orow)[n] = val;
+                }
             }
         }
     }
@@ -229,9 +304,10 @@ bool dense_tall_takes(uint32_t tokens, uint32_t rows, uint32_t columns, uint64_t
 }
 
 int launch_dense_tall(const DenseTallArgs& a, hipStream_t s) {
-    const uint32_t tiles = ((a.n + kTileN - 1) / kTileN) * ((a.m + kTileM - 1) / kTileM);
+    constexpr int WM = 1;
+    const uint32_t tiles = ((a.n + kTileN - 1) / kTileN) * ((a.m + 128 * WM - 1) / (128 * WM));
     const uint32_t groups = (tiles + 7) / 8 * 8;
-    TSP_LAUNCH("gemm_dense_tall", s, dense_tall_kernel<<<groups, kThreadsT, 0, s>>>(a));
+    TSP_LAUNCH("gemm_dense_tall", s, dense_tall_kernel<WM><<<groups, 256 * WM, 0, s>>>(a));
     return launch_status("dense_tall");
 }
 
