@@ -6,9 +6,10 @@
 // activation rows x 64 weight rows (four row tiles x two column tiles: 128 accumulator registers), so a weight is unpacked
 // once per 128 rows and a step of 64 columns is 32 MFMAs against ~180 vector instructions per wave.
 //
-//   * Arithmetic: the engine's for this path. A weight is its f32 value d * sc * q - dmin * mn rounded once to half (one
-//     v_cvt_f32_ubyte and one mixed-precision fused multiply-add per weight, exact in f32 before the rounding); activations
-//     are the bf16 values carried as halves; products accumulate in f32 on v_mfma_f32_32x32x16_f16.
+//   * Arithmetic: the engine's for this path. A weight is its f32 value d * sc * q - dmin * mn rounded once to half: the
+//     code q, masked out where it sits, is a subnormal half q * 2^-24, and one mixed-precision fused multiply-add per
+//     weight evaluates (d * sc * 2^24) * that - dmin * mn in f32 and rounds it to half; activations are the bf16 values
+//     carried as halves; products accumulate in f32 on v_mfma_f32_32x32x16_f16.
 //   * Activations: 256 rows x 128 bytes per step go global -> LDS directly, two steps ahead, into a ring of three slabs
 //     shared by the eight waves (16-byte chunk c of row r at position c ^ (r % 8)); one LDS-only barrier per step.
 //   * Weights: the step's 32 bytes of nibbles of the tile's 256 rows (8 KB, ring of four) and, once per super-block, the
@@ -37,6 +38,18 @@ __device__ __forceinline__ const uint8_t* uniform_pointer(const uint8_t* p) {
 // Byte N of a word as a float: one v_cvt_f32_ubyteN.
 template <int N>
 __device__ __forceinline__ float byte_as_float(uint32_t word) { return float((word >> (8 * N)) & 0xffu); }
+
+// Two weights from two codes sitting in the mantissas of two halves (`codes`: q or q << 4 per half, everything else zero: the
+// subnormal halves q * 2^-24 resp. q * 2^-20): each is scale * code + offset evaluated as one f32 fused multiply-add whose
+// result is rounded to half (v_fma_mix widens the half operand to f32 inside the instruction, subnormals included), one
+// instruction per weight and no separate conversion of the code to a float. With scale = d * sc * 2^24 (2^20) and offset =
+// -dmin * mn this is the f32 value d * sc * q - dmin * mn exactly, then rounded once.
+__device__ __forceinline__ uint32_t two_weights(uint32_t codes, float scale, float offset) {
+    uint32_t out;
+    asm volatile("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(out) : "v"(codes), "v"(scale), "v"(offset));
+    asm volatile("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(out) : "v"(codes), "v"(scale), "v"(offset));
+    return out;
+}
 
 constexpr int kTileN = 256, kStepK = 64, kRing = 3;
 constexpr int kQsBytes = kTileN * 32;
@@ -87,16 +100,21 @@ __global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))
     const uint32_t h_lane = h_row * row_bytes;
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds_raw));
     const uint32_t my_slab = lds0 + wave * 1024, my_qs = lds0 + kQsAt + wave * 1024, my_hdr = lds0 + kHdrAt + (wave % 4) * 1024;
-    auto request = [&](uint32_t step) {  // steps past the end ask for the last step again (nobody reads it)
+    // Step `step`'s bytes into ring slot step % 3. Steps past the end ask for the last step's bytes again (nobody reads them), and
+    // ask for headers where a real step would: the number of requests per step must not depend on where the matrix ends,
+    // the waits below count them.
+    auto request = [&](uint32_t step) {
+        const uint32_t slot = step % kRing, hdr_slot = (step / 4) % kHdrStages;
+        const bool with_headers = step % 4 == 0;
         step = step < steps ? step : steps - 1;
         const uint32_t b = step / 4, pair = step % 4;
         const uint8_t* a_base = uniform_pointer(reinterpret_cast<const uint8_t*>(a.a) + uint64_t(step) * (kStepK * 2));
-        const uint32_t slab = my_slab + (step % kRing) * kSlabBytes;
+        const uint32_t slab = my_slab + slot * kSlabBytes;
 #pragma unroll
         for (int i = 0; i < 4; ++i) load_to_lds_16(a_base, a_lane[i], slab + i * (kThreadsT * 16));
 #pragma unroll
-        for (int q = 0; q < QN; ++q) load_to_lds_16(a.w + uint64_t(b) * 144 + 16 + pair * 32, q_lane[q], my_qs + (step % kRing) * kQsBytes + q * (kThreadsT * 16));
-        if (pair == 0) load_to_lds_16(a.w + uint64_t(b) * 144, h_lane, my_hdr + (b % kHdrStages) * kHdrBytes);
+        for (int q = 0; q < QN; ++q) load_to_lds_16(a.w + uint64_t(b) * 144 + 16 + pair * 32, q_lane[q], my_qs + slot * kQsBytes + q * (kThreadsT * 16));
+        if (with_headers) load_to_lds_16(a.w + uint64_t(b) * 144, h_lane, my_hdr + hdr_slot * kHdrBytes);
     };
 
     f32x16 acc[4][2];
@@ -118,6 +136,8 @@ __global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))
         hdr_at[j] = kHdrAt + r * 16;
     }
 
+    struct { uint32_t low, high; } kc{0x000f000fu, 0x00f000f0u};  // kept in registers: as literals they would double the size of every mask instruction
+    asm volatile("" : "+s"(kc.low), "+s"(kc.high));
     float d[2], dmin[2];
     uint32_t sc[2][2], mn[2][2];  // eight scales and eight minima per weight row, one per byte
     auto step_fn = [&](uint32_t step, auto p_tag) {
@@ -142,18 +162,9 @@ __global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))
             }
         }
         // the lane's 16 bytes of the pair, per column tile: low nibbles are sub-block 2 P, high nibbles sub-block 2 P + 1
-        uint32_t nib[2][2][4];  // [column tile][low, high][word]: four codes per word, one per byte
+        u32x4 raw[2];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const u32x4 raw = *reinterpret_cast<const u32x4*>(qs + q_at[j]);
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                nib[j][0][w] = raw[w] & 0x0f0f0f0fu;
-                nib[j][1][w] = (raw[w] >> 4) & 0x0f0f0f0fu;
-                // kept as they are: left to itself the compiler digs every code out of the raw word again, a bit-field extract per weight
-                asm volatile("" : "+v"(nib[j][0][w]), "+v"(nib[j][1][w]));
-            }
-        }
+        for (int j = 0; j < 2; ++j) raw[j] = *reinterpret_cast<const u32x4*>(qs + q_at[j]);
         // The four k16 groups of the step, (low, high nibbles) x (first, second eight columns of the lane's sixteen). The
         // activation fragments of a group are read one group ahead, so that their LDS latency passes behind the unpacking
         // of the weights; left to itself the compiler reads them two at a time right before the MFMAs that use them.
@@ -178,22 +189,23 @@ __global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))
                     constexpr int B = (P % 2) * 2;
                     const float s8 = hi == 0 ? byte_as_float<B>(s4) : byte_as_float<B + 1>(s4);
                     const float m8 = hi == 0 ? byte_as_float<B>(m4) : byte_as_float<B + 1>(m4);
-                    scale[j] = d[j] * s8;
+                    scale[j] = (d[j] * s8) * (hi == 0 ? 16777216.0f : 1048576.0f);  // a power of two: no rounding
                     offset[j] = -(dmin[j] * m8);
                 }
             }
+            // A word holds four codes, one nibble of each byte; bytes (0, 2), then (1, 3), are masked out where they are: two halves
+            // whose only set bits are a code's. Eight columns come out in the order (0, 2, 1, 3, 4, 6, 5, 7), the activations' order.
             f16x8 b[2];
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const uint32_t w0 = nib[j][hi][2 * ff], w1 = nib[j][hi][2 * ff + 1];
-                b[j][0] = _Float16(__builtin_fmaf(byte_as_float<0>(w0), scale[j], offset[j]));
-                b[j][1] = _Float16(__builtin_fmaf(byte_as_float<1>(w0), scale[j], offset[j]));
-                b[j][2] = _Float16(__builtin_fmaf(byte_as_float<2>(w0), scale[j], offset[j]));
-                b[j][3] = _Float16(__builtin_fmaf(byte_as_float<3>(w0), scale[j], offset[j]));
-                b[j][4] = _Float16(__builtin_fmaf(byte_as_float<0>(w1), scale[j], offset[j]));
-                b[j][5] = _Float16(__builtin_fmaf(byte_as_float<1>(w1), scale[j], offset[j]));
-                b[j][6] = _Float16(__builtin_fmaf(byte_as_float<2>(w1), scale[j], offset[j]));
-                b[j][7] = _Float16(__builtin_fmaf(byte_as_float<3>(w1), scale[j], offset[j]));
+                u32x4 packed;
+#pragma unroll
+                for (int w = 0; w < 2; ++w) {
+                    const uint32_t word = raw[j][2 * ff + w], mask = hi == 0 ? kc.low : kc.high;
+                    packed[2 * w] = two_weights(word & mask, scale[j], offset[j]);
+                    packed[2 * w + 1] = two_weights((word >> 8) & mask, scale[j], offset[j]);
+                }
+                b[j] = __builtin_bit_cast(f16x8, packed);
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {

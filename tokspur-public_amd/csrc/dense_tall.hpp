@@ -6,7 +6,8 @@
 namespace tsp {
 
 struct DenseTallArgs {
-    const _Float16* a;   // activation rows as halves (bf16 values), a_stride halves apart, columns in their natural order
+    const _Float16* a;   // activation rows as halves (bf16 values), a_stride halves apart, columns of every eight in the order
+                         // (0, 2, 1, 3, 4, 6, 5, 7): the order in which a word of nibbles unpacks two at a time
     uint32_t a_stride;
     const uint8_t* w;    // [n rows][k / 256 blocks of 144 B]
     uint32_t m, n, k;
