@@ -1,26 +1,32 @@
 // Dense Q4_K GEMM for a thousand and more activation rows: out[m, n] = sum_k x[m, k] * half(dec(W[n, k])), f32 accumulation.
 //
-// With this many rows the product is bound by the matrix cores, provided the weights are not unpacked over and over: the
-// 64-row tiles of the general kernel (gemm.hip) unpack every weight once per 64 activation rows, and at 2048 rows spend
-// eight vector instructions per MFMA doing so. Here a workgroup of eight waves owns a 256 x 256 output tile, a wave 128
-// activation rows x 64 weight rows (four row tiles x two column tiles: 128 accumulator registers), so a weight is unpacked
-// once per 128 rows and a step of 64 columns is 32 MFMAs against ~180 vector instructions per wave.
+// With this many rows the weights must not be unpacked over and over: the 64-row tiles of the general kernel (gemm.hip)
+// unpack every weight once per 64 activation rows, and at 2048 rows spend eight vector instructions per MFMA doing so. Here
+// a workgroup of four waves owns a 128 x 256 (or 256 x 256) output tile, a wave all its activation rows x 64 weight rows
+// (four or eight row tiles x two column tiles: 128 or 256 accumulator registers), so a weight is unpacked once per 128 or
+// 256 rows. What bounds the loop is the rate at which a SIMD issues instructions next to its MFMAs (measured: one wave
+// issues one every ~8 cycles, two waves together one every ~4.6, and a mixed-precision multiply-add counts about double),
+// not the matrix pipe (about half busy), LDS (a fifth busy, no bank conflicts) or memory.
 //
 //   * Arithmetic: the engine's for this path. A weight is its f32 value d * sc * q - dmin * mn rounded once to half: the
 //     code q, masked out where it sits, is a subnormal half q * 2^-24, and one mixed-precision fused multiply-add per
 //     weight evaluates (d * sc * 2^24) * that - dmin * mn in f32 and rounds it to half; activations are the bf16 values
 //     carried as halves; products accumulate in f32 on v_mfma_f32_32x32x16_f16.
-//   * Activations: 256 rows x 128 bytes per step go global -> LDS directly, two steps ahead, into a ring of three slabs
-//     shared by the eight waves (16-byte chunk c of row r at position c ^ (r % 8)); one LDS-only barrier per step.
-//   * Weights: the step's 32 bytes of nibbles of the tile's 256 rows (8 KB, ring of four) and, once per super-block, the
+//   * Activations: the tile's rows x 128 bytes per step go global -> LDS directly, two steps ahead, into a ring of three
+//     slabs shared by the waves. 16-byte chunk c of row r sits at position c ^ ((r / 2) % 8): a 16-byte read by sixteen
+//     consecutive lanes (rows) then covers all 64 banks once (with c ^ (r % 8), rows r and r + 8 met in the same banks).
+//   * Weights: the step's 32 bytes of nibbles of the tile's 256 rows (8 KB, ring of three) and, once per super-block, the
 //     rows' 16 header bytes (d, dmin, packed scales and minima; ring of two) travel the same way. Every request in the
 //     loop is unconditional and issued by every thread (rows past the matrix's end repeat its last row), so each wave
 //     waits with an exact count.
+//   * One barrier per step, before the step's last group of MFMAs rather than between steps (see step_fn).
 //   * Workgroups are dealt to the XCDs in runs of consecutive tiles, column tiles fastest: the workgroups of one XCD
 //     share a slab of activation rows in its L2 and read every weight byte once.
 #include "dense_tall.hpp"
 
+#include <atomic>
 #include <type_traits>
+#include <utility>
 
 #include "mfma_quant.hpp"
 
@@ -45,28 +51,30 @@ __device__ __forceinline__ float byte_as_float(uint32_t word) { return float((wo
 // instruction per weight and no separate conversion of the code to a float. With scale = d * sc * 2^24 (2^20) and offset =
 // -dmin * mn this is the f32 value d * sc * q - dmin * mn exactly, then rounded once.
 __device__ __forceinline__ uint32_t two_weights(uint32_t codes, float scale, float offset) {
-    uint32_t out;
-    asm volatile("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(out) : "v"(codes), "v"(scale), "v"(offset));
-    asm volatile("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(out) : "v"(codes), "v"(scale), "v"(offset));
-    return out;
+    const f16x2 c = as_h2(codes);
+    const _Float16 lo = _Float16(__builtin_fmaf(float(c[0]), scale, offset)), hi = _Float16(__builtin_fmaf(float(c[1]), scale, offset));
+    return as_u32(f16x2{lo, hi});
 }
 
 constexpr int kTileN = 256, kStepK = 64, kRing = 3;
 constexpr int kQsBytes = kTileN * 32;
 constexpr int kHdrBytes = kTileN * 16, kHdrStages = 2;
 
-// WM: the workgroup's waves along the activation rows, 128 rows each (4 WM waves, a tile of 128 WM x 256).
-template <int WM>
-__global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))) void dense_tall_kernel(DenseTallArgs a) {
-    constexpr int kThreadsT = 256 * WM, kTileM = 128 * WM;
-    constexpr int kSlabBytes = kTileM * kStepK * 2;
+// RT x CT: the row tiles (32 activation rows each) and column tiles (32 weight rows each) of a wave, 16 accumulator registers
+// apiece. The four waves stand 8 / CT wide across the tile's 256 weight rows and CT / 2 high. With 128 accumulator registers
+// (4 x 2: a 128 x 256 tile) two workgroups share a compute unit, two waves a SIMD; with 256 (8 x 2: a 256 x 256 tile) a wave has
+// a SIMD and its 512 registers to itself, and every unpacked weight serves twice as many MFMAs.
+template <int RT, int CT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8 ? 1 : 2, RT * CT > 8 ? 1 : 2))) void dense_tall_kernel(DenseTallArgs a) {
+    constexpr int kThreadsT = 256, WN = 8 / CT, WM = 4 / WN, kTileM = WM * RT * 32;
+    constexpr int kSlabBytes = kTileM * kStepK * 2, kSlabPieces = kSlabBytes / (kThreadsT * 16);
     constexpr int kQsAt = kRing * kSlabBytes, kHdrAt = kQsAt + kRing * kQsBytes;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kHdrAt + kHdrStages * kHdrBytes];
-    static_assert(sizeof(lds_raw) * (2 / WM) <= 160 * 1024, "two waves per SIMD: one workgroup of eight waves or two of four per compute unit");
+    static_assert(sizeof(lds_raw) * (RT * CT > 8 ? 1 : 2) <= 160 * 1024, "the workgroups of a compute unit share 160 KB");
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const uint32_t col = lane % 32, khalf = (lane / 32) & 1;
-    const uint32_t wm = wave / 4, wn = wave % 4;  // the wave's 128 activation rows and 64 weight rows of the tile (wm < WM)
+    const uint32_t wm = wave / WN, wn = wave % WN;  // the wave's RT x 32 activation rows and CT x 32 weight rows of the tile
 
     // ---- the workgroup's tile: XCD x (workgroup id % 8) takes the x-th run of consecutive tiles
     const uint32_t n_tiles = (a.n + kTileN - 1) / kTileN, m_tiles = (a.m + kTileM - 1) / kTileM;
@@ -79,17 +87,17 @@ __global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     // ---- per-thread parts of the request addresses (the per-step parts are uniform)
     // activations: request i of thread t fills 16-byte position t + T i of the slab (T threads) = slot t % 8 of row (t + T i) / 8,
-    // with chunk (t % 8) ^ (row % 8) of that row
-    uint32_t a_lane[4];
+    // with chunk (t % 8) ^ ((row / 2) % 8) of that row
+    uint32_t a_lane[kSlabPieces];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kSlabPieces; ++i) {
         const uint32_t r = (tid + kThreadsT * i) / 8, row = m0 + r < a.m ? m0 + r : a.m - 1;
-        a_lane[i] = (row * a.a_stride + (((tid % 8) ^ (r & 7)) * 8)) * 2;
+        a_lane[i] = (row * a.a_stride + (((tid % 8) ^ ((r >> 1) & 7)) * 8)) * 2;
     }
     // nibbles: request q of thread t fills position u = t + T q of the stage = slot u % 2 of weight row u / 2, with chunk
     // (u % 2) ^ ((row / 8) % 2) of the step's 32 bytes of that row; headers: position t % 256 = weight row t % 256 (with eight
     // waves the two halves of the workgroup fetch the same)
-    constexpr int QN = 2 / WM;
+    constexpr int QN = 2;
     uint32_t q_lane[QN];
 #pragma unroll
     for (int q = 0; q < QN; ++q) {
@@ -111,80 +119,90 @@ __global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))
         const uint8_t* a_base = uniform_pointer(reinterpret_cast<const uint8_t*>(a.a) + uint64_t(step) * (kStepK * 2));
         const uint32_t slab = my_slab + slot * kSlabBytes;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_to_lds_16(a_base, a_lane[i], slab + i * (kThreadsT * 16));
+        for (int i = 0; i < kSlabPieces; ++i) load_to_lds_16(a_base, a_lane[i], slab + i * (kThreadsT * 16));
 #pragma unroll
         for (int q = 0; q < QN; ++q) load_to_lds_16(a.w + uint64_t(b) * 144 + 16 + pair * 32, q_lane[q], my_qs + slot * kQsBytes + q * (kThreadsT * 16));
         if (with_headers) load_to_lds_16(a.w + uint64_t(b) * 144, h_lane, my_hdr + hdr_slot * kHdrBytes);
     };
 
-    f32x16 acc[4][2];
+    f32x16 acc[RT][CT];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < CT; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
     // fragment reads: lane (col, khalf) takes chunk 4 hi + 2 khalf + ff of activation row col (+ 32 i) and the k-half's 16 bytes of
     // the nibbles of weight row col (+ 32 j)
-    const uint32_t a_row_at = (wm * 128 + col) * 128, a_swz = col & 7;
-    uint32_t q_at[2], hdr_at[2];
+    const uint32_t a_row_at = (wm * (RT * 32) + col) * 128, a_swz = (col >> 1) & 7;
+    uint32_t q_at[CT], hdr_at[CT];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const uint32_t r = wn * 64 + j * 32 + col;
+    for (int j = 0; j < CT; ++j) {
+        const uint32_t r = wn * (CT * 32) + j * 32 + col;
         q_at[j] = kQsAt + r * 32 + ((khalf ^ ((r >> 3) & 1)) * 16);
         hdr_at[j] = kHdrAt + r * 16;
     }
 
     struct { uint32_t low, high; } kc{0x000f000fu, 0x00f000f0u};  // kept in registers: as literals they would double the size of every mask instruction
     asm volatile("" : "+s"(kc.low), "+s"(kc.high));
-    float d[2], dmin[2];
-    uint32_t sc[2][2], mn[2][2];  // eight scales and eight minima per weight row, one per byte
-    auto step_fn = [&](uint32_t step, auto p_tag) {
-        constexpr int P = decltype(p_tag)::value;  // the pair of sub-blocks of the super-block: step % 4
-        // Wait for this thread's requests of the step (issued two steps ago); younger than those are the requests of the
-        // next step: four slab pieces, the nibbles, and at the last pair the next super-block's headers. Then the
-        // barrier: every thread's pieces have landed, and every wave has left the buffers that the next requests overwrite.
-        lds_barrier_after_loads<4 + QN + (P == 3 ? 1 : 0)>();
-        request(step + 2);
+    float d[CT], dmin[CT];
+    uint32_t sc[CT][2], mn[CT][2];  // eight scales and eight minima per weight row, one per byte
+    u32x4 raw[CT];                  // the lane's 16 bytes of the step's pair of sub-blocks, per column tile: low nibbles are sub-block 2 P, high nibbles 2 P + 1
+    f16x8 af[2][RT];                // activation fragments of the k16 group at work and of the one after it
+
+    // The four k16 groups of a step are (low, high nibbles) x (first, second eight columns of the lane's sixteen).
+    auto read_a = [&](uint32_t step, int g, f16x8 (&to)[RT]) {
         const uint8_t* slab = lds_raw + (step % kRing) * kSlabBytes;
-        const uint8_t* qs = lds_raw + (step % kRing) * kQsBytes;
-        if constexpr (P == 0) {
+        const uint32_t chunk = ((4 * (g / 2) + 2 * khalf + (g % 2)) ^ a_swz) * 16;
+#pragma unroll
+        for (int i = 0; i < RT; ++i) to[i] = *reinterpret_cast<const f16x8*>(slab + a_row_at + i * (32 * 128) + chunk);
+    };
+    // What a step needs before its first MFMA: its nibbles, the activation fragments of its first group, and at the first
+    // pair of a super-block the rows' scales and minima.
+    auto front = [&](uint32_t step, auto first_pair, u32x4 (&nibbles)[CT]) {
+        if constexpr (decltype(first_pair)::value) {
             const uint8_t* hdr = lds_raw + ((step / 4) % kHdrStages) * kHdrBytes;
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                RawHdrQ4 raw;
-                raw.words = *reinterpret_cast<const uint4*>(hdr + hdr_at[j]);
-                raw.dm = 0;
-                const HdrQ4 h = decode_hdr_q4k<B_Q4K_RAW>(raw);
+            for (int j = 0; j < CT; ++j) {
+                RawHdrQ4 words;
+                words.words = *reinterpret_cast<const uint4*>(hdr + hdr_at[j]);
+                words.dm = 0;
+                const HdrQ4 h = decode_hdr_q4k<B_Q4K_RAW>(words);
                 d[j] = h.d; dmin[j] = h.dmin;
                 sc[j][0] = h.sc[0]; sc[j][1] = h.sc[1]; mn[j][0] = h.mn[0]; mn[j][1] = h.mn[1];
             }
         }
-        // the lane's 16 bytes of the pair, per column tile: low nibbles are sub-block 2 P, high nibbles sub-block 2 P + 1
-        u32x4 raw[2];
+        const uint8_t* qs = lds_raw + (step % kRing) * kQsBytes;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) raw[j] = *reinterpret_cast<const u32x4*>(qs + q_at[j]);
-        // The four k16 groups of the step, (low, high nibbles) x (first, second eight columns of the lane's sixteen). The
-        // activation fragments of a group are read one group ahead, so that their LDS latency passes behind the unpacking
-        // of the weights; left to itself the compiler reads them two at a time right before the MFMAs that use them.
-        auto read_a = [&](int g, f16x8 (&af)[4]) {
-            const uint32_t chunk = ((4 * (g / 2) + 2 * khalf + (g % 2)) ^ a_swz) * 16;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const f16x8*>(slab + a_row_at + i * (32 * 128) + chunk);
-        };
-        f16x8 af[2][4];
-        read_a(0, af[0]);
-        float scale[2], offset[2];
+        for (int j = 0; j < CT; ++j) nibbles[j] = *reinterpret_cast<const u32x4*>(qs + q_at[j]);
+        read_a(step, 0, af[0]);
+    };
+
+    // One step. The workgroup's barrier does not sit between two steps but before a step's last group: by then a wave has
+    // every byte of the step in registers, so the step's ring slot can be given to the requests of step + 3, and the bytes of
+    // step + 1, asked for two steps ago, have landed in every wave's view after the barrier. The last group's MFMAs then
+    // cover the barrier, the requests and the next step's front; at the boundary between two steps nothing waits.
+    auto step_fn = [&](uint32_t step, auto p_tag) {
+        constexpr int P = decltype(p_tag)::value;  // the pair of sub-blocks of the super-block: step % 4
+        float scale[CT], offset[CT];
+        u32x4 next_raw[CT];
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const int hi = g / 2, ff = g % 2;
-            if (g < 3) read_a(g + 1, af[(g + 1) % 2]);
-            __builtin_amdgcn_sched_barrier(0);
+            // the activation fragments of a group are read one group ahead: their LDS latency passes behind the unpacking
+            if (g < 3) read_a(step, g + 1, af[(g + 1) % 2]);
+            if (g == 3) {
+                // Younger than the requests of step + 1 are those of step + 2: the slab's pieces, the nibbles, and the headers
+                // when step + 2 begins a super-block.
+                lds_barrier_after_loads<kSlabPieces + QN + (P == 2 ? 1 : 0)>();
+                request(step + 3);
+                front(step + 1, std::bool_constant<P == 3>{}, next_raw);
+            }
             if (ff == 0) {
                 // sub-block 2 P + hi; weight = half(d * sc * q - dmin * mn), the f32 value rounded once
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
+                for (int j = 0; j < CT; ++j) {
                     const uint32_t s4 = sc[j][P / 2], m4 = mn[j][P / 2];
                     constexpr int B = (P % 2) * 2;
                     const float s8 = hi == 0 ? byte_as_float<B>(s4) : byte_as_float<B + 1>(s4);
@@ -195,28 +213,47 @@ __global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))
             }
             // A word holds four codes, one nibble of each byte; bytes (0, 2), then (1, 3), are masked out where they are: two halves
             // whose only set bits are a code's. Eight columns come out in the order (0, 2, 1, 3, 4, 6, 5, 7), the activations' order.
-            f16x8 b[2];
+            // Two column tiles at a time, so that only two weight fragments are alive at once.
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                u32x4 packed;
+            for (int j0 = 0; j0 < CT; j0 += 2) {
+                f16x8 b[2];
 #pragma unroll
-                for (int w = 0; w < 2; ++w) {
-                    const uint32_t word = raw[j][2 * ff + w], mask = hi == 0 ? kc.low : kc.high;
-                    packed[2 * w] = two_weights(word & mask, scale[j], offset[j]);
-                    packed[2 * w + 1] = two_weights((word >> 8) & mask, scale[j], offset[j]);
+                for (int jj = 0; jj < 2; ++jj) {
+                    const int j = j0 + jj;
+                    u32x4 packed;
+#pragma unroll
+                    for (int w = 0; w < 2; ++w) {
+                        const uint32_t word = raw[j][2 * ff + w], mask = hi == 0 ? kc.low : kc.high;
+                        packed[2 * w] = two_weights(word & mask, scale[j], offset[j]);
+                        packed[2 * w + 1] = two_weights((word >> 8) & mask, scale[j], offset[j]);
+                    }
+                    b[jj] = __builtin_bit_cast(f16x8, packed);
                 }
-                b[j] = __builtin_bit_cast(f16x8, packed);
-            }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                acc[i][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[g % 2][i], b[0], acc[i][0], 0, 0, 0);
-                acc[i][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[g % 2][i], b[1], acc[i][1], 0, 0, 0);
+                for (int i = 0; i < RT; ++i) {
+                    acc[i][j0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[g % 2][i], b[0], acc[i][j0], 0, 0, 0);
+                    acc[i][j0 + 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[g % 2][i], b[1], acc[i][j0 + 1], 0, 0, 0);
+                }
             }
+        }
+#pragma unroll
+        for (int j = 0; j < CT; ++j) raw[j] = next_raw[j];
+        // A wave issues in order: eight MFMAs in a row hold it for eight times the matrix pipe's 32 cycles, with its own
+        // unpacking waiting behind them. Interleaved, one MFMA then four vector instructions (and an LDS read every other
+        // time), the unpacking of the next group runs in the shadow of this group's MFMAs.
+#pragma unroll
+        for (int k = 0; k < 4 * RT * CT; ++k) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, RT * CT > 8 ? 3 : 4, 0);
+            if (k % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
     };
 
     request(0);
     request(1);
+    request(2);
+    lds_barrier_after_loads<2 * (kSlabPieces + QN)>();  // step 0 has landed; the requests of steps 1 and 2 are the younger ones
+    front(0, std::true_type{}, raw);
     for (uint32_t b = 0; b < bpr; ++b) {
         step_fn(b * 4 + 0, std::integral_constant<int, 0>{});
         step_fn(b * 4 + 1, std::integral_constant<int, 1>{});
@@ -225,21 +262,23 @@ __global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     wait_all_loads();  // the last steps requested buffers that nobody reads: they must have landed before the LDS is given away
 
-    // ---- epilogue. Accumulator v of tile (i, j): row 32 i + 8 (v / 4) + 4 khalf + v % 4 of the wave's 128, weight row col of column tile j
+    // ---- epilogue. Accumulator v of tile (i, j): row 32 i + 8 (v / 4) + 4 khalf + v % 4 of the wave's rows, weight row col of column tile j
     uint32_t biggest = 0;  // the largest result's bits without the sign: anything not finite shows at the end
-    const uint32_t wave_m0 = m0 + wm * 128, wave_n0 = n0 + wn * 64;
-    const bool whole = wave_n0 + 64 <= a.n && reinterpret_cast<uintptr_t>(a.out) % 16 == 0 && a.out_stride % 16 == 0;  // uniform
+    const uint32_t wave_m0 = m0 + wm * (RT * 32), wave_n0 = n0 + wn * (CT * 32);
+    const bool whole = wave_n0 + CT * 32 <= a.n && reinterpret_cast<uintptr_t>(a.out) % 16 == 0 && a.out_stride % 16 == 0;  // uniform
     __syncthreads();  // every wave has left the rings, and every request into them has landed: the LDS is the epilogue's
     if (whole) {
-        // The wave's 128 x 64 results go out as whole 16-byte pieces, eight lanes to a row's 64 columns, after a turn through
-        // LDS that the wave has to itself (16 KB: all four row tiles as bf16, or two at a time as f32; a row pitch of 16 bytes
+        // The wave's results go out as whole 16-byte pieces, neighbouring lanes along a row, after a turn through LDS that the
+        // wave has to itself (18 KB: four row tiles of 64 results at a time as bf16, two as f32; a row pitch of 16 bytes
         // more than the row keeps the column-wise writes and the row-wise reads off each other's banks). A lane storing
         // its own 2- or 4-byte results one by one, 128 stores, took a fifth of the kernel's time.
         uint8_t* const mine = lds_raw + wave * (16 * 1024 + 2048);
         static_assert((kThreadsT / kWave) * (16 * 1024 + 2048) <= int(sizeof(lds_raw)));
-        auto pass = [&](auto bf16_tag, int first_tile) {
+        auto pass = [&](auto bf16_tag, auto first_tag) {
             constexpr bool BF16 = decltype(bf16_tag)::value;
-            constexpr int kTiles = BF16 ? 4 : 2, kElem = BF16 ? 2 : 4, kPitch = 64 * kElem + 16;
+            constexpr int first_tile = decltype(first_tag)::value;
+            constexpr int kTiles = (BF16 ? 8 : 4) / CT, kElem = BF16 ? 2 : 4, kPitch = CT * 32 * kElem + 16;
+            static_assert(kTiles * 32 * kPitch <= 16 * 1024 + 2048 && first_tile + kTiles <= RT);
 #pragma unroll
             for (int t = 0; t < kTiles; ++t) {
                 const int i = first_tile + t;
@@ -247,7 +286,7 @@ __global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))
                 for (int v = 0; v < 16; ++v) {
                     const uint32_t r = t * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
 #pragma unroll
-                    for (int j = 0; j < 2; ++j) {
+                    for (int j = 0; j < CT; ++j) {
                         const float val = acc[i][j][v];
                         const uint32_t vb = __float_as_uint(val), magnitude = vb & 0x7fffffffu;
                         biggest = biggest > magnitude ? biggest : magnitude;
@@ -261,7 +300,7 @@ __global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            constexpr int kPieces = 64 * kElem / 16;                    // 16-byte pieces per row
+            constexpr int kPieces = CT * 32 * kElem / 16;                    // 16-byte pieces per row
             constexpr int kRounds = kTiles * 32 * kPieces / kWave;      // pieces per lane
 #pragma unroll
             for (int q = 0; q < kRounds; ++q) {
@@ -275,23 +314,23 @@ __global__ __launch_bounds__(256 * WM) __attribute__((amdgpu_waves_per_eu(2, 2))
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         };
-        if (a.out_bf16) {
-            pass(std::true_type{}, 0);
-        } else {
-            pass(std::false_type{}, 0);
-            pass(std::false_type{}, 2);
-        }
+        // 8 / CT row tiles at a time as bf16, half as many as f32
+        auto passes = [&]<int... I>(auto bf16_tag, std::integer_sequence<int, I...>) {
+            (pass(bf16_tag, std::integral_constant<int, I * ((decltype(bf16_tag)::value ? 8 : 4) / CT)>{}), ...);
+        };
+        if (a.out_bf16) passes(std::true_type{}, std::make_integer_sequence<int, RT * CT / 8>{});
+        else passes(std::false_type{}, std::make_integer_sequence<int, RT * CT / 4>{});
     } else {
         // a ragged column tile or rows that 16 bytes do not align: element by element
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < RT; ++i) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const uint32_t row = wave_m0 + i * 32 + 8 * (v / 4) + 4 * khalf + (v % 4);
                 if (row >= a.m) continue;
                 uint8_t* orow = static_cast<uint8_t*>(a.out) + uint64_t(row) * a.out_stride;
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
+                for (int j = 0; j < CT; ++j) {
                     const uint32_t n = wave_n0 + j * 32 + col;
                     if (n >= a.n) continue;
                     const float val = acc[i][j][v];
@@ -316,10 +355,24 @@ bool dense_tall_takes(uint32_t tokens, uint32_t rows, uint32_t columns, uint64_t
 }
 
 int launch_dense_tall(const DenseTallArgs& a, hipStream_t s) {
-    constexpr int WM = 1;
-    const uint32_t tiles = ((a.n + kTileN - 1) / kTileN) * ((a.m + 128 * WM - 1) / (128 * WM));
-    const uint32_t groups = (tiles + 7) / 8 * 8;
-    TSP_LAUNCH("gemm_dense_tall", s, dense_tall_kernel<WM><<<groups, 256 * WM, 0, s>>>(a));
+    static std::atomic<uint64_t> seen{0};
+    static int units[64];
+    int device = 0;
+    if (first_use_on_device(seen, &device) || units[device] == 0) {
+        int n = 0;
+        TSP_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device));
+        units[device] = n >= 1 ? n : 1;
+    }
+    // 256-row tiles only where one round of them keeps nearly every compute unit busy (2048 x 8192 results on 256 units): there
+    // they are a few percent faster. Elsewhere 128-row tiles, two workgroups to a unit, lose less to the last, partly filled
+    // round, and a second round of 256-row tiles cannot start behind the first one's epilogue as a second workgroup can.
+    const uint32_t n_tiles = (a.n + kTileN - 1) / kTileN, cus = uint32_t(units[device]);
+    const uint32_t tall = n_tiles * ((a.m + 255) / 256), low = n_tiles * ((a.m + 127) / 128);
+    if (tall <= cus && uint64_t(tall) * 10 >= uint64_t(cus) * 9) {
+        TSP_LAUNCH("gemm_dense_tall", s, (dense_tall_kernel<8, 2><<<(tall + 7) / 8 * 8, 256, 0, s>>>(a)));
+    } else {
+        TSP_LAUNCH("gemm_dense_tall", s, (dense_tall_kernel<4, 2><<<(low + 7) / 8 * 8, 256, 0, s>>>(a)));
+    }
     return launch_status("dense_tall");
 }
 

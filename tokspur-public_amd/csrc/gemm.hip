@@ -662,7 +662,7 @@ extern "C" int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matr
     auto* xh = static_cast<_Float16*>(workspace);
     auto* sx = reinterpret_cast<_Float16*>(static_cast<uint8_t*>(workspace) + align256(uint64_t(tokens) * columns * 2));
     if (encoding == 12 && layout == TSP_LAYOUT_GGUF && dense_tall_takes(tokens, rows, columns, matrix_bytes)) {
-        // a thousand rows and more: 256 x 256 tiles, weights rounded once to half (the engine's arithmetic for this product)
+        // a thousand rows and more: tiles 128 or 256 rows high, weights rounded once to half (the engine's arithmetic for this product)
         int rc = convert_rows(input, input_stride_bytes, input_is_bf16, xh, sx, tokens, columns, error_word, s);  // with the sums come the swapped columns
         if (rc != TSP_OK) return rc;
         DenseTallArgs t{};
