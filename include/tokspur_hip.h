@@ -337,8 +337,10 @@ int tsp_planar_moe_routed_m8_shared(const tsp_small_moe* moe, const tsp_shared_r
  * factors whose block scales are applied in f32, f32 accumulation. The carry is exact for bf16 values of magnitude 2^-14
  * to 65504; smaller ones lose low bits (below 2^-24: zero), and a finite input above 65504 sets TSP_ERRBIT_NONFINITE like an
  * infinity would (the batch is refused rather than computed on a clipped value). The same holds for tsp_grouped_mm and
- * tsp_planar_nax_grouped_moe. Input rows are f32 or bf16, output rows f32 or
- * bf16 (RNE); strides in bytes. Q4_K raw GGUF rows or planar planes, Q6_K planes. `workspace` is caller
+ * tsp_planar_nax_grouped_moe. One shape differs: Q4_K raw GGUF rows against 1024 or more token rows enter the matrix cores as
+ * the engine's kernel stages them (test_moe_mm_many_gpu.cpp:54-63), each weight's f32 value d*sc*q - dmin*mn rounded once to
+ * half, which is what makes unpacking a weight once per 128 or 256 token rows possible. Input rows are f32 or bf16, output
+ * rows f32 or bf16 (RNE); strides in bytes. Q4_K raw GGUF rows or planar planes, Q6_K planes. `workspace` is caller
  * owned scratch of tsp_dense_mm_workspace_bytes(tokens, columns) bytes, 16-byte aligned. */
 uint64_t tsp_dense_mm_workspace_bytes(uint32_t tokens, uint32_t columns);
 int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matrix, uint64_t matrix_bytes, const void* input,

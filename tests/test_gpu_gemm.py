@@ -56,10 +56,11 @@ def test_dense_mm_q4k(gpu, tsp, orc, synth, layout, tokens, rows, cols):
     assert np.array_equal(got_b, synth.round_bf16(got)) and gpu.error() == 0
 
 
-@pytest.mark.parametrize("tokens,rows,cols", [(1024, 256, 256), (1100, 300, 512), (1300, 777, 1024)])
+# the last shape is 240 tiles of 256 rows, ragged on both sides: the one-wave-per-SIMD form of the kernel on a 256-unit GPU
+@pytest.mark.parametrize("tokens,rows,cols", [(1024, 256, 256), (1100, 300, 512), (1300, 777, 1024), (2000, 7500, 256)])
 def test_dense_mm_q4k_many_rows(gpu, tsp, orc, synth, tokens, rows, cols):
-    """Raw GGUF Q4_K rows against a thousand and more activation rows: the 256 x 256 tile kernel with ragged tiles on both
-    sides. Its arithmetic is the engine's (weights rounded once to half, bf16 activations, f32 accumulation): the
+    """Raw GGUF Q4_K rows against a thousand and more activation rows: the kernel with tiles 128 or 256 rows high, ragged on
+    both sides. Its arithmetic is the engine's (weights rounded once to half, bf16 activations, f32 accumulation): the
     half-staged reference is met to accumulation accuracy; strided rows and padding stay."""
     w = synth.matrix(12, 2300 + rows, rows, cols)
     x = synth.round_bf16(synth.activations_f32(2301 + tokens, (tokens, cols + 8)))
