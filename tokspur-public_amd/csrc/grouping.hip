@@ -68,87 +68,17 @@ __global__ __launch_bounds__(512) void grouped_tasks_kernel(const uint32_t* __re
                         tiles_scan, routes_scan);
 }
 
-// 128 threads, one per flat route (T*S <= 128). meta layout in 32-bit words: [0..7] header,
-// +8 experts[128], +136 counts[128], +264 tokens[128][8], +1288 routes[128][8].
+// 128 threads, one per flat route (T*S <= 128); the block's layout and arithmetic: union_block (grouping_device.hpp).
 __global__ __launch_bounds__(128) void union_build_kernel(const uint32_t* __restrict__ ids, uint32_t* __restrict__ meta,
                                                           uint32_t experts, uint32_t selected, uint32_t tokens, uint32_t hidden,
                                                           uint32_t channels, uint32_t* error_word) {
-    __shared__ __align__(16) uint32_t sid[128];
-    __shared__ __align__(16) uint32_t rank_of[128];
-    __shared__ __align__(16) uint32_t record_of[128];
-    __shared__ uint32_t wave_leaders[2];
-    __shared__ uint32_t any_bad;
-    const uint32_t f = threadIdx.x, total = tokens * selected;
-    const bool shape_ok = experts && experts <= 512 && experts % 2 == 0 && selected && selected <= 16 && selected <= experts &&
-                          tokens && tokens <= 8 && hidden && channels;
-    if (f == 0) any_bad = shape_ok ? 0u : 1u;
-    __syncthreads();
-    const bool live = shape_ok && f < total;
-    const uint32_t mine = live ? ids[f] : 0xffffffffu;
-    if (live && mine >= experts) any_bad = 1u;
-    sid[f] = mine;
-    __syncthreads();
-    if (any_bad) {
-        if (f < 8) meta[f] = 0;
-        if (f == 0) atomicOr(error_word, TSP_ERRBIT_INDEX);
-        return;
-    }
-    const uint32_t cap = tokens <= 4 ? 4u : 8u;
-    // All 128 slots are compared, four per LDS read and with no dependence between the reads, so the scan costs one LDS
-    // latency and not one per route; the slots past the last route hold 0xffffffff and match no live route.
-    uint32_t rank = 0, same = 0;
-#pragma unroll
-    for (uint32_t g = 0; g < 128; g += 4) {
-        const uint4 four = *reinterpret_cast<const uint4*>(&sid[g]);
-        const uint32_t id4[4] = {four.x, four.y, four.z, four.w};
-#pragma unroll
-        for (uint32_t i = 0; i < 4; ++i) {
-            const bool eq = id4[i] == mine;
-            rank += (eq && g + i < f) ? 1u : 0u;
-            same += eq ? 1u : 0u;
-        }
-    }
-    const bool leader = live && rank % cap == 0;
-    const uint64_t mask = __builtin_amdgcn_ballot_w64(leader);
-    const uint32_t lane = f % kWave, wave = f / kWave;
-    if (lane == 0) wave_leaders[wave] = __builtin_popcountll(mask);
-    __syncthreads();
-    const uint32_t record = (wave ? wave_leaders[0] : 0u) + __builtin_popcountll(mask & ((1ull << lane) - 1ull));
-    const uint32_t records = wave_leaders[0] + wave_leaders[1];
-    record_of[f] = leader ? record : 0xffffffffu;
-    rank_of[f] = rank;
-    __syncthreads();
-    if (live) {
-        // my record is the one opened by the route of my expert whose rank is rank - rank % cap
-        const uint32_t want = rank - rank % cap;
-        uint32_t rec = record;
-        if (!leader) {
-#pragma unroll
-            for (uint32_t g = 0; g < 128; g += 4) {
-                const uint4 id4 = *reinterpret_cast<const uint4*>(&sid[g]);
-                const uint4 rank4 = *reinterpret_cast<const uint4*>(&rank_of[g]);
-                const uint4 rec4 = *reinterpret_cast<const uint4*>(&record_of[g]);
-                if (id4.x == mine && rank4.x == want) rec = rec4.x;
-                if (id4.y == mine && rank4.y == want) rec = rec4.y;
-                if (id4.z == mine && rank4.z == want) rec = rec4.z;
-                if (id4.w == mine && rank4.w == want) rec = rec4.w;
-            }
-        }
-        const uint32_t slot = rank % cap;
-        meta[264 + rec * 8 + slot] = f / selected;
-        meta[1288 + rec * 8 + slot] = f;
-        if (leader) {
-            const uint32_t members = same - rank < cap ? same - rank : cap;
-            meta[8 + rec] = mine;
-            meta[136 + rec] = members;
-            for (uint32_t k = members; k < 8; ++k) { meta[264 + rec * 8 + k] = f / selected; meta[1288 + rec * 8 + k] = f; }
-        }
-    }
-    if (f == 0) {
-        meta[0] = (hidden + 7) / 8; meta[1] = records; meta[2] = 1;
-        meta[3] = (channels + 15) / 16; meta[4] = records; meta[5] = 1;
-        meta[6] = records; meta[7] = 0;
-    }
+    __shared__ __align__(16) uint32_t scratch[kUnionScratchWords];
+    const uint32_t f = threadIdx.x;
+    // the shape test comes again inside; here it only keeps the read of ids in bounds
+    const bool readable = tokens && tokens <= 8 && selected && selected <= 16 && f < tokens * selected;
+    const uint32_t mine = readable ? ids[f] : 0xffffffffu;
+    union_block(mine, f, 128u, experts, selected, tokens, hidden, channels, scratch,
+                [&](uint32_t word, uint32_t value) { meta[word] = value; }, [&]() { atomicOr(error_word, TSP_ERRBIT_INDEX); });
 }
 
 }  // namespace

@@ -22,7 +22,7 @@ struct SmallMoeArgs {
     const uint8_t* pair_hi;   // experts E/2..E-1
     const uint8_t* down;      // [experts] planar
     const uint32_t* ids;      // [tokens*selected]
-    const uint32_t* meta;     // union block, or nullptr for tokens == 1
+    uint32_t* meta;           // union block, or nullptr for tokens == 1
     const float* x;           // [tokens] rows, x_stride bytes apart
     float* h;                 // [tokens*selected] rows, h_stride bytes apart
     float* y;                 // [tokens*selected] rows, y_stride bytes apart
@@ -420,6 +420,13 @@ SkinnyMoe skinny_view(const SmallMoeArgs& a, const tsp_shared_rows* shared = nul
     return v;
 }
 
+// The record-resident gate/up launch builds the union records itself (and leaves them in `meta` for the down launch): no
+// launch of the union kernel goes before it.
+bool gate_up_builds_union(const SmallMoeArgs& a, const tsp_shared_rows* shared = nullptr) {
+    return skinny_moe_supported(a.gu.source_type, a.dn.source_type, a.channels, a.hidden, a.x, a.x_stride, a.h, a.h_stride, false) &&
+           record_gate_up_takes(skinny_view(a, shared));
+}
+
 int launch_gate_up(const SmallMoeArgs& a, hipStream_t s, const tsp_shared_rows* shared = nullptr) {
     const uint32_t records = record_slots(a);
     if (skinny_moe_supported(a.gu.source_type, a.dn.source_type, a.channels, a.hidden, a.x, a.x_stride, a.h, a.h_stride, false)) {
@@ -490,7 +497,7 @@ extern "C" int tsp_planar_moe_gate_up_swiglu_m8(const tsp_small_moe* m, void* st
     int rc = fill_common(m, &a, false);
     if (rc != TSP_OK) return rc;
     const auto s = static_cast<hipStream_t>(stream);
-    if (m->tokens > 1) {
+    if (m->tokens > 1 && !gate_up_builds_union(a)) {
         rc = tsp_planar_union_build(m->ids, m->union_meta, m->experts, m->selected, m->tokens, m->hidden, m->channels, m->error_word, stream);
         if (rc != TSP_OK) return rc;
     }
@@ -502,7 +509,7 @@ extern "C" int tsp_planar_moe_routed_m8(const tsp_small_moe* m, void* stream) {
     int rc = fill_common(m, &a, true);
     if (rc != TSP_OK) return rc;
     const auto s = static_cast<hipStream_t>(stream);
-    if (m->tokens > 1) {
+    if (m->tokens > 1 && !gate_up_builds_union(a)) {
         rc = tsp_planar_union_build(m->ids, m->union_meta, m->experts, m->selected, m->tokens, m->hidden, m->channels, m->error_word, stream);
         if (rc != TSP_OK) return rc;
     }
@@ -537,7 +544,7 @@ extern "C" int tsp_planar_moe_routed_m8_shared(const tsp_small_moe* m, const tsp
                     "planar v3 small MoE outputs overlap inputs");
     TSP_REQUIRE(!ranges_overlap(shared->h, h_span, shared->y, y_span), "planar v3 small MoE outputs overlap inputs");
     const auto s = static_cast<hipStream_t>(stream);
-    if (m->tokens > 1) {
+    if (m->tokens > 1 && !gate_up_builds_union(a, shared)) {
         rc = tsp_planar_union_build(m->ids, m->union_meta, m->experts, m->selected, m->tokens, m->hidden, m->channels, m->error_word, stream);
         if (rc != TSP_OK) return rc;
     }

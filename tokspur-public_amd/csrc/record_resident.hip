@@ -30,6 +30,7 @@
 
 #include <type_traits>
 
+#include "grouping_device.hpp"
 #include "mfma_quant.hpp"
 
 using namespace tsp;
@@ -48,7 +49,8 @@ struct RecordArgs {
     const uint8_t* shared_w0;  // the always-on expert: gate
     const uint8_t* shared_w1;  // up
     tsp_planar_spec spec;
-    const uint32_t* meta;      // the union block
+    const uint32_t* ids;       // the routes' expert ids, [tokens][selected]
+    uint32_t* meta;            // the union block: written by workgroup 0 for the launches that follow
     float* out;                // h rows by route, out_stride bytes apart
     uint64_t out_stride;
     float* shared_out;         // the always-on expert's h rows, by token
@@ -172,12 +174,14 @@ __device__ __forceinline__ float rows_to_fragments(const float4 (&v)[8], uint32_
 constexpr int kMetaBytes = 9280;  // the union block
 constexpr int kSlotBytes = 80;    // a record of the share: (index, expert, rows | flags), its 8 tokens, its 8 routes
 
-// The union block into LDS, all threads, one round trip (the caller's barrier follows).
-__device__ __forceinline__ void stage_union_block(const RecordArgs& a, uint8_t* lds, uint32_t tid) {
-    const uint4* block = reinterpret_cast<const uint4*>(a.meta);
-    uint4* staged = reinterpret_cast<uint4*>(lds);
-    staged[tid] = block[tid];
-    if (tid < kMetaBytes / 16 - kThreads) staged[kThreads + tid] = block[kThreads + tid];
+// The union block, built by every workgroup for itself in LDS from the routes' expert ids (one load per thread instead of a
+// launch of its own before this one); workgroup 0 also writes it to memory, where the down product's launch reads it. False
+// when an id is out of range: the block's header is then zero in memory, the error bit set, and every workgroup leaves.
+__device__ __forceinline__ bool build_union_block(const RecordArgs& a, uint32_t mine, uint32_t* block, uint32_t* scratch, uint32_t tid) {
+    const bool writer = blockIdx.x == 0;
+    return union_block(mine, tid, uint32_t(kThreads), a.experts, a.selected, a.tokens, a.n, 2048u, scratch,
+                       [&](uint32_t word, uint32_t value) { block[word] = value; if (writer) a.meta[word] = value; },
+                       [&]() { if (writer) atomicOr(a.error_word, TSP_ERRBIT_INDEX); });
 }
 
 // The launch's (record, unit) items, in record order, cut into equal contiguous shares, one per workgroup.
@@ -260,7 +264,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     const uint32_t units = a.n / 32;
     uint32_t bad = 0, phase = 0;
 
-    // ---- the tokens' rows, this wave's 256 columns of them (a kilobyte per row and request), and the union block: one round trip
+    // ---- the tokens' rows, this wave's 256 columns of them (a kilobyte per row and request)
+    // the thread's route id first: the union records are built from the ids while the rows travel
+    const uint32_t my_id = tid < a.tokens * a.selected ? a.ids[tid] : 0xffffffffu;
     float4 rows[8];
     {
 #pragma unroll
@@ -268,9 +274,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             const uint32_t token = uint32_t(j) < a.tokens ? j : 0;  // a token the batch does not have repeats the first; nobody reads its sums
             rows[j] = *reinterpret_cast<const float4*>(reinterpret_cast<const uint8_t*>(a.x) + uint64_t(token) * a.x_stride + (wave * 256 + lane * 4) * 4);
         }
-        stage_union_block(a, lds_raw, tid);
     }
-    __syncthreads();
+    static_assert(kUnionScratchWords * 4 <= kGuStages * kGuStageBytes);
+    if (!build_union_block(a, my_id, reinterpret_cast<uint32_t*>(lds_raw), reinterpret_cast<uint32_t*>(lds_raw + kStagesAt), tid)) return;
+    __syncthreads();  // the block is complete; the scratch (the first wave's ring of stages) is free again
     const uint32_t* meta = reinterpret_cast<const uint32_t*>(lds_raw);
     const Share sh = share_of(a, meta, units, tid);
     if (sh.it0 >= sh.it1) return;
@@ -479,7 +486,7 @@ bool record_gate_up_takes(const SkinnyMoe& m) {
 int launch_record_gate_up(const SkinnyMoe& m, hipStream_t s) {
     RecordArgs a{};
     a.x = m.x; a.x_stride = m.x_stride;
-    a.w0 = m.pair_lo; a.w1 = m.pair_hi; a.shared_w0 = m.shared_gate; a.shared_w1 = m.shared_up; a.spec = m.gu; a.meta = m.meta;
+    a.w0 = m.pair_lo; a.w1 = m.pair_hi; a.shared_w0 = m.shared_gate; a.shared_w1 = m.shared_up; a.spec = m.gu; a.ids = m.ids; a.meta = m.meta;
     a.out = m.h; a.out_stride = m.h_stride; a.shared_out = m.shared_h; a.shared_out_stride = m.shared_h_stride;
     a.experts = m.experts; a.tokens = m.tokens; a.selected = m.selected; a.records = m.records; a.n = m.hidden;
     a.error_word = m.error_word;

@@ -9,7 +9,7 @@ struct SkinnyMoe {
     const uint8_t* pair_hi;  // experts E/2..E-1
     const uint8_t* down;     // [experts] planar
     const uint32_t* ids;     // [tokens * selected]
-    const uint32_t* meta;    // union records, or nullptr for one route per task
+    uint32_t* meta;          // union records (the caller's scratch: the record-resident launch writes them), or nullptr for one route per task
     const float* x;          // token rows
     float* h;                // route rows
     float* y;                // route rows
