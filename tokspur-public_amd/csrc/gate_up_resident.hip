@@ -213,7 +213,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
             // the stage is free again: the tile two ahead goes there
             request_next();
             stage = stage + kStageBytes == kStages * kStageBytes ? 0 : stage + kStageBytes;
-            const float d = half_bits_to_float(dm & 0xffffu), dmin = half_bits_to_float(dm >> 16);
+            float d = half_bits_to_float(dm & 0xffffu), dmin = half_bits_to_float(dm >> 16);
+            asm volatile("" : "+v"(d), "+v"(dmin));  // as floats in registers: folded into the arithmetic as halves they make every multiply-add a mixed-precision one
 
             f32x16 blk[MT];
             auto steps = [&](auto p_tag) {
