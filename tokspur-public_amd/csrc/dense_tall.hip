@@ -95,8 +95,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
         a_lane[i] = (row * a.a_stride + (((tid % 8) ^ ((r >> 1) & 7)) * 8)) * 2;
     }
     // nibbles: request q of thread t fills position u = t + T q of the stage = slot u % 2 of weight row u / 2, with chunk
-    // (u % 2) ^ ((row / 8) % 2) of the step's 32 bytes of that row; headers: position t % 256 = weight row t % 256 (with eight
-    // waves the two halves of the workgroup fetch the same)
+    // (u % 2) ^ ((row / 8) % 2) of the step's 32 bytes of that row; headers: position t = weight row t
     constexpr int QN = 2;
     uint32_t q_lane[QN];
 #pragma unroll
@@ -108,7 +107,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
     const uint32_t h_lane = h_row * row_bytes;
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds_raw));
     const uint32_t my_slab = lds0 + wave * 1024, my_qs = lds0 + kQsAt + wave * 1024, my_hdr = lds0 + kHdrAt + (wave % 4) * 1024;
-    // Step `step`'s bytes into ring slot step % 3. Steps past the end ask for the last step's bytes again (nobody reads them), and
+    // Step `step`'s bytes into ring slot step % 3. Steps past the end ask for the last step's bytes again (read by the front of a step that never runs), and
     // ask for headers where a real step would: the number of requests per step must not depend on where the matrix ends,
     // the waits below count them.
     auto request = [&](uint32_t step) {
