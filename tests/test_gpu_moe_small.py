@@ -146,6 +146,17 @@ def test_routed_m8_sticky_errors_and_refusals(gpu, tsp, orc, synth):
     assert gpu.error() & tsp.ERRBIT_NONFINITE
     h, y = tsp.planar_moe_routed_m8(gpu, w, good, gpu.upload(x), 2, selected)  # the next batch is clean
     assert gpu.error() == 0 and np.isfinite(y.cpu().numpy()).all()
+    # the same through the launch that keeps the tokens resident and builds the union records itself (2048-column experts)
+    wide = tsp.PlanarMoeWeights(gpu, 12, 14, 2048, 256, experts, synth.matrix(12, 35, 256 * experts, 2048), synth.matrix(12, 36, 256 * experts, 2048),
+                                synth.matrix(14, 37, 2048 * experts, 256))
+    xw = synth.activations_f32(38, (2, 2048))
+    h, y = tsp.planar_moe_routed_m8(gpu, wide, good, gpu.upload(xw), 2, selected)
+    assert gpu.error() == 0 and np.isfinite(y.cpu().numpy()).all()
+    before = y.cpu().numpy().copy()
+    tsp.planar_moe_routed_m8(gpu, wide, gpu.upload(np.array([0, 1, 7, 3], dtype=np.uint32)), gpu.upload(xw), 2, selected, y=y)
+    assert gpu.error() & tsp.ERRBIT_INDEX and np.array_equal(y.cpu().numpy(), before)  # nothing ran on the bad batch
+    h, y2 = tsp.planar_moe_routed_m8(gpu, wide, good, gpu.upload(xw), 2, selected)
+    assert gpu.error() == 0 and np.array_equal(y2.cpu().numpy(), before)
     with pytest.raises(tsp.FormatError):
         tsp.planar_moe_routed_m8(gpu, w, good, gpu.upload(x), 9, selected)
     with pytest.raises(tsp.FormatError):
