@@ -57,14 +57,6 @@ __device__ __forceinline__ f16x8 scaled8_q4(uint32_t c0, uint32_t c1, f16x2 sc, 
     return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
 }
 
-// Eight codes 0..63: 0x5400 | (c << 4) = 64 + c, so (64 + c) * sc - 96 * sc = (c - 32) * sc.
-__device__ __forceinline__ f16x8 scaled8_q6(uint32_t c0, uint32_t c1, f16x2 sc, f16x2 bias) {
-    constexpr uint32_t K = 0x54005400u;
-    const f16x2 p0 = fma2(as_h2((spread01(c0, 0) << 4) | K), sc, bias), p1 = fma2(as_h2((spread23(c0, 0) << 4) | K), sc, bias);
-    const f16x2 p2 = fma2(as_h2((spread01(c1, 0) << 4) | K), sc, bias), p3 = fma2(as_h2((spread23(c1, 0) << 4) | K), sc, bias);
-    return f16x8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
-}
-
 // Eight int8 quants (two dwords) as exact halves: q ^ 0x80 = q + 128 in 0..255, 0x6400 | u = 1024 + u, minus 1152.
 __device__ __forceinline__ f16x8 quants8(uint32_t w0, uint32_t w1) {
     constexpr uint32_t K = 0x64646464u;
@@ -207,24 +199,27 @@ struct RawQ6 { u32x4 la, lb, qh; uint32_t sc[2]; };  // one section: low nibbles
 // the 16-weight group 2Q + h. Fragment f covers activation columns Q*32 + 16h + f*8 .. +8 of the section.
 template <int Q>
 __device__ __forceinline__ void frags_q6k(const RawQ6& r, uint32_t khalf, f16x8 frag[2]) {
-    constexpr uint32_t M4 = 0x0f0f0f0fu, M2 = 0x30303030u;
+    // A code c = low nibble | two high bits << 4 becomes the half 0x5400 | c << 4 = 64 + c, and (64 + c) * sc - 96 * sc =
+    // (c - 32) * sc in one fused multiply-add. The half is put together from its two bytes, four weights at a time: the low
+    // byte is the nibble << 4, the high byte 0x54 | the two high bits, and a byte permute pairs them up; the six-bit code
+    // itself is never formed (that took a shift and an or per pair of weights more).
+    constexpr uint32_t MH = 0xf0f0f0f0u, M2 = 0x03030303u;
+    uint32_t K = 0x54545454u;
+    asm("" : "+v"(K));  // in a vector register: with two scalar constants (x & M2) | K is two instructions, not one v_and_or_b32
     const u32x4& l = (Q & 1) ? r.lb : r.la;
     const uint32_t g = 2 * Q + khalf;
     const int sc = int(int8_t((r.sc[g >> 2] >> ((g & 3) * 8)) & 0xffu));
     const f16x2 s2 = splat(float(sc)), bias = s2 * splat(-96.0f);
-    uint32_t c[4];
+    f16x2 p[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const uint32_t low = Q < 2 ? l[i] & M4 : (l[i] >> 4) & M4;
-        uint32_t high;  // bits 2Q..2Q+1 of qh move to bits 4..5 of the code
-        if constexpr (Q == 0) high = r.qh[i] << 4;
-        else if constexpr (Q == 1) high = r.qh[i] << 2;
-        else if constexpr (Q == 2) high = r.qh[i];
-        else high = r.qh[i] >> 2;
-        c[i] = low | (high & M2);
+        const uint32_t low = Q < 2 ? (l[i] << 4) & MH : l[i] & MH;
+        const uint32_t high = ((Q == 0 ? r.qh[i] : r.qh[i] >> (2 * Q)) & M2) | K;  // bits 2Q..2Q+1 of every byte of qh
+        p[2 * i] = fma2(as_h2(__builtin_amdgcn_perm(high, low, 0x05010400u)), s2, bias);      // weights 0, 1 of the four
+        p[2 * i + 1] = fma2(as_h2(__builtin_amdgcn_perm(high, low, 0x07030602u)), s2, bias);  // weights 2, 3
     }
-    frag[0] = scaled8_q6(c[0], c[1], s2, bias);
-    frag[1] = scaled8_q6(c[2], c[3], s2, bias);
+    frag[0] = f16x8{p[0][0], p[0][1], p[1][0], p[1][1], p[2][0], p[2][1], p[3][0], p[3][1]};
+    frag[1] = f16x8{p[4][0], p[4][1], p[5][0], p[5][1], p[6][0], p[6][1], p[7][0], p[7][1]};
 }
 
 
