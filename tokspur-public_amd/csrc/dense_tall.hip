@@ -2,11 +2,12 @@
 //
 // With this many rows the weights must not be unpacked over and over: the 64-row tiles of the general kernel (gemm.hip)
 // unpack every weight once per 64 activation rows, and at 2048 rows spend eight vector instructions per MFMA doing so. Here
-// a workgroup of four waves owns a 128 x 256 (or 256 x 256) output tile, a wave all its activation rows x 64 weight rows
-// (four or eight row tiles x two column tiles: 128 or 256 accumulator registers), so a weight is unpacked once per 128 or
-// 256 rows. What bounds the loop is the rate at which a SIMD issues instructions next to its MFMAs (measured: one wave
-// issues one every ~8 cycles, two waves together one every ~4.6, and a mixed-precision multiply-add counts about double),
-// not the matrix pipe (about half busy), LDS (a fifth busy, no bank conflicts) or memory.
+// a workgroup owns a 128 x 256 output tile (four waves, each 128 activation rows x 64 weight rows) or a 256 x 256 tile (eight
+// waves, each 256 x 32): 128 accumulator registers per lane either way, two waves per SIMD, and a weight is unpacked once
+// per 128 or 256 rows. What bounds the loop is the rate at which a SIMD issues instructions next to its MFMAs (measured:
+// one wave issues one every ~8 cycles, two waves together one every ~4.6, a mixed-precision multiply-add counts about
+// double, a 16-byte LDS read from one wave every 17), not the matrix pipe (about half busy), LDS bandwidth (240-307 bytes
+// per cycle measured, a quarter of it used, no bank conflicts) or memory.
 //
 //   * Arithmetic: the engine's for this path. A weight is its f32 value d * sc * q - dmin * mn rounded once to half: the
 //     code q, masked out where it sits, is a subnormal half q * 2^-24, and one mixed-precision fused multiply-add per
@@ -60,17 +61,22 @@ constexpr int kTileN = 256, kStepK = 64, kRing = 3;
 constexpr int kQsBytes = kTileN * 32;
 constexpr int kHdrBytes = kTileN * 16, kHdrStages = 2;
 
+// waves per SIMD: 128-row tiles leave room for two workgroups per compute unit, 256-row tiles for one
+constexpr int tall_waves_per_simd(int rt, int ct, int waves) { return ((waves * ct / 8) * rt * 32 == 128 ? 2 : 1) * waves / 4; }
+
 // RT x CT: the row tiles (32 activation rows each) and column tiles (32 weight rows each) of a wave, 16 accumulator registers
-// apiece. The four waves stand 8 / CT wide across the tile's 256 weight rows and CT / 2 high. With 128 accumulator registers
-// (4 x 2: a 128 x 256 tile) two workgroups share a compute unit, two waves a SIMD; with 256 (8 x 2: a 256 x 256 tile) a wave has
-// a SIMD and its 512 registers to itself, and every unpacked weight serves twice as many MFMAs.
-template <int RT, int CT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8 ? 1 : 2, RT * CT > 8 ? 1 : 2))) void dense_tall_kernel(DenseTallArgs a) {
-    constexpr int kThreadsT = 256, WN = 8 / CT, WM = 4 / WN, kTileM = WM * RT * 32;
+// apiece; WAVES waves stand 8 / CT wide across the tile's 256 weight rows and WAVES CT / 8 high. Two forms are launched:
+//   4 x 2, four waves: a 128 x 256 tile; two workgroups share a compute unit.
+//   8 x 1, eight waves: a 256 x 256 tile; a weight is unpacked once per 256 rows, at the price of an LDS read per MFMA.
+// (8 x 2 with four waves, a wave alone on its SIMD with 256 accumulator registers, compiles too and measured in between.)
+template <int RT, int CT, int WAVES, int PER_SIMD = tall_waves_per_simd(RT, CT, WAVES)>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(PER_SIMD, PER_SIMD))) void dense_tall_kernel(DenseTallArgs a) {
+    constexpr int kThreadsT = 64 * WAVES, WN = 8 / CT, WM = WAVES / WN, kTileM = WM * RT * 32;
+    static_assert(WM >= 1 && WN * WM == WAVES);
     constexpr int kSlabBytes = kTileM * kStepK * 2, kSlabPieces = kSlabBytes / (kThreadsT * 16);
     constexpr int kQsAt = kRing * kSlabBytes, kHdrAt = kQsAt + kRing * kQsBytes;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kHdrAt + kHdrStages * kHdrBytes];
-    static_assert(sizeof(lds_raw) * (RT * CT > 8 ? 1 : 2) <= 160 * 1024, "the workgroups of a compute unit share 160 KB");
+    static_assert(sizeof(lds_raw) * (kTileM == 128 ? 2 : 1) <= 160 * 1024, "the workgroups of a compute unit share 160 KB");
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const uint32_t col = lane % 32, khalf = (lane / 32) & 1;
@@ -95,8 +101,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
         a_lane[i] = (row * a.a_stride + (((tid % 8) ^ ((r >> 1) & 7)) * 8)) * 2;
     }
     // nibbles: request q of thread t fills position u = t + T q of the stage = slot u % 2 of weight row u / 2, with chunk
-    // (u % 2) ^ ((row / 8) % 2) of the step's 32 bytes of that row; headers: position t = weight row t
-    constexpr int QN = 2;
+    // (u % 2) ^ ((row / 8) % 2) of the step's 32 bytes of that row; headers: position t % 256 = weight row t % 256 (with eight
+    // waves the two halves of the workgroup fetch the same bytes to the same place: every wave's count of requests is the same)
+    constexpr int QN = kQsBytes / (kThreadsT * 16);
     uint32_t q_lane[QN];
 #pragma unroll
     for (int q = 0; q < QN; ++q) {
@@ -148,7 +155,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
     float d[CT], dmin[CT];
     uint32_t sc[CT][2], mn[CT][2];  // eight scales and eight minima per weight row, one per byte
     u32x4 raw[CT];                  // the lane's 16 bytes of the step's pair of sub-blocks, per column tile: low nibbles are sub-block 2 P, high nibbles 2 P + 1
-    f16x8 af[2][RT];                // activation fragments of the k16 group at work and of the one after it
+    // activation fragments of the k16 group at work and of the one after it; with one column tile per wave a fragment serves
+    // one MFMA only, and its register is refilled for the next group right behind that MFMA instead (half the registers)
+    constexpr bool kRolling = CT == 1;
+    f16x8 af[kRolling ? 1 : 2][RT];
 
     // The four k16 groups of a step are (low, high nibbles) x (first, second eight columns of the lane's sixteen).
     auto read_a = [&](uint32_t step, int g, f16x8 (&to)[RT]) {
@@ -157,6 +167,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
 #pragma unroll
         for (int i = 0; i < RT; ++i) to[i] = *reinterpret_cast<const f16x8*>(slab + a_row_at + i * (32 * 128) + chunk);
     };
+    // The lane's byte position of row tile 0 of a group's fragments, as one opaque register per group: the row tiles then are
+    // immediate offsets of the read. Left to fold the slot's offset (up to 64 KB) and the row tile's into one constant, the
+    // compiler overflows the 16-bit offset field and keeps a separate address register for every fragment of a step.
+    auto group_at = [&](uint32_t step, int g) {
+        uint32_t at = a_row_at + (((4 * (g / 2) + 2 * khalf + (g % 2)) ^ a_swz) * 16) + (step % kRing) * kSlabBytes;
+        asm volatile("" : "+v"(at));
+        return at;
+    };
+    auto read_a_one = [&](uint32_t at, int i) { return *reinterpret_cast<const f16x8*>(lds_raw + at + i * (32 * 128)); };
     // What a step needs before its first MFMA: its nibbles, the activation fragments of its first group, and at the first
     // pair of a super-block the rows' scales and minima.
     auto front = [&](uint32_t step, auto first_pair, u32x4 (&nibbles)[CT]) {
@@ -175,7 +194,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
         const uint8_t* qs = lds_raw + (step % kRing) * kQsBytes;
 #pragma unroll
         for (int j = 0; j < CT; ++j) nibbles[j] = *reinterpret_cast<const u32x4*>(qs + q_at[j]);
-        read_a(step, 0, af[0]);
+        if constexpr (!kRolling) read_a(step, 0, af[0]);
     };
 
     // One step. The workgroup's barrier does not sit between two steps but before a step's last group: by then a wave has
@@ -190,13 +209,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
         for (int g = 0; g < 4; ++g) {
             const int hi = g / 2, ff = g % 2;
             // the activation fragments of a group are read one group ahead: their LDS latency passes behind the unpacking
-            if (g < 3) read_a(step, g + 1, af[(g + 1) % 2]);
+            if (!kRolling && g < 3) read_a(step, g + 1, af[(g + 1) % 2]);
             if (g == 3) {
                 // Younger than the requests of step + 1 are those of step + 2: the slab's pieces, the nibbles, and the headers
                 // when step + 2 begins a super-block.
                 lds_barrier_after_loads<kSlabPieces + QN + (P == 2 ? 1 : 0)>();
                 request(step + 3);
-                front(step + 1, std::bool_constant<P == 3>{}, next_raw);
+                if constexpr (!kRolling) front(step + 1, std::bool_constant<P == 3>{}, next_raw);
             }
             if (ff == 0) {
                 // sub-block 2 P + hi; weight = half(d * sc * q - dmin * mn), the f32 value rounded once
@@ -212,12 +231,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
             }
             // A word holds four codes, one nibble of each byte; bytes (0, 2), then (1, 3), are masked out where they are: two halves
             // whose only set bits are a code's. Eight columns come out in the order (0, 2, 1, 3, 4, 6, 5, 7), the activations' order.
-            // Two column tiles at a time, so that only two weight fragments are alive at once.
+            // At most two column tiles at a time, so that only two weight fragments are alive at once.
+            constexpr int JB = CT >= 2 ? 2 : 1;
 #pragma unroll
-            for (int j0 = 0; j0 < CT; j0 += 2) {
-                f16x8 b[2];
+            for (int j0 = 0; j0 < CT; j0 += JB) {
+                f16x8 b[JB];
 #pragma unroll
-                for (int jj = 0; jj < 2; ++jj) {
+                for (int jj = 0; jj < JB; ++jj) {
                     const int j = j0 + jj;
                     u32x4 packed;
 #pragma unroll
@@ -228,23 +248,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
                     }
                     b[jj] = __builtin_bit_cast(f16x8, packed);
                 }
+                // with one column tile the step's last unpacking has just freed the nibbles' registers: the next step's go there
+                if constexpr (kRolling) if (g == 3) front(step + 1, std::bool_constant<P == 3>{}, raw);
+                uint32_t next_at = 0;
+                if constexpr (kRolling) next_at = g < 3 ? group_at(step, g + 1) : group_at(step + 1, 0);
 #pragma unroll
                 for (int i = 0; i < RT; ++i) {
-                    acc[i][j0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[g % 2][i], b[0], acc[i][j0], 0, 0, 0);
-                    acc[i][j0 + 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[g % 2][i], b[1], acc[i][j0 + 1], 0, 0, 0);
+#pragma unroll
+                    for (int jj = 0; jj < JB; ++jj)
+                        acc[i][j0 + jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[kRolling ? 0 : g % 2][i], b[jj], acc[i][j0 + jj], 0, 0, 0);
+                    // the next group's fragment into the register this MFMA has read (after the barrier of the last group:
+                    // the next step's first group)
+                    if constexpr (kRolling) af[0][i] = read_a_one(next_at, i);
                 }
             }
         }
+        if constexpr (!kRolling) {
 #pragma unroll
-        for (int j = 0; j < CT; ++j) raw[j] = next_raw[j];
+            for (int j = 0; j < CT; ++j) raw[j] = next_raw[j];
+        }
         // A wave issues in order: eight MFMAs in a row hold it for eight times the matrix pipe's 32 cycles, with its own
         // unpacking waiting behind them. Interleaved, one MFMA then four vector instructions (and an LDS read every other
         // time), the unpacking of the next group runs in the shadow of this group's MFMAs.
 #pragma unroll
         for (int k = 0; k < 4 * RT * CT; ++k) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, RT * CT > 8 ? 3 : 4, 0);
-            if (k % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, CT == 1 ? 2 : RT * CT > 8 ? 3 : 4, 0);
+            if (CT == 1 || k % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
     };
 
@@ -253,6 +283,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
     request(2);
     lds_barrier_after_loads<2 * (kSlabPieces + QN)>();  // step 0 has landed; the requests of steps 1 and 2 are the younger ones
     front(0, std::true_type{}, raw);
+    if constexpr (kRolling) {
+        const uint32_t at = group_at(0, 0);
+#pragma unroll
+        for (int i = 0; i < RT; ++i) af[0][i] = read_a_one(at, i);
+    }
     for (uint32_t b = 0; b < bpr; ++b) {
         step_fn(b * 4 + 0, std::integral_constant<int, 0>{});
         step_fn(b * 4 + 1, std::integral_constant<int, 1>{});
@@ -268,16 +303,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
     __syncthreads();  // every wave has left the rings, and every request into them has landed: the LDS is the epilogue's
     if (whole) {
         // The wave's results go out as whole 16-byte pieces, neighbouring lanes along a row, after a turn through LDS that the
-        // wave has to itself (18 KB: four row tiles of 64 results at a time as bf16, two as f32; a row pitch of 16 bytes
+        // wave has to itself (16 or 18 KB: a few row tiles at a time; a row pitch of 16 bytes
         // more than the row keeps the column-wise writes and the row-wise reads off each other's banks). A lane storing
         // its own 2- or 4-byte results one by one, 128 stores, took a fifth of the kernel's time.
-        uint8_t* const mine = lds_raw + wave * (16 * 1024 + 2048);
-        static_assert((kThreadsT / kWave) * (16 * 1024 + 2048) <= int(sizeof(lds_raw)));
+        constexpr int kRegion = WAVES == 8 ? 16 * 1024 : 16 * 1024 + 2048;
+        uint8_t* const mine = lds_raw + wave * kRegion;
+        static_assert(WAVES * kRegion <= int(sizeof(lds_raw)));
         auto pass = [&](auto bf16_tag, auto first_tag) {
             constexpr bool BF16 = decltype(bf16_tag)::value;
             constexpr int first_tile = decltype(first_tag)::value;
-            constexpr int kTiles = (BF16 ? 8 : 4) / CT, kElem = BF16 ? 2 : 4, kPitch = CT * 32 * kElem + 16;
-            static_assert(kTiles * 32 * kPitch <= 16 * 1024 + 2048 && first_tile + kTiles <= RT);
+            constexpr int kTiles = CT == 1 ? (BF16 ? 4 : 2) : (BF16 ? 8 : 4) / CT, kElem = BF16 ? 2 : 4, kPitch = CT * 32 * kElem + 16;
+            static_assert(kTiles * 32 * kPitch <= kRegion && first_tile + kTiles <= RT);
 #pragma unroll
             for (int t = 0; t < kTiles; ++t) {
                 const int i = first_tile + t;
@@ -313,12 +349,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(RT * CT > 8
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         };
-        // 8 / CT row tiles at a time as bf16, half as many as f32
+        // four row tiles at a time as bf16, two as f32 (with two column tiles per wave; twice that with four, and four and two with one)
+        constexpr int kTilesB = CT == 1 ? 4 : 8 / CT, kTilesF = CT == 1 ? 2 : 4 / CT;
         auto passes = [&]<int... I>(auto bf16_tag, std::integer_sequence<int, I...>) {
-            (pass(bf16_tag, std::integral_constant<int, I * ((decltype(bf16_tag)::value ? 8 : 4) / CT)>{}), ...);
+            (pass(bf16_tag, std::integral_constant<int, I * (decltype(bf16_tag)::value ? kTilesB : kTilesF)>{}), ...);
         };
-        if (a.out_bf16) passes(std::true_type{}, std::make_integer_sequence<int, RT * CT / 8>{});
-        else passes(std::false_type{}, std::make_integer_sequence<int, RT * CT / 4>{});
+        if (a.out_bf16) passes(std::true_type{}, std::make_integer_sequence<int, RT / kTilesB>{});
+        else passes(std::false_type{}, std::make_integer_sequence<int, RT / kTilesF>{});
     } else {
         // a ragged column tile or rows that 16 bytes do not align: element by element
 #pragma unroll
@@ -368,9 +405,9 @@ int launch_dense_tall(const DenseTallArgs& a, hipStream_t s) {
     const uint32_t n_tiles = (a.n + kTileN - 1) / kTileN, cus = uint32_t(units[device]);
     const uint32_t tall = n_tiles * ((a.m + 255) / 256), low = n_tiles * ((a.m + 127) / 128);
     if (tall <= cus && uint64_t(tall) * 10 >= uint64_t(cus) * 9) {
-        TSP_LAUNCH("gemm_dense_tall", s, (dense_tall_kernel<8, 2><<<(tall + 7) / 8 * 8, 256, 0, s>>>(a)));
+        TSP_LAUNCH("gemm_dense_tall", s, (dense_tall_kernel<8, 1, 8><<<(tall + 7) / 8 * 8, 512, 0, s>>>(a)));
     } else {
-        TSP_LAUNCH("gemm_dense_tall", s, (dense_tall_kernel<4, 2><<<(low + 7) / 8 * 8, 256, 0, s>>>(a)));
+        TSP_LAUNCH("gemm_dense_tall", s, (dense_tall_kernel<4, 2, 4><<<(low + 7) / 8 * 8, 256, 0, s>>>(a)));
     }
     return launch_status("dense_tall");
 }
