@@ -799,6 +799,123 @@ void test_encode_moe_mm_many_raw_arm() {
     }
     release_moe_mm_many_scratch(g, scratch);
 }
+// native/tests/test_profile.cpp: the opt-in per-operator profile. Same fixture (an F32 GEMV, SiLU, a product and an RMS
+// norm), same checks: rows only when asked for, one per operator with the engine's labels and shape metadata, nothing
+// allocated while encoding and no output changed, calibration never fails a batch, a batch longer than one sample chunk,
+// the capacity refusal while encoding, no stale profile after a device error, the payload on the ledger and its release.
+double checked_timings(const GraphProfile& profile) {
+    const double mismatch = profile.cpu_clock_mismatch_fraction;
+    const bool calibrated = std::isfinite(mismatch) && mismatch >= 0 && mismatch <= 0.03;
+    EXPECT(profile.timings_valid == calibrated);
+    double maximum = 0, sum = 0;
+    bool ticks = true, millis = true;
+    uint64_t previous = 0;
+    for (const auto& t : profile.kernels) {
+        ticks = ticks && t.start && t.end >= t.start && t.start >= previous;
+        previous = t.end;
+        if (profile.timings_valid) {
+            millis = millis && std::isfinite(t.milliseconds) && t.milliseconds >= 0;
+            maximum = std::max(maximum, t.milliseconds);
+            sum += t.milliseconds;
+        } else millis = millis && std::isnan(t.milliseconds);
+    }
+    EXPECT(ticks && millis);
+    if (profile.timings_valid) EXPECT(profile.gpu_tick_nanoseconds > 0 && std::isfinite(profile.sampled_milliseconds) && profile.sampled_milliseconds == sum);
+    else EXPECT(std::isnan(profile.gpu_tick_nanoseconds) && std::isnan(profile.sampled_milliseconds));
+    return maximum;
+}
+void test_profile() {
+    EXPECT(profile_calibration_valid(1.0, 0.03) && !profile_calibration_valid(1.0, 0.0301) && !profile_calibration_valid(0.0, 0.0) &&
+           !profile_calibration_valid(std::numeric_limits<double>::quiet_NaN(), 0.0) && !profile_calibration_valid(1.0, -0.1));
+    HipGraph graph("unused", 128u << 20);
+    constexpr uint32_t columns = 4096, rows = 2048;
+    std::vector<float> matrix(size_t(columns) * rows), x(columns), ones(rows, 1);
+    for (size_t i = 0; i < matrix.size(); ++i) matrix[i] = float(int((i * 13 + 5) % 251) - 125) / 32768;
+    for (size_t i = 0; i < x.size(); ++i) x[i] = float(int((i * 17 + 3) % 257) - 128) / 128;
+    const GpuView weights = graph.upload(bytes_of(matrix), "profile fixture weights"), input = graph.upload(bytes_of(x), "profile fixture input");
+    const GpuView gain = graph.upload(bytes_of(ones), "profile fixture gain");
+    const GpuView output = graph.zeros(rows * 4, "profile fixture output"), norm = graph.zeros(rows * 4, "profile fixture norm");
+    const uint64_t base = graph.memory().live_bytes;
+    const auto encode = [&] {
+        graph.gemv(0, weights, input, output, columns, rows);
+        graph.activate(output, output, Activation::silu);
+        graph.multiply(output, gain, output);
+        graph.rms(output, gain, norm, 64, 1e-6f);
+    };
+    graph.begin(); encode(); (void)graph.submit();
+    const auto expected = graph.read(norm);
+    EXPECT(graph.last_profile().kernels.empty() && graph.last_profile().mode == ProfileMode::disabled);
+    const ProfileMode mode = graph.configure_profiling(4096);
+    EXPECT(mode == ProfileMode::dispatch_boundary && graph.memory().profile_counter_payload_bytes == 2 * 32768 &&
+           graph.memory().live_bytes == base + 65536);
+    double maximum = 0, gemv_ms = 0;
+    for (uint32_t repeat = 0; repeat < 8; ++repeat) {
+        const uint64_t allocations = graph.memory().allocations;
+        graph.begin();
+        EXPECT(throws_format([&] { (void)graph.last_profile(); }));
+        EXPECT(throws_format([&] { (void)graph.configure_profiling(0); }));
+        encode();
+        const BatchResult batch = graph.submit();
+        const GraphProfile& profile = graph.last_profile();
+        EXPECT(batch.dispatches == 4 && profile.kernels.size() == 4 && profile.mode == mode);
+        EXPECT(graph.memory().allocations == allocations && graph.read(norm) == expected);
+        if (profile.kernels.size() == 4) {
+            EXPECT(profile.kernels[0].kernel == "graph_quantized_gemv" && profile.kernels[0].encoding == 0 && profile.kernels[0].shape[0] == columns &&
+                   profile.kernels[0].shape[1] == rows);
+            EXPECT(profile.kernels[1].kernel == "graph_activate" && profile.kernels[2].kernel == "graph_multiply" && profile.kernels[3].kernel == "graph_rms");
+            // the raw samples order the operators whether or not the batch calibrated; the 32 MB GEMV is the long one
+            EXPECT(profile.kernels[0].end - profile.kernels[0].start > profile.kernels[1].end - profile.kernels[1].start);
+            EXPECT(profile.kernels[3].end <= uint64_t(batch.gpu_ms * 1e6) + 1000);
+            if (profile.timings_valid) gemv_ms = std::max(gemv_ms, profile.kernels[0].milliseconds);
+        }
+        maximum = std::max(maximum, checked_timings(profile));
+    }
+    // a batch long enough to calibrate, and longer than one chunk of 2048 samples
+    graph.begin(); encode();
+    for (uint32_t i = 0; i < 2050; ++i) graph.activate(norm, norm, Activation::identity);
+    const BatchResult crossing = graph.submit();
+    EXPECT(crossing.dispatches == 2054 && graph.last_profile().kernels.size() == 2054 && graph.read(norm) == expected);
+    EXPECT(graph.last_profile().kernels.size() == 2054 && graph.last_profile().kernels[2048].kernel == "graph_activate");
+    maximum = std::max(maximum, checked_timings(graph.last_profile()));
+    {
+        const GraphProfile& profile = graph.last_profile();
+        std::printf("   profile of %zu operators: valid %d, clock mismatch %.4f, sampled %.3f ms of %.3f ms on the GPU; GEMV row %.1f us\n", profile.kernels.size(),
+                    int(profile.timings_valid), profile.cpu_clock_mismatch_fraction, profile.sampled_milliseconds, crossing.gpu_ms,
+                    double(profile.kernels[0].end - profile.kernels[0].start) / 1e3);
+        // the rows tile the batch: their raw spans add up to the GPU's span of it, first boundary to end
+        uint64_t span = 0;
+        for (const auto& t : profile.kernels) span += t.end - t.start;
+        EXPECT(std::fabs(double(span) / 1e6 - crossing.gpu_ms) <= 0.05 * crossing.gpu_ms + 0.05);
+    }
+    EXPECT(throws_format([&] { (void)graph.configure_profiling(16385); }));
+    const auto before = graph.read(output);
+    (void)graph.configure_profiling(1);
+    graph.begin();
+    graph.gemv(0, weights, input, output, columns, rows);
+    EXPECT(throws_format([&] { graph.activate(output, output, Activation::silu); }));  // past the capacity: refused, nothing launched
+    graph.abort();
+    EXPECT(graph.last_profile().kernels.empty());
+    (void)before;  // the GEMV of the aborted batch was launched as it was encoded (operators are not deferred here): its output is the same product
+    (void)graph.configure_profiling(8);
+    const std::vector<float> infinity(rows, std::numeric_limits<float>::infinity());
+    const GpuView invalid = graph.upload(bytes_of(infinity), "profile invalid input");
+    graph.begin();
+    graph.activate(invalid, output, Activation::sigmoid);
+    EXPECT(throws_format([&] { (void)graph.submit(); }));
+    EXPECT(graph.last_profile().kernels.empty());  // no stale successful profile after a device error
+    graph.begin(); encode(); (void)graph.submit();
+    EXPECT(graph.read(norm) == expected && graph.last_profile().kernels.size() == 4);
+    graph.release(invalid);
+    (void)graph.configure_profiling(0);
+    EXPECT(graph.memory().live_bytes == base && graph.memory().profile_counter_payload_bytes == 0);
+    graph.begin(); encode(); (void)graph.submit();
+    EXPECT(graph.last_profile().kernels.empty() && graph.read(norm) == expected);
+    HipGraph limited(16384);
+    const uint64_t low = limited.memory().live_bytes;
+    EXPECT(throws_format([&] { (void)limited.configure_profiling(16384); }));  // 262144 bytes of samples against a 16 KB budget
+    EXPECT(limited.memory().live_bytes == low && limited.last_profile().kernels.empty() && limited.memory().profile_counter_payload_bytes == 0);
+    std::printf("   maximum sampled operator %.4f ms, F32 GEMV %.4f ms\n", maximum, gemv_ms);
+}
 }  // namespace
 
 int main() {
@@ -812,7 +929,8 @@ int main() {
                                                          {"router projection: plan, selection, bounds, refusals", test_router_projection_controls},
                                                          {"pack v3: build, adopt, upload a block, encode_moe_mm_many on it", test_pack_v3_block_on_graph},
                                                          {"RMS, activation, residual streams; partial commit", test_residual_streams_and_partial_commit},
-                                                         {"encode_moe_mm_many, raw-GGUF arm; prepare twice; Q8_0 registration", test_encode_moe_mm_many_raw_arm}};
+                                                         {"encode_moe_mm_many, raw-GGUF arm; prepare twice; Q8_0 registration", test_encode_moe_mm_many_raw_arm},
+                                                         {"per-operator profile", test_profile}};
     for (const auto& [name, fn] : tests) {
         std::printf("== %s\n", name);
         std::fflush(stdout);

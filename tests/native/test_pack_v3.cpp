@@ -10,6 +10,7 @@
 #include <unistd.h>
 
 #include "gguf_writer.hpp"
+#include "hip_graph.hpp"
 #include "pack_v3.hpp"
 #include "tokspur_hip.h"
 #include "tokspur_oracle.h"
@@ -271,6 +272,53 @@ void test_build_adopt_tamper(const Shards& s) {
     // a pack cannot be packed again
     EXPECT(refuses([&] { (void)plan_derived_pack_v3(*adopted.model); }));
 }
+// include/tokspur/grouped_mm.hpp:22-26: the C++ planners, against the restated ones (themselves bit-equal to the compiled
+// reference) on the engine's shapes and on every encoding / layout pair, and the engine's refusals
+void test_grouped_mm_planners() {
+    static_assert(sizeof(GroupedMmArgs) == 56);
+    const auto same = [](const GroupedMmPlan& a, const orc_grouped_mm_plan& b) {
+        return std::memcmp(&a.args, &b.args, 56) == 0 && a.matrix_bytes == b.matrix_bytes && a.indices_bytes == b.indices_bytes &&
+               a.input_bytes == b.input_bytes && a.output_bytes == b.output_bytes && a.token_map_bytes == b.token_map_bytes &&
+               a.counts_bytes == b.counts_bytes && a.tasks_bytes == b.tasks_bytes && a.grid_x == b.grid_x && a.grid_y == b.grid_y;
+    };
+    const std::pair<uint32_t, PrefillWeightLayout> pairs[] = {{7, PrefillWeightLayout::gguf}, {8, PrefillWeightLayout::gguf}, {12, PrefillWeightLayout::gguf},
+                                                              {13, PrefillWeightLayout::gguf}, {8, PrefillWeightLayout::q8_lanes_v1}};
+    for (const auto& [type, layout] : pairs)
+        for (const uint32_t tokens : {1u, 31u, 32u, 33u, 512u, 2048u})
+            for (const bool broadcast : {false, true}) {
+                const bool big = tokens > 512;
+                const uint32_t experts = layout == PrefillWeightLayout::q8_lanes_v1 && !big ? 1 : 64, selected = experts == 1 ? 1 : 10;
+                orc_grouped_mm_plan want{};
+                EXPECT(orc_grouped_mm_plan_make(type, uint32_t(layout), 2560, 640, experts, selected, tokens, 10240, 2560, broadcast, big, &want) == 0);
+                const auto got = grouped_mm_plan(type, layout, 2560, 640, experts, selected, tokens, 10240, 2560, broadcast, big);
+                EXPECT(same(got, want) && std::string(got.kernel) == "graph_grouped_mm" && got.threads == 128 && got.threadgroup_bytes == 8192);
+            }
+    {   // the engine's Q5_1 lane geometry: 640 columns, more than one expert
+        orc_grouped_mm_plan want{};
+        EXPECT(orc_grouped_mm_plan_make(7, 2, 640, 2560, 512, 10, 512, 2560, 10240, 0, 0, &want) == 0);
+        EXPECT(same(grouped_mm_plan(7, PrefillWeightLayout::q51_lanes_v1, 640, 2560, 512, 10, 512, 2560, 10240, false), want));
+        EXPECT(refuses([] { (void)grouped_mm_plan(7, PrefillWeightLayout::q51_lanes_v1, 672, 2560, 512, 10, 512, 2688, 10240, false); }));
+    }
+    // config 1's dense product as the engine would plan it (experts = 1, selected = 1, broadcast)
+    const auto c1 = grouped_mm_plan(12, PrefillWeightLayout::gguf, 2048, 8192, 1, 1, 512, 8192, 32768, true);
+    EXPECT(c1.args.row_bytes == 1152 && c1.matrix_bytes == 9437184 && c1.grid_x == 128 && c1.grid_y == 17 && c1.args.maximum_tasks == 17);
+    const auto d = dense_mm_q8_plan(PrefillWeightLayout::gguf, 2048, 4096, 100, 8192, 16384);
+    EXPECT(d.indices_bytes == 0 && d.token_map_bytes == 0 && d.counts_bytes == 0 && d.tasks_bytes == 0 && d.args.maximum_tasks == 4 && d.grid_y == 4 &&
+           d.args.row_bytes == 2176 && std::string(d.kernel) == "graph_dense_mm_q8");
+    EXPECT(std::string(grouped_mm_kernel(13, PrefillWeightLayout::gguf)) == "graph_grouped_mm");
+    EXPECT(std::string(dense_mm_q8_kernel(PrefillWeightLayout::q8_lanes_v1)) == "graph_dense_mm_q8");
+    EXPECT(refuses([] { (void)grouped_mm_kernel(14, PrefillWeightLayout::gguf); }));                 // encoding
+    EXPECT(refuses([] { (void)grouped_mm_kernel(12, PrefillWeightLayout::q8_lanes_v1); }));          // layout / encoding
+    EXPECT(refuses([] { (void)dense_mm_q8_kernel(PrefillWeightLayout::q51_lanes_v1); }));
+    EXPECT(refuses([] { (void)grouped_mm_plan(12, PrefillWeightLayout::gguf, 2048, 512, 512, 10, 513, 8192, 2048, true); }));        // rows beyond 512 need allow_nax_2k
+    EXPECT(refuses([] { (void)grouped_mm_plan(12, PrefillWeightLayout::gguf, 2048, 512, 512, 10, 2049, 8192, 2048, true, true); }));
+    EXPECT(refuses([] { (void)grouped_mm_plan(12, PrefillWeightLayout::gguf, 2000, 512, 512, 10, 8, 8192, 2048, true); }));          // whole blocks
+    EXPECT(refuses([] { (void)grouped_mm_plan(12, PrefillWeightLayout::gguf, 2048, 512, 513, 10, 8, 8192, 2048, true); }));
+    EXPECT(refuses([] { (void)grouped_mm_plan(12, PrefillWeightLayout::gguf, 2048, 512, 8, 10, 8, 8192, 2048, true); }));            // selected beyond experts
+    EXPECT(refuses([] { (void)grouped_mm_plan(12, PrefillWeightLayout::gguf, 2048, 512, 512, 10, 8, 8188, 2048, true); }));          // stride below a row / not in 16s
+    EXPECT(refuses([] { (void)grouped_mm_plan(12, PrefillWeightLayout::gguf, 2048, 512, 512, 10, 8, 8192, 2040, true); }));
+    EXPECT(refuses([] { (void)dense_mm_q8_plan(PrefillWeightLayout::q8_lanes_v1, 544, 64, 8, 2176, 256); }));                        // lanes: 256s or under 512
+}
 }  // namespace
 
 int main() {
@@ -278,6 +326,7 @@ int main() {
     const std::pair<const char*, std::function<void()>> tests[] = {
         {"SHA-256 known answers", test_sha256_known_answers},
         {"GGUF reader", test_gguf_reader},
+        {"grouped_mm_plan / dense_mm_q8_plan", test_grouped_mm_planners},
         {"pack v3: plan, header, build, adoption, tamper", [] { const Shards s; test_plan_and_header(s); test_build_adopt_tamper(s); }}};
     for (const auto& [name, fn] : tests) {
         std::printf("== %s\n", name);

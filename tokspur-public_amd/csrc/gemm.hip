@@ -794,10 +794,11 @@ NaxLayout nax_layout(uint32_t tokens, uint32_t selected, uint32_t experts, uint3
     return l;
 }
 
-// The planar kinds the matrix-core kernels have no unpacking for (Q5_K / Q8_0 gate and up, Q5_1 / Q8_0 down) run
-// through the routed kernels for at most eight tokens, a chunk of eight tokens at a time: the same routes, tasks and
-// expert_down rows, computed in f32 on the vector units. h of a chunk (8 * selected rows of f32) borrows the buffer the
-// matrix-core path keeps its h rows in, which is never smaller.
+// Every gate/up pair of one encoding (Q4_K, Q5_K or Q8_0 co-located halves) and every down kind runs on the matrix cores
+// below. What is left for this arm are gate and up tensors of DIFFERENT encodings (this entry point takes any gate kind
+// beside any up kind; the engine's is_planar_moe asks for one encoding, so its compositions never come here): they run through the routed kernels for at most eight tokens, a chunk of eight tokens at a
+// time: the same routes, tasks and expert_down rows, computed in f32 on the vector units. h of a chunk (8 * selected rows of
+// f32) borrows the buffer the matrix-core path keeps its h rows in, which is never smaller.
 int grouped_moe_in_eights(const tsp_grouped_moe* m, const NaxLayout& l, void* stream) {
     auto* ws = static_cast<uint8_t*>(m->workspace);
     TSP_REQUIRE(uint64_t(8) * m->selected * m->hidden * 4 <= l.meta - l.hbuf, "planar v3 NAX scratch too small for requested batch");  // before anything is enqueued

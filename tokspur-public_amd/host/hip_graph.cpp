@@ -8,6 +8,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cstring>
+#include <limits>
 #include <thread>
 
 #include "tokspur_hip.h"
@@ -75,16 +76,62 @@ struct HipGraph::Impl {
     uint64_t q8_workspace_bytes = 0;
     uint32_t prepared_gate_up = 0, prepared_down = 0;
     bool router_batch = false, router_batch_prepared = false;
+    // per-operator timing: boundary b is recorded on the stream before operator b; the batch's end closes the last one
+    struct Mark { const char* kernel; uint32_t encoding; std::array<uint32_t, 4> shape; };
+    uint32_t profile_capacity = 0;
+    uint64_t profile_payload = 0;
+    std::vector<hipEvent_t> boundaries;  // profile_capacity + 1 once configured
+    std::vector<Mark> marks;
+    GraphProfile profile;
 
     void same_thread() const { require(std::this_thread::get_id() == thread, "GPU graph used from another thread"); }
     void idle() const {
         same_thread();
         require(!encoding, "GPU graph operation requires an idle graph");
     }
-    void active() {
+    void active(const char* kernel, uint32_t type = uint32_t(-1), std::array<uint32_t, 4> shape = {}) {
         same_thread();
         require(encoding, "GPU graph operator outside begin/submit");
+        if (profile_capacity) {
+            require(dispatches < profile_capacity && marks.size() == dispatches, "GPU profiler dispatch bookkeeping failed");
+            marks.push_back({kernel, type, shape});  // reserved while idle: no allocation here
+            hip(hipEventRecord(boundaries[dispatches], stream), "hipEventRecord");
+        }
         ++dispatches;
+    }
+    void drop_profile() {
+        profile.mode = ProfileMode::disabled;
+        profile.timings_valid = profile.cpu_clock_is_mach = false;
+        profile.gpu_tick_nanoseconds = profile.cpu_clock_mismatch_fraction = profile.sampled_milliseconds = 0;
+        profile.kernels.clear();  // keeps its reserved capacity
+        marks.clear();
+    }
+    void collect_profile(double gpu_ms, double wall_ms) {
+        require(marks.size() == dispatches, "GPU counter mark/dispatch bookkeeping differs");
+        const double unavailable = std::numeric_limits<double>::quiet_NaN();
+        const bool spans = gpu_ms > 0 && wall_ms > 0;
+        const double mismatch = spans ? std::abs(gpu_ms - wall_ms) / wall_ms : unavailable;
+        profile.mode = ProfileMode::dispatch_boundary;
+        profile.timings_valid = profile_calibration_valid(1.0, mismatch);
+        profile.gpu_tick_nanoseconds = profile.timings_valid ? 1.0 : unavailable;
+        profile.cpu_clock_mismatch_fraction = mismatch;
+        profile.sampled_milliseconds = profile.timings_valid ? 0 : unavailable;
+        uint64_t previous = 1;
+        for (size_t i = 0; i < marks.size(); ++i) {
+            float to_end = 0;  // boundary i + 1, or the batch's end for the last operator
+            hip(hipEventElapsedTime(&to_end, started, i + 1 < marks.size() ? boundaries[i + 1] : finished), "hipEventElapsedTime");
+            const uint64_t end = std::max(previous, uint64_t(1) + uint64_t(std::llround(std::max(0.0, double(to_end)) * 1e6)));
+            if (i == 0) {
+                float to_start = 0;
+                hip(hipEventElapsedTime(&to_start, started, boundaries[0]), "hipEventElapsedTime");
+                previous = uint64_t(1) + uint64_t(std::llround(std::max(0.0, double(to_start)) * 1e6));
+            }
+            const uint64_t start = std::min(previous, end);
+            const double ms = profile.timings_valid ? double(end - start) / 1e6 : unavailable;
+            profile.kernels.push_back({marks[i].kernel, marks[i].encoding, marks[i].shape, start, end, ms});
+            profile.sampled_milliseconds += ms;
+            previous = end;
+        }
     }
     const Allocation& allocation(const GpuView& v, bool writable = false) const {
         require(v.owner == owner && v.slot < slots.size() && slots[v.slot].live, "released or foreign GPU view");
@@ -167,6 +214,7 @@ HipGraph::~HipGraph() {
         if (a.live) (void)hipFree(a.device);
     for (void* p : {impl_->union_meta, impl_->nax_workspace, impl_->dense_workspace, impl_->grouped_workspace, impl_->q8_workspace, static_cast<void*>(impl_->error_word)})
         if (p) (void)hipFree(p);
+    for (hipEvent_t e : impl_->boundaries) (void)hipEventDestroy(e);
     (void)hipEventDestroy(impl_->started);
     (void)hipEventDestroy(impl_->finished);
     (void)hipStreamDestroy(impl_->stream);
@@ -225,7 +273,48 @@ void HipGraph::release(GpuView full_buffer) {
     slot.device = nullptr;
 }
 
-GraphMemory HipGraph::memory() const { return {impl_->budget, impl_->live_bytes, impl_->peak_bytes, impl_->allocations}; }
+GraphMemory HipGraph::memory() const { return {impl_->budget, impl_->live_bytes, impl_->peak_bytes, impl_->allocations, impl_->profile_payload}; }
+
+// include/tokspur/graph.hpp:503 (src/graph.mm:2669-2750)
+ProfileMode HipGraph::configure_profiling(uint32_t capacity) {
+    auto& p = *impl_; p.idle();
+    require(capacity <= 16384, "GPU profiling capacity limit");
+    const auto release = [&p] {
+        for (hipEvent_t e : p.boundaries) (void)hipEventDestroy(e);
+        p.boundaries.clear();
+        p.live_bytes -= p.profile_payload;
+        p.profile_payload = 0;
+        p.profile_capacity = 0;
+        p.drop_profile();
+    };
+    if (!capacity) { release(); return ProfileMode::disabled; }
+    constexpr uint32_t chunk = 2048;  // the engine sizes its sample buffers per 2048 dispatches, whole pages each
+    uint64_t payload = 0;
+    for (uint32_t first = 0; first < capacity; first += chunk) payload += (uint64_t(std::min(chunk, capacity - first)) * 16 + 4095) / 4096 * 4096;
+    require(payload <= p.budget - std::min(p.budget, p.live_bytes) + p.profile_payload, "GPU counter payload exceeds graph budget");
+    release();
+    std::vector<hipEvent_t> fresh;
+    fresh.reserve(size_t(capacity) + 1);
+    for (uint32_t i = 0; i <= capacity; ++i) {
+        hipEvent_t e = nullptr;
+        const hipError_t status = hipEventCreate(&e);
+        if (status != hipSuccess) {
+            for (hipEvent_t made : fresh) (void)hipEventDestroy(made);
+            hip(status, "hipEventCreate");
+        }
+        fresh.push_back(e);
+    }
+    p.boundaries = std::move(fresh);
+    p.marks.reserve(capacity);
+    p.profile.kernels.reserve(capacity);
+    p.profile_capacity = capacity;
+    p.profile_payload = payload;
+    p.live_bytes += payload;
+    p.peak_bytes = std::max(p.peak_bytes, p.live_bytes);
+    ++p.allocations;
+    return ProfileMode::dispatch_boundary;
+}
+const GraphProfile& HipGraph::last_profile() const { impl_->idle(); return impl_->profile; }
 
 std::string HipGraph::device_name() const {
     int device = 0;
@@ -245,6 +334,49 @@ void HipGraph::validate_disjoint(std::span<const GpuView> inputs, std::span<cons
     }
     for (size_t a = 0; a < destinations.size(); ++a)
         for (size_t b = a + 1; b < destinations.size(); ++b) require(!Impl::overlaps(destinations[a], destinations[b]), "unsupported GPU buffer alias");
+}
+
+// ------------------------------------------------------------------ planners of grouped_mm / dense_mm_q8
+namespace {
+GroupedMmPlan plan_from(const tsp_grouped_mm_plan_t& c, const char* kernel) {
+    GroupedMmPlan plan;
+    static_assert(sizeof(GroupedMmArgs) == sizeof(tsp_grouped_mm_args_t), "argument blocks differ");
+    std::memcpy(&plan.args, &c.args, sizeof plan.args);
+    plan.matrix_bytes = c.matrix_bytes;
+    plan.indices_bytes = c.indices_bytes;
+    plan.input_bytes = c.input_bytes;
+    plan.output_bytes = c.output_bytes;
+    plan.token_map_bytes = c.token_map_bytes;
+    plan.counts_bytes = c.counts_bytes;
+    plan.tasks_bytes = c.tasks_bytes;
+    plan.grid_x = c.grid_x;
+    plan.grid_y = c.grid_y;
+    plan.kernel = kernel;
+    return plan;
+}
+}  // namespace
+
+const char* grouped_mm_kernel(uint32_t encoding, PrefillWeightLayout layout) {
+    require(grouped_mm_takes(encoding, layout) && layout != PrefillWeightLayout::planar_v3,
+            encoding == 7 || encoding == 8 || encoding == 12 || encoding == 13 ? "grouped mm layout/encoding mismatch" : "grouped mm encoding");
+    return "graph_grouped_mm";
+}
+const char* dense_mm_q8_kernel(PrefillWeightLayout layout) {
+    (void)grouped_mm_kernel(8, layout);
+    return "graph_dense_mm_q8";
+}
+GroupedMmPlan grouped_mm_plan(uint32_t encoding, PrefillWeightLayout layout, uint32_t columns, uint32_t rows, uint32_t experts, uint32_t selected,
+                              uint32_t tokens, uint64_t input_stride_bytes, uint64_t output_stride_bytes, bool broadcast, bool allow_nax_2k) {
+    tsp_grouped_mm_plan_t c{};
+    check(tsp_grouped_mm_plan(encoding, uint32_t(layout), columns, rows, experts, selected, tokens, input_stride_bytes, output_stride_bytes, broadcast,
+                              allow_nax_2k, &c));
+    return plan_from(c, grouped_mm_kernel(encoding, layout));
+}
+GroupedMmPlan dense_mm_q8_plan(PrefillWeightLayout layout, uint32_t columns, uint32_t rows, uint32_t tokens, uint64_t input_stride_bytes,
+                               uint64_t output_stride_bytes, bool allow_nax_2k) {
+    tsp_grouped_mm_plan_t c{};
+    check(tsp_dense_mm_q8_plan(uint32_t(layout), columns, rows, tokens, input_stride_bytes, output_stride_bytes, allow_nax_2k, &c));
+    return plan_from(c, dense_mm_q8_kernel(layout));
 }
 
 // ------------------------------------------------------------------ Pack v3 registration
@@ -323,8 +455,11 @@ void HipGraph::begin() {
     impl_->locked = true;
     impl_->encoding = true;
     impl_->dispatches = 0;
-    impl_->wall_start = std::chrono::steady_clock::now();
+    impl_->drop_profile();
     hip(hipEventRecord(impl_->started, impl_->stream), "hipEventRecord");
+    // with a profile asked for, the GPU's clock and the host's start the batch together: the stream is idle here, so the wait is short
+    if (impl_->profile_capacity) hip(hipEventSynchronize(impl_->started), "hipEventSynchronize");
+    impl_->wall_start = std::chrono::steady_clock::now();
 }
 
 void HipGraph::abort() {
@@ -334,6 +469,7 @@ void HipGraph::abort() {
     hip(hipStreamSynchronize(impl_->stream), "hipStreamSynchronize");
     hip(hipMemset(impl_->error_word, 0, 4), "hipMemset");
     impl_->encoding = false;
+    impl_->drop_profile();
 }
 
 BatchResult HipGraph::submit() {
@@ -341,22 +477,24 @@ BatchResult HipGraph::submit() {
     require(impl_->encoding, "no GPU batch to submit");
     hip(hipEventRecord(impl_->finished, impl_->stream), "hipEventRecord");
     hip(hipStreamSynchronize(impl_->stream), "hipStreamSynchronize");
+    const double wall_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - impl_->wall_start).count();
     impl_->encoding = false;
     uint32_t word = 0;
     hip(hipMemcpy(&word, impl_->error_word, 4, hipMemcpyDeviceToHost), "hipMemcpy");
     if (word) {
         hip(hipMemset(impl_->error_word, 0, 4), "hipMemset");  // later batches are unaffected
+        impl_->drop_profile();
         throw FormatError("GPU graph produced nonfinite values or invalid gates");
     }
     float gpu_ms = 0;
     hip(hipEventElapsedTime(&gpu_ms, impl_->started, impl_->finished), "hipEventElapsedTime");
-    const double wall_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - impl_->wall_start).count();
+    if (impl_->profile_capacity) impl_->collect_profile(gpu_ms, wall_ms);
     return {impl_->dispatches, wall_ms, gpu_ms};
 }
 
 // ------------------------------------------------------------------ operators
 void HipGraph::gemv(uint32_t encoding, GpuView matrix, GpuView input, GpuView output, uint32_t columns, uint32_t rows) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_quantized_gemv", encoding, {columns, rows, 0, 0});
     require(input.bytes == uint64_t(columns) * 4 && output.bytes == uint64_t(rows) * 4, "GEMV vector byte span mismatch");
     const std::array in{matrix, input};
     validate_disjoint(in, std::array{output});
@@ -366,7 +504,7 @@ void HipGraph::gemv(uint32_t encoding, GpuView matrix, GpuView input, GpuView ou
 }
 
 void HipGraph::gemv_rows(uint32_t encoding, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_quantized_gemv_rows", encoding, {input.columns, output.columns, input.rows, 0});
     p.rows_fit(input, "GEMV rows geometry mismatch");
     p.rows_fit(output, "GEMV rows geometry mismatch");
     require(input.rows == output.rows, "GEMV rows geometry mismatch");
@@ -391,7 +529,7 @@ bool HipGraph::commit_partial() {
 }
 
 void HipGraph::rms(GpuView input, GpuView gains, GpuView output, uint32_t group_width, float epsilon) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_rms");
     const uint64_t count = floats(input);
     require(group_width && count % group_width == 0 && group_width <= 65536 && floats(output) == count &&
                 (floats(gains) == count || floats(gains) == group_width) && std::isfinite(epsilon) && epsilon > 0,
@@ -401,7 +539,7 @@ void HipGraph::rms(GpuView input, GpuView gains, GpuView output, uint32_t group_
                   count, group_width, gains.bytes == uint64_t(group_width) * 4 && count != group_width, epsilon, p.error_word, p.stream));
 }
 void HipGraph::rms_sigmoid_gate(GpuView input, GpuView gains, GpuView gate, GpuView output, uint32_t group_width, float epsilon) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_rms_sigmoid_gate");
     const uint64_t count = floats(input);
     require(group_width && count % group_width == 0 && group_width <= 65536 && floats(gate) == count && floats(output) == count &&
                 (floats(gains) == count || floats(gains) == group_width) && std::isfinite(epsilon) && epsilon > 0,
@@ -412,7 +550,7 @@ void HipGraph::rms_sigmoid_gate(GpuView input, GpuView gains, GpuView gate, GpuV
                                gains.bytes == uint64_t(group_width) * 4 && count != group_width, epsilon, p.error_word, p.stream));
 }
 void HipGraph::activate(GpuView input, GpuView output, Activation kind, float scale) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_activate");
     const uint64_t count = floats(input);
     require(floats(output) == count && uint32_t(kind) <= 3 && std::isfinite(scale), "graph activation shape/mode mismatch");
     // the output may be the input itself, not a view that merely overlaps it: the C ABI refuses that
@@ -420,14 +558,14 @@ void HipGraph::activate(GpuView input, GpuView output, Activation kind, float sc
                        p.error_word, p.stream));
 }
 void HipGraph::multiply(GpuView input, GpuView gate, GpuView output, bool sigmoid_gate) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_multiply");
     const uint64_t count = floats(input);
     require(floats(gate) == count && floats(output) == count, "graph multiplication shape mismatch");
     check(tsp_multiply(reinterpret_cast<const float*>(p.device(input)), reinterpret_cast<const float*>(p.device(gate)),
                        reinterpret_cast<float*>(p.device(output, true)), count, sigmoid_gate, p.error_word, p.stream));
 }
 void HipGraph::residual_read(GpuView normalized, GpuView scores, GpuView inject, GpuView output, GpuView scales, uint32_t branches, uint32_t channels) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_residual_read");
     require(branches && branches <= 64 && channels && channels <= 65536 && floats(normalized) == checked_mul(branches, channels) &&
                 floats(scores) == floats(normalized) && floats(inject) == branches && floats(output) == channels && floats(scales) == branches,
             "graph residual-read shape mismatch");
@@ -437,7 +575,7 @@ void HipGraph::residual_read(GpuView normalized, GpuView scores, GpuView inject,
                             reinterpret_cast<float*>(p.device(scales, true)), branches, channels, p.error_word, p.stream));
 }
 void HipGraph::residual_write(GpuView streams, GpuView input, GpuView scales, GpuView destination) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_residual_write");
     const uint64_t channels = floats(input), branches = floats(scales);
     require(branches && branches <= 64 && channels && channels <= 65536 && floats(streams) == checked_mul(branches, channels) && floats(destination) == floats(streams),
             "graph residual-write shape mismatch");
@@ -462,7 +600,7 @@ void HipGraph::prepare_moe_router_f32_batch() {
     p.router_batch_prepared = true;
 }
 void HipGraph::moe_router_f32_batch(GpuView matrix, GpuRowsF32 input, GpuRowsF32 output) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active(moe_router_f32_kernel, uint32_t(-1), {input.columns, output.columns, input.rows, 0});
     require(p.router_batch && p.router_batch_prepared, "router FP32 batch requires explicit idle selection/preparation and direct batches");
     require(input.rows == output.rows, "router FP32 batch row count mismatch");
     const auto plan = moe_router_f32_plan(input.columns, output.columns, input.rows, input.stride_bytes, output.stride_bytes, false);
@@ -481,7 +619,7 @@ void HipGraph::prepare_q8_matvec_many(uint32_t width) {
 }
 
 void HipGraph::q8_matvec_many(GpuView matrix, GpuView input, GpuView output, uint32_t columns, uint32_t rows, uint32_t width) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_q8_matvec_many", uint32_t(-1), {columns, rows, width, 0});
     require(input.bytes == uint64_t(columns) * width * 4 && output.bytes == uint64_t(rows) * width * 4, "Q8-many vector byte span mismatch");
     validate_disjoint(std::array{matrix, input}, std::array{output});
     check(tsp_q8_matvec_many(TSP_LAYOUT_GGUF, p.device(matrix), matrix.bytes, reinterpret_cast<const float*>(p.device(input)),
@@ -489,7 +627,7 @@ void HipGraph::q8_matvec_many(GpuView matrix, GpuView input, GpuView output, uin
 }
 
 void HipGraph::route(GpuView logits, GpuView indices, GpuView weights, uint32_t selected, RouterMode mode, bool normalize_selected) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_route");
     require(logits.bytes % 4 == 0 && logits.bytes / 4 <= 4096 && indices.bytes == uint64_t(selected) * 4 && weights.bytes == uint64_t(selected) * 4,
             "graph router shape/mode mismatch");
     validate_disjoint(std::array{logits}, std::array{indices, weights});
@@ -500,7 +638,7 @@ void HipGraph::route(GpuView logits, GpuView indices, GpuView weights, uint32_t 
 
 void HipGraph::prefill_route_batch(GpuView logits, GpuView indices, GpuView weights, uint32_t experts, uint32_t selected, uint32_t tokens,
                                    RouterMode mode, bool normalize_selected) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_route_batch", uint32_t(-1), {experts, selected, tokens, uint32_t(mode)});
     require(logits.bytes == checked_mul(checked_mul(tokens, experts), 4) && indices.bytes == checked_mul(checked_mul(tokens, selected), 4) &&
                 weights.bytes == indices.bytes,
             "prefill route batch geometry/mode mismatch");
@@ -512,7 +650,7 @@ void HipGraph::prefill_route_batch(GpuView logits, GpuView indices, GpuView weig
 
 void HipGraph::routed_gemv(uint32_t encoding, GpuView matrices, GpuView indices, GpuView input, GpuView output, uint32_t columns, uint32_t rows,
                            uint32_t experts, bool broadcast_input) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_routed_gemv", encoding, {columns, rows, experts, 0});
     require(indices.bytes % 4 == 0 && indices.bytes >= 4, "routed GEMV index span mismatch");
     const uint32_t selected = uint32_t(indices.bytes / 4);
     require(input.bytes == uint64_t(columns) * 4 * (broadcast_input ? 1 : selected) && output.bytes == uint64_t(rows) * 4 * selected,
@@ -524,7 +662,7 @@ void HipGraph::routed_gemv(uint32_t encoding, GpuView matrices, GpuView indices,
 }
 
 void HipGraph::swiglu(GpuView gate, GpuView up, GpuView output, float scale) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_swiglu", uint32_t(-1), {uint32_t(gate.bytes / 4), 0, 0, 0});
     require(gate.bytes == up.bytes && gate.bytes == output.bytes && gate.bytes % 4 == 0 && gate.bytes > 0, "graph SwiGLU shape/scale mismatch");
     (void)p.allocation(gate); (void)p.allocation(up);
     check(tsp_swiglu(reinterpret_cast<const float*>(p.device(gate)), reinterpret_cast<const float*>(p.device(up)),
@@ -532,7 +670,7 @@ void HipGraph::swiglu(GpuView gate, GpuView up, GpuView output, float scale) {
 }
 
 void HipGraph::mixture(GpuView expert_outputs, GpuView weights, GpuView shared_output, GpuView shared_logit, GpuView output) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_mixture");
     require(output.bytes % 4 == 0 && output.bytes > 0 && weights.bytes % 4 == 0 && weights.bytes > 0 && shared_output.bytes == output.bytes &&
                 shared_logit.bytes == 4 && expert_outputs.bytes == checked_mul(output.bytes, weights.bytes / 4),
             "mixture shape mismatch");
@@ -543,7 +681,7 @@ void HipGraph::mixture(GpuView expert_outputs, GpuView weights, GpuView shared_o
 }
 
 void HipGraph::prefill_mixture_batch(GpuView experts, GpuView weights, GpuView shared, GpuView shared_logit, GpuRowsF32 output, uint32_t selected) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_mixture_batch", uint32_t(-1), {output.columns, selected, output.rows, 0});
     p.rows_fit(output, "mixture shape mismatch");
     const uint64_t tokens = output.rows, channels = output.columns;
     require(selected >= 1 && experts.bytes == checked_mul(checked_mul(tokens * selected, channels), 4) && weights.bytes == tokens * selected * 4 &&
@@ -562,7 +700,7 @@ struct PlanarTriple { PlanarMatrixShape lo, hi, dn; };
 
 void HipGraph::planar_moe_gate_up_swiglu_m8(GpuView pair_lo, GpuView pair_hi, GpuView indices, GpuRowsF32 input, GpuRowsF32 expert_hidden,
                                             uint32_t experts, uint32_t selected) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("planar_moe_gate_up_swiglu_m8", uint32_t(-1), {input.columns, expert_hidden.columns, experts, input.rows});
     const PlanarEntry* lo = p.planar_of(pair_lo);
     const PlanarEntry* hi = p.planar_of(pair_hi);
     require(lo && hi && p.union_meta, "planar v3 MoE requires registered matrices and prepare_planar_moe_v3");
@@ -586,7 +724,7 @@ void HipGraph::planar_moe_gate_up_swiglu_m8(GpuView pair_lo, GpuView pair_hi, Gp
 
 void HipGraph::planar_moe_routed_m8(GpuView pair_lo, GpuView pair_hi, GpuView down_weights, GpuView indices, GpuRowsF32 input,
                                     GpuRowsF32 expert_hidden, GpuRowsF32 expert_down, uint32_t experts, uint32_t selected) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("planar_moe_routed_m8", uint32_t(-1), {input.columns, expert_down.columns, experts, input.rows});
     const PlanarEntry* lo = p.planar_of(pair_lo);
     const PlanarEntry* hi = p.planar_of(pair_hi);
     const PlanarEntry* dn = p.planar_of(down_weights);
@@ -616,7 +754,7 @@ void HipGraph::planar_moe_routed_m8(GpuView pair_lo, GpuView pair_hi, GpuView do
 void HipGraph::planar_nax_grouped_moe(GpuView pair_lo, GpuView pair_hi, GpuView down_weights, GpuView indices, GpuRowsF32 input,
                                       GpuRowsF32 expert_down, GpuView token_map, GpuView counts, GpuView tasks, uint32_t experts,
                                       uint32_t selected, const SharedPlanarExpert* shared) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("planar_nax_grouped_moe", uint32_t(-1), {input.columns, expert_down.columns, experts, input.rows});
     const PlanarEntry* lo = p.planar_of(pair_lo);
     const PlanarEntry* hi = p.planar_of(pair_hi);
     const PlanarEntry* dn = p.planar_of(down_weights);
@@ -683,7 +821,7 @@ void HipGraph::prepare_grouped_mm(uint32_t encoding, PrefillWeightLayout layout,
 
 void HipGraph::grouped_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView matrices, GpuView indices, GpuRowsF32 input, GpuRowsF32 output,
                           GpuView token_map, GpuView counts, GpuView tasks, uint32_t experts, uint32_t selected, bool broadcast) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_grouped_mm", encoding, {input.columns, output.columns, experts, input.rows});
     require(p.grouped_workspace, "grouped prefill requires idle preparation and direct batches");
     require(selected && output.rows % selected == 0, "grouped prefill route-row count mismatch");
     const uint32_t tokens = output.rows / selected;
@@ -704,7 +842,7 @@ void HipGraph::grouped_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView
 }
 
 void HipGraph::dense_mm(uint32_t encoding, PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_dense_mm", encoding, {input.columns, output.columns, 1, input.rows});
     require(p.dense_workspace, "dense dequant-GEMM requires prepare_dense_mm");
     p.rows_fit(input, "dense dequant-GEMM geometry");
     p.rows_fit(output, "dense dequant-GEMM geometry");
@@ -727,7 +865,7 @@ void HipGraph::prepare_dense_mm_q8(PrefillWeightLayout layout, uint32_t max_toke
 }
 
 void HipGraph::dense_mm_q8(PrefillWeightLayout layout, GpuView matrix, GpuRowsF32 input, GpuRowsF32 output, bool) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("graph_dense_mm_q8", 8, {input.columns, output.columns, input.rows, uint32_t(layout)});
     require(layout == PrefillWeightLayout::gguf || layout == PrefillWeightLayout::q8_lanes_v1, "dense Q8_0 GEMM layout");
     p.rows_fit(input, "dense Q8_0 GEMM geometry");
     p.rows_fit(output, "dense Q8_0 GEMM geometry");
@@ -774,7 +912,7 @@ void HipGraph::prepare_logit_topk() {
 }
 
 void HipGraph::logit_topk(GpuRowsF32 logits, GpuView partial_scratch, GpuView out_rows) {
-    auto& p = *impl_; p.active();
+    auto& p = *impl_; p.active("logit_topk", uint32_t(-1), {logits.rows, logits.columns, 0, 64});
     require(p.topk_prepared, "GPU logit top-k requires prepared direct batches");
     p.rows_fit(logits, "GPU logit top-k geometry mismatch");
     validate_disjoint(std::array{logits.view}, std::array{partial_scratch, out_rows});

@@ -16,6 +16,7 @@
 #pragma once
 
 #include <array>
+#include <cmath>
 #include <cstddef>
 #include <cstdint>
 #include <memory>
@@ -60,6 +61,35 @@ struct GraphMemory {
     uint64_t live_bytes = 0;
     uint64_t peak_bytes = 0;
     uint64_t allocations = 0;
+    uint64_t profile_counter_payload_bytes = 0;  // what configure_profiling holds, part of live_bytes
+};
+// include/tokspur/graph.hpp:337-344,353-359,386-400: opt-in timing of every operator of a batch. A row of `kernels` is one
+// operator call, in encoding order: the label the engine gives that operator's kernel where it has a single one, the
+// operator's own name where it launches several, and the engine's encoding / shape metadata. `start` and `end` are
+// nanoseconds on the GPU's event clock counted from the batch's first boundary (+ 1, so that a sample is never zero), hence
+// gpu_tick_nanoseconds is 1 in a calibrated profile. Calibration compares the GPU's span of the batch with steady_clock's
+// between begin() and the return of submit(): a short batch can miss the 3 % tolerance through submission latency alone;
+// its raw samples are kept, its milliseconds are NaN, and the batch itself never fails on that account.
+enum class ProfileMode { disabled, dispatch_boundary, encoder_boundary };
+inline bool profile_calibration_valid(double tick_nanoseconds, double mismatch_fraction) {
+    return std::isfinite(tick_nanoseconds) && tick_nanoseconds > 0 && std::isfinite(mismatch_fraction) && mismatch_fraction >= 0 &&
+           mismatch_fraction <= 0.03;
+}
+struct KernelTiming {
+    std::string kernel;
+    uint32_t encoding;
+    std::array<uint32_t, 4> shape;
+    uint64_t start, end;
+    double milliseconds;
+};
+struct GraphProfile {
+    ProfileMode mode = ProfileMode::disabled;
+    bool timings_valid = false;
+    bool cpu_clock_is_mach = false;
+    double gpu_tick_nanoseconds = 0;
+    double cpu_clock_mismatch_fraction = 0;
+    double sampled_milliseconds = 0;
+    std::vector<KernelTiming> kernels;
 };
 // include/tokspur/graph.hpp:270-275
 struct BatchResult {
@@ -99,6 +129,12 @@ public:
     void read(GpuView source, std::span<std::byte> destination) const;
     void release(GpuView full_buffer);
     [[nodiscard]] GraphMemory memory() const;
+    // graph.hpp:503,528. Idle only; zero disables; at most 16384 operators per batch. The boundary events are charged to the
+    // byte budget (16 bytes per operator in whole pages per 2048 operators, the engine's accounting) and a request beyond the
+    // budget is refused with nothing changed. An operator past the capacity is refused while encoding. last_profile() is the
+    // last successfully submitted batch's; begin(), abort() and a batch refused for a device error leave it empty.
+    ProfileMode configure_profiling(uint32_t max_dispatches);
+    [[nodiscard]] const GraphProfile& last_profile() const;
     [[nodiscard]] std::string device_name() const;
     void validate_disjoint(std::span<const GpuView> inputs, std::span<const GpuView> destinations) const;  // graph.hpp:671
 
@@ -188,6 +224,31 @@ private:
     struct Impl;
     std::unique_ptr<Impl> impl_;
 };
+
+// ---- include/tokspur/grouped_mm.hpp:8-26: the argument block (56 bytes, as the engine's kernels take it) and the pure
+// geometry / byte-bound planners of grouped_mm and dense_mm_q8. They refuse what the engine refuses, with FormatError and the
+// engine's wording; `threads` / `threadgroup_bytes` are the engine's launch constants, kept so that callers that print a plan
+// compile unchanged.
+struct GroupedMmArgs {
+    uint32_t columns, rows, row_bytes, experts;
+    uint32_t selected, tokens, broadcast, maximum_tasks;
+    uint64_t expert_stride_bytes, input_stride_bytes, output_stride_bytes;
+};
+static_assert(sizeof(GroupedMmArgs) == 56, "GroupedMmArgs ABI");
+struct GroupedMmPlan {
+    GroupedMmArgs args{};
+    uint64_t matrix_bytes = 0, indices_bytes = 0, input_bytes = 0, output_bytes = 0;
+    uint64_t token_map_bytes = 0, counts_bytes = 0, tasks_bytes = 0;
+    uint32_t grid_x = 0, grid_y = 0, threads = 128, threadgroup_bytes = 8192;
+    const char* kernel = nullptr;
+};
+GroupedMmPlan grouped_mm_plan(uint32_t encoding, PrefillWeightLayout layout, uint32_t columns, uint32_t rows, uint32_t experts,
+                              uint32_t selected, uint32_t tokens, uint64_t input_stride_bytes, uint64_t output_stride_bytes, bool broadcast,
+                              bool allow_nax_2k = false);
+GroupedMmPlan dense_mm_q8_plan(PrefillWeightLayout layout, uint32_t columns, uint32_t rows, uint32_t tokens, uint64_t input_stride_bytes,
+                               uint64_t output_stride_bytes, bool allow_nax_2k = false);
+const char* grouped_mm_kernel(uint32_t encoding, PrefillWeightLayout layout);
+const char* dense_mm_q8_kernel(PrefillWeightLayout layout);
 
 // ---- the MoE sublayer for one token, include/tokspur/moe.hpp:9-45, src/moe.cpp:13-83
 struct GpuMatrix { GpuView view; uint32_t encoding; };
