@@ -241,9 +241,15 @@ int tsp_swiglu(const float* gate, const float* up, float* output, uint64_t count
 
 /* ------------------------------------------------------------------ device: the f32 operators around the sublayer */
 
+/* What a destination holds after a batch these operators refused is what the engine's holds (kernels/graph.metal:18-21
+ * `checked_store`): a non-finite RESULT sets TSP_ERRBIT_NONFINITE and is stored; where an operator tests its operands first
+ * (a group's sum of squares in rms, the normalised value and the gate in rms_sigmoid_gate, both factors in multiply, the
+ * branch values, scores and inject logits in residual_read) a non-finite operand sets the bit and that element, group or
+ * thread stores nothing. */
+
 /* include/tokspur/graph.hpp:983 `rms` (src/graph.mm:7399-7409; kernels/graph.metal:222-247): independent groups of `group_width`
  * values, out = x * rsqrt(mean(x^2) + epsilon) * gain; `gains` holds one gain per element, or `group_width` gains shared by
- * every group (shared_gains). A non-finite sum or result sets TSP_ERRBIT_NONFINITE and is not stored. */
+ * every group (shared_gains). */
 int tsp_rms(const float* input, const float* gains, float* output, uint64_t count, uint32_t group_width, int shared_gains, float epsilon,
             uint32_t* error_word, void* stream);
 /* include/tokspur/graph.hpp:984 `rms_sigmoid_gate` (kernels/graph.metal:249-282): the same times sigmoid(gate), in one pass. */

@@ -53,6 +53,21 @@ def test_routed_m8_reference_cases(gpu, tsp, orc, gu, dn):
         assert np.array_equal(only_h.cpu().numpy(), h.cpu().numpy())
 
 
+@pytest.mark.parametrize("dn,hidden", [(7, 160), (8, 96)])
+@pytest.mark.parametrize("tokens", [2, 5, 8])
+def test_routed_m8_2048_columns_narrow_experts(gpu, tsp, orc, dn, hidden, tokens):
+    """Experts of 2048 columns whose hidden width is no multiple of 128 (five and three 32-unit tiles) on the kernel that keeps
+    the step's token rows resident: the share split by 32-unit tiles and the hand-off to a Q5_1 / Q8_0 down product."""
+    channels, experts, selected = 2048, 8, 3
+    gate, up, down, w = build(tsp, gpu, orc, 12, dn, channels, hidden, experts)
+    x = lcg_inputs(555 + tokens * 17 + hidden, tokens * channels).reshape(tokens, channels)
+    ids = np.array([[(t * 2 + s * 3) % experts for s in range(selected)] for t in range(tokens)], dtype=np.uint32).reshape(-1)
+    h, y = tsp.planar_moe_routed_m8(gpu, w, gpu.upload(ids), gpu.upload(x), tokens, selected)
+    ref_h, ref_y = orc.moe_routed_reference(12, dn, gate, up, down, channels, hidden, experts, ids, tokens, selected, x, threads=4)
+    assert nmse(h.cpu().numpy(), ref_h) <= 1e-6 and nmse(y.cpu().numpy(), ref_y) <= 1e-6
+    assert gpu.error() == 0
+
+
 @pytest.mark.parametrize("gu,dn", [(12, 7), (8, 8)])
 def test_routed_m8_all_singletons(gpu, tsp, orc, gu, dn):
     # native/tests/test_planar_pack_v3.cpp:553-627: 32 experts, every route a distinct expert, hidden = 416 (13 blocks).

@@ -333,12 +333,13 @@ def test_rms_activate_multiply(gpu, orc, tsp):
     y = gpu.multiply(gpu.upload(x), gpu.upload(x[::-1].copy())).cpu().numpy()
     assert np.array_equal(y, x * x[::-1])
     assert gpu.error() == 0
-    # error contract: a non-finite input raises the flag and leaves its destination alone; refusals on the host
+    # error contract (kernels/graph.metal:18-21, 284-311): activate stores the non-finite operand itself and raises the flag;
+    # multiply tests its operands first and leaves that destination alone; refusals on the host
     bad = x.copy()
     bad[3] = np.inf
     out = gpu.full(bad.size, -5.0)
     gpu.activate(gpu.upload(bad), 2, out=out)
-    assert gpu.error() == 1 and out.cpu().numpy()[3] == -5.0 and out.cpu().numpy()[4] != -5.0
+    assert gpu.error() == 1 and out.cpu().numpy()[3] == np.inf and out.cpu().numpy()[4] != -5.0
     out = gpu.full(bad.size, -5.0)
     gpu.multiply(gpu.upload(x), gpu.upload(bad), out=out)
     assert gpu.error() == 1 and out.cpu().numpy()[3] == -5.0
@@ -351,3 +352,64 @@ def test_rms_activate_multiply(gpu, orc, tsp):
                  lambda: gpu.activate(d, 4), lambda: gpu.activate(d, 1, float("inf")), lambda: gpu.residual_read(d, d, d, 65, 4), lambda: gpu.residual_write(d, d, d, 2, 70000)):
         with pytest.raises(tsp.FormatError):
             call()
+
+
+def test_destination_contents_after_a_refused_batch(gpu, tsp):
+    """kernels/graph.metal:18-21 `checked_store` stores a non-finite result and raises the flag; the operators that test their
+    operands first (graph.metal:258-311, 340-347) raise it and store nothing for that element. A caller that looks at its
+    buffers after a refused batch finds what the engine leaves there, in place forms included."""
+    inf, nan = np.float32(np.inf), np.float32(np.nan)
+    x = np.array([1.0, inf, -2.0, nan, 0.5, -inf, 3.0, 4.0], dtype=np.float32)
+    for kind in (0, 1, 2, 3):  # activate: the scaled operand itself is what lands, never sigmoid(inf) = 1
+        buf = gpu.upload(x)
+        gpu.activate(buf, kind, 1.0, out=buf)
+        got = buf.cpu().numpy()
+        assert gpu.error() == tsp.ERRBIT_NONFINITE
+        gpu.clear_error()
+        assert got[1] == inf and np.isnan(got[3]) and got[5] == -inf and np.isfinite(got[[0, 2, 4, 6, 7]]).all()
+    gate = np.array([1.0, 1.0, inf, 1.0, 2.0, 1.0, 1.0, 3e38], dtype=np.float32)
+    big = np.array([1.0, 2.0, 3.0, 4.0, 5.0, 6.0, 7.0, 3e38], dtype=np.float32)
+    out = gpu.full((8,), -9.0)
+    gpu.multiply(gpu.upload(big), gpu.upload(gate), False, out=out)
+    got = out.cpu().numpy()
+    assert gpu.error() == tsp.ERRBIT_NONFINITE
+    gpu.clear_error()
+    assert got[2] == -9.0 and got[7] == inf and got[4] == 10.0  # bad operand: untouched; overflowing product: stored
+    buf = gpu.upload(x)
+    gpu.multiply(buf, gpu.upload(np.ones(8, dtype=np.float32)), False, out=buf)  # in place: the bad elements stay what they were
+    got = buf.cpu().numpy()
+    gpu.clear_error()
+    assert got[1] == inf and np.isnan(got[3]) and got[0] == 1.0
+    # rms: a group whose sum of squares is not finite stores nothing; a finite group beside it is normalised
+    groups = np.array([1.0, 2.0, inf, 4.0, 3.0, 4.0, 0.0, 0.0], dtype=np.float32)
+    out = gpu.full((8,), -9.0)
+    gpu.rms(gpu.upload(groups), gpu.upload(np.ones(4, dtype=np.float32)), 4, 1e-6, out=out)
+    got = out.cpu().numpy()
+    assert gpu.error() == tsp.ERRBIT_NONFINITE
+    gpu.clear_error()
+    assert (got[:4] == -9.0).all() and abs(got[4] - 3.0 / np.sqrt(6.25)) <= 1e-6
+    # rms_sigmoid_gate: a non-finite gate skips its element only
+    out = gpu.full((4,), -9.0)
+    gpu.rms(gpu.upload(np.array([3.0, 4.0, 0.0, 0.0], dtype=np.float32)), gpu.upload(np.ones(4, dtype=np.float32)), 4, 1e-6,
+            gate=gpu.upload(np.array([0.0, nan, 0.0, 0.0], dtype=np.float32)), out=out)
+    got = out.cpu().numpy()
+    assert gpu.error() == tsp.ERRBIT_NONFINITE
+    gpu.clear_error()
+    assert got[1] == -9.0 and abs(got[0] - 0.5 * 3.0 / np.sqrt(6.25)) <= 1e-6
+    # residual_read: the thread of a bad channel writes neither its channel nor the scale of the same index
+    branches, channels = 2, 3
+    normalized = np.array([[1.0, inf, 3.0], [1.0, 1.0, 1.0]], dtype=np.float32)
+    scores = np.zeros((branches, channels), dtype=np.float32)
+    read, scales = gpu.full((channels,), -9.0), gpu.full((branches,), -7.0)
+    gpu.residual_read(gpu.upload(normalized), gpu.upload(scores), gpu.upload(np.zeros(branches, dtype=np.float32)), branches, channels, out=read, scales=scales)
+    got, got_s = read.cpu().numpy(), scales.cpu().numpy()
+    assert gpu.error() == tsp.ERRBIT_NONFINITE
+    gpu.clear_error()
+    assert got[0] == 0.5 and got[1] == -9.0 and got[2] == 1.0 and got_s[0] == 1.0 and got_s[1] == -7.0
+    # residual_write: an overflowing sum is stored
+    streams = np.array([3e38, 1.0], dtype=np.float32)
+    written = gpu.residual_write(gpu.upload(streams), gpu.upload(np.array([3e38, 1.0], dtype=np.float32)), gpu.upload(np.array([1.0], dtype=np.float32)), 1, 2)
+    got = written.cpu().numpy()
+    assert gpu.error() == tsp.ERRBIT_NONFINITE
+    gpu.clear_error()
+    assert got[0] == inf and got[1] == 2.0

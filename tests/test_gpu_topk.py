@@ -53,6 +53,19 @@ def test_topk_refusals(gpu, tsp):
     assert tsp.logit_topk_scratch_bytes(16, 151936) == 16 * 38 * 528 and tsp.logit_topk_output_bytes(16) == 16 * 528
 
 
+def check_sampled_logits(orc, w, x, logits, columns, vocabulary, seed, what, samples=2048):
+    """GPU logits of `samples` random vocabulary rows, plus the first and the last, against `reference_gemv` for every token row."""
+    row_bytes = columns // 32 * 34
+    sel = np.unique(np.concatenate([np.random.default_rng(seed).choice(vocabulary, size=samples, replace=False), [0, vocabulary - 1]]))
+    sub = np.ascontiguousarray(w.reshape(vocabulary, row_bytes)[sel]).reshape(-1)
+    worst = 0.0
+    for r in range(x.shape[0]):
+        ref = orc.reference_gemv(8, sub, columns, len(sel), x[r])
+        worst = max(worst, float(np.max(np.abs(ref - logits[r, sel]) / np.maximum(1.0, np.abs(ref)))))
+    print(f"{what}: {len(sel)} sampled vocabulary rows x {x.shape[0]} token rows, reference metric {worst:.2e}")
+    assert worst <= 5e-5
+
+
 def test_config4_lm_head_argmax(gpu, tsp, orc, synth):
     """BASELINE config 4 at full size for M = 1, 4, 8, 16: Q8_0 LM head 151 936 x 2048 -> logits -> top-64 rows.
     The arg-max (rank 0) is compared with the CPU arg-max of the same GPU logits bit for bit, and with the arg-max of the
@@ -80,7 +93,9 @@ def test_config4_lm_head_argmax(gpu, tsp, orc, synth):
             want = orc.logit_topk_row(logits[r])
             assert np.array_equal(rows[r]["ids"], np.array(want.ids, dtype=np.uint32)) and rows[r]["count"] == 64
             assert rows[r]["ids"][0] == int(np.argmax(logits[r]))
-        # the reference logits for the top candidates of row 0 (a full CPU GEMV is 3e8 multiply-adds per row)
+        # reference logits of 2048 random vocabulary rows (and the first and last one) for EVERY token row, the engine's
+        # |a - e| / max(1, |e|) <= 5e-5 (native/tools/ffn_check.cpp:48-56); a full CPU GEMV is 3e8 multiply-adds per row
+        check_sampled_logits(orc, w, x, logits, C, V, seed=40 + m, what=f"config4 M={m} raw rows")
         cand = rows[0]["ids"][:8].astype(np.int64)
         ref = np.array([orc.reference_gemv(8, w[int(c) * (C // 32) * 34:(int(c) + 1) * (C // 32) * 34], C, 1, x[0])[0] for c in cand])
         assert np.max(np.abs(ref - rows[0]["logits"][:8]) / np.maximum(1.0, np.abs(ref))) <= 5e-5
@@ -100,6 +115,7 @@ def test_config4_lm_head_argmax(gpu, tsp, orc, synth):
         assert gpu.error() == 0
         a, b = raw_rows.cpu().numpy(), lane_rows.cpu().numpy()
         assert float(np.max(np.abs(a - b) / np.maximum(1.0, np.abs(a)))) <= 5e-5
+        check_sampled_logits(orc, w, x, b, C, V, seed=90 + m, what=f"config4 M={m} q8_lanes_v1 rows")
         top = tsp.logit_topk(gpu, lane_rows, m, V).cpu().numpy().view(tsp.TOPK_ROW_DTYPE)
         for r in range(m):
             assert top[r]["ids"][0] == int(np.argmax(b[r]))

@@ -23,9 +23,13 @@ def test_static_scratch_topk_matches_the_scratch_argument_form(gpu, tsp, orc):
         logits = _rows(seed, rows, vocab)
         d = gpu.upload(logits)
         out = gpu.empty(tsp.logit_topk_output_bytes(rows), "uint8")
-        before = torch.cuda.memory_allocated()
+        torch.cuda.synchronize()
+        # device-wide free bytes, not torch's own counter: a hipMalloc inside the library would not move the latter. The first
+        # call on a device looks the array's address up (no allocation either: the array is part of the loaded code object).
+        before, reserved = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
         tsp.logit_topk_static(gpu, d, rows, vocab, out=out)
-        assert torch.cuda.memory_allocated() == before
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == before and torch.cuda.memory_reserved() == reserved
         got = out.cpu().numpy().view(tsp.TOPK_ROW_DTYPE)
         ref = tsp.logit_topk(gpu, d, rows, vocab).cpu().numpy().view(tsp.TOPK_ROW_DTYPE)
         for name in fields:
@@ -36,6 +40,37 @@ def test_static_scratch_topk_matches_the_scratch_argument_form(gpu, tsp, orc):
             assert got[r]["first_nonfinite_col"] == want.first_nonfinite_col and got[r]["first_subnormal_col"] == want.first_subnormal_col
             assert np.array_equal(got[r]["ids"], np.array(want.ids, dtype=np.uint32))
             assert np.array_equal(got[r]["logits"].view(np.uint32), np.array(want.logits, dtype=np.float32).view(np.uint32))
+
+
+def test_static_scratch_topk_under_stream_capture(gpu, tsp, orc):
+    """The use the entry point is for: after one eager call on the device, a call recorded into a HIP graph and replayed.
+    Every replay, with new logits copied in between and eager work of the program's own around it, gives the rows of
+    `tsp_logit_topk` bit for bit."""
+    import torch
+    fields = ("vocabulary", "count", "first_nonfinite_col", "first_subnormal_col", "ids", "logits")
+    rows, vocab = 4, 40000
+    d = gpu.upload(_rows(10, rows, vocab))
+    out = gpu.empty(tsp.logit_topk_output_bytes(rows), "uint8")
+    tsp.logit_topk_static(gpu, d, rows, vocab, out=out)  # eager: the address look-up happens here, outside capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        tsp.logit_topk_static(gpu, d, rows, vocab, out=out)
+    for replay in range(4):
+        logits = _rows(20 + replay, rows, vocab)
+        d.copy_(gpu.upload(logits))
+        out.fill_(0xEE)
+        torch.cuda.synchronize()
+        free = torch.cuda.mem_get_info()[0]
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free
+        got = out.cpu().numpy().view(tsp.TOPK_ROW_DTYPE)
+        ref = tsp.logit_topk(gpu, d, rows, vocab).cpu().numpy().view(tsp.TOPK_ROW_DTYPE)
+        for name in fields:
+            assert np.array_equal(got[name].view(np.uint32), ref[name].view(np.uint32)), (replay, name)
+        want = orc.logit_topk_row(logits[0])
+        assert np.array_equal(got[0]["ids"], np.array(want.ids, dtype=np.uint32))
 
 
 def test_static_scratch_topk_refuses_what_does_not_fit(gpu, tsp):

@@ -353,8 +353,9 @@ class Device:
         check(dll().tsp_multiply(self.ptr(x), self.ptr(gate), self.ptr(out), C.c_uint64(x.numel()), C.c_int(bool(sigmoid_gate)), self.ptr(self.err), self.stream()))
         return out
 
-    def residual_read(self, normalized, scores, inject, branches, channels):
-        out, scales = self.empty(channels), self.empty(branches)
+    def residual_read(self, normalized, scores, inject, branches, channels, out=None, scales=None):
+        out = self.empty(channels) if out is None else out
+        scales = self.empty(branches) if scales is None else scales
         check(dll().tsp_residual_read(self.ptr(normalized), self.ptr(scores), self.ptr(inject), self.ptr(out), self.ptr(scales), C.c_uint32(branches),
                                       C.c_uint32(channels), self.ptr(self.err), self.stream()))
         return out, scales

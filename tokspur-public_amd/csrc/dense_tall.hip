@@ -394,10 +394,11 @@ int launch_dense_tall(const DenseTallArgs& a, hipStream_t s) {
     static std::atomic<uint64_t> seen{0};
     static int units[64];
     int device = 0;
-    if (first_use_on_device(seen, &device) || units[device] == 0) {
+    if (setup_pending(seen, &device)) {
         int n = 0;
         TSP_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device));
         units[device] = n >= 1 ? n : 1;
+        setup_done(seen, device);
     }
     // 256-row tiles only where one round of them keeps nearly every compute unit busy (2048 x 8192 results on 256 units): there
     // they are a few percent faster. Elsewhere 128-row tiles, two workgroups to a unit, lose less to the last, partly filled

@@ -425,10 +425,11 @@ int launch_resident_down(const ResidentDownArgs& a, hipStream_t s) {
     static std::atomic<uint64_t> seen{0};
     static int cus[64];
     int device = 0;
-    if (first_use_on_device(seen, &device) || cus[device] == 0) {
+    if (setup_pending(seen, &device)) {
         int n = 0;
         TSP_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device));
         cus[device] = n >= 8 ? n / 8 * 8 : 8;
+        setup_done(seen, device);
     }
     if (a.spec.source_type == kQ6) TSP_LAUNCH("gemm_down", s, down_resident_kernel<kQ6><<<cus[device], kThreads, 0, s>>>(a));
     else if (a.spec.source_type == kQ8) TSP_LAUNCH("gemm_down", s, down_resident_kernel<kQ8><<<cus[device], kThreads, 0, s>>>(a));

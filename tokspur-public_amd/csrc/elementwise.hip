@@ -1,7 +1,9 @@
 // The small f32 operators that sit either side of the MoE sublayer in a layer (kernels/graph.metal:222-361): grouped RMS
 // normalisation (alone and fused with a sigmoid gate), activations, gated multiplication, and the read / write of the gated
 // residual streams. All are a few bytes per element and bound by memory or by launch latency; they follow the engine's error
-// contract: a non-finite input or result sets the sticky bit, and the value is not stored.
+// contract: a non-finite result sets the sticky bit and is stored all the same (kernels/graph.metal:18-21), so after a refused
+// batch a destination holds what the engine's holds; a non-finite INPUT of the operators that test their inputs first
+// (multiply, the gated RMS, residual_read) sets the bit and leaves that element of the destination as it was.
 #include "tsp_common.hpp"
 
 using namespace tsp;
@@ -19,11 +21,10 @@ __device__ __forceinline__ float softplus_value(float x) {
     // log1p by compensation: 1 + z rounds, (sum - 1) is what was actually added; a sum that rounds to 1 keeps its tiny tail
     return fmaxf(x, 0.0f) + (sum == 1.0f ? z : logf(sum) * (z / (sum - 1.0f)));
 }
-// a finite value is stored; anything else raises the flag and leaves the destination as it was
+// kernels/graph.metal:18-21: the value is stored whatever it is; a non-finite one raises the flag as well
 __device__ __forceinline__ uint32_t checked_store(float* out, uint64_t i, float v) {
-    if (nonfinite(v)) return TSP_ERRBIT_NONFINITE;
     out[i] = v;
-    return 0;
+    return nonfinite(v) ? TSP_ERRBIT_NONFINITE : 0u;
 }
 
 // One wave per group of `width` values: out = x * rsqrt(mean(x^2) + eps) * gain, gains per element or shared by all groups;
@@ -85,9 +86,9 @@ __global__ __launch_bounds__(256) void residual_read_kernel(const float* __restr
                                                             uint32_t branches, uint32_t channels, uint32_t* error_word) {
     const uint32_t channel = blockIdx.x * blockDim.x + threadIdx.x;
     uint32_t bad = 0;
+    bool ok = true;  // a thread that met a non-finite operand writes nothing more, neither its channel nor its scale (graph.metal:340)
     if (channel < channels) {
         float total = 0;
-        bool ok = true;
         for (uint32_t b = 0; b < branches && ok; ++b) {
             const float n = normalised[uint64_t(b) * channels + channel], s = scores[uint64_t(b) * channels + channel];
             if (nonfinite(n) || nonfinite(s)) { bad = TSP_ERRBIT_NONFINITE; ok = false; break; }
@@ -95,7 +96,7 @@ __global__ __launch_bounds__(256) void residual_read_kernel(const float* __restr
         }
         if (ok) bad |= checked_store(output, channel, total / float(branches));
     }
-    if (channel < branches) {
+    if (ok && channel < branches) {
         const float v = inject[channel];
         if (nonfinite(v)) bad = TSP_ERRBIT_NONFINITE;
         else bad |= checked_store(scales, channel, 2.0f * sigmoid_value(v / float(branches)));

@@ -322,10 +322,11 @@ int launch_resident_gate_up(const ResidentGateUpArgs& a, hipStream_t s) {
     static std::atomic<uint64_t> seen{0};
     static int cus[64];
     int device = 0;
-    if (first_use_on_device(seen, &device) || cus[device] == 0) {
+    if (setup_pending(seen, &device)) {
         int n = 0;
         TSP_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device));
         cus[device] = n >= 8 ? n / 8 * 8 : 8;
+        setup_done(seen, device);
     }
     TSP_LAUNCH("gemm_gate_up_swiglu", s, gate_up_resident_kernel<<<cus[device], kThreads, 0, s>>>(a));
     return launch_status("gate_up_resident");

@@ -156,8 +156,11 @@ int launch(uint32_t layout, const Q8Args& a, hipStream_t stream) {
     const uint64_t lds_bytes = uint64_t(M) * (a.columns + 4) * 4;
     if (a.columns % 64 == 0 && reinterpret_cast<uintptr_t>(a.matrix) % 4 == 0 && lds_bytes <= 96 * 1024) {
         static std::atomic<uint64_t> raised{0};  // one per instantiation (M)
-        if (lds_bytes > 48 * 1024 && first_use_on_device(raised))
+        int device = 0;
+        if (lds_bytes > 48 * 1024 && setup_pending(raised, &device)) {
             TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_flat<M>), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+            setup_done(raised, device);
+        }
         TSP_LAUNCH("q8_flat", stream, q8_flat<M><<<grid, 256, lds_bytes, stream>>>(a));
         return launch_status("q8_flat");
     }

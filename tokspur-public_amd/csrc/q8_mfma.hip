@@ -501,12 +501,13 @@ int q8_mfma(const void* matrix, const float* x, float* y, uint32_t columns, uint
     static std::atomic<uint64_t> raised{0};
     static int units_of[64] = {};
     int device = 0;
-    if (first_use_on_device(raised, &device)) {
+    if (setup_pending(raised, &device)) {
         const int most = int(2 * 8 * 2048 * 2 + kWaves * kTileBytes);
         TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<1, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
         TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<2, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
         TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_mfma_kernel<2, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
         TSP_HIP(hipDeviceGetAttribute(&units_of[device], hipDeviceAttributeMultiprocessorCount, device));
+        setup_done(raised, device);
     }
     const int compute_units = units_of[device];
     const uint32_t tiles = (rows + 31) / 32;
@@ -539,11 +540,12 @@ int q8_lanes_mfma(const void* matrix, const float* x, float* y, uint32_t columns
     static std::atomic<uint64_t> raised{0};
     static int units_of[64] = {};
     int device = 0;
-    if (first_use_on_device(raised, &device)) {
+    if (setup_pending(raised, &device)) {
         const int most = int(2 * 8 * 2048 * 2 + kWaves * kLaneTileBytes);
         TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_lanes_mfma_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
         TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_lanes_mfma_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
         TSP_HIP(hipDeviceGetAttribute(&units_of[device], hipDeviceAttributeMultiprocessorCount, device));
+        setup_done(raised, device);
     }
     const int compute_units = units_of[device];
     const uint32_t tiles = (rows + kLaneRows - 1) / kLaneRows;

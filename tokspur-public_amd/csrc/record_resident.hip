@@ -457,10 +457,11 @@ int compute_units(int* out) {
     static std::atomic<uint64_t> seen{0};
     static int cus[64];
     int device = 0;
-    if (first_use_on_device(seen, &device) || cus[device] == 0) {
+    if (setup_pending(seen, &device)) {
         int n = 0;
         TSP_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device));
         cus[device] = n >= 1 ? n : 1;
+        setup_done(seen, device);
     }
     *out = cus[device];
     return TSP_OK;

@@ -148,8 +148,11 @@ extern "C" int tsp_router_f32_batch(const float* weights, const float* input, ui
     const uint64_t w_span = uint64_t(columns) * experts * 4;
     TSP_REQUIRE(!ranges_overlap(output, out_span, input, in_span) && !ranges_overlap(output, out_span, weights, w_span),
                 "router f32 batch output overlaps an input");
-    if (first_use_on_device(g_lds_raised))
+    int device = 0;
+    if (setup_pending(g_lds_raised, &device)) {
         TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(router_f32_gemm), hipFuncAttributeMaxDynamicSharedMemorySize, int(kLdsBytes)));
+        setup_done(g_lds_raised, device);
+    }
     RouterArgs a{};
     a.weights = weights; a.input = input; a.output = output;
     a.input_stride = input_stride_bytes / 4; a.output_stride = output_stride_bytes / 4;

@@ -827,13 +827,15 @@ int launch_flat(const char* name, const SkinnyArgs& a, uint32_t tasks, hipStream
     const uint32_t bpr = a.k / 256, waves = bpr < 4 ? 4 : bpr, ucols = waves / bpr;
     const uint32_t per_group = ucols * (OUT == OUT_SWIGLU ? 32 : 64), col_tiles = (a.n + per_group - 1) / per_group;
     static std::atomic<uint64_t> raised{0};
-    if (first_use_on_device(raised)) {
+    int device = 0;
+    if (setup_pending(raised, &device)) {
         if constexpr (BKIND == B_Q6K_PLANAR)
             TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&flat16_kernel<BKIND, OUT, SRC>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         int(8 * kWaveLds)));
         else
             TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&flat_kernel<BKIND, OUT, SRC>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                         int(8 * kWaveLds)));
+        setup_done(raised, device);
     }
     if constexpr (BKIND == B_Q6K_PLANAR) TSP_LAUNCH(name, s, flat16_kernel<BKIND, OUT, SRC><<<dim3(col_tiles, tasks), waves * kWave, waves * kWaveLds, s>>>(a));
     else TSP_LAUNCH(name, s, flat_kernel<BKIND, OUT, SRC><<<dim3(col_tiles, tasks), waves * kWave, waves * kWaveLds, s>>>(a));
@@ -846,9 +848,12 @@ template <int BKIND, int OUT, int SRC, int KS>
 int launch_sliced(const char* name, const SkinnyArgs& a, uint32_t col_tiles, uint32_t tasks, hipStream_t s) {
     const uint32_t bytes = lds_bytes(a.k, BKIND != B_Q6K_PLANAR);
     static std::atomic<uint64_t> raised{0};
-    if (first_use_on_device(raised))
+    int device = 0;
+    if (setup_pending(raised, &device)) {
         TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&skinny_kernel<BKIND, OUT, SRC, KS>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     int(lds_bytes(kMaxColumns, true))));
+        setup_done(raised, device);
+    }
     TSP_LAUNCH(name, s, skinny_kernel<BKIND, OUT, SRC, KS><<<dim3(col_tiles, tasks), 256 * KS, bytes, s>>>(a));
     return launch_status(name);
 }

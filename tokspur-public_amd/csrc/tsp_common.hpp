@@ -30,15 +30,16 @@ void set_error(const char* fmt, ...);
 
 inline bool mul_overflows(uint64_t a, uint64_t b) { return a && b > UINT64_MAX / a; }
 
-// Per-device set-up (a kernel's dynamic LDS limit is raised on the device that is current): `seen` has one bit per device
-// ordinal; true the first time the current device asks. Two threads racing both run the set-up, which is harmless.
-inline bool first_use_on_device(std::atomic<uint64_t>& seen, int* ordinal = nullptr) {
+// Per-device set-up (a kernel's dynamic LDS limit is raised on the device that is current, its compute units are counted):
+// `done` has one bit per device ordinal, set by setup_done() only AFTER the set-up has run. Two threads that race both run
+// it, which is harmless (the calls are idempotent), and neither launches before it has run.
+inline bool setup_pending(const std::atomic<uint64_t>& done, int* ordinal = nullptr) {
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess || device < 0 || device > 63) device = 0;
     if (ordinal) *ordinal = device;
-    const uint64_t bit = 1ull << device;
-    return (seen.fetch_or(bit, std::memory_order_relaxed) & bit) == 0;
+    return (done.load(std::memory_order_acquire) & (1ull << device)) == 0;
 }
+inline void setup_done(std::atomic<uint64_t>& done, int device) { done.fetch_or(1ull << device, std::memory_order_release); }
 
 inline bool ranges_overlap(const void* a, uint64_t an, const void* b, uint64_t bn) {
     const auto x = reinterpret_cast<uintptr_t>(a), y = reinterpret_cast<uintptr_t>(b);
