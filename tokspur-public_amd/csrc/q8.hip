@@ -208,13 +208,15 @@ extern "C" int tsp_dense_mm_q8(uint32_t layout, const void* matrix, uint64_t mat
     // width sequence of src/q8_many.cpp:20-29); rows with padding between them go one by one.
     const bool packed = input_stride_bytes == uint64_t(columns) * 4 && output_stride_bytes == uint64_t(rows) * 4;
     // Nine or more packed rows left: up to sixteen go through the matrix-core kernel in one pass over the weights.
-    const bool sixteen = packed && layout == TSP_LAYOUT_GGUF && matrix && error_word && columns % 32 == 0 && rows <= 1000000 &&
-                         uint64_t(columns / 32) * rows * 34 == matrix_bytes && q8_mfma_supported_16(matrix, input, output, columns, rows);
+    const bool whole = packed && matrix && error_word && columns % 32 == 0 && rows <= 1000000 && uint64_t(columns / 32) * rows * 34 == matrix_bytes;
+    const bool lanes = layout == TSP_LAYOUT_Q8_LANES_V1;
+    const bool sixteen = whole && (layout == TSP_LAYOUT_GGUF ? q8_mfma_supported_16(matrix, input, output, columns, rows)
+                                                            : lanes && q8_lanes_mfma_supported_16(matrix, input, output, columns, rows));
     for (uint32_t done = 0; done < tokens;) {
         if (sixteen && tokens - done > 8) {
             const uint32_t width = tokens - done < 16 ? tokens - done : 16;
-            const int rc = q8_mfma(matrix, input + uint64_t(done) * columns, output + uint64_t(done) * rows, columns, rows, width, error_word,
-                                   static_cast<hipStream_t>(stream));
+            const int rc = (lanes ? q8_lanes_mfma : q8_mfma)(matrix, input + uint64_t(done) * columns, output + uint64_t(done) * rows, columns, rows, width,
+                                                             error_word, static_cast<hipStream_t>(stream));
             if (rc != TSP_OK) return rc;
             done += width;
             continue;

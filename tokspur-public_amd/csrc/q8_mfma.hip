@@ -319,16 +319,22 @@ constexpr uint32_t kRunBlocks = 16, kRunChunks = 2 + 32;  // 32 B of scales + 51
 constexpr uint32_t kLaneRows = 16, kLaneStride = 560, kLaneTileBytes = kLaneRows * kLaneStride;  // 8 960 B per wave
 constexpr uint32_t kLaneLoads = (kLaneRows * kRunChunks + kWave - 1) / kWave;  // 9 chunk loads per lane and run (the last half used)
 
-template <int DEPTH>
+// ROWS = token rows staged: 8 (all of K per workgroup) or 16 (even workgroups the first half of a row's runs, odd ones the second,
+// each pair over its share of the tiles, both adding their f32 sums into an output the host cleared: the matrix is read once).
+template <int DEPTH, int ROWS>
 __global__ __launch_bounds__(kThreads, 1) void q8_lanes_mfma_kernel(Q8MfmaArgs a) {
-    constexpr int kRows = 8;
+    constexpr int kRows = ROWS;
+    constexpr uint32_t KSPLIT = ROWS / 8;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [hi plane][lo plane][8 weight tiles]
     __shared__ float wave_max[kWaves];
     __shared__ uint32_t next_tile;
 
     const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const uint32_t n16 = lane % 16, kq = lane / 16;
-    const uint32_t K = a.columns, chunks = K / 8, blocks = K / 32, runs = blocks / kRunBlocks, row_bytes = blocks * 34;
+    // K: the columns this workgroup multiplies, runs run0 .. run0 + runs - 1 of every row
+    const uint32_t K = a.columns / KSPLIT, chunks = K / 8, blocks = a.columns / 32, runs = blocks / kRunBlocks / KSPLIT, row_bytes = blocks * 34;
+    const uint32_t run0 = (blockIdx.x % KSPLIT) * runs;
+    const uint32_t sharer = blockIdx.x / KSPLIT, sharers = gridDim.x / KSPLIT;  // the host launches a multiple of KSPLIT
     const uint32_t tiles = (a.rows + kLaneRows - 1) / kLaneRows;
     if (tid == 0) next_tile = 0;
     __syncthreads();
@@ -338,7 +344,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_lanes_mfma_kernel(Q8MfmaArgs a
 
     uint32_t bad = 0;
     float4 xv[kMine][2];
-    request_token_rows<kRows>(a, K, 0, xv);
+    request_token_rows<kRows>(a, K, run0 * (kRunBlocks * 32), xv);
 
     // chunk `id` of a tile: row id / 34 of the wave's 16, piece id % 34 of that row's run: pieces 0 and 1 are the run's scales
     // (32 bytes per run from the row's start), pieces 2 .. 33 its quants (512 bytes per run after all the scales).
@@ -350,7 +356,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_lanes_mfma_kernel(Q8MfmaArgs a
     for (uint32_t t = 0; t < kLaneLoads; ++t) {
         uint32_t id = t * kWave + lane;
         id = id < kLaneRows * kRunChunks ? id : kLaneRows * kRunChunks - 1;  // the tail lanes repeat the last chunk
-        chunk_at[t] = piece_at(id / kRunChunks, id % kRunChunks, 0);
+        chunk_at[t] = piece_at(id / kRunChunks, id % kRunChunks, run0);
         chunk_step[t] = id % kRunChunks < 2 ? 32 : 512;
     }
     uint2 stage[DEPTH][kLaneLoads][2];
@@ -365,7 +371,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_lanes_mfma_kernel(Q8MfmaArgs a
                 uint32_t id = t * kWave + lane;
                 id = id < kLaneRows * kRunChunks ? id : kLaneRows * kRunChunks - 1;
                 const uint32_t row = row0 + id / kRunChunks < a.rows ? id / kRunChunks : a.rows - 1 - row0;
-                at = piece_at(row, id % kRunChunks, run);
+                at = piece_at(row, id % kRunChunks, run0 + run);
             }
             const uint4 v = *reinterpret_cast<const uint4*>(from + at);
             stage[SET][t][0] = uint2{v.x, v.y};
@@ -376,7 +382,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_lanes_mfma_kernel(Q8MfmaArgs a
     auto take_tile = [&]() {
         uint32_t t = 0;
         if (lane == 0) t = atomicAdd(&next_tile, 1u);
-        return uint32_t(__builtin_amdgcn_readfirstlane(int(t))) * gridDim.x + blockIdx.x;
+        return uint32_t(__builtin_amdgcn_readfirstlane(int(t))) * sharers + sharer;
     };
     uint32_t t = take_tile(), t_next = take_tile();
     if (t < share_end) {
@@ -387,11 +393,12 @@ __global__ __launch_bounds__(kThreads, 1) void q8_lanes_mfma_kernel(Q8MfmaArgs a
     const float inv_scale = stage_token_rows<kRows>(xv, K, a_hi, a_lo, wave_max, bad);
 
     // the activation chunk of block B of run g, columns 8 kq .. 8 kq + 7: chunk g * 64 + B * 4 + kq of row `arow`, kept at
-    // chunk ^ arow; arow < 8 flips the three low bits, which B % 2 and kq decide
+    // chunk ^ arow; arow < kRows flips the three or four low bits, which B % kVariants and kq decide
     const uint32_t arow = n16 & (kRows - 1);
-    uint32_t a_at[2];
+    constexpr uint32_t kVariants = kRows / 4;
+    uint32_t a_at[kVariants];
 #pragma unroll
-    for (uint32_t v = 0; v < 2; ++v) a_at[v] = (arow * chunks + ((v * 4 + kq) ^ arow)) * 8;
+    for (uint32_t v = 0; v < kVariants; ++v) a_at[v] = (arow * chunks + ((v * 4 + kq) ^ arow)) * 8;
     auto store_run = [&](auto set_tag) {
         constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
@@ -448,7 +455,7 @@ __global__ __launch_bounds__(kThreads, 1) void q8_lanes_mfma_kernel(Q8MfmaArgs a
                     const int B = kBase + b;
                     const f16x8 b_frag = quants8(w[b][0], w[b][1]);
                     const float scale_d = half_bits_to_float((scales[B / 2] >> (16 * (B % 2))) & 0xffffu);
-                    const uint32_t at = a_at[B % 2] + (g * 64 + (B / 2) * 8) * 8;  // columns g * 512 + B * 32 + 8 kq of the lane's token row
+                    const uint32_t at = a_at[B % kVariants] + (g * 64 + (B / kVariants) * kVariants * 4) * 8;  // columns g * 512 + B * 32 + 8 kq of the lane's token row
                     const f16x8 ah = *reinterpret_cast<const f16x8*>(a_hi + at), al = *reinterpret_cast<const f16x8*>(a_lo + at);
                     const f32x4 zero{};
                     const f32x4 part_lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, b_frag, zero, 0, 0, 0);
@@ -469,11 +476,12 @@ __global__ __launch_bounds__(kThreads, 1) void q8_lanes_mfma_kernel(Q8MfmaArgs a
         const uint32_t r = row0 + n16;
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            const uint32_t m = 4 * kq + v;  // lanes with kq >= 2 hold repeats of rows 0 .. 7
+            const uint32_t m = 4 * kq + v;  // with eight token rows the lanes with kq >= 2 hold repeats of rows 0 .. 7
             if (m < kRows && m < a.m && r < a.rows) {
                 const float val = acc[v] * inv_scale;
                 if (nonfinite(val)) bad = TSP_ERRBIT_NONFINITE;
-                a.y[uint64_t(m) * a.rows + r] = val;
+                if constexpr (KSPLIT == 1) a.y[uint64_t(m) * a.rows + r] = val;
+                else unsafeAtomicAdd(a.y + uint64_t(m) * a.rows + r, val);
             }
         }
     }
@@ -533,6 +541,11 @@ bool q8_lanes_mfma_supported(const void* matrix, const float* x, uint32_t column
            reinterpret_cast<uintptr_t>(x) % 16 == 0;
 }
 
+bool q8_lanes_mfma_supported_16(const void* matrix, const float* x, const float* y, uint32_t columns, uint32_t rows) {
+    return q8_lanes_mfma_supported(matrix, x, columns, rows) && columns % 1024 == 0 && rows >= 32 && rows % 4 == 0 &&
+           reinterpret_cast<uintptr_t>(y) % 16 == 0;
+}
+
 int q8_lanes_mfma(const void* matrix, const float* x, float* y, uint32_t columns, uint32_t rows, uint32_t width, uint32_t* error_word,
                   hipStream_t s) {
     const Q8MfmaArgs a{static_cast<const uint8_t*>(matrix), x, y, columns, rows, width, error_word};
@@ -542,17 +555,29 @@ int q8_lanes_mfma(const void* matrix, const float* x, float* y, uint32_t columns
     int device = 0;
     if (setup_pending(raised, &device)) {
         const int most = int(2 * 8 * 2048 * 2 + kWaves * kLaneTileBytes);
-        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_lanes_mfma_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
-        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_lanes_mfma_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_lanes_mfma_kernel<1, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_lanes_mfma_kernel<2, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_lanes_mfma_kernel<1, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        TSP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_lanes_mfma_kernel<2, 16>), hipFuncAttributeMaxDynamicSharedMemorySize, most));
         TSP_HIP(hipDeviceGetAttribute(&units_of[device], hipDeviceAttributeMultiprocessorCount, device));
         setup_done(raised, device);
     }
     const int compute_units = units_of[device];
     const uint32_t tiles = (rows + kLaneRows - 1) / kLaneRows;
     uint32_t grid = uint32_t(compute_units > 0 ? compute_units : 256);
+    if (width > 8) {
+        // two workgroups (one per half of a row's runs) share each stretch of tiles; the output starts at zero
+        uint32_t pairs = grid / 2 ? grid / 2 : 1;
+        if (pairs * kWaves > tiles) pairs = (tiles + kWaves - 1) / kWaves;
+        const uint64_t count4 = uint64_t(width) * rows / 4;
+        TSP_LAUNCH("clear_rows", s, clear_rows<<<uint32_t((count4 + 255) / 256), 256, 0, s>>>(reinterpret_cast<float4*>(y), count4));
+        if ((columns / 1024) % 2 == 0) TSP_LAUNCH("q8_lanes_mfma", s, q8_lanes_mfma_kernel<2, 16><<<2 * pairs, kThreads, lds_bytes, s>>>(a));
+        else TSP_LAUNCH("q8_lanes_mfma", s, q8_lanes_mfma_kernel<1, 16><<<2 * pairs, kThreads, lds_bytes, s>>>(a));
+        return launch_status("q8_lanes_mfma");
+    }
     if (grid * kWaves > tiles) grid = (tiles + kWaves - 1) / kWaves;
-    if ((columns / 512) % 2 == 0) TSP_LAUNCH("q8_lanes_mfma", s, q8_lanes_mfma_kernel<2><<<grid, kThreads, lds_bytes, s>>>(a));
-    else TSP_LAUNCH("q8_lanes_mfma", s, q8_lanes_mfma_kernel<1><<<grid, kThreads, lds_bytes, s>>>(a));
+    if ((columns / 512) % 2 == 0) TSP_LAUNCH("q8_lanes_mfma", s, q8_lanes_mfma_kernel<2, 8><<<grid, kThreads, lds_bytes, s>>>(a));
+    else TSP_LAUNCH("q8_lanes_mfma", s, q8_lanes_mfma_kernel<1, 8><<<grid, kThreads, lds_bytes, s>>>(a));
     return launch_status("q8_lanes_mfma");
 }
 
