@@ -358,6 +358,23 @@ def main():
         k0 = profiled(capi, torch, gemv_rot, 120)
         configs["c0_gemv_q4k"]["kernel_us"] = round(min(v["avg_us"] for v in k0.values()), 2)
         del copies
+        # NOT a BASELINE configuration: the same Q4_K GEMV kernel at sizes where HBM, not launch latency, bounds it (the 4.7 MB of
+        # config 0 cannot show the kernel's bandwidth). Weights: config 0's rows repeated; two copies alternate.
+        for big_rows in (65536, 262144):
+            wb = np.tile(w0, big_rows // 4096)
+            pair = [gpu.upload(wb), gpu.upload(wb)]
+            yb = gpu.empty(big_rows)
+            state["i"] = 0
+
+            def gemv_big():
+                gpu.gemv(12, pair[state["i"] % 2], x0, C, big_rows, y=yb)
+                state["i"] += 1
+
+            ms = timed(torch, gemv_big, 40, 10)
+            bb = big_rows * 8 * 144 + 8192 + big_rows * 4
+            configs[f"gemv_q4k_{big_rows}x2048_not_a_baseline_config"] = {"us": ms * 1e3, "hbm_gbps": bb / (ms * 1e-3) / 1e9,
+                                                                           "hbm_frac": bb / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "bytes": bb}
+            del pair, wb, yb
         # config 2: MoE verify T = 8 on the config-3 experts; eight router inputs in rotation so the ~150 MB of
         # selected experts differ from step to step and do not sit in the 256 MB last-level cache
         T2 = 8

@@ -72,9 +72,11 @@ def test_dense_mm_q4k(gpu, tsp, orc, synth, layout, tokens, rows, cols):
 
 
 # the last shape is 240 tiles of 256 rows, ragged on both sides: the one-wave-per-SIMD form of the kernel on a 256-unit GPU
-@pytest.mark.parametrize("tokens,rows,cols", [(1024, 256, 256), (1100, 300, 512), (1300, 777, 1024), (2000, 7500, 256)])
+# (512, 300, 256), (600, 1000, 512) and (1000, 256, 1024): fewer than 1024 rows take 128 x 128 tiles, ragged on both sides
+@pytest.mark.parametrize("tokens,rows,cols", [(1024, 256, 256), (1100, 300, 512), (1300, 777, 1024), (2000, 7500, 256),
+                                              (512, 300, 256), (600, 1000, 512), (1000, 256, 1024)])
 def test_dense_mm_q4k_many_rows(gpu, tsp, orc, synth, tokens, rows, cols):
-    """Raw GGUF Q4_K rows against a thousand and more activation rows: the kernel with tiles 128 or 256 rows high, ragged on
+    """Raw GGUF Q4_K rows against 512 and more activation rows: the kernel with tiles 128 or 256 rows high, ragged on
     both sides. Its arithmetic is the engine's (weights rounded once to half, bf16 activations, f32 accumulation): the
     half-staged reference is met to accumulation accuracy; strided rows and padding stay."""
     w = synth.matrix(12, 2300 + rows, rows, cols)
@@ -158,8 +160,8 @@ def test_config1_dense_q4k_gemm(gpu, tsp, orc, synth, tokens):
     err, err_un = max_rel_error(out_f32[:, sel], want), max_rel_error(out_f32[:, sel], unstaged)
     print(f"config1 M={tokens}: max rel error vs half-staged reference {err:.2e}, vs f32-dequantised {err_un:.2e}, "
           f"NMSE vs f32-dequantised {nmse(out_f32[:, sel], unstaged):.2e}")
-    if tokens >= 1024:
-        # a thousand rows and more take the 256 x 256 tile kernel, which rounds every weight once to half like the engine's
+    if tokens >= 512:
+        # 512 rows and more take the many-row kernel (128 x 128, 128 x 256 or 256 x 256 tiles), which rounds every weight once to half like the engine's
         # own kernel: the half-staged reference is met to accumulation accuracy, the f32-dequantised one within the engine's
         # rel-L2 limit for that comparison
         assert err <= 5e-6 and rel_l2(out_f32[:, sel], unstaged) <= 5e-3
@@ -168,10 +170,10 @@ def test_config1_dense_q4k_gemm(gpu, tsp, orc, synth, tokens):
     # the engine's own metric, |a - e| / max(1, |e|), against the reference that rounds nothing: outputs are O(500) here, so
     # an f32-accumulated product is well inside the configuration's 2e-3
     # (for the kernel that stages weights as halves, against the reference staged the same way, as the engine's own tests do)
-    value, at, actual, expected, row_rms = reference_metric(out_f32[:, sel], want if tokens >= 1024 else unstaged)
+    value, at, actual, expected, row_rms = reference_metric(out_f32[:, sel], want if tokens >= 512 else unstaged)
     print(f"config1 M={tokens}: reference metric {value:.2e} at element {at} (got {actual:.6g}, reference {expected:.6g}, row rms {row_rms:.3g})")
     assert value <= 2e-3
-    # and against the reference that rounds nothing, whatever the kernel stages. The integer-factor kernel (fewer than 1024
+    # and against the reference that rounds nothing, whatever the kernel stages. The integer-factor kernel (fewer than 512
     # rows) meets the configuration's 2e-3 in the engine's own metric with a factor of twenty to spare. The many-row kernel
     # rounds every weight once to half, as the engine's kernel for this product does: 2^-12 per weight, which over 2048 terms
     # is ~1.4e-4 of the row's scale for a typical element and 1.8e-3 at the extreme of the 393 216 sampled ones, inside 2e-3 in
@@ -182,7 +184,7 @@ def test_config1_dense_q4k_gemm(gpu, tsp, orc, synth, tokens):
     print(f"config1 M={tokens}: against the f32-dequantised reference: {err_un:.2e} of the row scale; engine's metric {value_un:.2e} at element {at_un} "
           f"(got {actual_un:.6g}, reference {expected_un:.6g}, row rms {rms_un:.3g})")
     assert err_un <= 2e-3
-    if tokens < 1024:
+    if tokens < 512:
         assert value_un <= 2e-3
     # every column: permuting the token rows permutes the output rows bit for bit (tiles hold no row state)
     perm = np.random.default_rng(1).permutation(tokens)
@@ -191,26 +193,26 @@ def test_config1_dense_q4k_gemm(gpu, tsp, orc, synth, tokens):
 
 
 def test_dense_mm_across_the_many_row_threshold(gpu, tsp, orc, synth):
-    """`tsp_dense_mm` on Q4_K GGUF rows changes arithmetic at 1024 token rows: below, exact integer factors with f32 block
+    """`tsp_dense_mm` on Q4_K GGUF rows changes arithmetic at 512 token rows: below, exact integer factors with f32 block
     scales; from there on, every weight rounded once to half (the engine's staging). The same token rows through both arms
-    (1023 of them, then 1024) must agree within what that rounding allows, and each arm with its own reference: a caller that
+    (511 of them, then 512) must agree within what that rounding allows, and each arm with its own reference: a caller that
     chunks a prompt differently gets results that differ by this much and no more."""
     rows, cols = 512, 2048
     w = synth.matrix(12, 2601, rows, cols)
-    x = synth.round_bf16(synth.activations_f32(2602, (1024, cols)))
+    x = synth.round_bf16(synth.activations_f32(2602, (512, cols)))
     dw = gpu.upload(w)
-    below = tsp.dense_mm(gpu, 12, tsp.LAYOUT_GGUF, dw, gpu.upload(np.ascontiguousarray(x[:1023])), 1023, cols, rows).cpu().numpy()
-    above = tsp.dense_mm(gpu, 12, tsp.LAYOUT_GGUF, dw, gpu.upload(x), 1024, cols, rows).cpu().numpy()
+    below = tsp.dense_mm(gpu, 12, tsp.LAYOUT_GGUF, dw, gpu.upload(np.ascontiguousarray(x[:511])), 511, cols, rows).cpu().numpy()
+    above = tsp.dense_mm(gpu, 12, tsp.LAYOUT_GGUF, dw, gpu.upload(x), 512, cols, rows).cpu().numpy()
     assert gpu.error() == 0
     sel = np.arange(0, rows, 4, dtype=np.uint32)
     exact = orc.staged_gemm(12, w, cols, x, rows_sel=sel, stage_f16=False)
     staged = orc.staged_gemm(12, w, cols, x, rows_sel=sel)
-    assert max_rel_error(below[:, sel], exact[:1023]) <= 2e-5 and max_rel_error(above[:, sel], staged) <= 5e-6
-    across = max_rel_error(below, above[:1023])
-    value = reference_metric(below, above[:1023])[0]
-    print(f"dense_mm 1023 rows against 1024 rows: max difference {across:.2e} of the row scale, {value:.2e} in the engine's metric")
+    assert max_rel_error(below[:, sel], exact[:511]) <= 2e-5 and max_rel_error(above[:, sel], staged) <= 5e-6
+    across = max_rel_error(below, above[:511])
+    value = reference_metric(below, above[:511])[0]
+    print(f"dense_mm 511 rows against 512 rows: max difference {across:.2e} of the row scale, {value:.2e} in the engine's metric")
     # half staging: 2^-12 per weight, ~2.8e-4 of the row scale in the mean square over 2048 terms, 1.5e-3 at the extreme of
-    # these 523 776 elements (the engine's metric, which divides an element that cancels to nearly nothing by 1, is printed only)
+    # these 261 632 elements (the engine's metric, which divides an element that cancels to nearly nothing by 1, is printed only)
     assert across <= 2e-3 and max_rel_error(above[:, sel], exact) <= 2e-3
 
 

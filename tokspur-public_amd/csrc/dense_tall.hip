@@ -57,22 +57,24 @@ __device__ __forceinline__ uint32_t two_weights(uint32_t codes, float scale, flo
     return as_u32(f16x2{lo, hi});
 }
 
-constexpr int kTileN = 256, kStepK = 64, kRing = 3;
-constexpr int kQsBytes = kTileN * 32;
-constexpr int kHdrBytes = kTileN * 16, kHdrStages = 2;
+constexpr int kStepK = 64, kRing = 3, kHdrStages = 2;
 
 // waves per SIMD: 128-row tiles leave room for two workgroups per compute unit, 256-row tiles for one
-constexpr int tall_waves_per_simd(int rt, int ct, int waves) { return ((waves * ct / 8) * rt * 32 == 128 ? 2 : 1) * waves / 4; }
+constexpr int tall_waves_per_simd(int rt, int ct, int waves, int tn) { return ((waves * ct * 32 / tn) * rt * 32 == 128 ? 2 : 1) * waves / 4; }
 
 // RT x CT: the row tiles (32 activation rows each) and column tiles (32 weight rows each) of a wave, 16 accumulator registers
 // apiece; WAVES waves stand 8 / CT wide across the tile's 256 weight rows and WAVES CT / 8 high. Two forms are launched:
 //   4 x 2, four waves: a 128 x 256 tile; two workgroups share a compute unit.
 //   8 x 1, eight waves: a 256 x 256 tile; a weight is unpacked once per 256 rows, at the price of an LDS read per MFMA.
 // (8 x 2 with four waves, a wave alone on its SIMD with 256 accumulator registers, compiles too and measured in between.)
-template <int RT, int CT, int WAVES, int PER_SIMD = tall_waves_per_simd(RT, CT, WAVES)>
+// TN = weight rows of a tile: 256, or 128 for
+//   4 x 1, four waves: a 128 x 128 tile, for 512 to 1023 activation rows, where 256 weight rows per tile would leave half of
+//     the compute units without a tile (512 x 8192 results are 256 such tiles); 64 accumulator registers per lane.
+template <int RT, int CT, int WAVES, int TN = 256, int PER_SIMD = tall_waves_per_simd(RT, CT, WAVES, TN)>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(PER_SIMD, PER_SIMD))) void dense_tall_kernel(DenseTallArgs a) {
-    constexpr int kThreadsT = 64 * WAVES, WN = 8 / CT, WM = WAVES / WN, kTileM = WM * RT * 32;
-    static_assert(WM >= 1 && WN * WM == WAVES);
+    constexpr int kTileN = TN, kQsBytes = kTileN * 32, kHdrBytes = kTileN * 16;
+    constexpr int kThreadsT = 64 * WAVES, WN = TN / 32 / CT, WM = WAVES / WN, kTileM = WM * RT * 32;
+    static_assert(WM >= 1 && WN * WM == WAVES && kQsBytes % (kThreadsT * 16) == 0);
     constexpr int kSlabBytes = kTileM * kStepK * 2, kSlabPieces = kSlabBytes / (kThreadsT * 16);
     constexpr int kQsAt = kRing * kSlabBytes, kHdrAt = kQsAt + kRing * kQsBytes;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[kHdrAt + kHdrStages * kHdrBytes];
@@ -110,10 +112,10 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(PER_
         const uint32_t u = tid + kThreadsT * q, q_r = u / 2, q_row = n0 + q_r < a.n ? n0 + q_r : a.n - 1;
         q_lane[q] = q_row * row_bytes + (((u % 2) ^ ((q_r >> 3) & 1)) * 16);
     }
-    const uint32_t h_r = tid % 256, h_row = n0 + h_r < a.n ? n0 + h_r : a.n - 1;
+    const uint32_t h_r = tid % kTileN, h_row = n0 + h_r < a.n ? n0 + h_r : a.n - 1;
     const uint32_t h_lane = h_row * row_bytes;
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds_raw));
-    const uint32_t my_slab = lds0 + wave * 1024, my_qs = lds0 + kQsAt + wave * 1024, my_hdr = lds0 + kHdrAt + (wave % 4) * 1024;
+    const uint32_t my_slab = lds0 + wave * 1024, my_qs = lds0 + kQsAt + wave * 1024, my_hdr = lds0 + kHdrAt + (wave % (kTileN / 64)) * 1024;
     // Step `step`'s bytes into ring slot step % 3. Steps past the end ask for the last step's bytes again (read by the front of a step that never runs), and
     // ask for headers where a real step would: the number of requests per step must not depend on where the matrix ends,
     // the waits below count them.
@@ -306,7 +308,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(PER_
         // wave has to itself (16 or 18 KB: a few row tiles at a time; a row pitch of 16 bytes
         // more than the row keeps the column-wise writes and the row-wise reads off each other's banks). A lane storing
         // its own 2- or 4-byte results one by one, 128 stores, took a fifth of the kernel's time.
-        constexpr int kRegion = WAVES == 8 ? 16 * 1024 : 16 * 1024 + 2048;
+        constexpr int kRegion = CT == 1 && WAVES == 4 ? 12 * 1024 : WAVES == 8 ? 16 * 1024 : 16 * 1024 + 2048;
         uint8_t* const mine = lds_raw + wave * kRegion;
         static_assert(WAVES * kRegion <= int(sizeof(lds_raw)));
         auto pass = [&](auto bf16_tag, auto first_tag) {
@@ -386,7 +388,7 @@ __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(PER_
 namespace tsp {
 
 bool dense_tall_takes(uint32_t tokens, uint32_t rows, uint32_t columns, uint64_t matrix_bytes) {
-    return tokens >= 1024 && rows >= kTileN && columns % 256 == 0 && columns >= 256 && matrix_bytes < (1ull << 32) &&
+    return tokens >= 512 && rows >= 256 && columns % 256 == 0 && columns >= 256 && matrix_bytes < (1ull << 32) &&
            uint64_t(tokens) * columns * 2 < (1ull << 32);
 }
 
@@ -403,9 +405,13 @@ int launch_dense_tall(const DenseTallArgs& a, hipStream_t s) {
     // 256-row tiles only where one round of them keeps nearly every compute unit busy (2048 x 8192 results on 256 units): there
     // they are a few percent faster. Elsewhere 128-row tiles, two workgroups to a unit, lose less to the last, partly filled
     // round, and a second round of 256-row tiles cannot start behind the first one's epilogue as a second workgroup can.
-    const uint32_t n_tiles = (a.n + kTileN - 1) / kTileN, cus = uint32_t(units[device]);
+    const uint32_t n_tiles = (a.n + 255) / 256, cus = uint32_t(units[device]);
     const uint32_t tall = n_tiles * ((a.m + 255) / 256), low = n_tiles * ((a.m + 127) / 128);
-    if (tall <= cus && uint64_t(tall) * 10 >= uint64_t(cus) * 9) {
+    const uint32_t narrow = ((a.n + 127) / 128) * ((a.m + 127) / 128);
+    if (a.m < 1024 && low < cus) {
+        // too few 128 x 256 tiles for the chip: 128 x 128 tiles, one workgroup of four waves each
+        TSP_LAUNCH("gemm_dense_tall", s, (dense_tall_kernel<4, 1, 4, 128><<<(narrow + 7) / 8 * 8, 256, 0, s>>>(a)));
+    } else if (tall <= cus && uint64_t(tall) * 10 >= uint64_t(cus) * 9) {
         TSP_LAUNCH("gemm_dense_tall", s, (dense_tall_kernel<8, 1, 8><<<(tall + 7) / 8 * 8, 512, 0, s>>>(a)));
     } else {
         TSP_LAUNCH("gemm_dense_tall", s, (dense_tall_kernel<4, 2, 4><<<(low + 7) / 8 * 8, 256, 0, s>>>(a)));
