@@ -5,6 +5,7 @@
 #include "../../include/tokspur_hip.h"
 
 #include <algorithm>
+#include <array>
 #include <atomic>
 #include <cerrno>
 #include <cstring>
@@ -211,57 +212,110 @@ std::span<const std::byte> Gguf::tensor_bytes(const Tensor& tensor) const {
     return data_.subspan(size_t(tensor.offset), size_t(tensor.bytes));
 }
 
-void Gguf::parse() {
-    Reader r{data_};
-    require(r.number(4) == 0x46554747 && r.number(4) == 3, "expected little-endian GGUF v3");
+// The header is taken apart in four stages, each over the table the stage before it left, so that reading the bytes and
+// judging what they say stay apart: (1) walk the records and note where each one lies (nothing is judged beyond what finding
+// the next record needs); (2) admit the metadata keys; (3) admit the tensor records against the alignment the metadata
+// declares; (4) lay the data section out behind the header and check every tensor's bytes against the file and each other.
+namespace {
+struct MetadataRecord { std::string_view key; Metadata value; };
+struct TensorRecord {
+    std::string_view name;
+    uint32_t rank = 0, type = 0;
+    std::array<uint64_t, 4> extent{};
+    uint64_t offset = 0;  // from the start of the data section
+};
+struct HeaderWalk {
+    std::vector<MetadataRecord> metadata;
+    std::vector<TensorRecord> tensors;
+    uint64_t end = 0;  // first byte behind the last record
+};
+
+// stage 1: where the records lie. A record that cannot be walked over (a string past its limit, a value of no known type, a rank
+// with no extents to count) stops the walk; everything else about a record is left to the stages that follow.
+HeaderWalk walk_header(std::span<const std::byte> bytes) {
+    Reader r{bytes};
+    const uint64_t magic = r.number(4), version = r.number(4);
+    require(magic == 0x46554747 && version == 3, "expected little-endian GGUF v3");
     const uint64_t tensor_count = r.number(8), metadata_count = r.number(8);
     require(tensor_count <= kRecordLimit && metadata_count <= kRecordLimit, "GGUF record limit exceeded");
-    // the shortest tensor record is 33 bytes, the shortest metadata record 14
-    require(checked_add(checked_mul(tensor_count, 33), checked_mul(metadata_count, 14)) <= data_.size() - r.at, "GGUF counts exceed available file bytes");
-    for (uint64_t i = 0; i < metadata_count; ++i) {
-        const std::string key(r.text(65535));
-        require(key_ok(key), "invalid GGUF metadata key");
-        const Metadata m = r.value(uint32_t(r.number(4)));
-        require(metadata_.emplace(key, m).second, "duplicate GGUF metadata key");
+    // no record is shorter than its fixed fields: 8 + 4 + 8 + 4 + 8 + one name byte for a tensor, 8 + 4 + one key byte + one
+    // value byte for a metadata item; counts that cannot fit in what is left of the file are refused before any table grows
+    const uint64_t least = checked_add(checked_mul(tensor_count, 33), checked_mul(metadata_count, 14));
+    require(least <= bytes.size() - r.at, "GGUF counts exceed available file bytes");
+    HeaderWalk walk;
+    walk.metadata.resize(size_t(metadata_count));
+    for (MetadataRecord& item : walk.metadata) {
+        item.key = r.text(65535);
+        require(key_ok(item.key), "invalid GGUF metadata key");  // the key decides whether the value's bytes mean anything at all
+        item.value = r.value(uint32_t(r.number(4)));
     }
-    const uint64_t alignment = find("general.alignment") ? unsigned_value("general.alignment") : 32;
-    require(alignment && alignment <= 65536 && !(alignment & (alignment - 1)), "unsupported GGUF alignment");
-    tensors_.reserve(size_t(tensor_count));
-    std::set<std::string, std::less<>> names;
-    for (uint64_t i = 0; i < tensor_count; ++i) {
-        Tensor t;
-        t.name = std::string(r.text(64));
-        require(!t.name.empty() && names.insert(t.name).second, "empty or duplicate tensor name");
-        for (const unsigned char c : t.name) require(c >= 0x21 && c <= 0x7e, "non-ASCII tensor name");
-        const uint64_t rank = r.number(4);
-        require(rank >= 1 && rank <= 4, "unsupported GGUF tensor rank");
-        t.elements = 1;
-        for (uint64_t d = 0; d < rank; ++d) {
-            const uint64_t extent = r.number(8);
-            require(extent != 0, "zero tensor dimension");
-            t.dimensions.push_back(extent);
-            t.elements = checked_mul(t.elements, extent);
-        }
+    walk.tensors.resize(size_t(tensor_count));
+    for (TensorRecord& t : walk.tensors) {
+        t.name = r.text(64);
+        t.rank = uint32_t(r.number(4));
+        require(t.rank >= 1 && t.rank <= 4, "unsupported GGUF tensor rank");
+        for (uint32_t d = 0; d < t.rank; ++d) t.extent[d] = r.number(8);
         t.type = uint32_t(r.number(4));
-        const Encoding& e = encoding(t.type);
-        require(t.dimensions.front() % e.elements_per_block == 0, "quantized tensor row is not block-aligned");
-        t.bytes = checked_mul(t.elements / e.elements_per_block, e.bytes_per_block);
         t.offset = r.number(8);
-        require(t.offset % alignment == 0, "unaligned GGUF tensor offset");
+    }
+    walk.end = r.at;
+    return walk;
+}
+
+// stage 3, one record: names are printable ASCII, extents positive, rows whole blocks of the encoding
+Tensor admit_tensor(const TensorRecord& record, uint64_t alignment) {
+    require(!record.name.empty(), "empty or duplicate tensor name");
+    for (const unsigned char c : record.name) require(c >= 0x21 && c <= 0x7e, "non-ASCII tensor name");
+    Tensor t;
+    t.name = std::string(record.name);
+    t.type = record.type;
+    t.elements = 1;
+    for (uint32_t d = 0; d < record.rank; ++d) {
+        require(record.extent[d] != 0, "zero tensor dimension");
+        t.dimensions.push_back(record.extent[d]);
+        t.elements = checked_mul(t.elements, record.extent[d]);
+    }
+    const Encoding& e = encoding(t.type);
+    require(t.dimensions.front() % e.elements_per_block == 0, "quantized tensor row is not block-aligned");
+    t.bytes = checked_mul(t.elements / e.elements_per_block, e.bytes_per_block);
+    require(record.offset % alignment == 0, "unaligned GGUF tensor offset");
+    t.offset = record.offset;
+    return t;
+}
+}  // namespace
+
+void Gguf::parse() {
+    const HeaderWalk walk = walk_header(data_);
+    // stage 2: the metadata index
+    for (const MetadataRecord& item : walk.metadata) require(metadata_.emplace(std::string(item.key), item.value).second, "duplicate GGUF metadata key");
+    uint64_t alignment = 32;
+    if (find("general.alignment")) alignment = unsigned_value("general.alignment");
+    require(alignment != 0 && alignment <= 65536 && (alignment & (alignment - 1)) == 0, "unsupported GGUF alignment");
+    // stage 3: the tensor table, in file order
+    tensors_.reserve(walk.tensors.size());
+    std::set<std::string_view> seen;
+    for (const TensorRecord& record : walk.tensors) {
+        Tensor t = admit_tensor(record, alignment);
+        require(seen.insert(record.name).second, "empty or duplicate tensor name");
         tensors_.push_back(std::move(t));
     }
-    data_offset_ = checked_add(r.at, alignment - 1) & ~(alignment - 1);
-    if (!tensor_count) data_offset_ = std::min<uint64_t>(data_offset_, data_.size());  // a metadata-only shard has no data section to pad to
+    // stage 4: the data section starts at the next multiple of the alignment behind the header (a shard of metadata alone has
+    // none and need not be padded); every tensor lies inside the file and no two share a byte
+    data_offset_ = checked_add(walk.end, alignment - 1) / alignment * alignment;
+    if (tensors_.empty() && data_offset_ > data_.size()) data_offset_ = data_.size();
     require(data_offset_ <= data_.size(), "truncated GGUF header padding");
-    std::vector<std::pair<uint64_t, uint64_t>> spans;
-    for (auto& t : tensors_) {
-        t.offset = checked_add(data_offset_, t.offset);
-        const uint64_t end = checked_add(t.offset, t.bytes);
-        require(end <= data_.size(), "truncated GGUF tensor data");
-        spans.emplace_back(t.offset, end);
+    std::vector<size_t> by_offset(tensors_.size());
+    for (size_t i = 0; i < tensors_.size(); ++i) {
+        by_offset[i] = i;
+        tensors_[i].offset = checked_add(data_offset_, tensors_[i].offset);
+        require(checked_add(tensors_[i].offset, tensors_[i].bytes) <= data_.size(), "truncated GGUF tensor data");
     }
-    std::sort(spans.begin(), spans.end());
-    for (size_t i = 1; i < spans.size(); ++i) require(spans[i].first >= spans[i - 1].second, "overlapping GGUF tensors");
+    std::sort(by_offset.begin(), by_offset.end(), [&](size_t a, size_t b) { return tensors_[a].offset < tensors_[b].offset; });
+    uint64_t used_to = 0;
+    for (const size_t i : by_offset) {
+        require(tensors_[i].offset >= used_to, "overlapping GGUF tensors");
+        used_to = tensors_[i].offset + tensors_[i].bytes;
+    }
 }
 
 ModelFiles::ModelFiles(const std::vector<std::filesystem::path>& paths) {
