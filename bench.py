@@ -331,6 +331,32 @@ def main():
         configs["c3_routed_q4k_gate_up_q8_down"] = {"ms": ms, "tok_per_s": T / (ms * 1e-3),
                                                     "kernels_us": {k: round(v["avg_us"], 2) for k, v in profiled(capi, torch, routed_q8_down, 5).items()}}
         del w8
+        # NOT a BASELINE configuration: the engine's own expert shape (2560 channels, 640 hidden units: src/moe_mm_many_plan.cpp:7,31)
+        # with its kinds, Q4_K co-located gate/up and Q8_0 planes down, 2048 tokens, 512 experts, top-10, uniform router. Neither
+        # resident kernel takes this shape (they want 2048 columns resp. 512 hidden units): gate/up runs on the general
+        # integer-factor kernel, down on the staged kernel. 64 synthetic experts repeated eight times.
+        Ce, He = 2560, 640
+        rep = E // 64
+        ge = np.tile(synth.matrix(12, synth.tensor_seed(3, 30), He * 64, Ce), rep)
+        ue = np.tile(synth.matrix(12, synth.tensor_seed(3, 31), He * 64, Ce), rep)
+        de = np.tile(synth.matrix(8, synth.tensor_seed(3, 32), Ce * 64, He), rep)
+        we = capi.PlanarMoeWeights(gpu, 12, 8, Ce, He, E, ge, ue, de)
+        del ge, ue, de
+        xe = gpu.upload(synth.round_bf16(synth.activations_f32(synth.tensor_seed(3, 33), (T, Ce))))
+        ids_e, wts_e = gpu.zeros((T, S), "int32"), gpu.zeros((T, S))
+        gpu.route(gpu.upload(synth.activations_f32(synth.tensor_seed(3, 34), (T, E))), S, 0, True, tokens=T, out=(ids_e, wts_e))
+        scratch_e, ye = capi.GroupedScratch(gpu, T, S, E, Ce, He), gpu.empty((T * S, Ce))
+
+        def routed_engine_shape():
+            capi.planar_nax_grouped_moe(gpu, we, ids_e, xe, T, S, scratch_e, y=ye)
+
+        ms = timed(torch, routed_engine_shape, k2, 2)
+        fl_e = T * S * 3 * 2.0 * Ce * He
+        configs["engine_shape_2560x640_q4k_gate_up_q8_down_not_a_baseline_config"] = {
+            "ms": ms, "tok_per_s": T / (ms * 1e-3), "tflops": fl_e / (ms * 1e-3) / 1e12,
+            "kernels_us": {k: round(v["avg_us"], 2) for k, v in profiled(capi, torch, routed_engine_shape, 5).items()}}
+        assert gpu.error() == 0
+        del we, xe, scratch_e, ye
         # config 0: dense Q4_K GEMV over a rotation of distinct weight copies (> 512 MB) so every read comes from HBM
         w0 = synth.matrix(12, synth.tensor_seed(0, 1), 4096, C)
         x0, y0 = gpu.upload(synth.activations_f32(synth.tensor_seed(0, 2), C)), gpu.empty(4096)

@@ -591,13 +591,16 @@ def test_grouped_moe_exact_when_products_fit_half(gpu, tsp, orc, synth):
 @pytest.mark.parametrize("gu_type,dn_type,channels,hidden", [(13, 7, 256, 256), (8, 8, 256, 256), (12, 8, 256, 256), (13, 14, 256, 256), (12, 7, 512, 160),
                                                              (8, 7, 96, 64), (8, 14, 160, 256), (12, 8, 256, 512), (8, 8, 384, 512),
                                                              (13, 8, 2048, 512), (12, 7, 256, 512), (8, 7, 768, 512),
-                                                             (12, 7, 2048, 160), (12, 8, 2048, 96)])
+                                                             (12, 7, 2048, 160), (12, 8, 2048, 96),
+                                                             (12, 8, 2560, 640), (12, 7, 2560, 640), (13, 8, 2560, 640), (8, 7, 2560, 640)])
 def test_grouped_moe_other_planar_kinds(gpu, tsp, orc, synth, gu_type, dn_type, channels, hidden):
     """The planar kinds of include/tokspur/moe.hpp:27-29 beside Q4_K gate/up and Q6_K down (Q5_K / Q8_0 gate and up, Q5_1 / Q8_0
     down) run on the matrix cores as well, their weights decoded to halves on the fly; any gate/up kind combines with any down
     kind (experts of 512 hidden units with Q8_0 planes down take the kernel that keeps a task's h rows in registers). Same
     token_map / counts / tasks; expert_down rows against the reference with the declared staging: activations as
-    bf16 values, h as 256 * half(h / 256), weights of the staged kinds rounded to half (Q4_K / Q6_K keep their integer factors)."""
+    bf16 values, h as 256 * half(h / 256), weights of the staged kinds rounded to half (Q4_K / Q6_K keep their integer factors).
+    The last four shapes are the engine's own expert, 2560 channels and 640 hidden units (native/src/moe_mm_many_plan.cpp:7,31),
+    with each of its gate/up and down kinds."""
     experts, selected, n = 6, 3, 75  # an expert with more than 64 routes, one with more than 32, ragged tails
     gate = synth.matrix(gu_type, 3301, hidden * experts, channels)
     up = synth.matrix(gu_type, 3302, hidden * experts, channels)
