@@ -5,7 +5,10 @@
 //
 //  gemv_generic   wave per row, any decodable encoding and any K: the scalar control arm.
 //  gemv_q4k       Q4_K, raw GGUF rows or one planar v3 expert; a lane owns one 32-byte nibble pair
-//                 (two 32-weight sub-blocks), 4 lanes per super-block.
+//                 (two 32-weight sub-blocks), 4 lanes per super-block. The lane's 64 activations are
+//                 kept as three planes of signed bytes under a per-sub-block scale (24 bits of each
+//                 value), and the nibbles multiply them four at a time with v_dot4_i32_i8: the sums
+//                 of q * x are exact integers, scaled by d * sc in f32 once per sub-block.
 //  gemv_q8        Q8_0 raw rows as a flat dword stream (row bytes are a multiple of 4).
 //  gemv_q6k       Q6_K planar expert planes.
 #include "decode.hpp"
@@ -65,7 +68,6 @@ __global__ __launch_bounds__(256) void gemv_generic(GemvArgs a) {
 }
 
 // ------------------------------------------------------------------------------------ Q4_K
-__device__ __forceinline__ float ub(uint32_t w, int i) { return float((w >> (8 * i)) & 0xffu); }
 
 // Sum over aligned groups of N lanes (N = 8, 16, 32, 64); every lane of a group gets the sum.
 template <int N>
@@ -139,14 +141,48 @@ __global__ __launch_bounds__(256) void gemv_q4k(GemvArgs a) {
         if (kQuads % 256 == 0 || threadIdx.x + j * 256 < kQuads) reinterpret_cast<float4*>(xs)[threadIdx.x + j * 256] = xv[j];
     __syncthreads();
 
-    float xa[32], xb[32];
-    float sxa = 0, sxb = 0;
+    // The lane's 64 activations become integers: per sub-block of 32 one scale that brings the largest magnitude to 8 290 000
+    // (just under 127 * 2^16 + 2^15, the most that three signed bytes hold), every value rounded to the nearest integer of
+    // that grid (2^-24 of the sub-block's largest value: the precision of the f32 operand itself for the values that matter)
+    // and written as three signed base-256 digits, x = (a 2^16 + b 2^8 + c) / scale with a, b, c in [-128, 127]. Four
+    // activations' digits share a dword, in the order of the four bytes of a word of nibbles, so that v_dot4_i32_i8 multiplies
+    // four weights per instruction and plane: three integer instructions per four weights where the f32 form spends a
+    // conversion and a multiply-add per weight. The integer sums are exact; the three of a sub-block recombine in f32.
+    uint32_t pa[3][8], pb[3][8];
+    float sxa = 0, sxb = 0, inv_a, inv_b;
+    bool x_bad = false;
     {
         const float* src = xs + blk_in_row * 256 + pair * 64;
+        auto planes = [&](const float* v32, uint32_t (&p)[3][8], float& sum, float& inv) {
+            float biggest = 0;
 #pragma unroll
-        for (int i = 0; i < 32; ++i) { xa[i] = src[i]; sxa += xa[i]; }
+            for (int i = 0; i < 32; ++i) {
+                const float v = v32[i];
+                sum += v;
+                x_bad = x_bad || nonfinite(v);
+                biggest = fmaxf(biggest, fabsf(v));
+            }
+            // a sub-block of zeros, of subnormals only, or with something not finite in it keeps scale 1 (its integers are zeros)
+            const bool usable = biggest >= 1.1754944e-38f && !nonfinite(biggest);
+            const float scale = usable ? 8290000.0f / biggest : 1.0f;
+            inv = usable ? biggest / 8290000.0f : 1.0f;
 #pragma unroll
-        for (int i = 0; i < 32; ++i) { xb[i] = src[32 + i]; sxb += xb[i]; }
+            for (int k = 0; k < 8; ++k) {
+                uint32_t w2 = 0, w1 = 0, w0 = 0;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int xi = usable ? __float2int_rn(v32[4 * k + j] * scale) : 0;
+                    const int c = ((xi + 128) & 255) - 128, upper = (xi - c) >> 8;
+                    const int b = ((upper + 128) & 255) - 128, a = (upper - b) >> 8;
+                    w2 |= uint32_t(a & 0xff) << (8 * j);
+                    w1 |= uint32_t(b & 0xff) << (8 * j);
+                    w0 |= uint32_t(c & 0xff) << (8 * j);
+                }
+                p[2][k] = w2; p[1][k] = w1; p[0][k] = w0;
+            }
+        };
+        planes(src, pa, sxa, inv_a);
+        planes(src + 32, pb, sxb, inv_b);
     }
 
     for (; step < steps; step += waves) {
@@ -175,22 +211,24 @@ __global__ __launch_bounds__(256) void gemv_q4k(GemvArgs a) {
             }
         }
         const uint32_t words[8] = {now.q0.x, now.q0.y, now.q0.z, now.q0.w, now.q1.x, now.q1.y, now.q1.z, now.q1.w};
-        float dot_a0 = 0, dot_a1 = 0, dot_b0 = 0, dot_b1 = 0;
+        int a2 = 0, a1 = 0, a0 = 0, b2 = 0, b1 = 0, b0 = 0;
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            const uint32_t lo = words[k] & 0x0f0f0f0fu, hi = (words[k] >> 4) & 0x0f0f0f0fu;
-            dot_a0 = __builtin_fmaf(ub(lo, 0), xa[4 * k + 0], dot_a0);
-            dot_a1 = __builtin_fmaf(ub(lo, 1), xa[4 * k + 1], dot_a1);
-            dot_a0 = __builtin_fmaf(ub(lo, 2), xa[4 * k + 2], dot_a0);
-            dot_a1 = __builtin_fmaf(ub(lo, 3), xa[4 * k + 3], dot_a1);
-            dot_b0 = __builtin_fmaf(ub(hi, 0), xb[4 * k + 0], dot_b0);
-            dot_b1 = __builtin_fmaf(ub(hi, 1), xb[4 * k + 1], dot_b1);
-            dot_b0 = __builtin_fmaf(ub(hi, 2), xb[4 * k + 2], dot_b0);
-            dot_b1 = __builtin_fmaf(ub(hi, 3), xb[4 * k + 3], dot_b1);
+            const int lo = int(words[k] & 0x0f0f0f0fu), hi = int((words[k] >> 4) & 0x0f0f0f0fu);
+            a2 = __builtin_amdgcn_sdot4(lo, int(pa[2][k]), a2, false);
+            a1 = __builtin_amdgcn_sdot4(lo, int(pa[1][k]), a1, false);
+            a0 = __builtin_amdgcn_sdot4(lo, int(pa[0][k]), a0, false);
+            b2 = __builtin_amdgcn_sdot4(hi, int(pb[2][k]), b2, false);
+            b1 = __builtin_amdgcn_sdot4(hi, int(pb[1][k]), b1, false);
+            b0 = __builtin_amdgcn_sdot4(hi, int(pb[0][k]), b0, false);
         }
+        // each plane's sum is below 2^16 and exact as a float; the three recombine with two roundings to f32
+        const float dot_a = __builtin_fmaf(float(a2), 65536.0f, __builtin_fmaf(float(a1), 256.0f, float(a0))) * inv_a;
+        const float dot_b = __builtin_fmaf(float(b2), 65536.0f, __builtin_fmaf(float(b1), 256.0f, float(b0))) * inv_b;
         // sum_c ((d*sc)*q - dmin*mn) * x = (d*sc) * sum q x - (dmin*mn) * sum x, per sub-block
-        float part = (d * float(sc_a)) * (dot_a0 + dot_a1) - (dmin * float(mn_a)) * sxa;
-        part += (d * float(sc_b)) * (dot_b0 + dot_b1) - (dmin * float(mn_b)) * sxb;
+        float part = (d * float(sc_a)) * dot_a - (dmin * float(mn_a)) * sxa;
+        part += (d * float(sc_b)) * dot_b - (dmin * float(mn_b)) * sxb;
+        if (x_bad) part = __uint_as_float(0x7fc00000u);  // a non-finite activation: the row's sum is not a number, and the batch is refused
         const float total = group_sum<LPR>(part);
         if (live && lane % LPR == 0) {
             if (nonfinite(total)) atomicOr(a.error_word, TSP_ERRBIT_NONFINITE);
@@ -212,7 +250,12 @@ int launch_gemv(uint32_t encoding, uint32_t layout, GemvArgs a, hipStream_t stre
         const bool planar = layout == TSP_LAYOUT_PLANAR_V3;
 #define TSP_Q4K_CASE(N)                                                                                                   \
     if (bpr == N) {                                                                                                       \
-        const dim3 grid(grid_rows((a.rows + 64 / (4 * N) - 1) / (64 / (4 * N)), 4), a.count);                             \
+        /* at most 768 workgroups, three per compute unit of a 256-unit GPU: a wave's set-up (its 64 activations turned into */ \
+        /* digit planes) is worth many steps, and twelve waves per unit with a step in flight each keep memory as busy as */  \
+        /* thirty-two do (measured at 65 536 and 262 144 rows of 2048 columns: 21.5 and 66 us against 29 and 71) */            \
+        uint32_t blocks = grid_rows((a.rows + 64 / (4 * N) - 1) / (64 / (4 * N)), 4);                                     \
+        if (a.count == 1 && blocks > 768) blocks = 768;                                                                   \
+        const dim3 grid(blocks, a.count);                                                                                 \
         if (planar) TSP_LAUNCH("gemv_q4k", stream, gemv_q4k<N, true><<<grid, 256, 0, stream>>>(a));                                                       \
         else TSP_LAUNCH("gemv_q4k", stream, gemv_q4k<N, false><<<grid, 256, 0, stream>>>(a));                                                             \
         return launch_status("gemv_q4k");                                                                                 \
