@@ -88,7 +88,9 @@ template <int BPR, bool PLANAR>
 __global__ __launch_bounds__(256) void gemv_q4k(GemvArgs a) {
     constexpr int LPR = 4 * BPR;        // lanes per row
     constexpr int RPS = kWave / LPR;    // rows per wave step
-    __shared__ __attribute__((aligned(16))) float xs[BPR * 256];
+    // per sub-block of 32 activations: three planes of eight dwords (four signed bytes each), then 1 / scale, the sum, a flag
+    constexpr uint32_t kSubWords = 3 * 8 + 4;
+    __shared__ __attribute__((aligned(16))) uint32_t planes[BPR * 8 * kSubWords];
     const uint8_t* w; const float* x; float* y;
     if (!resolve(a, w, x, y)) return;
     const uint32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -136,53 +138,66 @@ __global__ __launch_bounds__(256) void gemv_q4k(GemvArgs a) {
     }
     uint32_t step = blockIdx.x * (blockDim.x / kWave) + wave;
     Raw cur = fetch(step < steps ? step : 0);
+    // The activations become integers, once per workgroup: per sub-block of 32 one scale that brings the largest magnitude to
+    // 8 290 000 (just under 127 * 2^16 + 2^15, the most that three signed bytes hold), every value rounded to the nearest
+    // integer of that grid (2^-24 of the sub-block's largest value: the precision of the f32 operand itself for the values
+    // that matter) and written as three signed base-256 digits, x = (a 2^16 + b 2^8 + c) / scale with a, b, c in [-128, 127].
+    // Four activations' digits share a dword, in the order of the four bytes of a word of nibbles, so that v_dot4_i32_i8
+    // multiplies four weights per instruction and plane: three integer instructions per four weights where the f32 form
+    // spends a conversion and a multiply-add per weight. The integer sums are exact; the three of a sub-block recombine in f32.
+    // A thread turns the quads it loaded into digits; the eight threads of a sub-block are neighbours and agree on its scale
+    // with three cross-lane steps.
 #pragma unroll
-    for (uint32_t j = 0; j < kMine; ++j)
-        if (kQuads % 256 == 0 || threadIdx.x + j * 256 < kQuads) reinterpret_cast<float4*>(xs)[threadIdx.x + j * 256] = xv[j];
+    for (uint32_t j = 0; j < kMine; ++j) {
+        const uint32_t quad = threadIdx.x + j * 256;
+        const bool mine = kQuads % 256 == 0 || quad < kQuads;  // uniform over every group of eight lanes
+        const float v4[4] = {mine ? xv[j].x : 0.0f, mine ? xv[j].y : 0.0f, mine ? xv[j].z : 0.0f, mine ? xv[j].w : 0.0f};
+        float biggest = fmaxf(fmaxf(fabsf(v4[0]), fabsf(v4[1])), fmaxf(fabsf(v4[2]), fabsf(v4[3])));
+        float sum = (v4[0] + v4[1]) + (v4[2] + v4[3]);
+        uint32_t flag = (nonfinite(v4[0]) || nonfinite(v4[1]) || nonfinite(v4[2]) || nonfinite(v4[3])) ? 1u : 0u;
+        biggest = dpp_max<0xB1>(biggest); biggest = dpp_max<0x4E>(biggest); biggest = dpp_max<0x141>(biggest);
+        sum = octet_sum(sum);
+        flag |= uint32_t(__builtin_amdgcn_update_dpp(0, int(flag), 0xB1, 0xf, 0xf, true));
+        flag |= uint32_t(__builtin_amdgcn_update_dpp(0, int(flag), 0x4E, 0xf, 0xf, true));
+        flag |= uint32_t(__builtin_amdgcn_update_dpp(0, int(flag), 0x141, 0xf, 0xf, true));
+        // a sub-block of zeros, of subnormals only, or with something not finite in it keeps scale 1 (its integers are zeros)
+        const bool usable = biggest >= 1.1754944e-38f && !nonfinite(biggest) && flag == 0;
+        const float scale = usable ? 8290000.0f / biggest : 1.0f;
+        uint32_t w2 = 0, w1 = 0, w0 = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int xi = usable ? __float2int_rn(v4[e] * scale) : 0;
+            const int c = ((xi + 128) & 255) - 128, upper = (xi - c) >> 8;
+            const int b = ((upper + 128) & 255) - 128, a8 = (upper - b) >> 8;
+            w2 |= uint32_t(a8 & 0xff) << (8 * e);
+            w1 |= uint32_t(b & 0xff) << (8 * e);
+            w0 |= uint32_t(c & 0xff) << (8 * e);
+        }
+        if (mine) {
+            uint32_t* sub = planes + (quad / 8) * kSubWords;
+            sub[16 + quad % 8] = w2; sub[8 + quad % 8] = w1; sub[quad % 8] = w0;
+            if (quad % 8 == 0) {
+                sub[24] = __float_as_uint(usable ? biggest / 8290000.0f : 1.0f);
+                sub[25] = __float_as_uint(sum);
+                sub[26] = flag;
+            }
+        }
+    }
     __syncthreads();
 
-    // The lane's 64 activations become integers: per sub-block of 32 one scale that brings the largest magnitude to 8 290 000
-    // (just under 127 * 2^16 + 2^15, the most that three signed bytes hold), every value rounded to the nearest integer of
-    // that grid (2^-24 of the sub-block's largest value: the precision of the f32 operand itself for the values that matter)
-    // and written as three signed base-256 digits, x = (a 2^16 + b 2^8 + c) / scale with a, b, c in [-128, 127]. Four
-    // activations' digits share a dword, in the order of the four bytes of a word of nibbles, so that v_dot4_i32_i8 multiplies
-    // four weights per instruction and plane: three integer instructions per four weights where the f32 form spends a
-    // conversion and a multiply-add per weight. The integer sums are exact; the three of a sub-block recombine in f32.
     uint32_t pa[3][8], pb[3][8];
-    float sxa = 0, sxb = 0, inv_a, inv_b;
-    bool x_bad = false;
+    float sxa, sxb, inv_a, inv_b;
+    bool x_bad;
     {
-        const float* src = xs + blk_in_row * 256 + pair * 64;
-        auto planes = [&](const float* v32, uint32_t (&p)[3][8], float& sum, float& inv) {
-            float biggest = 0;
+        const uint32_t* sa = planes + (blk_in_row * 8 + pair * 2) * kSubWords;
+        const uint32_t* sb = sa + kSubWords;
 #pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                const float v = v32[i];
-                sum += v;
-                x_bad = x_bad || nonfinite(v);
-                biggest = fmaxf(biggest, fabsf(v));
-            }
-            // a sub-block of zeros, of subnormals only, or with something not finite in it keeps scale 1 (its integers are zeros)
-            const bool usable = biggest >= 1.1754944e-38f && !nonfinite(biggest);
-            const float scale = usable ? 8290000.0f / biggest : 1.0f;
-            inv = usable ? biggest / 8290000.0f : 1.0f;
+        for (int p = 0; p < 3; ++p)
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                uint32_t w2 = 0, w1 = 0, w0 = 0;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int xi = usable ? __float2int_rn(v32[4 * k + j] * scale) : 0;
-                    const int c = ((xi + 128) & 255) - 128, upper = (xi - c) >> 8;
-                    const int b = ((upper + 128) & 255) - 128, a = (upper - b) >> 8;
-                    w2 |= uint32_t(a & 0xff) << (8 * j);
-                    w1 |= uint32_t(b & 0xff) << (8 * j);
-                    w0 |= uint32_t(c & 0xff) << (8 * j);
-                }
-                p[2][k] = w2; p[1][k] = w1; p[0][k] = w0;
-            }
-        };
-        planes(src, pa, sxa, inv_a);
-        planes(src + 32, pb, sxb, inv_b);
+            for (int k = 0; k < 8; ++k) { pa[p][k] = sa[p * 8 + k]; pb[p][k] = sb[p * 8 + k]; }
+        inv_a = __uint_as_float(sa[24]); sxa = __uint_as_float(sa[25]);
+        inv_b = __uint_as_float(sb[24]); sxb = __uint_as_float(sb[25]);
+        x_bad = (sa[26] | sb[26]) != 0;
     }
 
     for (; step < steps; step += waves) {
@@ -250,11 +265,12 @@ int launch_gemv(uint32_t encoding, uint32_t layout, GemvArgs a, hipStream_t stre
         const bool planar = layout == TSP_LAYOUT_PLANAR_V3;
 #define TSP_Q4K_CASE(N)                                                                                                   \
     if (bpr == N) {                                                                                                       \
-        /* at most 768 workgroups, three per compute unit of a 256-unit GPU: a wave's set-up (its 64 activations turned into */ \
-        /* digit planes) is worth many steps, and twelve waves per unit with a step in flight each keep memory as busy as */  \
-        /* thirty-two do (measured at 65 536 and 262 144 rows of 2048 columns: 21.5 and 66 us against 29 and 71) */            \
+        /* at most 1024 workgroups, four per compute unit of a 256-unit GPU: sixteen waves per unit with a step in flight each */ \
+        /* keep memory as busy as thirty-two do, and a workgroup's set-up (the activations' digit planes) serves more steps */    \
+        /* (measured at 65 536 and 262 144 rows of 2048 columns: 15.2 and 59.4 us against 16.3 and 60.0; two steps in flight */   \
+        /* per wave: no faster) */                                                                                              \
         uint32_t blocks = grid_rows((a.rows + 64 / (4 * N) - 1) / (64 / (4 * N)), 4);                                     \
-        if (a.count == 1 && blocks > 768) blocks = 768;                                                                   \
+        if (a.count == 1 && blocks > 1024) blocks = 1024;                                                                 \
         const dim3 grid(blocks, a.count);                                                                                 \
         if (planar) TSP_LAUNCH("gemv_q4k", stream, gemv_q4k<N, true><<<grid, 256, 0, stream>>>(a));                                                       \
         else TSP_LAUNCH("gemv_q4k", stream, gemv_q4k<N, false><<<grid, 256, 0, stream>>>(a));                                                             \
