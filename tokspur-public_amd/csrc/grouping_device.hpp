@@ -5,6 +5,36 @@
 
 namespace tsp {
 
+// Inclusive sums over the 512 values of a block of 512 threads (one per thread), two or three sequences at once: each wave
+// scans its 64 values with six shuffles, the eight wave totals meet in LDS (`totals`: 8 words per sequence), one barrier on
+// the way in and one on the way out, where a step-by-step scan through LDS takes eighteen. Returns the scan at this thread;
+// `grand[i]` receives the sum of all 512.
+template <int N>
+__device__ __forceinline__ void scan512(uint32_t (&v)[N], uint32_t (&grand)[N], uint32_t* totals) {
+    const uint32_t tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+#pragma unroll
+        for (int step = 1; step < kWave; step <<= 1) {
+            const uint32_t below = uint32_t(__shfl_up(int(v[i]), step, kWave));
+            if (lane >= uint32_t(step)) v[i] += below;
+        }
+    }
+    __syncthreads();  // whoever still reads `totals` from an earlier call has left
+    if (lane == kWave - 1)
+#pragma unroll
+        for (int i = 0; i < N; ++i) totals[i * 8 + wave] = v[i];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        uint32_t before = 0, all = 0;
+#pragma unroll
+        for (uint32_t w = 0; w < 8; ++w) { const uint32_t t = totals[i * 8 + w]; if (w < wave) before += t; all += t; }
+        v[i] += before;
+        grand[i] = all;
+    }
+}
+
 // One block of 512 threads writes one list; experts <= 512. tiles(e) = ceil(min(counts[e], T) / tile), exclusive scan over
 // the experts, task i of expert e is (e, i * tile); unused slots up to the bound are 0xFFFFFFFF. The two scan arrays (512
 // words each) are the caller's LDS.
@@ -20,18 +50,11 @@ __device__ __forceinline__ void grouped_tasks_block(const uint32_t* __restrict__
     const uint32_t count = tid < experts ? counts[tid] : 0;
     if (count > tokens) bad = TSP_ERRBIT_INDEX;
     const uint32_t n = ((count < tokens ? count : tokens) + tile - 1) / tile;
-    tiles_scan[tid] = n;
-    routes_scan[tid] = count;
-    __syncthreads();
-    for (uint32_t step = 1; step < 512; step <<= 1) {  // inclusive Hillis-Steele scan
-        const uint32_t a = tid >= step ? tiles_scan[tid - step] : 0, b = tid >= step ? routes_scan[tid - step] : 0;
-        __syncthreads();
-        tiles_scan[tid] += a;
-        routes_scan[tid] += b;
-        __syncthreads();
-    }
-    const uint32_t total = tiles_scan[511], routes = routes_scan[511];
-    const uint32_t offset = tiles_scan[tid] - n;
+    uint32_t scans[2] = {n, count}, sums[2];
+    scan512(scans, sums, tiles_scan);
+    (void)routes_scan;
+    const uint32_t total = sums[0], routes = sums[1];
+    const uint32_t offset = scans[0] - n;
     for (uint32_t i = tid; i < bound; i += 512) { tasks[2 + 2 * i] = 0xffffffffu; tasks[3 + 2 * i] = 0xffffffffu; }
     __syncthreads();
     if (tid < experts)
@@ -61,21 +84,11 @@ __device__ __forceinline__ void task_class_lists_block(const uint32_t* __restric
     const uint32_t count = tid < experts ? (counts[tid] < tokens ? counts[tid] : tokens) : 0;
     const uint32_t n = (count + tile - 1) / tile;
     const uint32_t small = n && count - (n - 1) * tile <= 32 ? 1 : 0;  // the last task is a small one
-    __syncthreads();
-    scan_all[tid] = n;
-    scan_small[tid] = small;
-    scan_large[tid] = n - small;
-    __syncthreads();
-    for (uint32_t step = 1; step < 512; step <<= 1) {
-        const uint32_t a = tid >= step ? scan_all[tid - step] : 0, b = tid >= step ? scan_small[tid - step] : 0, c = tid >= step ? scan_large[tid - step] : 0;
-        __syncthreads();
-        scan_all[tid] += a;
-        scan_small[tid] += b;
-        scan_large[tid] += c;
-        __syncthreads();
-    }
-    const uint32_t total = scan_all[511], total_small = scan_small[511], total_large = scan_large[511];
-    const uint32_t first = scan_all[tid] - n, first_small = scan_small[tid] - small, first_large = scan_large[tid] - (n - small);
+    uint32_t scans[3] = {n, small, n - small}, sums[3];
+    scan512(scans, sums, scan_all);
+    (void)scan_small; (void)scan_large;
+    const uint32_t total = sums[0], total_small = sums[1], total_large = sums[2];
+    const uint32_t first = scans[0] - n, first_small = scans[1] - small, first_large = scans[2] - (n - small);
     uint32_t* list_small = out + 2;
     uint32_t* list_large = out + 2 + bound;
     for (uint32_t i = 0; i < n; ++i) {
