@@ -185,8 +185,8 @@ int tsp_q8_matvec_many(uint32_t layout, const void* matrix, uint64_t matrix_byte
 /* include/tokspur/graph.hpp:860 `dense_mm_q8` (kernels/grouped_mm.metal:239-243; planner src/grouped_mm.cpp:48-54):
  * out[t, :] = W in[t, :] for a dense Q8_0 matrix in GGUF rows (layout 0) or q8_lanes_v1 rows (layout 1), f32 rows in
  * and out with byte strides. Decoded and accumulated in f32 (the engine stages halves); token rows that lie back to
- * back share each weight read eight at a time, and up to sixteen at a time for GGUF rows of 1024 or 2048 columns
- * (16-byte aligned buffers, at least 64 rows, a multiple of 4). */
+ * back share each weight read eight at a time, and up to sixteen at a time for rows of 1024 or 2048 columns in either
+ * layout (16-byte aligned buffers, at least 64 matrix rows, 32 for the lanes layout, in multiples of 4). */
 int tsp_dense_mm_q8(uint32_t layout, const void* matrix, uint64_t matrix_bytes, const float* input, uint64_t input_stride_bytes,
                     float* output, uint64_t output_stride_bytes, uint32_t tokens, uint32_t columns, uint32_t rows,
                     uint32_t* error_word, void* stream);
@@ -343,7 +343,7 @@ int tsp_planar_moe_routed_m8_shared(const tsp_small_moe* moe, const tsp_shared_r
  * factors whose block scales are applied in f32, f32 accumulation. The carry is exact for bf16 values of magnitude 2^-14
  * to 65504; smaller ones lose low bits (below 2^-24: zero), and a finite input above 65504 sets TSP_ERRBIT_NONFINITE like an
  * infinity would (the batch is refused rather than computed on a clipped value). The same holds for tsp_grouped_mm and
- * tsp_planar_nax_grouped_moe. One shape differs: Q4_K raw GGUF rows against 1024 or more token rows enter the matrix cores as
+ * tsp_planar_nax_grouped_moe. One shape differs: Q4_K raw GGUF rows against 512 or more token rows enter the matrix cores as
  * the engine's kernel stages them (test_moe_mm_many_gpu.cpp:54-63), each weight's f32 value d*sc*q - dmin*mn rounded once to
  * half, which is what makes unpacking a weight once per 128 or 256 token rows possible. Input rows are f32 or bf16, output
  * rows f32 or bf16 (RNE); strides in bytes. Q4_K raw GGUF rows or planar planes, Q6_K planes. `workspace` is caller

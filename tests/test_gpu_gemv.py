@@ -143,7 +143,7 @@ def test_config0_dense_q4k_gemv(gpu, tsp, orc, synth):
     # the two arms share their arithmetic: identical bits (the engine's block path is held to this too,
     # native/tests/test_block_gemv.cpp:94)
     assert np.array_equal(bits(got), bits(got_p))
-    # The configuration's bar is max scaled error 2e-3 with f32 accumulation. Measured: 9.2e-5, on an element of magnitude ~1
+    # The configuration's bar is max scaled error 2e-3 with f32 accumulation. Measured: 6.2e-5, on an element of magnitude ~1
     # in a vector whose entries reach several hundred (weights up to ~19, 2048 products): 3e-7 of the vector's scale, which
     # is what f32 accumulation leaves. The engine's 5e-5 (native/src/main.cpp:165) is quoted on outputs of magnitude ~1 and
     # holds at those (test_gemv_shapes, test_gemv_all_encodings_reference_fixture); here the bound asserted is 2e-4.
