@@ -9,6 +9,7 @@ the decode-side numbers (configs 0, 2, 4 as HBM GB/s), config 1 (dense dequant-G
 dominant kernel measured live with events around each launch, and a CPU baseline timed on this host.
 """
 import argparse
+import copy
 import importlib
 import json
 import os
@@ -401,9 +402,16 @@ def main():
             configs[f"gemv_q4k_{big_rows}x2048_not_a_baseline_config"] = {"us": ms * 1e3, "hbm_gbps": bb / (ms * 1e-3) / 1e9,
                                                                            "hbm_frac": bb / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "bytes": bb}
             del pair, wb, yb
-        # config 2: MoE verify T = 8 on the config-3 experts; eight router inputs in rotation so the ~150 MB of
-        # selected experts differ from step to step and do not sit in the 256 MB last-level cache
+        # config 2: MoE verify T = 8 on the config-3 experts. Eight router inputs in rotation select different experts from step
+        # to step, and four copies of the whole 1.06 GB expert set take turns as well: any one copy is read every fourth step,
+        # with ~450 MB of other copies' experts in between, so no expert's planes are still in the 256 MB last-level cache
+        # when a step asks for them (with one copy, a quarter of a step's experts had been read one or two steps before)
         T2 = 8
+        expert_sets = [w]
+        for _ in range(3):
+            twin = copy.copy(w)
+            twin.pair_lo, twin.pair_hi, twin.down, twin.union_meta = w.pair_lo.clone(), w.pair_hi.clone(), w.down.clone(), w.union_meta.clone()
+            expert_sets.append(twin)
         sets = []
         for i in range(8):
             lg = gpu.upload(synth.activations_f32(synth.tensor_seed(2, 100 + i), (T2, E)))
@@ -418,21 +426,23 @@ def main():
 
         def step_c2_two_streams():  # the shared expert as a routed call of its own beside the routed experts
             lg, xx = sets[state["i"] % len(sets)]
+            w2 = expert_sets[state["i"] % len(expert_sets)]
             state["i"] += 1
             main = torch.cuda.current_stream()
             side.wait_stream(main)
             with torch.cuda.stream(side):
                 capi.planar_moe_routed_m8(gpu, ws, ids_s2, xx, T2, 1, h=hs2, y=ys2)
             gpu.route(lg, S, 0, True, tokens=T2, out=(ids2, wts2))
-            capi.planar_moe_routed_m8(gpu, w, ids2, xx, T2, S, h=h2, y=y2)
+            capi.planar_moe_routed_m8(gpu, w2, ids2, xx, T2, S, h=h2, y=y2)
             main.wait_stream(side)
             gpu.mixture(y2, wts2, ys2, sl2, C, S, tokens=T2, out=out2)
 
         def step_c2():  # the shared expert as one more record of the routed experts' two launches
             lg, xx = sets[state["i"] % len(sets)]
+            w2 = expert_sets[state["i"] % len(expert_sets)]
             state["i"] += 1
             gpu.route(lg, S, 0, True, tokens=T2, out=(ids2, wts2))
-            capi.planar_moe_routed_m8(gpu, w, ids2, xx, T2, S, h=h2, y=y2, shared=shared, shared_h=hs2, shared_y=ys2)
+            capi.planar_moe_routed_m8(gpu, w2, ids2, xx, T2, S, h=h2, y=y2, shared=shared, shared_h=hs2, shared_y=ys2)
             gpu.mixture(y2, wts2, ys2, sl2, C, S, tokens=T2, out=out2)
 
         two_streams_ms = None
@@ -462,8 +472,10 @@ def main():
                                        "two_streams_us": None if two_streams_ms is None else two_streams_ms * 1e3}
         state["i"] = 0
         configs["c2_moe_verify_t8"]["kernels_us"] = {k: round(v["avg_us"], 2) for k, v in profiled(capi, torch, step_c2, 8).items()}
+        configs["c2_moe_verify_t8"]["note"] = "eight router inputs x four copies of the expert set in rotation: every expert plane comes from HBM"
+        del expert_sets, graph2
         # config 4: Q8_0 LM head, vocab 151936 x 2048, both arms: raw GGUF rows and the same matrix as q8_lanes_v1 rows. M = 16 goes
-        # through the dense Q8_0 GEMM entry point (raw rows: one pass, K halves summed; lanes rows: two passes of eight)
+        # through the dense Q8_0 GEMM entry point (either layout: one pass, K halves summed)
         V = 151936
         w4_host = synth.matrix(8, synth.tensor_seed(4, 1), V, C)
         w4 = gpu.upload(w4_host)

@@ -5,6 +5,7 @@
 #include <cstdio>
 #include <cstring>
 #include <fcntl.h>
+#include <fstream>
 #include <functional>
 #include <sys/stat.h>
 #include <unistd.h>
@@ -274,6 +275,71 @@ void test_build_adopt_tamper(const Shards& s) {
 }
 // include/tokspur/grouped_mm.hpp:22-26: the C++ planners, against the restated ones (themselves bit-equal to the compiled
 // reference) on the engine's shapes and on every encoding / layout pair, and the engine's refusals
+// native/tests/test_planar_pack_v3.cpp:324-327 and native/tests/test_derived_pack.cpp:390-401: the budget report of a plan, and a
+// build interrupted through its cancellation hook, which must leave the directory as it found it.
+int g_chunks_before_cancel = 0;
+void cancel_after_some_chunks() {
+    if (g_chunks_before_cancel-- == 0) throw FormatError("interrupted test build");
+}
+void test_budget_and_cancellation(const Shards& s) {
+    const BudgetReportV3 budget = measure_pack_v3_budget(*s.source, s.sidecar.get(), s.dir.path, {}, 2, 1 << 20);
+    const PackPlanV3 plan = plan_derived_pack_v3(*s.source, s.sidecar.get());
+    EXPECT(budget.ram_ceiling_satisfied && budget.reserve_satisfied);
+    EXPECT(budget.original_12b_scale_header_bytes * 4 == budget.expanded_16b_scale_header_bytes * 3 && budget.expanded_16b_scale_header_bytes > 0);
+    EXPECT(budget.planned_pack_v3_file_bytes == plan.file_bytes && budget.planned_pack_v3_payload_bytes == plan.payload_bytes);
+    EXPECT(budget.required_reserve_bytes == (1 << 20) && budget.existing_pack_v2_file_bytes == 0);
+    EXPECT(budget.free_after_pack_v3_bytes + plan.file_bytes == budget.filesystem_available_bytes);
+    // the families add up to the planar tensors of the plan, each counted once
+    uint64_t planar = 0, biggest_chunk = 0;
+    for (const auto& t : plan.tensors) {
+        if (!is_planar_v3_kind(t.kind)) continue;
+        planar += t.bytes;
+        tsp_planar_spec spec{};
+        EXPECT(tsp_make_expert_spec(t.source_type, uint32_t(t.source_dimensions[0]), uint32_t(t.source_dimensions[1]), &spec) == TSP_OK);
+        biggest_chunk = std::max<uint64_t>(biggest_chunk, (spec.planar_expert_bytes + 2 * spec.source_expert_bytes) * 2 * (is_coloc_gate_kind(t.kind) ? 2 : 1));
+    }
+    EXPECT(planar > 0 && budget.q4k_planar_bytes + budget.q5k_planar_bytes + budget.q51_planar_bytes + budget.q8_planar_moe_bytes == planar);
+    EXPECT(budget.streaming_ring_buffer_bytes == std::max<uint64_t>(biggest_chunk, 2 * derived_pack::default_chunk_bytes));
+    // a block plan with the smallest chunk: the buffers of the plain and lane tensors still count (two chunks)
+    const PackPlanV3 block = plan_block_pack_v3(*s.source, s.sidecar.get(), 0);
+    const auto existing = s.dir.path / "older-pack.bin";
+    { std::ofstream(existing, std::ios::binary) << std::string(777, 'x'); }
+    const BudgetReportV3 small = measure_pack_v3_budget(block, s.dir.path, existing, 2, 0, 32768);
+    EXPECT(small.planned_pack_v3_file_bytes == block.file_bytes && small.streaming_ring_buffer_bytes >= 65536 && small.existing_pack_v2_file_bytes == 777);
+    EXPECT(measure_pack_v3_budget(block, s.dir.path, s.dir.path, 2, 0, 32768).existing_pack_v2_file_bytes == 0);  // a directory is no pack
+    EXPECT(!measure_pack_v3_budget(block, s.dir.path, {}, 2, ~0ull >> 1, 32768).reserve_satisfied);
+    EXPECT(refuses([&] { (void)measure_pack_v3_budget(block, s.dir.path, {}, 0, 0, 32768); }));
+    EXPECT(refuses([&] { (void)measure_pack_v3_budget(block, s.dir.path, {}, 65, 0, 32768); }));
+    EXPECT(refuses([&] { (void)measure_pack_v3_budget(block, s.dir.path, {}, 2, 0, 32767); }));
+    EXPECT(refuses([&] { (void)measure_pack_v3_budget(block, s.dir.path / "no-such-directory", {}, 2, 0, 32768); }));
+    std::filesystem::remove(existing);
+
+    // cancellation at the first chunk, in the middle and just before publication: refused, nothing left behind, and the
+    // same build goes through afterwards
+    const auto entries = [&] { size_t n = 0; for (const auto& e : std::filesystem::directory_iterator(s.dir.path)) { (void)e; ++n; } return n; };
+    const size_t before = entries();
+    const auto output = s.dir.path / "cancelled.asa.gguf";
+    int chunks = 0;
+    g_chunks_before_cancel = 1 << 30;
+    {   // count the hook's calls on a build that completes
+        (void)build_block_pack_v3(s.source, s.sidecar, 0, output, 2, 0, 32768, cancel_after_some_chunks);
+        chunks = (1 << 30) - g_chunks_before_cancel;
+        EXPECT(chunks >= 3 && std::filesystem::exists(output));
+        EXPECT(::chmod(output.c_str(), 0600) == 0 && std::filesystem::remove(output));
+    }
+    for (const int at : {0, chunks / 2, chunks - 1}) {
+        g_chunks_before_cancel = at;
+        bool interrupted = false;
+        try { (void)build_block_pack_v3(s.source, s.sidecar, 0, output, 2, 0, 32768, cancel_after_some_chunks); }
+        catch (const FormatError& e) { interrupted = std::string(e.what()).find("interrupted test build") != std::string::npos; }
+        EXPECT(interrupted && !std::filesystem::exists(output) && entries() == before);
+    }
+    g_chunks_before_cancel = 1 << 30;
+    const PackPlanV3 rebuilt = build_block_pack_v3(s.source, s.sidecar, 0, output, 2, 0, 32768, cancel_after_some_chunks);
+    EXPECT(rebuilt.file_bytes == block.file_bytes && std::filesystem::file_size(output) == block.file_bytes);
+    EXPECT(::chmod(output.c_str(), 0600) == 0 && std::filesystem::remove(output) && entries() == before);
+}
+
 void test_grouped_mm_planners() {
     static_assert(sizeof(GroupedMmArgs) == 56);
     const auto same = [](const GroupedMmPlan& a, const orc_grouped_mm_plan& b) {
@@ -327,7 +393,8 @@ int main() {
         {"SHA-256 known answers", test_sha256_known_answers},
         {"GGUF reader", test_gguf_reader},
         {"grouped_mm_plan / dense_mm_q8_plan", test_grouped_mm_planners},
-        {"pack v3: plan, header, build, adoption, tamper", [] { const Shards s; test_plan_and_header(s); test_build_adopt_tamper(s); }}};
+        {"pack v3: plan, header, build, adoption, tamper", [] { const Shards s; test_plan_and_header(s); test_build_adopt_tamper(s); }},
+        {"pack v3: budget report, cancelled build", [] { const Shards s; test_budget_and_cancellation(s); }}};
     for (const auto& [name, fn] : tests) {
         std::printf("== %s\n", name);
         std::fflush(stdout);

@@ -871,8 +871,61 @@ PackPlanV3 plan_block_pack_v3(const ModelFiles& source, const ModelFiles* sideca
     return plan_filtered(source, sidecar, "blk." + std::to_string(block_id) + ".", block_recipe_prefix_v3 + std::to_string(block_id), byte_budget);
 }
 
+BudgetReportV3 measure_pack_v3_budget(const PackPlanV3& plan, const std::filesystem::path& output_directory,
+                                      const std::filesystem::path& existing_pack_v2_path, uint32_t experts_per_chunk, uint64_t reserve_bytes,
+                                      uint64_t chunk_bytes) {
+    require(experts_per_chunk >= 1 && experts_per_chunk <= 64, "experts_per_chunk must be in 1..64");
+    require(chunk_bytes >= 32'768 && chunk_bytes <= 67'108'864, "invalid chunk_bytes bound");
+    BudgetReportV3 report;
+    {
+        const int dir = ::open(output_directory.c_str(), O_RDONLY | O_DIRECTORY | O_CLOEXEC);
+        require(dir >= 0, "cannot open pack v3 directory");
+        struct statvfs v{};
+        const bool ok = ::fstatvfs(dir, &v) == 0;
+        ::close(dir);
+        require(ok, "cannot query free space for pack v3");
+        report.filesystem_available_bytes = checked_mul(uint64_t(v.f_bavail), uint64_t(v.f_frsize));
+    }
+    if (!existing_pack_v2_path.empty()) {
+        struct stat info{};
+        if (::stat(existing_pack_v2_path.c_str(), &info) == 0 && S_ISREG(info.st_mode)) report.existing_pack_v2_file_bytes = uint64_t(info.st_size);
+    }
+    report.planned_pack_v3_payload_bytes = plan.payload_bytes;
+    report.planned_pack_v3_file_bytes = plan.file_bytes;
+    report.required_reserve_bytes = reserve_bytes;
+    report.original_12b_scale_header_bytes = plan.original_12b_scale_header_bytes;
+    report.expanded_16b_scale_header_bytes = plan.expanded_16b_scale_header_bytes;
+    // which family's counter a planar kind adds to (plain and lane tensors: none)
+    uint64_t* const family[10] = {nullptr, nullptr, &report.q4k_planar_bytes, &report.q4k_planar_bytes, &report.q5k_planar_bytes,
+                                  &report.q5k_planar_bytes, &report.q8_planar_moe_bytes, &report.q8_planar_moe_bytes,
+                                  &report.q51_planar_bytes, &report.q8_planar_moe_bytes};
+    // a plain or lane tensor streams through one written and one read-back buffer of chunk_bytes; a planar tensor through
+    // the packed chunk, its read-back and the restored source, per expert (a co-located pair counts twice)
+    uint64_t buffers = checked_mul(chunk_bytes, 2);
+    for (const PackTensorV3& t : plan.tensors) {
+        require(uint32_t(t.kind) < std::size(family), "unknown PlanarKind");
+        if (uint64_t* const counter = family[uint32_t(t.kind)]) *counter = checked_add(*counter, t.bytes);
+        if (!is_planar_v3_kind(t.kind)) continue;
+        require(t.source_dimensions.size() >= 2, "planar v3 tensor without expert dimensions");
+        const tsp_planar_spec spec = expert_spec(t.source_type, t.source_dimensions[0], t.source_dimensions[1]);
+        const uint64_t per_expert = checked_add(spec.planar_expert_bytes, checked_mul(spec.source_expert_bytes, 2));
+        buffers = std::max(buffers, checked_mul(per_expert, uint64_t(experts_per_chunk) * (is_coloc_gate_kind(t.kind) ? 2 : 1)));
+    }
+    report.streaming_ring_buffer_bytes = buffers;
+    report.reserve_satisfied = derived_pack::check_disk_reserve(report.filesystem_available_bytes, plan.file_bytes, reserve_bytes);
+    report.free_after_pack_v3_bytes = report.filesystem_available_bytes >= plan.file_bytes ? report.filesystem_available_bytes - plan.file_bytes : 0;
+    report.ram_ceiling_satisfied = buffers <= report.streaming_ram_ceiling_bytes;
+    return report;
+}
+BudgetReportV3 measure_pack_v3_budget(const ModelFiles& source, const ModelFiles* sidecar, const std::filesystem::path& output_directory,
+                                      const std::filesystem::path& existing_pack_v2_path, uint32_t experts_per_chunk, uint64_t reserve_bytes) {
+    return measure_pack_v3_budget(plan_derived_pack_v3(source, sidecar), output_directory, existing_pack_v2_path, experts_per_chunk, reserve_bytes,
+                                  derived_pack::default_chunk_bytes);
+}
+
 PackPlanV3 build_pack_v3_from_plan(PackPlanV3 plan, std::shared_ptr<const ModelFiles> source, std::shared_ptr<const ModelFiles> sidecar,
-                                   const std::filesystem::path& output, uint32_t experts_per_chunk, uint64_t reserve_bytes, uint64_t chunk_bytes) {
+                                   const std::filesystem::path& output, uint32_t experts_per_chunk, uint64_t reserve_bytes, uint64_t chunk_bytes,
+                                   void (*check_cancelled)()) {
     require(bool(source), "missing source model files for pack v3");
     require(experts_per_chunk >= 1 && experts_per_chunk <= 64, "experts_per_chunk must be in 1..64");
     require(chunk_bytes >= 32'768 && chunk_bytes <= 67'108'864, "invalid chunk_bytes bound");
@@ -891,6 +944,7 @@ PackPlanV3 build_pack_v3_from_plan(PackPlanV3 plan, std::shared_ptr<const ModelF
     };
     // one chunk: written, read back from the file, and what was read back is what gets unpacked, compared and hashed
     const auto commit = [&](std::span<const std::byte> chunk, std::span<std::byte> readback) {
+        if (check_cancelled) check_cancelled();  // throws to cancel: the temporary goes with its owner
         write_at(tmp.fd, chunk, end);
         read_into(tmp.fd, readback, end);
         end = checked_add(end, chunk.size());
@@ -994,6 +1048,7 @@ PackPlanV3 build_pack_v3_from_plan(PackPlanV3 plan, std::shared_ptr<const ModelF
         t.packed_sha256 = packed_digest.finish();
     }
     require(end == plan.file_bytes, "pack v3 final byte size mismatch");
+    if (check_cancelled) check_cancelled();
     const Bytes final_header = build_header_v3(plan);
     require(final_header.size() == first_header.size(), "pack v3 manifest changed header size");
     write_at(tmp.fd, final_header, 0);
@@ -1010,16 +1065,19 @@ PackPlanV3 build_pack_v3_from_plan(PackPlanV3 plan, std::shared_ptr<const ModelF
 }
 
 PackPlanV3 build_derived_pack_v3(std::shared_ptr<const ModelFiles> source, std::shared_ptr<const ModelFiles> sidecar, const std::filesystem::path& output,
-                                 uint32_t experts_per_chunk, uint64_t reserve_bytes, uint64_t chunk_bytes) {
+                                 uint32_t experts_per_chunk, uint64_t reserve_bytes, uint64_t chunk_bytes, void (*check_cancelled)()) {
     require(bool(source), "missing source model files for pack v3");
     auto plan = plan_derived_pack_v3(*source, sidecar.get());
-    return build_pack_v3_from_plan(std::move(plan), std::move(source), std::move(sidecar), output, experts_per_chunk, reserve_bytes, chunk_bytes);
+    return build_pack_v3_from_plan(std::move(plan), std::move(source), std::move(sidecar), output, experts_per_chunk, reserve_bytes, chunk_bytes,
+                                   check_cancelled);
 }
 PackPlanV3 build_block_pack_v3(std::shared_ptr<const ModelFiles> source, std::shared_ptr<const ModelFiles> sidecar, uint32_t block_id,
-                               const std::filesystem::path& output, uint32_t experts_per_chunk, uint64_t reserve_bytes, uint64_t chunk_bytes) {
+                               const std::filesystem::path& output, uint32_t experts_per_chunk, uint64_t reserve_bytes, uint64_t chunk_bytes,
+                               void (*check_cancelled)()) {
     require(bool(source), "missing source model files for pack v3");
     auto plan = plan_block_pack_v3(*source, sidecar.get(), block_id);
-    return build_pack_v3_from_plan(std::move(plan), std::move(source), std::move(sidecar), output, experts_per_chunk, reserve_bytes, chunk_bytes);
+    return build_pack_v3_from_plan(std::move(plan), std::move(source), std::move(sidecar), output, experts_per_chunk, reserve_bytes, chunk_bytes,
+                                   check_cancelled);
 }
 
 namespace {

@@ -196,6 +196,22 @@ struct AdoptedPackV3 {
 
 [[nodiscard]] std::vector<std::byte> build_header_v3(const PackPlanV3& plan);  // src/planar_pack_v3.cpp:898-920
 
+// include/tokspur/planar_pack_v3.hpp:108-125: what building a plan would cost, before a byte is written
+struct BudgetReportV3 {
+    uint64_t filesystem_available_bytes = 0;
+    uint64_t existing_pack_v2_file_bytes = 0;  // size of a regular file at the given path, 0 if there is none
+    uint64_t planned_pack_v3_payload_bytes = 0;
+    uint64_t planned_pack_v3_file_bytes = 0;
+    uint64_t free_after_pack_v3_bytes = 0;
+    uint64_t required_reserve_bytes = derived_pack::default_reserve_bytes;
+    uint64_t streaming_ring_buffer_bytes = 0;  // the largest packed + read-back + restored buffers a chunk needs
+    uint64_t streaming_ram_ceiling_bytes = 4'000'000'000ull;
+    uint64_t q4k_planar_bytes = 0, q5k_planar_bytes = 0, q51_planar_bytes = 0, q8_planar_moe_bytes = 0;
+    uint64_t original_12b_scale_header_bytes = 0, expanded_16b_scale_header_bytes = 0;
+    bool reserve_satisfied = false;
+    bool ram_ceiling_satisfied = false;
+};
+
 // src/planar_pack_v3.cpp:394-499: every GPU tensor of the source (and of the optional sidecar), in name order; a
 // *.ffn_gate_exps.weight is emitted together with its *.ffn_up_exps.weight as a co-located pair when both are eligible,
 // *.ffn_down_exps.weight in Q5_1 / Q8_0 as planes, dense Q8_0 matrices in q8_lanes_v1 rows, everything else as it is.
@@ -204,21 +220,33 @@ struct AdoptedPackV3 {
 [[nodiscard]] PackPlanV3 plan_block_pack_v3(const ModelFiles& source, const ModelFiles* mtp_sidecar, uint32_t block_id,
                                             uint64_t byte_budget = 4'000'000'000ull);
 
+// src/planar_pack_v3.cpp:931-1000: free space of the output directory against the plan's file size plus the reserve,
+// planar bytes per family, and the host buffers one streaming chunk needs against the RAM ceiling. Writes nothing.
+[[nodiscard]] BudgetReportV3 measure_pack_v3_budget(const PackPlanV3& plan, const std::filesystem::path& output_directory,
+                                                    const std::filesystem::path& existing_pack_v2_path, uint32_t experts_per_chunk,
+                                                    uint64_t reserve_bytes, uint64_t chunk_bytes);
+[[nodiscard]] BudgetReportV3 measure_pack_v3_budget(const ModelFiles& source, const ModelFiles* mtp_sidecar,
+                                                    const std::filesystem::path& output_directory,
+                                                    const std::filesystem::path& existing_pack_v2_path = {}, uint32_t experts_per_chunk = 8,
+                                                    uint64_t reserve_bytes = derived_pack::default_reserve_bytes);
+
 // src/planar_pack_v3.cpp:1002-1237: streams the plan into a temporary beside `output`, reads every chunk back and proves the
 // byte-exact inverse against the source before hashing it, writes the final header (now with digests), makes the file
 // read-only and publishes it under `output` without replacing anything. Returns the plan with digests.
+// `check_cancelled` (src/planar_pack_v3.cpp:1010,1080-1229), when given, is called before every chunk is written and once
+// more before publication; it cancels by throwing, and whatever it throws leaves the directory as it was found.
 [[nodiscard]] PackPlanV3 build_pack_v3_from_plan(PackPlanV3 plan, std::shared_ptr<const ModelFiles> source,
                                                  std::shared_ptr<const ModelFiles> mtp_sidecar, const std::filesystem::path& output,
                                                  uint32_t experts_per_chunk = 8, uint64_t reserve_bytes = derived_pack::default_reserve_bytes,
-                                                 uint64_t chunk_bytes = derived_pack::default_chunk_bytes);
+                                                 uint64_t chunk_bytes = derived_pack::default_chunk_bytes, void (*check_cancelled)() = nullptr);
 [[nodiscard]] PackPlanV3 build_derived_pack_v3(std::shared_ptr<const ModelFiles> source, std::shared_ptr<const ModelFiles> mtp_sidecar,
                                                const std::filesystem::path& output, uint32_t experts_per_chunk = 8,
                                                uint64_t reserve_bytes = derived_pack::default_reserve_bytes,
-                                               uint64_t chunk_bytes = derived_pack::default_chunk_bytes);
+                                               uint64_t chunk_bytes = derived_pack::default_chunk_bytes, void (*check_cancelled)() = nullptr);
 [[nodiscard]] PackPlanV3 build_block_pack_v3(std::shared_ptr<const ModelFiles> source, std::shared_ptr<const ModelFiles> mtp_sidecar,
                                              uint32_t block_id, const std::filesystem::path& output, uint32_t experts_per_chunk = 8,
                                              uint64_t reserve_bytes = derived_pack::default_reserve_bytes,
-                                             uint64_t chunk_bytes = derived_pack::default_chunk_bytes);
+                                             uint64_t chunk_bytes = derived_pack::default_chunk_bytes, void (*check_cancelled)() = nullptr);
 
 // src/planar_pack_v3.cpp:1268-1643: the file must be a read-only regular file with one link and exactly the planned size;
 // its header must equal the canonical header of the plan (with the manifest's digests); every tensor is unpacked and
