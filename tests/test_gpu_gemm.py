@@ -50,7 +50,11 @@ def rel_l2(got, ref):
 # ---------------------------------------------------------------------------------- dense
 
 @pytest.mark.parametrize("layout", ["raw", "planar"])
-@pytest.mark.parametrize("tokens,rows,cols", [(1, 64, 256), (33, 96, 512), (128, 256, 2048), (130, 300, 1024), (257, 512, 768)])
+# GGUF rows of 512, 1024 or 2048 columns against at most 384 rows take 64 x 64 tiles with the columns split over the waves:
+# (33, 96, 512), (128, 256, 2048), (130, 300, 1024), (200, 100, 2048), (384, 132, 1024) and (1, 68, 2048) are its shapes (ragged on either
+# side, one to three rounds of tiles); (385, 64, 2048) and (257, 512, 768) stay with the general kernel
+@pytest.mark.parametrize("tokens,rows,cols", [(1, 64, 256), (33, 96, 512), (128, 256, 2048), (130, 300, 1024), (257, 512, 768),
+                                              (200, 100, 2048), (384, 132, 1024), (1, 68, 2048), (385, 64, 2048)])
 def test_dense_mm_q4k(gpu, tsp, orc, synth, layout, tokens, rows, cols):
     if layout == "planar" and rows % 4:
         pytest.skip("planar experts need rows % 4 == 0")

@@ -24,6 +24,7 @@
 //     two and three steps ahead, into a ring of four slabs; one LDS-only barrier per K step.
 //   * For gate/up the two column tiles of a wave are the gate rows and the up rows of the same 32 hidden
 //     units, so SwiGLU is an element-wise epilogue on accumulator registers.
+#include "dense_ksplit.hpp"
 #include "dense_tall.hpp"
 #include "down_resident.hpp"
 #include "gate_up_resident.hpp"
@@ -672,6 +673,13 @@ extern "C" int tsp_dense_mm(uint32_t encoding, uint32_t layout, const void* matr
     }
     int rc = convert_rows(input, input_stride_bytes, input_is_bf16, xh, encoding == 12 ? sx : nullptr, tokens, columns, error_word, s);
     if (rc != TSP_OK) return rc;
+    if (encoding == 12 && layout == TSP_LAYOUT_GGUF && dense_ksplit_takes(tokens, rows, columns)) {
+        // few rows: 64 x 64 tiles with the columns split over a workgroup's waves, so that the chip has tiles enough
+        DenseKsplitArgs t{};
+        t.a = xh; t.sx = sx; t.w = static_cast<const uint8_t*>(matrix); t.m = tokens; t.n = rows; t.k = columns;
+        t.out = output; t.out_stride = output_stride_bytes; t.out_bf16 = output_is_bf16; t.error_word = error_word;
+        return launch_dense_ksplit(t, s);
+    }
     a.a = xh; a.a_stride = columns; a.sx = sx; a.w0 = static_cast<const uint8_t*>(matrix); a.experts = 1;
     a.m = tokens; a.n = rows; a.k = columns; a.out = output; a.out_stride = output_stride_bytes; a.out_scale = 1.0f;
     a.error_word = error_word;
